@@ -1,0 +1,274 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-Linear hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Headline workload (the one the metric is quoted on): the INT4 AWQ-style W4 GEMV,
+M=1, K=4096, N=4096, group size 128, f32 activations, f32 scale + f32
+zero-point per group (the reference's storage).  A step is one GEMV launch over
+one weight set; the run rotates through 64 distinct weight sets (> 600 MB) so
+that the 256 MB Infinity Cache cannot serve the weights, with all inputs
+resident in HBM before the timed region.  The INT8 prefill GEMM
+(2048 x 4096 x 11008 on the i8 matrix cores) is timed in the same run and
+reported under "secondary".  One JSON line is printed on stdout.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+I8_PEAK_TOPS = 5000.0        # MI355X dense int8 MFMA, published
+F16_PEAK_TFLOPS = 2500.0     # MI355X dense f16 MFMA, published
+
+M, K, N, G = 1, 4096, 4096, 128
+GROUPS = K // G
+# algorithmic bytes of one GEMV: packed nibbles + scales + zero-points + x + y, each once
+BYTES_F32_ZP = K * N // 2 + 2 * GROUPS * N * 4 + K * 4 + N * 4           # 9,469,952 (layout executed)
+BYTES_U4_ZP = K * N // 2 + GROUPS * N * 4 + GROUPS * N // 2 + K * 4 + N * 4  # 9,011,200 (u4 zero-points)
+WEIGHT_SETS = 64
+
+
+def log(msg):
+    print(msg, file=sys.stderr, flush=True)
+
+
+def time_graph(torch, launch_all, launches_per_replay, steps, warmup):
+    """Capture `launch_all` (a burst of launches) in a HIP graph and time replays with HIP events
+    on the stream the kernels run on.  Returns (seconds_total, launches_timed, used_graph)."""
+    stream = torch.cuda.current_stream()
+    graph = None
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(stream)
+        with torch.cuda.stream(side):
+            launch_all()                       # warm the capture stream
+        stream.wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            launch_all()
+        graph = g
+    except Exception as e:  # capture is an optimisation of the launch path only
+        log(f"[bench] HIP graph capture unavailable ({e!r}); timing direct launches")
+        torch.cuda.synchronize()
+    run = graph.replay if graph is not None else launch_all
+    for _ in range(max(1, -(-warmup // launches_per_replay))):
+        run()
+    torch.cuda.synchronize()
+    replays = max(1, -(-steps // launches_per_replay))
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(replays):
+        run()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) * 1e-3, replays * launches_per_replay, graph is not None
+
+
+def bench_gemv(torch, ops, steps, warmup):
+    from rumus_amd import workloads
+    dev = torch.device("cuda:0")
+    w0, x0 = workloads.w4_gemv(0)
+    x = torch.from_numpy(x0).to(dev)
+    sets = []
+    gen = torch.Generator(device=dev).manual_seed(0)
+    for i in range(WEIGHT_SETS):
+        if i == 0:
+            w = torch.from_numpy(w0).to(dev)
+        else:
+            w = torch.randn((K, N), generator=gen, device=dev, dtype=torch.float32) * 0.02
+        sets.append(ops.w4_quantize_pack(w, G))
+        del w
+    ys = [torch.empty((M, N), dtype=torch.float32, device=dev) for _ in range(WEIGHT_SETS)]
+    torch.cuda.synchronize()
+
+    def burst_rotating():
+        for (p, s, z), y in zip(sets, ys):
+            ops.qmatmul_int4(x, p, s, z, K, G, out=y)
+
+    def burst_resident():
+        p, s, z = sets[0]
+        for y in ys:
+            ops.qmatmul_int4(x, p, s, z, K, G, out=y)
+
+    # the timed region of record: EXACTLY `steps` launches, bracketed by device syncs
+    sec, launches, used_graph = time_graph(torch, burst_rotating, WEIGHT_SETS, steps, warmup)
+    sec_res, launches_res, _ = time_graph(torch, burst_resident, WEIGHT_SETS, steps, warmup)
+    return {
+        "sec": sec, "launches": launches, "graph": used_graph,
+        "sec_resident": sec_res, "launches_resident": launches_res,
+        "x": x0, "w": w0, "y0": ys[0].cpu().numpy(),
+    }
+
+
+def bench_i8_gemm(torch, ops, steps=30, warmup=5):
+    m, k, n = 2048, 4096, 11008
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev).manual_seed(1)
+    x = torch.randn((m, k), generator=gen, device=dev)
+    w = torch.randn((k, n), generator=gen, device=dev) * 0.02
+    xq, sx = ops.i8_quantize_rows(x)
+    wq, sw = ops.i8_quantize_cols_t(w)
+    del w
+    y = torch.empty((m, n), dtype=torch.float32, device=dev)
+    for _ in range(warmup):
+        ops.i8_gemm(xq, wq, sx, sw, None, out=y)
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        ops.i8_gemm(xq, wq, sx, sw, None, out=y)
+    end.record()
+    torch.cuda.synchronize()
+    sec = start.elapsed_time(end) * 1e-3 / steps
+    ops_per = 2.0 * m * k * n
+    # dynamic activation quantizer, timed separately (it precedes every GEMM in a forward)
+    start.record()
+    for _ in range(steps):
+        ops.i8_quantize_rows(x)
+    end.record()
+    torch.cuda.synchronize()
+    sec_q = start.elapsed_time(end) * 1e-3 / steps
+    tops = ops_per / sec / 1e12
+    return {
+        "workload": "int8_gemm_2048x4096x11008", "ms_per_launch": sec * 1e3, "tops": tops,
+        "roofline": {"bound": "mfma", "achieved": tops, "peak": I8_PEAK_TOPS, "unit": "TOP/s",
+                     "frac": tops / I8_PEAK_TOPS, "traffic": None},
+        "act_quantize_rows_ms": sec_q * 1e3,
+        "act_quantize_rows_gbs": (m * k * 5 + m * 4) / sec_q / 1e9,
+    }
+
+
+def bench_w4_gemm(torch, ops, m, steps=50, warmup=5):
+    """W4 GEMM with act-order (GPTQ style), K=4096, N=11008, g128, symmetric zp=8."""
+    k, n = 4096, 11008
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev).manual_seed(2)
+    w = torch.randn((k, n), generator=gen, device=dev) * 0.02
+    packed, scales, zp = ops.w4_quantize_pack(w, G, symmetric=True)
+    del w
+    g_idx = (torch.randperm(k, generator=gen, device=dev) // G).to(torch.int32)
+    packed_sorted, perm = ops.w4_actorder_prepare(packed, g_idx, G)
+    x = torch.randn((m, k), generator=gen, device=dev)
+    y = torch.empty((m, n), dtype=torch.float32, device=dev)
+    for _ in range(warmup):
+        ops.qmatmul_int4_perm(x, packed_sorted, scales, zp, k, G, perm=perm, out=y)
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        ops.qmatmul_int4_perm(x, packed_sorted, scales, zp, k, G, perm=perm, out=y)
+    end.record()
+    torch.cuda.synchronize()
+    sec = start.elapsed_time(end) * 1e-3 / steps
+    nbytes = k * n // 2 + (k // G) * n * 4 + k * 4 + m * k * 4 + m * n * 4
+    flops = 2.0 * m * k * n
+    return {"workload": f"w4_gemm_actorder_{m}x4096x11008_g128", "ms_per_launch": sec * 1e3,
+            "gbs": nbytes / sec / 1e9, "hbm_frac": nbytes / sec / 1e9 / HBM_PEAK_GBS,
+            "tflops": flops / sec / 1e12, "f16_mfma_frac": flops / sec / 1e12 / F16_PEAK_TFLOPS}
+
+
+def cpu_baseline(x, w, budget_s=12.0):
+    """The CPU restatement of the reference kernels on the host cores: single thread (the
+    reference CpuBackend's contract) for `value`, all cores as an extra figure."""
+    import oracle
+    t0 = time.perf_counter()
+    packed, scales, zp = oracle.w4_from_f32(w, G)
+    t_pack = time.perf_counter() - t0
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 5 and (time.perf_counter() - t_start) < budget_s:
+        t0 = time.perf_counter()
+        y = oracle.qmatmul_int4(x, packed, scales, zp, K, G, threads=1)
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    cores = os.cpu_count() or 1
+    cores = min(cores, 16)
+    t0 = time.perf_counter()
+    oracle.qmatmul_int4(x, packed, scales, zp, K, G, threads=cores)
+    t_mt = time.perf_counter() - t0
+    return {
+        "value": BYTES_F32_ZP / med / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+        "sample": f"{len(times)} full 1x4096x4096 g128 GEMVs, median, scalar C restatement of "
+                  "qmatmul_int4.wgsl (reference has no CPU kernel for this op)",
+        "ms_per_gemv": med * 1e3,
+        "all_cores": {"value": BYTES_F32_ZP / t_mt / 1e9, "cores": cores, "ms_per_gemv": t_mt * 1e3},
+        "quantize_pack_from_f32_s": t_pack,
+    }, y
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=6400)
+    ap.add_argument("--warmup", type=int, default=640)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only-gemv", action="store_true", help="skip the secondary workloads")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build targets one GPU; --gpus above 1 is not supported "
+                 "(no collectives or sharding are part of it)")
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
+    from rumus_amd import _lib, ops
+    _lib.call("rumus_hip_init", 0)
+    torch.cuda.set_device(0)
+
+    steps = max(WEIGHT_SETS, (args.steps // WEIGHT_SETS) * WEIGHT_SETS)
+    warmup = max(0, args.warmup)
+
+    torch.cuda.synchronize()
+    wall0 = time.perf_counter()
+    r = bench_gemv(torch, ops, steps, warmup)
+    wall = time.perf_counter() - wall0
+    log(f"[bench] gemv leg wall {wall:.1f}s (includes building {WEIGHT_SETS} weight sets)")
+
+    per_launch = r["sec"] / r["launches"]
+    gbs = BYTES_F32_ZP / per_launch / 1e9
+    per_launch_res = r["sec_resident"] / r["launches_resident"]
+
+    out = {
+        "metric": "W4 GEMV GB/s (%HBM peak) @1x4096x4096; INT8 GEMM TOPS (%MFMA peak)",
+        "value": gbs, "unit": "GB/s", "n_gpus": 1, "steps": r["launches"], "warmup": warmup,
+        "ms_per_step": per_launch * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "w4_gemv_1x4096x4096_g128_awq_f32zp", "weight_sets_rotated": WEIGHT_SETS,
+                   "hip_graph": r["graph"], "bytes_per_step": BYTES_F32_ZP},
+        "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": gbs / HBM_PEAK_GBS, "traffic": None},
+        "gbs_at_u4_zero_point_bytes": BYTES_U4_ZP / per_launch / 1e9,
+        "cache_resident": {"gbs": BYTES_F32_ZP / per_launch_res / 1e9,
+                           "ms_per_step": per_launch_res * 1e3,
+                           "note": "single weight set, served by Infinity Cache / L2; not HBM"},
+    }
+
+    if not args.only_gemv:
+        out["secondary"] = bench_i8_gemm(torch, ops)
+        out["w4_gemm"] = [bench_w4_gemm(torch, ops, 16), bench_w4_gemm(torch, ops, 128)]
+
+    if not args.no_cpu:
+        cb, y_cpu = cpu_baseline(r["x"], r["w"])
+        out["cpu_baseline"] = cb
+        err = np.abs(r["y0"] - y_cpu)
+        tol = 1e-4 + 1e-3 * np.abs(y_cpu)
+        out["parity_vs_cpu"] = {"max_abs_err": float(err.max()), "within_tol": bool((err <= tol).all())}
+    else:
+        out["cpu_baseline"] = None
+
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,183 @@
+/*
+ * rumus_hip.h -- C ABI of librumus_hip.so: the MI355X (gfx950) device code for
+ * RUMUS's quantized-Linear path.
+ *
+ * Every entry point is what a RUMUS dispatch function for this path would bind
+ * through FFI; the reference interface each one replaces is cited as
+ * file:line relative to the RUMUS checkout.  Entry points marked EXTENSION
+ * have no reference counterpart (the W8A8 INT8 engine, symmetric / act-order
+ * INT4) and follow the closed forms given in their comments.
+ *
+ * Conventions
+ *   - every pointer is a caller-owned DEVICE pointer (hipMalloc'd) unless it
+ *     is said to be a host pointer; the library never frees caller memory and
+ *     allocates nothing on the launch path;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *     launches are asynchronous on that stream, like wgpu's queue.submit
+ *     (rumus/src/backend/gpu/compute.rs:1981);
+ *   - every function returns 0 on success or a RUMUS_HIP_E* code, and
+ *     rumus_hip_last_error() then returns a thread-local message.  The
+ *     reference panics on the same preconditions (assert!/expect); a Rust
+ *     shim turns a non-zero status into panic! to keep that behaviour;
+ *   - functions are re-entrant and thread-safe.
+ */
+#ifndef RUMUS_HIP_H
+#define RUMUS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RUMUS_HIP_OK 0
+#define RUMUS_HIP_EINVAL 1 /* a precondition the reference asserts does not hold */
+#define RUMUS_HIP_EHIP 2   /* a HIP runtime call failed */
+
+typedef void* rumus_hip_stream_t;
+
+/* ---- runtime ------------------------------------------------------------ */
+
+/* GpuContext::get() (rumus/src/backend/gpu/context.rs:779-820): select the
+ * device and cache its properties.  Optional: launches work without it on the
+ * current device. */
+int rumus_hip_init(int device);
+
+/* Message for the last non-zero status returned on this thread. */
+const char* rumus_hip_last_error(void);
+
+/* "rumus-hip <version> gfx950" */
+const char* rumus_hip_version(void);
+
+/* device.poll(Wait) (context.rs:840-850): block until `stream` is idle. */
+int rumus_hip_sync(rumus_hip_stream_t stream);
+
+/* ---- INT8 engine, reference Q8 block format ----------------------------- */
+
+/* DType::Q8{block_size}.gpu_buf_size(numel) (rumus/src/tensor/core.rs:87-98):
+ * num_blocks*(4+block_size) bytes rounded up to 4. */
+uint64_t rumus_hip_q8_buf_size(uint64_t numel, uint32_t block_size);
+
+/* quantize_dispatch (compute.rs:1948-1982) + quantize_kernel
+ * (shaders/quantize.wgsl:29-100).  in: numel f32, already in the order to be
+ * blocked.  out: per block one header word (f16 scale in the low 16 bits) and
+ * block_size/4 data words of little-endian signed bytes.
+ * EINVAL unless block_size > 0 and block_size % 4 == 0 (ops.rs:2291). */
+int rumus_hip_q8_quantize(const float* in, uint32_t* out, uint32_t numel,
+                          uint32_t block_size, rumus_hip_stream_t stream);
+
+/* dequantize_dispatch (compute.rs:1985-2018) + dequantize_kernel
+ * (shaders/dequantize.wgsl:32-52): out[i] = f32(q[i]) * f16scale(block i/bs). */
+int rumus_hip_q8_dequantize(const uint32_t* in, float* out, uint32_t numel,
+                            uint32_t block_size, rumus_hip_stream_t stream);
+
+/* matmul_q8_dispatch (compute.rs:2021-2060) + matmul_q8_kernel
+ * (shaders/matmul_q8.wgsl:37-98): c[m,n] = a[m,k] f32 x Q8 b, where column j
+ * of b is the run of ceil(k/block_size) blocks starting at word
+ * j*blocks_per_col*stride. */
+int rumus_hip_matmul_q8(const float* a, const uint32_t* b, float* c, uint32_t m,
+                        uint32_t k, uint32_t n, uint32_t block_size,
+                        rumus_hip_stream_t stream);
+
+/* Tensor::add_bias (rumus/src/tensor/ops.rs:885-931, shaders/bias.wgsl:18-25):
+ * out[i,j] = mat[i,j] + bias[j].  out may alias mat. */
+int rumus_hip_add_bias(const float* mat, const float* bias, float* out,
+                       uint32_t m, uint32_t n, rumus_hip_stream_t stream);
+
+/* transpose(-2,-1).contiguous() that Tensor::quantize runs first
+ * (ops.rs:2307): out[c,r] = in[r,c]. */
+int rumus_hip_transpose_f32(const float* in, float* out, uint32_t rows,
+                            uint32_t cols, rumus_hip_stream_t stream);
+
+/* ---- INT8 engine, W8A8 (EXTENSION) -------------------------------------- */
+
+/* Dynamic per-row quantizer: for each row r of x[rows,cols]
+ *   amax = max|x[r,:]|; scale[r] = amax==0 ? 1 : amax/127;
+ *   inv = amax==0 ? 0 : 127/amax; xq[r,c] = clamp(rint(x[r,c]*inv),-128,127)
+ * i.e. quantize.wgsl:66-67,93 per row, with the scale kept in f32. */
+int rumus_hip_i8_quantize_rows(const float* x, int8_t* xq, float* scale,
+                               uint32_t rows, uint32_t cols,
+                               rumus_hip_stream_t stream);
+
+/* Per-output-channel weight quantizer for a Linear weight w[k,n] ([in,out],
+ * rumus/src/nn/linear.rs:39-46): same formula per COLUMN of w; the result is
+ * written transposed, wq[n,k] (K contiguous), with sw[n]. */
+int rumus_hip_i8_quantize_cols_t(const float* w, int8_t* wq, float* sw,
+                                 uint32_t k, uint32_t n, rumus_hip_stream_t stream);
+
+/* acc[m,n] = sum_k xq[m,k]*wq[n,k] on the i8 matrix cores (exact i32), then
+ * y[m,n] = (f32(acc)*sx[m])*sw[n] (+ bias[n]).
+ * acc may be NULL (accumulators not stored); y may be NULL (only acc stored,
+ * sx/sw/bias ignored); bias may be NULL.  EINVAL unless k % 16 == 0. */
+int rumus_hip_i8_gemm(const int8_t* xq, const int8_t* wq, const float* sx,
+                      const float* sw, const float* bias, int32_t* acc, float* y,
+                      uint32_t m, uint32_t k, uint32_t n, rumus_hip_stream_t stream);
+
+/* ---- INT4 engine --------------------------------------------------------- */
+
+/* QuantizedTensor::from_f32 (rumus-vision/src/quant.rs:42-102) on the device:
+ * w[k,n] f32 -> packed u32 [(padded_k/8), n], scales and zero_points f32
+ * [num_groups, n], with padded_k = ceil(k/group_size)*group_size.
+ * EINVAL unless group_size % 8 == 0 (quant.rs:43). */
+int rumus_hip_w4_quantize_pack(const float* w, uint32_t k, uint32_t n,
+                               uint32_t group_size, uint32_t* packed,
+                               float* scales, float* zero_points,
+                               rumus_hip_stream_t stream);
+
+/* EXTENSION: symmetric 4-bit, zero-point 8: scale = max|w|/7 per (group,col)
+ * (1 for an all-zero group), q = clamp(round_half_away(w/scale)+8, 0, 15).
+ * zero_points (may be NULL) is filled with 8.0f. */
+int rumus_hip_w4_quantize_pack_sym(const float* w, uint32_t k, uint32_t n,
+                                   uint32_t group_size, uint32_t* packed,
+                                   float* scales, float* zero_points,
+                                   rumus_hip_stream_t stream);
+
+/* custom_forward(&QMatMulINT4FwdOp, [x, packed, scales, zp]) followed by
+ * add_bias (rumus-vision/src/quant.rs:191-221,228-256; kernel
+ * shaders/qmatmul_int4.wgsl:40-87).  The six scalars are the op's uniform
+ * (quant.rs:243-249).  y[m,n] = x[m,k] . dequant(W) (+ bias[n]),
+ * dequant = (q - zp[g,n]) * scales[g,n], g = row/group_size.
+ * bias may be NULL.  EXTENSION: g_idx (device int32[k], may be NULL) replaces
+ * g by g_idx[row] (act-order).
+ * EINVAL unless group_size % 8 == 0, padded_k == num_groups*group_size,
+ * k <= padded_k < k+group_size. */
+int rumus_hip_qmatmul_int4(const float* x, const uint32_t* packed,
+                           const float* scales, const float* zero_points,
+                           const float* bias, const int32_t* g_idx, float* y,
+                           uint32_t m, uint32_t k, uint32_t n, uint32_t padded_k,
+                           uint32_t group_size, uint32_t num_groups,
+                           rumus_hip_stream_t stream);
+
+/* custom_forward(&QMatMulINT4TransposeOp, [grad_y, packed, scales, zp])
+ * (quant.rs:262-317; kernel shaders/qmatmul_int4_transpose.wgsl:37-74):
+ * out[m,k] = a[m,n] . dequant(W)^T. */
+int rumus_hip_qmatmul_int4_t(const float* a, const uint32_t* packed,
+                             const float* scales, const float* zero_points,
+                             float* out, uint32_t m, uint32_t k, uint32_t n,
+                             uint32_t padded_k, uint32_t group_size,
+                             uint32_t num_groups, rumus_hip_stream_t stream);
+
+/* EXTENSION (act-order, done once per weight): stable-sort the rows of W by
+ * g_idx so that every group is contiguous.  perm[j] (int32[padded_k]) is the
+ * original row stored at sorted position j; packed_sorted has the layout of
+ * packed.  EINVAL unless every group holds exactly group_size rows. */
+int rumus_hip_w4_actorder_prepare(const uint32_t* packed, const int32_t* g_idx,
+                                  uint32_t padded_k, uint32_t n, uint32_t group_size,
+                                  uint32_t* packed_sorted, int32_t* perm,
+                                  rumus_hip_stream_t stream);
+
+/* EXTENSION: qmatmul_int4 on a weight prepared by rumus_hip_w4_actorder_prepare:
+ * y[m,n] = sum_j x[m,perm[j]] * (q_sorted[j,n]-zp[j/gs,n])*scales[j/gs,n].
+ * perm == NULL means the identity.  Requires k == padded_k when perm != NULL. */
+int rumus_hip_qmatmul_int4_perm(const float* x, const uint32_t* packed_sorted,
+                                const float* scales, const float* zero_points,
+                                const float* bias, const int32_t* perm, float* y,
+                                uint32_t m, uint32_t k, uint32_t n, uint32_t padded_k,
+                                uint32_t group_size, uint32_t num_groups,
+                                rumus_hip_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

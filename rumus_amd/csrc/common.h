@@ -1,0 +1,41 @@
+// Shared helpers for the gfx950 kernels of librumus_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "rumus_hip.h"
+
+namespace rumus {
+
+// Records a thread-local message and returns `code`.
+int set_error(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+// Converts a HIP status into a return code (0 when hipSuccess).
+int check_hip(hipError_t e, const char* what);
+
+// hipGetLastError() after a kernel launch.
+inline int check_launch(const char* kernel) { return check_hip(hipGetLastError(), kernel); }
+
+inline hipStream_t as_stream(rumus_hip_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+constexpr int kWave = 64;       // CDNA wavefront width
+constexpr int kXcds = 8;        // MI355X: 8 accelerator dies, each with its own L2
+
+inline uint32_t ceil_div(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
+
+// Workgroups are handed to the 8 XCDs round-robin (workgroup b runs on XCD
+// b % 8).  This maps b to a logical tile index so that each XCD owns one
+// contiguous range of tiles: neighbouring tiles then share an L2.
+__device__ __forceinline__ uint32_t xcd_contiguous(uint32_t b, uint32_t total) {
+    uint32_t x = b % kXcds, l = b / kXcds;
+    uint32_t q = total / kXcds, r = total % kXcds;
+    return x * q + (x < r ? x : r) + l;
+}
+
+}  // namespace rumus
+
+#define RUMUS_REQUIRE(cond, ...)                                         \
+    do {                                                                 \
+        if (!(cond)) return ::rumus::set_error(RUMUS_HIP_EINVAL, __VA_ARGS__); \
+    } while (0)

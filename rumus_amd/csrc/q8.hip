@@ -1,0 +1,316 @@
+// INT8 engine, reference Q8 block format: quantize, dequantize, W8A32 matmul,
+// plus the bias add and the transpose that surround them in the reference.
+//
+// Buffer format (rumus/src/tensor/core.rs:61-98): per block one header word
+// (f16 scale in the low half) followed by block_size signed bytes.
+#include <hip/hip_fp16.h>
+
+#include "common.h"
+
+namespace rumus {
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+    return v;
+}
+
+__device__ __forceinline__ int quant_i8(float v, float inv) {
+    // quantize.wgsl:93: clamp(i32(round(v*inv)), -128, 127), round = half-even.
+    float t = rintf(__fmul_rn(v, inv));
+    t = fminf(fmaxf(t, -128.0f), 127.0f);
+    return (int)t;
+}
+
+// One wave per block: abs-max by wave reduction, then quantize and pack.
+// quantize.wgsl:29-100.
+__global__ __launch_bounds__(256) void q8_quantize_kernel(const float* __restrict__ in,
+                                                          uint32_t* __restrict__ out,
+                                                          uint32_t numel, uint32_t bs,
+                                                          uint32_t num_blocks, uint32_t stride) {
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t block = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (block >= num_blocks) return;
+    const uint64_t start = (uint64_t)block * bs;
+    const uint32_t words = bs / 4;
+    const bool full = start + bs <= numel && ((reinterpret_cast<uintptr_t>(in) & 15) == 0);
+
+    float amax = 0.0f;
+    if (full) {
+        const float4* p = reinterpret_cast<const float4*>(in + start);
+        for (uint32_t w = lane; w < words; w += 64) {
+            float4 v = p[w];
+            amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+        }
+    } else {
+        for (uint32_t i = lane; i < bs; i += 64)
+            if (start + i < numel) amax = fmaxf(amax, fabsf(in[start + i]));
+    }
+    amax = wave_max(amax);
+
+    const float scale = amax == 0.0f ? 1.0f : __fdiv_rn(amax, 127.0f);  // :66
+    const float inv = amax == 0.0f ? 0.0f : __fdiv_rn(127.0f, amax);    // :67
+    uint32_t* ob = out + (uint64_t)block * stride;
+    if (lane == 0) ob[0] = (uint32_t)__half_as_ushort(__float2half_rn(scale));  // :71-74
+
+    if (full) {
+        const float4* p = reinterpret_cast<const float4*>(in + start);
+        for (uint32_t w = lane; w < words; w += 64) {
+            float4 v = p[w];
+            uint32_t word = ((uint32_t)quant_i8(v.x, inv) & 0xFFu) |
+                            (((uint32_t)quant_i8(v.y, inv) & 0xFFu) << 8) |
+                            (((uint32_t)quant_i8(v.z, inv) & 0xFFu) << 16) |
+                            (((uint32_t)quant_i8(v.w, inv) & 0xFFu) << 24);
+            ob[1 + w] = word;
+        }
+    } else {
+        for (uint32_t w = lane; w < words; w += 64) {
+            uint32_t word = 0;
+            for (uint32_t b = 0; b < 4; b++) {
+                uint64_t gi = start + w * 4 + b;
+                int q = gi < numel ? quant_i8(in[gi], inv) : 0;
+                word |= ((uint32_t)q & 0xFFu) << (8 * b);
+            }
+            ob[1 + w] = word;
+        }
+    }
+}
+
+__device__ __forceinline__ float header_scale(uint32_t header) {
+    return __half2float(__ushort_as_half((unsigned short)(header & 0xFFFFu)));
+}
+
+// One thread per data word (4 elements).  dequantize.wgsl:32-52.
+__global__ __launch_bounds__(256) void q8_dequantize_kernel(const uint32_t* __restrict__ in,
+                                                            float* __restrict__ out,
+                                                            uint32_t numel, uint32_t bs,
+                                                            uint32_t stride) {
+    const uint64_t w = (uint64_t)blockIdx.x * 256 + threadIdx.x;  // data-word index
+    const uint64_t e0 = w * 4;
+    if (e0 >= numel) return;
+    const uint32_t block = (uint32_t)(e0 / bs);
+    const uint32_t pos = (uint32_t)(e0 % bs);
+    const uint32_t* ib = in + (uint64_t)block * stride;
+    const float scale = header_scale(ib[0]);
+    const uint32_t word = ib[1 + pos / 4];
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+        if (e0 + b < numel) {
+            int q = (int)(int8_t)((word >> (8 * b)) & 0xFFu);
+            out[e0 + b] = __fmul_rn((float)q, scale);
+        }
+    }
+}
+
+// W8A32 matmul, 64x64 tile per workgroup, 4x4 outputs per thread, K in steps
+// of 16.  Arithmetic follows matmul_q8.wgsl:77-80 per element:
+// sum += (a * f32(q)) * scale.  Requires block_size % 16 == 0 so that a run of
+// 16 bytes never straddles a block.
+constexpr int kQ8Tile = 64;
+constexpr int kQ8K = 16;
+
+__global__ __launch_bounds__(256) void matmul_q8_tiled_kernel(
+    const float* __restrict__ a, const uint32_t* __restrict__ b, float* __restrict__ c,
+    uint32_t m, uint32_t k, uint32_t n, uint32_t bs, uint32_t stride, uint32_t blocks_per_col) {
+    __shared__ float as[kQ8K][kQ8Tile + 4];
+    __shared__ float ws[kQ8K][kQ8Tile + 4];   // f32(q)
+    __shared__ float ss[kQ8Tile];             // block scale per column for this K step
+    const uint32_t tid = threadIdx.x;
+    const uint32_t row0 = blockIdx.y * kQ8Tile, col0 = blockIdx.x * kQ8Tile;
+    const uint32_t tx = tid % 16, ty = tid / 16;
+    float acc[4][4] = {};
+
+    for (uint32_t k0 = 0; k0 < k; k0 += kQ8K) {
+        // A tile: 64 rows x 16 k; thread loads 4 consecutive k of one row.
+        {
+            uint32_t r = tid / 4, kq = (tid % 4) * 4;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                uint32_t kk = k0 + kq + i;
+                float v = 0.0f;
+                if (row0 + r < m && kk < k) v = a[(uint64_t)(row0 + r) * k + kk];
+                as[kq + i][r] = v;
+            }
+        }
+        // B tile: 64 columns x 16 k = one word per (column, k-quad).
+        {
+            uint32_t cidx = tid / 4, kq = (tid % 4) * 4;
+            uint32_t col = col0 + cidx;
+            uint32_t kk = k0 + kq;
+            uint32_t word = 0;
+            float sc = 0.0f;
+            if (col < n && kk < k) {
+                uint32_t blk = kk / bs, pos = kk % bs;
+                const uint32_t* bb = b + ((uint64_t)col * blocks_per_col + blk) * stride;
+                word = bb[1 + pos / 4];
+                sc = header_scale(bb[0]);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                float q = (float)(int)(int8_t)((word >> (8 * i)) & 0xFFu);
+                ws[kq + i][cidx] = (k0 + kq + i < k) ? q : 0.0f;
+            }
+            if (kq == 0) ss[cidx] = sc;
+        }
+        __syncthreads();
+        float sc[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) sc[j] = ss[tx * 4 + j];
+#pragma unroll
+        for (int kk = 0; kk < kQ8K; kk++) {
+            float av[4], wv[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) av[i] = as[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; j++) wv[j] = ws[kk][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    acc[i][j] = __fadd_rn(acc[i][j], __fmul_rn(__fmul_rn(av[i], wv[j]), sc[j]));
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        uint32_t r = row0 + ty * 4 + i;
+        if (r >= m) continue;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            uint32_t cc = col0 + tx * 4 + j;
+            if (cc < n) c[(uint64_t)r * n + cc] = acc[i][j];
+        }
+    }
+}
+
+// Any block_size % 4 == 0: one thread per output, the reference's own loop.
+__global__ __launch_bounds__(256) void matmul_q8_naive_kernel(
+    const float* __restrict__ a, const uint32_t* __restrict__ b, float* __restrict__ c,
+    uint32_t m, uint32_t k, uint32_t n, uint32_t bs, uint32_t stride, uint32_t blocks_per_col) {
+    const uint32_t col = blockIdx.x * 64 + threadIdx.x % 64;
+    const uint32_t row = blockIdx.y * 4 + threadIdx.x / 64;
+    if (row >= m || col >= n) return;
+    float sum = 0.0f;
+    uint32_t k_off = 0;
+    for (uint32_t blk = 0; blk < blocks_per_col; blk++) {
+        const uint32_t* bb = b + ((uint64_t)col * blocks_per_col + blk) * stride;
+        const float sc = header_scale(bb[0]);
+        const uint32_t len = min(bs, k - k_off);
+        for (uint32_t r = 0; r < len; r++) {
+            int q = (int)(int8_t)((bb[1 + r / 4] >> (8 * (r % 4))) & 0xFFu);
+            sum = __fadd_rn(sum, __fmul_rn(__fmul_rn(a[(uint64_t)row * k + k_off + r], (float)q), sc));
+        }
+        k_off += bs;
+    }
+    c[(uint64_t)row * n + col] = sum;
+}
+
+// bias.wgsl:18-25, four columns per thread when n % 4 == 0.
+__global__ __launch_bounds__(256) void add_bias_kernel(const float* __restrict__ mat,
+                                                       const float* __restrict__ bias,
+                                                       float* __restrict__ out, uint64_t total,
+                                                       uint32_t n) {
+    uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    out[i] = __fadd_rn(mat[i], bias[i % n]);
+}
+
+// 32x32 tile transpose through LDS.
+__global__ __launch_bounds__(256) void transpose_kernel(const float* __restrict__ in,
+                                                        float* __restrict__ out, uint32_t rows,
+                                                        uint32_t cols) {
+    __shared__ float t[32][33];
+    const uint32_t tx = threadIdx.x % 32, ty = threadIdx.x / 32;  // 32 x 8
+    const uint32_t r0 = blockIdx.y * 32, c0 = blockIdx.x * 32;
+#pragma unroll
+    for (int i = 0; i < 32; i += 8) {
+        uint32_t r = r0 + ty + i, cc = c0 + tx;
+        if (r < rows && cc < cols) t[ty + i][tx] = in[(uint64_t)r * cols + cc];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 32; i += 8) {
+        uint32_t cc = c0 + ty + i, r = r0 + tx;
+        if (r < rows && cc < cols) out[(uint64_t)cc * rows + r] = t[tx][ty + i];
+    }
+}
+
+}  // namespace rumus
+
+using namespace rumus;
+
+extern "C" {
+
+uint64_t rumus_hip_q8_buf_size(uint64_t numel, uint32_t block_size) {
+    if (block_size == 0) return 0;
+    uint64_t num_blocks = (numel + block_size - 1) / block_size;
+    return (num_blocks * (4 + (uint64_t)block_size) + 3) & ~(uint64_t)3;
+}
+
+int rumus_hip_q8_quantize(const float* in, uint32_t* out, uint32_t numel, uint32_t block_size,
+                          rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE(block_size > 0 && block_size % 4 == 0,
+                  "quantize: block_size must be > 0 and divisible by 4 (got %u)", block_size);
+    RUMUS_REQUIRE(in && out, "quantize: null buffer");
+    if (numel == 0) return RUMUS_HIP_OK;
+    uint32_t num_blocks = ceil_div(numel, block_size);
+    uint32_t stride = (4 + block_size + 3) / 4;
+    hipLaunchKernelGGL(q8_quantize_kernel, dim3(ceil_div(num_blocks, 4)), dim3(256), 0,
+                       as_stream(stream), in, out, numel, block_size, num_blocks, stride);
+    return check_launch("q8_quantize_kernel");
+}
+
+int rumus_hip_q8_dequantize(const uint32_t* in, float* out, uint32_t numel, uint32_t block_size,
+                            rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE(block_size > 0 && block_size % 4 == 0,
+                  "dequantize: block_size must be > 0 and divisible by 4 (got %u)", block_size);
+    RUMUS_REQUIRE(in && out, "dequantize: null buffer");
+    if (numel == 0) return RUMUS_HIP_OK;
+    uint32_t stride = (4 + block_size + 3) / 4;
+    uint32_t words = ceil_div(numel, 4);
+    hipLaunchKernelGGL(q8_dequantize_kernel, dim3(ceil_div(words, 256)), dim3(256), 0,
+                       as_stream(stream), in, out, numel, block_size, stride);
+    return check_launch("q8_dequantize_kernel");
+}
+
+int rumus_hip_matmul_q8(const float* a, const uint32_t* b, float* c, uint32_t m, uint32_t k,
+                        uint32_t n, uint32_t block_size, rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE(block_size > 0 && block_size % 4 == 0,
+                  "matmul_q8: block_size must be > 0 and divisible by 4 (got %u)", block_size);
+    RUMUS_REQUIRE(a && b && c, "matmul_q8: null buffer");
+    if (m == 0 || n == 0) return RUMUS_HIP_OK;
+    RUMUS_REQUIRE(k > 0, "matmul_q8: k must be > 0");
+    uint32_t blocks_per_col = ceil_div(k, block_size);
+    uint32_t stride = (4 + block_size + 3) / 4;
+    if (block_size % 16 == 0) {
+        dim3 grid(ceil_div(n, kQ8Tile), ceil_div(m, kQ8Tile));
+        hipLaunchKernelGGL(matmul_q8_tiled_kernel, grid, dim3(256), 0, as_stream(stream), a, b, c,
+                           m, k, n, block_size, stride, blocks_per_col);
+        return check_launch("matmul_q8_tiled_kernel");
+    }
+    dim3 grid(ceil_div(n, 64), ceil_div(m, 4));
+    hipLaunchKernelGGL(matmul_q8_naive_kernel, grid, dim3(256), 0, as_stream(stream), a, b, c, m,
+                       k, n, block_size, stride, blocks_per_col);
+    return check_launch("matmul_q8_naive_kernel");
+}
+
+int rumus_hip_add_bias(const float* mat, const float* bias, float* out, uint32_t m, uint32_t n,
+                       rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE(mat && bias && out, "add_bias: null buffer");
+    uint64_t total = (uint64_t)m * n;
+    if (total == 0) return RUMUS_HIP_OK;
+    hipLaunchKernelGGL(add_bias_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0,
+                       as_stream(stream), mat, bias, out, total, n);
+    return check_launch("add_bias_kernel");
+}
+
+int rumus_hip_transpose_f32(const float* in, float* out, uint32_t rows, uint32_t cols,
+                            rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE(in && out, "transpose: null buffer");
+    if (rows == 0 || cols == 0) return RUMUS_HIP_OK;
+    dim3 grid(ceil_div(cols, 32), ceil_div(rows, 32));
+    hipLaunchKernelGGL(transpose_kernel, grid, dim3(256), 0, as_stream(stream), in, out, rows, cols);
+    return check_launch("transpose_kernel");
+}
+
+}  // extern "C"

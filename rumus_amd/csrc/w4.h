@@ -1,0 +1,36 @@
+// Internal interface between the INT4 matmul kernels and their dispatcher.
+#pragma once
+
+#include "common.h"
+
+namespace rumus {
+
+// Arguments of one fused INT4 dequant-matmul, y[m,n] = x[m,k] . dequant(W).
+// `perm` (or null) gathers the activation column for sorted row j; `g_idx`
+// (or null) picks the metadata row per original row (generic kernel only).
+struct W4Args {
+    const float* x;
+    const uint32_t* packed;
+    const float* scales;
+    const float* zp;
+    const float* bias;
+    const int32_t* g_idx;
+    const int32_t* perm;
+    float* y;
+    uint32_t m, k, n, padded_k, group_size, num_groups;
+};
+
+// Reference-order kernel: any shape, g_idx and perm; one thread per column.
+int w4_launch_generic(const W4Args& a, hipStream_t s);
+
+// Bandwidth kernel for m <= 8 (needs n % 4 == 0, 16-byte aligned buffers,
+// m * padded_k floats of LDS, no g_idx).
+bool w4_gemv_supported(const W4Args& a);
+int w4_launch_gemv(const W4Args& a, hipStream_t s);
+
+// f16 MFMA kernel for larger m (needs group_size % 32 == 0, n % 4 == 0,
+// 16-byte aligned buffers, no g_idx).
+bool w4_gemm_supported(const W4Args& a);
+int w4_launch_gemm(const W4Args& a, hipStream_t s);
+
+}  // namespace rumus

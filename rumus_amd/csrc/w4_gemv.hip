@@ -1,0 +1,347 @@
+// INT4 engine: fused dequant-matmul kernels that are bound by HBM bandwidth
+// (decode shapes, m <= 8), the reference-order kernel for every other case the
+// MFMA kernel does not take, the transpose kernel for grad_x, and the entry
+// points that pick between them.
+//
+// Packed layout (rumus-vision/src/quant.rs:98-100): word (k/8)*N + col holds
+// rows 8*(k/8)..+7 of column col; scales / zero_points are f32 [groups, N].
+#include "w4.h"
+
+namespace rumus {
+
+// ---------------------------------------------------------------------------
+// Reference-order kernel.  One thread per column, MR rows per thread, strictly
+// ascending k, w = (f32(q) - zp) * scale then sum += x * w with every
+// operation rounded separately (qmatmul_int4.wgsl:50-84): the result is
+// bit-identical to a scalar CPU loop in the same order.
+// ---------------------------------------------------------------------------
+template <int MR>
+__global__ __launch_bounds__(64) void w4_generic_kernel(W4Args a) {
+    const uint32_t col = blockIdx.x * 64 + threadIdx.x;
+    const uint32_t row0 = blockIdx.y * MR;
+    if (col >= a.n) return;
+    float sum[MR];
+#pragma unroll
+    for (int r = 0; r < MR; r++) sum[r] = 0.0f;
+    const uint32_t wpg = a.group_size / 8;
+    for (uint32_t g = 0; g < a.num_groups; g++) {
+        float scale = a.scales[(uint64_t)g * a.n + col];
+        float z = a.zp[(uint64_t)g * a.n + col];
+        for (uint32_t w = 0; w < wpg; w++) {
+            const uint32_t k_base = g * a.group_size + w * 8;
+            if (k_base >= a.k) break;
+            const uint32_t word = a.packed[(uint64_t)(k_base / 8) * a.n + col];
+            for (uint32_t j = 0; j < 8; j++) {
+                const uint32_t kk = k_base + j;
+                if (kk >= a.k) break;  // padding rows (qmatmul_int4.wgsl:71)
+                const float q = (float)((word >> (4 * j)) & 0xFu);
+                if (a.g_idx) {
+                    const uint64_t mi = (uint64_t)a.g_idx[kk] * a.n + col;
+                    scale = a.scales[mi];
+                    z = a.zp[mi];
+                }
+                const float wv = __fmul_rn(__fsub_rn(q, z), scale);
+                const uint32_t xk = a.perm ? (uint32_t)a.perm[kk] : kk;
+#pragma unroll
+                for (int r = 0; r < MR; r++) {
+                    if (row0 + r < a.m) {
+                        const float xv = a.x[(uint64_t)(row0 + r) * a.k + xk];
+                        sum[r] = __fadd_rn(sum[r], __fmul_rn(xv, wv));
+                    }
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < MR; r++) {
+        if (row0 + r < a.m) {
+            float v = sum[r];
+            if (a.bias) v = __fadd_rn(v, a.bias[col]);
+            a.y[(uint64_t)(row0 + r) * a.n + col] = v;
+        }
+    }
+}
+
+int w4_launch_generic(const W4Args& a, hipStream_t s) {
+    constexpr int MR = 4;
+    hipLaunchKernelGGL((w4_generic_kernel<MR>), dim3(ceil_div(a.n, 64), ceil_div(a.m, MR)), dim3(64),
+                       0, s, a);
+    return check_launch("w4_generic_kernel");
+}
+
+// ---------------------------------------------------------------------------
+// Bandwidth kernel, m <= 8.
+//
+// A workgroup owns 16 adjacent columns over the whole of K, so no partial
+// sums cross workgroups (no atomics, no zero-fill, deterministic).  Four lanes
+// cover the 16 columns with one 128-bit load each (4 words = 4 columns x 8
+// rows); the other lane bits and the four waves walk the K/8 word rows 64 at
+// a time.  A word row is then a 64-byte segment per workgroup: the XCD-
+// contiguous workgroup order puts the workgroup that reads the other half of
+// each 128-byte line on the same L2.  All loads of a pass are issued before
+// any arithmetic.  Per (word, column) the kernel forms d = sum_j x_j * q_j in
+// f32 straight from the nibbles (v_cvt_f32_ubyte on masked words) and applies
+// scale * (d - zp * sum_j x_j), which equals sum_j x_j * (q_j - zp) * scale.
+// Rows of x live in LDS (zero beyond k, so padded nibbles contribute nothing).
+// ---------------------------------------------------------------------------
+constexpr int kGemvCols = 16;   // columns per workgroup
+constexpr int kGemvRows = 64;   // word rows per pass (256 threads / 4 column lanes)
+constexpr int kGemvUnroll = 8;  // passes whose loads are in flight together
+
+__device__ __forceinline__ float ubyte(uint32_t v, int i) { return (float)((v >> (8 * i)) & 0xFFu); }
+
+template <int M>
+__global__ __launch_bounds__(256) void w4_gemv_kernel(W4Args a, uint32_t nchunks) {
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    float* xs = smem;                            // [M][padded_k]
+    float* red = smem + (size_t)M * a.padded_k;  // [4 waves][M][16]
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t chunk = xcd_contiguous(blockIdx.x, nchunks);
+    const uint32_t c0 = chunk * kGemvCols;
+
+    for (uint32_t i = tid; i < M * a.padded_k; i += 256) {
+        const uint32_t r = i / a.padded_k, j = i - r * a.padded_k;
+        float v = 0.0f;
+        if (j < a.k) v = a.x[(uint64_t)r * a.k + (a.perm ? (uint32_t)a.perm[j] : j)];
+        xs[i] = v;
+    }
+    __syncthreads();
+
+    const uint32_t cq = tid & 3, rsub = tid >> 2;
+    const uint32_t col = c0 + 4 * cq;
+    const bool col_ok = col < a.n;  // n % 4 == 0: all four columns in or out
+    const uint32_t R = a.padded_k / 8;
+
+    float acc[M][4];
+#pragma unroll
+    for (int m = 0; m < M; m++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) acc[m][c] = 0.0f;
+
+    for (uint32_t r0 = 0; r0 < R; r0 += kGemvRows * kGemvUnroll) {
+        uint4 w[kGemvUnroll];
+        float4 sc[kGemvUnroll], z[kGemvUnroll];
+#pragma unroll
+        for (int u = 0; u < kGemvUnroll; u++) {
+            const uint32_t r = r0 + u * kGemvRows + rsub;
+            if (col_ok && r < R) {
+                const uint32_t g = (r * 8) / a.group_size;
+                w[u] = *reinterpret_cast<const uint4*>(a.packed + (uint64_t)r * a.n + col);
+                sc[u] = *reinterpret_cast<const float4*>(a.scales + (uint64_t)g * a.n + col);
+                z[u] = *reinterpret_cast<const float4*>(a.zp + (uint64_t)g * a.n + col);
+            } else {
+                w[u] = make_uint4(0, 0, 0, 0);
+                sc[u] = make_float4(0, 0, 0, 0);
+                z[u] = make_float4(0, 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kGemvUnroll; u++) {
+            const uint32_t r = min(r0 + u * kGemvRows + rsub, R - 1);
+            const uint32_t wv[4] = {w[u].x, w[u].y, w[u].z, w[u].w};
+            const float scv[4] = {sc[u].x, sc[u].y, sc[u].z, sc[u].w};
+            const float zv[4] = {z[u].x, z[u].y, z[u].z, z[u].w};
+            float q[4][8];
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const uint32_t lo = wv[c] & 0x0F0F0F0Fu, hi = (wv[c] >> 4) & 0x0F0F0F0Fu;
+#pragma unroll
+                for (int b = 0; b < 4; b++) {
+                    q[c][2 * b] = ubyte(lo, b);
+                    q[c][2 * b + 1] = ubyte(hi, b);
+                }
+            }
+#pragma unroll
+            for (int m = 0; m < M; m++) {
+                const float4 xa = *reinterpret_cast<const float4*>(xs + (size_t)m * a.padded_k + r * 8);
+                const float4 xb = *reinterpret_cast<const float4*>(xs + (size_t)m * a.padded_k + r * 8 + 4);
+                const float xv[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+                const float xsum = ((xa.x + xa.y) + (xa.z + xa.w)) + ((xb.x + xb.y) + (xb.z + xb.w));
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    float d = 0.0f;
+#pragma unroll
+                    for (int j = 0; j < 8; j++) d = fmaf(xv[j], q[c][j], d);
+                    acc[m][c] = fmaf(scv[c], fmaf(-zv[c], xsum, d), acc[m][c]);
+                }
+            }
+        }
+    }
+
+    // lanes that share cq hold partial sums of the same columns: fold lane bits 2..5
+#pragma unroll
+    for (int m = 0; m < M; m++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            float v = acc[m][c];
+            v += __shfl_xor(v, 4);
+            v += __shfl_xor(v, 8);
+            v += __shfl_xor(v, 16);
+            v += __shfl_xor(v, 32);
+            acc[m][c] = v;
+        }
+    const uint32_t lane = tid & 63, wave = tid >> 6;
+    if (lane < 4) {
+#pragma unroll
+        for (int m = 0; m < M; m++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) red[(wave * M + m) * kGemvCols + lane * 4 + c] = acc[m][c];
+    }
+    __syncthreads();
+    if (tid < M * kGemvCols) {
+        const uint32_t m = tid / kGemvCols, c = tid % kGemvCols;
+        if (c0 + c < a.n) {
+            float v = (red[(0 * M + m) * kGemvCols + c] + red[(1 * M + m) * kGemvCols + c]) +
+                      (red[(2 * M + m) * kGemvCols + c] + red[(3 * M + m) * kGemvCols + c]);
+            if (a.bias) v += a.bias[c0 + c];
+            a.y[(uint64_t)m * a.n + c0 + c] = v;
+        }
+    }
+}
+
+static size_t gemv_lds_bytes(const W4Args& a) {
+    return ((size_t)a.m * a.padded_k + 4 * (size_t)a.m * kGemvCols) * sizeof(float);
+}
+
+bool w4_gemv_supported(const W4Args& a) {
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(a.packed) | reinterpret_cast<uintptr_t>(a.scales) |
+                           reinterpret_cast<uintptr_t>(a.zp);
+    return a.m >= 1 && a.m <= 8 && a.n % 4 == 0 && (bits & 15) == 0 && !a.g_idx &&
+           gemv_lds_bytes(a) <= 64 * 1024;
+}
+
+template <int M>
+static int launch_gemv_m(const W4Args& a, hipStream_t s) {
+    const uint32_t nchunks = ceil_div(a.n, kGemvCols);
+    hipLaunchKernelGGL((w4_gemv_kernel<M>), dim3(nchunks), dim3(256), gemv_lds_bytes(a), s, a, nchunks);
+    return check_launch("w4_gemv_kernel");
+}
+
+int w4_launch_gemv(const W4Args& a, hipStream_t s) {
+    switch (a.m) {
+        case 1: return launch_gemv_m<1>(a, s);
+        case 2: return launch_gemv_m<2>(a, s);
+        case 3: return launch_gemv_m<3>(a, s);
+        case 4: return launch_gemv_m<4>(a, s);
+        case 5: return launch_gemv_m<5>(a, s);
+        case 6: return launch_gemv_m<6>(a, s);
+        case 7: return launch_gemv_m<7>(a, s);
+        case 8: return launch_gemv_m<8>(a, s);
+    }
+    return set_error(RUMUS_HIP_EINVAL, "w4 gemv: m = %u out of range", a.m);
+}
+
+// ---------------------------------------------------------------------------
+// Transpose kernel (grad_x): out[m,k] = sum_n a[m,n] * dequant(W)[k,n]
+// (qmatmul_int4_transpose.wgsl:37-74).  A workgroup owns one word row (8
+// output columns k) and MR rows of a; threads stride over n, so packed words,
+// scales and zero-points are read once per workgroup row block, coalesced.
+// ---------------------------------------------------------------------------
+template <int MR>
+__global__ __launch_bounds__(256) void w4_transpose_kernel(
+    const float* __restrict__ a, const uint32_t* __restrict__ packed,
+    const float* __restrict__ scales, const float* __restrict__ zp, float* __restrict__ out,
+    uint32_t m, uint32_t k, uint32_t n, uint32_t gs) {
+    __shared__ float red[4][MR][8];
+    const uint32_t kr = blockIdx.x, row0 = blockIdx.y * MR, tid = threadIdx.x;
+    const uint32_t g = (kr * 8) / gs;
+    float acc[MR][8];
+#pragma unroll
+    for (int r = 0; r < MR; r++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) acc[r][j] = 0.0f;
+    for (uint32_t c = tid; c < n; c += 256) {
+        const uint32_t word = packed[(uint64_t)kr * n + c];
+        const float sc = scales[(uint64_t)g * n + c], z = zp[(uint64_t)g * n + c];
+        float wv[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) wv[j] = ((float)((word >> (4 * j)) & 0xFu) - z) * sc;
+#pragma unroll
+        for (int r = 0; r < MR; r++) {
+            if (row0 + r < m) {
+                const float av = a[(uint64_t)(row0 + r) * n + c];
+#pragma unroll
+                for (int j = 0; j < 8; j++) acc[r][j] = fmaf(av, wv[j], acc[r][j]);
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < MR; r++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            float v = acc[r][j];
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+            if ((tid & 63) == 0) red[tid >> 6][r][j] = v;
+        }
+    __syncthreads();
+    if (tid < MR * 8) {
+        const uint32_t r = tid / 8, j = tid % 8;
+        const uint32_t kk = kr * 8 + j;
+        if (row0 + r < m && kk < k)
+            out[(uint64_t)(row0 + r) * k + kk] = (red[0][r][j] + red[1][r][j]) + (red[2][r][j] + red[3][r][j]);
+    }
+}
+
+static int validate(const W4Args& a, const char* who) {
+    RUMUS_REQUIRE(a.group_size > 0 && a.group_size % 8 == 0,
+                  "%s: group_size must be a multiple of 8 (got %u)", who, a.group_size);
+    RUMUS_REQUIRE(a.padded_k == a.num_groups * a.group_size,
+                  "%s: padded_k %u != num_groups %u * group_size %u", who, a.padded_k, a.num_groups,
+                  a.group_size);
+    RUMUS_REQUIRE(a.k <= a.padded_k && a.padded_k < a.k + a.group_size,
+                  "%s: padded_k %u does not pad k %u to group_size %u", who, a.padded_k, a.k,
+                  a.group_size);
+    RUMUS_REQUIRE(a.x && a.packed && a.scales && a.zp && a.y, "%s: null buffer", who);
+    return RUMUS_HIP_OK;
+}
+
+static int dispatch(const W4Args& a, hipStream_t s) {
+    if (a.m == 0 || a.n == 0) return RUMUS_HIP_OK;
+    RUMUS_REQUIRE(a.k > 0, "qmatmul_int4: k must be > 0");
+    if (w4_gemv_supported(a)) return w4_launch_gemv(a, s);
+    if (w4_gemm_supported(a)) return w4_launch_gemm(a, s);
+    return w4_launch_generic(a, s);
+}
+
+}  // namespace rumus
+
+using namespace rumus;
+
+extern "C" {
+
+int rumus_hip_qmatmul_int4(const float* x, const uint32_t* packed, const float* scales,
+                           const float* zero_points, const float* bias, const int32_t* g_idx,
+                           float* y, uint32_t m, uint32_t k, uint32_t n, uint32_t padded_k,
+                           uint32_t group_size, uint32_t num_groups, rumus_hip_stream_t stream) {
+    W4Args a{x, packed, scales, zero_points, bias, g_idx, nullptr, y, m, k, n, padded_k, group_size, num_groups};
+    if (int rc = validate(a, "qmatmul_int4")) return rc;
+    return dispatch(a, as_stream(stream));
+}
+
+int rumus_hip_qmatmul_int4_perm(const float* x, const uint32_t* packed_sorted, const float* scales,
+                                const float* zero_points, const float* bias, const int32_t* perm,
+                                float* y, uint32_t m, uint32_t k, uint32_t n, uint32_t padded_k,
+                                uint32_t group_size, uint32_t num_groups, rumus_hip_stream_t stream) {
+    W4Args a{x, packed_sorted, scales, zero_points, bias, nullptr, perm, y, m, k, n, padded_k, group_size, num_groups};
+    if (int rc = validate(a, "qmatmul_int4_perm")) return rc;
+    RUMUS_REQUIRE(!perm || k == padded_k, "qmatmul_int4_perm: perm needs k == padded_k (%u vs %u)", k,
+                  padded_k);
+    return dispatch(a, as_stream(stream));
+}
+
+int rumus_hip_qmatmul_int4_t(const float* a, const uint32_t* packed, const float* scales,
+                             const float* zero_points, float* out, uint32_t m, uint32_t k,
+                             uint32_t n, uint32_t padded_k, uint32_t group_size,
+                             uint32_t num_groups, rumus_hip_stream_t stream) {
+    W4Args v{a, packed, scales, zero_points, nullptr, nullptr, nullptr, out, m, k, n, padded_k, group_size, num_groups};
+    if (int rc = validate(v, "qmatmul_int4_t")) return rc;
+    if (m == 0 || k == 0) return RUMUS_HIP_OK;
+    constexpr int MR = 4;
+    hipLaunchKernelGGL((w4_transpose_kernel<MR>), dim3(ceil_div(k, 8), ceil_div(m, MR)), dim3(256), 0,
+                       as_stream(stream), a, packed, scales, zero_points, out, m, k, n, group_size);
+    return check_launch("w4_transpose_kernel");
+}
+
+}  // extern "C"

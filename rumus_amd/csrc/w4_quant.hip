@@ -1,0 +1,159 @@
+// INT4 engine, weight preparation: min/max group quantizer + nibble packer
+// (QuantizedTensor::from_f32, rumus-vision/src/quant.rs:42-102), its symmetric
+// variant, and the one-time act-order row sort.
+//
+// Packed layout (quant.rs:98-100): word (row/8)*N + col holds rows
+// 8*(row/8) .. +7 of column col, row r in bits 4*(r%8) .. +3.
+#include <vector>
+
+#include "common.h"
+
+namespace rumus {
+
+// Thread = one column of one group; workgroup = 256 adjacent columns, so every
+// row read and every word store is one contiguous 1 KiB segment per wave
+// quad.  The group is read twice (min/max, then quantize); the second read is
+// served by L2.
+template <bool SYM>
+__global__ __launch_bounds__(256) void w4_quantize_pack_kernel(
+    const float* __restrict__ w, uint32_t k, uint32_t n, uint32_t gs,
+    uint32_t* __restrict__ packed, float* __restrict__ scales, float* __restrict__ zps) {
+    const uint32_t col = blockIdx.x * 256 + threadIdx.x;
+    const uint32_t g = blockIdx.y;
+    if (col >= n) return;
+    const uint32_t r0 = g * gs;
+
+    float scale, zp;
+    if (SYM) {
+        float amax = 0.0f;
+        for (uint32_t r = r0; r < r0 + gs && r < k; r++)
+            amax = fmaxf(amax, fabsf(w[(uint64_t)r * n + col]));
+        scale = amax > 0.0f ? __fdiv_rn(amax, 7.0f) : 1.0f;
+        zp = 8.0f;
+    } else {
+        // quant.rs:66-74; rows >= k are the zero padding of quant.rs:50-56
+        float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
+        for (uint32_t r = r0; r < r0 + gs; r++) {
+            float v = r < k ? w[(uint64_t)r * n + col] : 0.0f;
+            if (v < mn) mn = v;
+            if (v > mx) mx = v;
+        }
+        const float range = __fsub_rn(mx, mn);
+        const bool live = range > 1e-10f;                       // quant.rs:77-79
+        scale = live ? __fdiv_rn(range, 15.0f) : 1.0f;
+        zp = live ? __fdiv_rn(-mn, scale) : 0.0f;
+    }
+    scales[(uint64_t)g * n + col] = scale;
+    if (zps) zps[(uint64_t)g * n + col] = zp;
+
+    for (uint32_t wr = 0; wr < gs / 8; wr++) {
+        uint32_t word = 0;
+#pragma unroll
+        for (uint32_t j = 0; j < 8; j++) {
+            const uint32_t r = r0 + wr * 8 + j;
+            const float v = r < k ? w[(uint64_t)r * n + col] : 0.0f;
+            float t;
+            if (SYM) {
+                t = __fadd_rn(roundf(__fdiv_rn(v, scale)), 8.0f);
+            } else {
+                t = roundf(__fadd_rn(__fdiv_rn(v, scale), zp));  // quant.rs:96, half away
+            }
+            t = fminf(fmaxf(t, 0.0f), 15.0f);                    // NaN -> 0 like `as i32`
+            word |= (uint32_t)t << (4 * j);
+        }
+        packed[(uint64_t)(r0 / 8 + wr) * n + col] = word;
+    }
+}
+
+// packed_sorted word (jr, col) gathers the nibbles of original rows
+// perm[8*jr .. 8*jr+7].
+__global__ __launch_bounds__(256) void w4_gather_rows_kernel(const uint32_t* __restrict__ packed,
+                                                             const int32_t* __restrict__ perm,
+                                                             uint32_t n,
+                                                             uint32_t* __restrict__ out) {
+    const uint32_t col = blockIdx.x * 256 + threadIdx.x;
+    const uint32_t jr = blockIdx.y;
+    if (col >= n) return;
+    uint32_t word = 0;
+#pragma unroll
+    for (uint32_t i = 0; i < 8; i++) {
+        const uint32_t r = (uint32_t)perm[jr * 8 + i];
+        const uint32_t src = packed[(uint64_t)(r / 8) * n + col];
+        word |= ((src >> (4 * (r % 8))) & 0xFu) << (4 * i);
+    }
+    out[(uint64_t)jr * n + col] = word;
+}
+
+template <bool SYM>
+static int quantize_pack(const float* w, uint32_t k, uint32_t n, uint32_t gs, uint32_t* packed,
+                         float* scales, float* zps, hipStream_t s) {
+    RUMUS_REQUIRE(gs > 0 && gs % 8 == 0, "group_size must be a multiple of 8 (got %u)", gs);
+    RUMUS_REQUIRE(w && packed && scales && (SYM || zps), "w4_quantize_pack: null buffer");
+    if (n == 0 || k == 0) return RUMUS_HIP_OK;
+    const uint32_t groups = ceil_div(k, gs);
+    hipLaunchKernelGGL((w4_quantize_pack_kernel<SYM>), dim3(ceil_div(n, 256), groups), dim3(256), 0,
+                       s, w, k, n, gs, packed, scales, zps);
+    return check_launch("w4_quantize_pack_kernel");
+}
+
+}  // namespace rumus
+
+using namespace rumus;
+
+extern "C" {
+
+int rumus_hip_w4_quantize_pack(const float* w, uint32_t k, uint32_t n, uint32_t group_size,
+                               uint32_t* packed, float* scales, float* zero_points,
+                               rumus_hip_stream_t stream) {
+    return quantize_pack<false>(w, k, n, group_size, packed, scales, zero_points, as_stream(stream));
+}
+
+int rumus_hip_w4_quantize_pack_sym(const float* w, uint32_t k, uint32_t n, uint32_t group_size,
+                                   uint32_t* packed, float* scales, float* zero_points,
+                                   rumus_hip_stream_t stream) {
+    return quantize_pack<true>(w, k, n, group_size, packed, scales, zero_points, as_stream(stream));
+}
+
+// Synchronous by design (runs once per weight): g_idx is copied to the host,
+// validated and stably sorted there, and the row gather runs on the device.
+int rumus_hip_w4_actorder_prepare(const uint32_t* packed, const int32_t* g_idx, uint32_t padded_k,
+                                  uint32_t n, uint32_t group_size, uint32_t* packed_sorted,
+                                  int32_t* perm, rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE(group_size > 0 && group_size % 8 == 0,
+                  "group_size must be a multiple of 8 (got %u)", group_size);
+    RUMUS_REQUIRE(padded_k > 0 && padded_k % group_size == 0,
+                  "actorder_prepare: padded_k %u is not a multiple of group_size %u", padded_k,
+                  group_size);
+    RUMUS_REQUIRE(packed && g_idx && packed_sorted && perm, "actorder_prepare: null buffer");
+    RUMUS_REQUIRE(packed != packed_sorted, "actorder_prepare: cannot sort in place");
+    hipStream_t s = as_stream(stream);
+    const uint32_t groups = padded_k / group_size;
+    std::vector<int32_t> gi(padded_k), pm(padded_k);
+    if (int rc = check_hip(hipMemcpyAsync(gi.data(), g_idx, padded_k * sizeof(int32_t),
+                                          hipMemcpyDeviceToHost, s), "copy g_idx"))
+        return rc;
+    if (int rc = check_hip(hipStreamSynchronize(s), "sync g_idx")) return rc;
+    std::vector<uint32_t> count(groups, 0);
+    for (uint32_t r = 0; r < padded_k; r++) {
+        RUMUS_REQUIRE(gi[r] >= 0 && (uint32_t)gi[r] < groups, "actorder_prepare: g_idx[%u] = %d out of range",
+                      r, gi[r]);
+        count[gi[r]]++;
+    }
+    for (uint32_t g = 0; g < groups; g++)
+        RUMUS_REQUIRE(count[g] == group_size, "actorder_prepare: group %u holds %u rows, expected %u", g,
+                      count[g], group_size);
+    std::vector<uint32_t> next(groups);
+    for (uint32_t g = 0; g < groups; g++) next[g] = g * group_size;
+    for (uint32_t r = 0; r < padded_k; r++) pm[next[gi[r]]++] = (int32_t)r;  // stable
+    if (int rc = check_hip(hipMemcpyAsync(perm, pm.data(), padded_k * sizeof(int32_t),
+                                          hipMemcpyHostToDevice, s), "copy perm"))
+        return rc;
+    if (int rc = check_hip(hipStreamSynchronize(s), "sync perm")) return rc;
+    if (n == 0) return RUMUS_HIP_OK;
+    hipLaunchKernelGGL(w4_gather_rows_kernel, dim3(ceil_div(n, 256), padded_k / 8), dim3(256), 0, s,
+                       packed, perm, n, packed_sorted);
+    if (int rc = check_launch("w4_gather_rows_kernel")) return rc;
+    return check_hip(hipStreamSynchronize(s), "sync gather");
+}
+
+}  // extern "C"

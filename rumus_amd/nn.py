@@ -1,0 +1,185 @@
+"""Host-side mirror of the reference's module API for the quantized-Linear path.
+
+Same names, argument meaning and error behaviour as the reference (which
+panics; here a failed precondition raises ``RumusError``/``ValueError``):
+
+* ``Linear``             rumus/src/nn/linear.rs:44-104   (weight ``[in, out]``)
+* ``QuantizedTensor``    rumus-vision/src/quant.rs:24-127
+* ``QLinear``            rumus-vision/src/quant.rs:165-222
+* ``Q8Tensor`` + ``quantize`` / ``dequantize`` / ``matmul``
+                         rumus/src/tensor/ops.rs:516-545,2290-2357 (``DType::Q8``)
+* ``Int8Linear``         the W8A8 engine (no reference counterpart)
+
+torch tensors are only the device-memory handles; all arithmetic is done by the
+HIP library through ``rumus_amd.ops``.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from . import ops
+
+
+class Linear:
+    """``y = x @ weight + bias`` with ``weight`` of shape ``[in_features, out_features]``."""
+
+    def __init__(self, weight: torch.Tensor, bias: Optional[torch.Tensor] = None):
+        if weight.dim() != 2:
+            raise ValueError("Linear: weight must be 2-D [in, out]")
+        self.weight = weight
+        self.bias = bias
+
+    @property
+    def in_features(self) -> int:
+        return self.weight.shape[0]
+
+    @property
+    def out_features(self) -> int:
+        return self.weight.shape[1]
+
+
+# ---- INT4 ------------------------------------------------------------------------
+
+class QuantizedTensor:
+    """INT4 weight with group-wise metadata (quant.rs:24-38)."""
+
+    def __init__(self, k, n, padded_k, group_size, num_groups, packed, scales, zp,
+                 perm: Optional[torch.Tensor] = None):
+        self.k, self.n, self.padded_k = k, n, padded_k
+        self.group_size, self.num_groups = group_size, num_groups
+        self.packed_tensor, self.scales_tensor, self.zp_tensor = packed, scales, zp
+        self.perm = perm  # act-order: original row held at each sorted position
+
+    @classmethod
+    def from_f32(cls, data: torch.Tensor, k: int, n: int, group_size: int,
+                 symmetric: bool = False) -> "QuantizedTensor":
+        """quant.rs:42-102 on the device.  ``data`` is ``[k, n]`` row-major (any shape with k*n elements)."""
+        if group_size <= 0 or group_size % 8 != 0:
+            raise ValueError("group_size must be a multiple of 8")
+        if data.numel() != k * n:
+            raise ValueError("data length mismatch")
+        w = data.reshape(k, n).contiguous()
+        packed, scales, zp = ops.w4_quantize_pack(w, group_size, symmetric)
+        padded_k, groups = ops.w4_geometry(k, group_size)
+        return cls(k, n, padded_k, group_size, groups, packed, scales, zp)
+
+    @classmethod
+    def from_packed(cls, packed, scales, zp, k: int, group_size: int,
+                    g_idx: Optional[torch.Tensor] = None) -> "QuantizedTensor":
+        """Adopt pre-quantized arrays (AWQ/GPTQ style).  With ``g_idx`` the rows are sorted once
+        so that groups are contiguous (act-order)."""
+        padded_k, groups = ops.w4_geometry(k, group_size)
+        if packed.shape[0] * 8 != padded_k or scales.shape != (groups, packed.shape[1]):
+            raise ValueError("from_packed: array shapes do not match k / group_size")
+        perm = None
+        if g_idx is not None:
+            if k != padded_k:
+                raise ValueError("act-order needs k to be a multiple of group_size")
+            packed, perm = ops.w4_actorder_prepare(packed, g_idx, group_size)
+        return cls(k, packed.shape[1], padded_k, group_size, groups, packed, scales, zp, perm)
+
+
+class QLinear:
+    """Linear layer with frozen INT4 weights and optional bias (quant.rs:165-222)."""
+
+    def __init__(self, weight: QuantizedTensor, bias: Optional[torch.Tensor]):
+        self.weight = weight
+        self.bias = bias
+        self.in_features = weight.k
+        self.out_features = weight.n
+
+    @classmethod
+    def from_linear(cls, linear: Linear, group_size: int) -> "QLinear":
+        k, n = linear.weight.shape
+        return cls(QuantizedTensor.from_f32(linear.weight, k, n, group_size), linear.bias)
+
+    def forward(self, x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``y = x @ dequant(W) + bias`` in one launch (the reference runs a second add_bias pass)."""
+        w = self.weight
+        return ops.qmatmul_int4_perm(x, w.packed_tensor, w.scales_tensor, w.zp_tensor, w.k,
+                                     w.group_size, bias=self.bias, perm=w.perm, out=out)
+
+    def backward_input(self, grad_output: torch.Tensor) -> torch.Tensor:
+        """grad_x = grad_y @ dequant(W)^T (QLinearBackward, quant.rs:298-317)."""
+        w = self.weight
+        if w.perm is not None:
+            raise NotImplementedError("grad_x for act-order weights")
+        return ops.qmatmul_int4_t(grad_output, w.packed_tensor, w.scales_tensor, w.zp_tensor, w.k,
+                                  w.group_size)
+
+    __call__ = forward
+
+
+# ---- INT8, reference block format -----------------------------------------------
+
+@dataclass
+class Q8Tensor:
+    """A ``DType::Q8{block_size}`` tensor: fused header+data buffer, logical shape ``[K, N]``."""
+    buffer: torch.Tensor
+    shape: tuple
+    block_size: int
+
+    def numel(self) -> int:
+        return self.shape[0] * self.shape[1]
+
+
+def quantize(t, block_size: int) -> Q8Tensor:
+    """``Tensor::quantize`` (ops.rs:2290-2327): transpose the last two dims, then block-quantize."""
+    if isinstance(t, Q8Tensor):
+        raise ValueError("quantize: input is already quantized")
+    if block_size <= 0 or block_size % 4 != 0:
+        raise ValueError("quantize: block_size must be > 0 and divisible by 4")
+    if t.dim() != 2:
+        raise ValueError("quantize: tensor must be 2-D for column-major repacking")
+    tt = ops.transpose_f32(t.contiguous())
+    return Q8Tensor(ops.q8_quantize(tt.reshape(-1), block_size), tuple(t.shape), block_size)
+
+
+def dequantize(q: Q8Tensor) -> torch.Tensor:
+    """``Tensor::dequantize`` (ops.rs:2332-2357).  Like the reference, the values come back in
+    the transposed ``[N, K]`` order of the buffer under the original ``[K, N]`` shape."""
+    if not isinstance(q, Q8Tensor):
+        raise ValueError("dequantize: tensor is not Q8")
+    return ops.q8_dequantize(q.buffer, q.numel(), q.block_size).reshape(q.shape)
+
+
+def matmul(lhs: torch.Tensor, rhs) -> torch.Tensor:
+    """``Tensor::matmul`` with a Q8 right-hand side (ops.rs:516-545)."""
+    if isinstance(lhs, Q8Tensor):
+        raise ValueError("matmul: Q8 activations (lhs) not supported")
+    if not isinstance(rhs, Q8Tensor):
+        raise ValueError("matmul: this path handles Q8 weights only")
+    if lhs.dim() != 2 or lhs.shape[1] != rhs.shape[0]:
+        raise ValueError("matmul: inner dimension mismatch")
+    return ops.matmul_q8(lhs.contiguous(), rhs.buffer, rhs.shape[0], rhs.shape[1], rhs.block_size)
+
+
+def linear_forward(linear: Linear, x: torch.Tensor, weight_q8: Q8Tensor) -> torch.Tensor:
+    """``Linear::forward`` (nn/linear.rs:76-103) with the weight replaced by its Q8 form."""
+    out = matmul(x, weight_q8)
+    return ops.add_bias(out, linear.bias) if linear.bias is not None else out
+
+
+# ---- INT8, W8A8 -------------------------------------------------------------------
+
+class Int8Linear:
+    """Per-output-channel int8 weights, per-row dynamic int8 activations, i32 accumulate."""
+
+    def __init__(self, wq: torch.Tensor, sw: torch.Tensor, bias: Optional[torch.Tensor]):
+        self.wq, self.sw, self.bias = wq, sw, bias
+        self.out_features, self.in_features = wq.shape
+
+    @classmethod
+    def from_linear(cls, linear: Linear) -> "Int8Linear":
+        wq, sw = ops.i8_quantize_cols_t(linear.weight.contiguous())
+        return cls(wq, sw, linear.bias)
+
+    def forward(self, x: torch.Tensor, want_acc: bool = False):
+        xq, sx = ops.i8_quantize_rows(x.contiguous())
+        y, acc = ops.i8_gemm(xq, self.wq, sx, self.sw, self.bias, want_acc=want_acc)
+        return (y, acc) if want_acc else y
+
+    __call__ = forward

@@ -1,0 +1,190 @@
+"""Thin Python front end of the C ABI: one function per entry point.
+
+torch is used for device memory and streams only (``data_ptr()`` of CUDA/HIP
+tensors, ``torch.cuda.current_stream()``); every computation happens inside
+``librumus_hip.so``.  Shapes and dtypes are checked here because raw pointers
+carry none; numeric preconditions are checked by the library itself.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from ._lib import RumusError, call
+
+__all__ = [
+    "q8_buf_size", "q8_quantize", "q8_dequantize", "matmul_q8", "add_bias", "transpose_f32",
+    "i8_quantize_rows", "i8_quantize_cols_t", "i8_gemm", "w4_quantize_pack", "qmatmul_int4",
+    "qmatmul_int4_t", "w4_actorder_prepare", "qmatmul_int4_perm", "w4_geometry", "RumusError",
+]
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(t: torch.Tensor, dtype, name: str) -> int:
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise TypeError(f"{name}: expected a GPU tensor")
+    if t.dtype != dtype:
+        raise TypeError(f"{name}: expected {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name}: tensor must be contiguous")
+    return t.data_ptr()
+
+
+def _opt(t, dtype, name):
+    return None if t is None else _dev(t, dtype, name)
+
+
+def w4_geometry(k: int, group_size: int):
+    padded_k = ((k + group_size - 1) // group_size) * group_size
+    return padded_k, padded_k // group_size
+
+
+# ---- INT8, reference block format -------------------------------------------
+
+def q8_buf_size(numel: int, block_size: int) -> int:
+    return int(_lib.lib().rumus_hip_q8_buf_size(numel, block_size))
+
+
+def q8_quantize(flat: torch.Tensor, block_size: int) -> torch.Tensor:
+    """f32 [numel] -> Q8 buffer as int32 words (header word + bs/4 data words per block)."""
+    numel = flat.numel()
+    nbytes = q8_buf_size(numel, block_size) if block_size > 0 else 4
+    out = torch.empty(max(nbytes // 4, 1), dtype=torch.int32, device=flat.device)
+    call("rumus_hip_q8_quantize", _dev(flat, torch.float32, "in"), out.data_ptr(), numel,
+         block_size, _stream())
+    return out
+
+
+def q8_dequantize(words: torch.Tensor, numel: int, block_size: int) -> torch.Tensor:
+    out = torch.empty(numel, dtype=torch.float32, device=words.device)
+    call("rumus_hip_q8_dequantize", _dev(words, torch.int32, "in"), out.data_ptr(), numel,
+         block_size, _stream())
+    return out
+
+
+def matmul_q8(a: torch.Tensor, words: torch.Tensor, k: int, n: int, block_size: int) -> torch.Tensor:
+    m = a.shape[0]
+    if a.dim() != 2 or a.shape[1] != k:
+        raise ValueError("matmul: inner dimension mismatch")
+    c = torch.empty((m, n), dtype=torch.float32, device=a.device)
+    call("rumus_hip_matmul_q8", _dev(a, torch.float32, "a"), _dev(words, torch.int32, "b"),
+         c.data_ptr(), m, k, n, block_size, _stream())
+    return c
+
+
+def add_bias(mat: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    m, n = mat.shape
+    if bias.numel() != n:
+        raise ValueError("add_bias: bias length mismatch")
+    out = torch.empty_like(mat)
+    call("rumus_hip_add_bias", _dev(mat, torch.float32, "mat"), _dev(bias, torch.float32, "bias"),
+         out.data_ptr(), m, n, _stream())
+    return out
+
+
+def transpose_f32(t: torch.Tensor) -> torch.Tensor:
+    rows, cols = t.shape
+    out = torch.empty((cols, rows), dtype=torch.float32, device=t.device)
+    call("rumus_hip_transpose_f32", _dev(t, torch.float32, "in"), out.data_ptr(), rows, cols, _stream())
+    return out
+
+
+# ---- INT8, W8A8 ---------------------------------------------------------------
+
+def i8_quantize_rows(x: torch.Tensor):
+    rows, cols = x.shape
+    xq = torch.empty((rows, cols), dtype=torch.int8, device=x.device)
+    s = torch.empty(rows, dtype=torch.float32, device=x.device)
+    call("rumus_hip_i8_quantize_rows", _dev(x, torch.float32, "x"), xq.data_ptr(), s.data_ptr(),
+         rows, cols, _stream())
+    return xq, s
+
+
+def i8_quantize_cols_t(w: torch.Tensor):
+    """w [k,n] -> wq int8 [n,k], sw f32 [n]."""
+    k, n = w.shape
+    wq = torch.empty((n, k), dtype=torch.int8, device=w.device)
+    sw = torch.empty(n, dtype=torch.float32, device=w.device)
+    call("rumus_hip_i8_quantize_cols_t", _dev(w, torch.float32, "w"), wq.data_ptr(), sw.data_ptr(),
+         k, n, _stream())
+    return wq, sw
+
+
+def i8_gemm(xq, wq, sx=None, sw=None, bias=None, want_acc=False, want_y=True, out=None):
+    m, k = xq.shape
+    n = wq.shape[0]
+    if wq.shape[1] != k:
+        raise ValueError("i8_gemm: inner dimension mismatch")
+    acc = torch.empty((m, n), dtype=torch.int32, device=xq.device) if want_acc else None
+    y = None
+    if want_y:
+        y = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=xq.device)
+    call("rumus_hip_i8_gemm", _dev(xq, torch.int8, "xq"), _dev(wq, torch.int8, "wq"),
+         _opt(sx, torch.float32, "sx"), _opt(sw, torch.float32, "sw"), _opt(bias, torch.float32, "bias"),
+         None if acc is None else acc.data_ptr(), None if y is None else _dev(y, torch.float32, "y"),
+         m, k, n, _stream())
+    return y, acc
+
+
+# ---- INT4 -----------------------------------------------------------------------
+
+def w4_quantize_pack(w: torch.Tensor, group_size: int, symmetric: bool = False):
+    k, n = w.shape
+    gs = max(group_size, 1)
+    padded_k, groups = w4_geometry(k, gs)
+    packed = torch.empty((max(padded_k // 8, 1), n), dtype=torch.int32, device=w.device)
+    scales = torch.empty((groups, n), dtype=torch.float32, device=w.device)
+    zp = torch.empty((groups, n), dtype=torch.float32, device=w.device)
+    name = "rumus_hip_w4_quantize_pack_sym" if symmetric else "rumus_hip_w4_quantize_pack"
+    call(name, _dev(w, torch.float32, "w"), k, n, group_size, packed.data_ptr(), scales.data_ptr(),
+         zp.data_ptr(), _stream())
+    return packed, scales, zp
+
+
+def _w4_call(name, x, packed, scales, zp, bias, extra, k, group_size, out=None):
+    m = x.shape[0]
+    n = packed.shape[1]
+    if x.dim() != 2 or x.shape[1] != k:
+        raise ValueError("qmatmul_int4: x must be [m, k]")
+    padded_k, groups = w4_geometry(k, group_size) if group_size > 0 else (k, 0)
+    y = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=x.device)
+    call(name, _dev(x, torch.float32, "x"), _dev(packed, torch.int32, "packed"),
+         _dev(scales, torch.float32, "scales"), _dev(zp, torch.float32, "zero_points"),
+         _opt(bias, torch.float32, "bias"), _opt(extra, torch.int32, "g_idx/perm"),
+         _dev(y, torch.float32, "y"), m, k, n, padded_k, group_size, groups, _stream())
+    return y
+
+
+def qmatmul_int4(x, packed, scales, zp, k, group_size, bias=None, g_idx=None, out=None):
+    return _w4_call("rumus_hip_qmatmul_int4", x, packed, scales, zp, bias, g_idx, k, group_size, out)
+
+
+def qmatmul_int4_perm(x, packed_sorted, scales, zp, k, group_size, bias=None, perm=None, out=None):
+    return _w4_call("rumus_hip_qmatmul_int4_perm", x, packed_sorted, scales, zp, bias, perm, k,
+                    group_size, out)
+
+
+def qmatmul_int4_t(a, packed, scales, zp, k, group_size):
+    m, n = a.shape
+    if packed.shape[1] != n:
+        raise ValueError("qmatmul_int4_t: a must be [m, n]")
+    padded_k, groups = w4_geometry(k, group_size)
+    out = torch.empty((m, k), dtype=torch.float32, device=a.device)
+    call("rumus_hip_qmatmul_int4_t", _dev(a, torch.float32, "a"), _dev(packed, torch.int32, "packed"),
+         _dev(scales, torch.float32, "scales"), _dev(zp, torch.float32, "zero_points"),
+         out.data_ptr(), m, k, n, padded_k, group_size, groups, _stream())
+    return out
+
+
+def w4_actorder_prepare(packed, g_idx, group_size):
+    rows, n = packed.shape
+    padded_k = rows * 8
+    out = torch.empty_like(packed)
+    perm = torch.empty(padded_k, dtype=torch.int32, device=packed.device)
+    call("rumus_hip_w4_actorder_prepare", _dev(packed, torch.int32, "packed"),
+         _dev(g_idx, torch.int32, "g_idx"), padded_k, n, group_size, out.data_ptr(), perm.data_ptr(),
+         _stream())
+    return out, perm

@@ -1,0 +1,68 @@
+"""The C-ABI library loads without a GPU and exports exactly what the header declares."""
+import os
+import re
+import subprocess
+
+import pytest
+
+from rumus_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "rumus_hip.h")
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(rumus_hip_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def library():
+    if not os.path.exists(_lib.LIB_PATH):
+        _lib.build()
+    return _lib.lib()
+
+
+def test_header_and_binding_agree():
+    assert _declared() == sorted(_lib.PROTOTYPES)
+
+
+def test_every_declared_symbol_is_exported(library):
+    out = subprocess.check_output(["nm", "-D", "--defined-only", _lib.LIB_PATH], text=True)
+    exported = {line.split()[-1] for line in out.splitlines() if " T " in line}
+    missing = [s for s in _declared() if s not in exported]
+    assert not missing, missing
+    for name in _declared():
+        assert getattr(library, name) is not None
+
+
+def test_version_and_pure_host_entry_points(library):
+    assert library.rumus_hip_version().decode().endswith("gfx950")
+    # tensor/core.rs:87-98
+    assert library.rumus_hip_q8_buf_size(512 * 512, 512) == 512 * 516
+    assert library.rumus_hip_q8_buf_size(10, 4) == 24
+
+
+def test_preconditions_are_rejected_before_any_launch(library):
+    # null pointers are fine here: validation runs first and nothing is launched
+    rc = library.rumus_hip_q8_quantize(None, None, 16, 6, None)
+    assert rc == _lib.EINVAL and b"divisible by 4" in library.rumus_hip_last_error()
+    rc = library.rumus_hip_w4_quantize_pack(None, 16, 4, 12, None, None, None, None)
+    assert rc == _lib.EINVAL and b"multiple of 8" in library.rumus_hip_last_error()
+    rc = library.rumus_hip_qmatmul_int4(None, None, None, None, None, None, None,
+                                        1, 100, 4, 128, 64, 3, None)
+    assert rc == _lib.EINVAL and b"padded_k" in library.rumus_hip_last_error()
+    rc = library.rumus_hip_i8_gemm(None, None, None, None, None, None, None, 4, 24, 4, None)
+    assert rc == _lib.EINVAL
+    with pytest.raises(_lib.RumusError):
+        _lib.call("rumus_hip_matmul_q8", None, None, None, 1, 8, 1, 3, None)
+
+
+def test_product_package_does_not_touch_the_oracle():
+    pkg = os.path.join(ROOT, "rumus_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp", ".hpp")) or f == "Makefile":
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.replace("test oracle", ""), os.path.join(dirpath, f)

@@ -1,0 +1,203 @@
+"""GPU parity for the INT8 engine: reference Q8 block format and the W8A8 extension."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from rumus_amd import workloads
+
+from gpu_util import assert_close, dev, host, host_u32, say
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(__file__), "golden", "q8_kat.json")
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from rumus_amd import ops as o
+    return o
+
+
+def test_q8_quantize_known_answers(ops):
+    for case in json.load(open(GOLD))["cases"]:
+        say(f"q8_quantize KAT {case['name']}")
+        x = np.array(case["x"], np.float32)
+        words = host_u32(ops.q8_quantize(dev(x), case["block_size"]))
+        assert f"{words[0]:08x}" == case["header_hex"]
+        assert words[1:].view(np.int8).tolist() == case["q"]
+        xq, s = ops.i8_quantize_rows(dev(x.reshape(1, -1)))
+        assert host(xq)[0].tolist() == case["q"]
+
+
+@pytest.mark.parametrize("numel,bs", [(64 * 5 + 20, 64), (512 * 512, 512), (4096 * 24, 4096),
+                                      (1000, 8), (36, 4)])
+def test_q8_quantize_dequantize_bit_exact(ops, numel, bs):
+    say(f"q8 quantize/dequantize numel={numel} bs={bs}")
+    rng = np.random.default_rng(numel + bs)
+    x = rng.normal(0, 0.02, numel).astype(np.float32)
+    x[: min(bs, numel) // 2] *= 50
+    if numel > 3 * bs:
+        x[2 * bs: 3 * bs] = 0.0          # an all-zero block
+    want = oracle.q8_quantize(x, bs)
+    got = ops.q8_quantize(dev(x), bs)
+    assert got.numel() * 4 == ops.q8_buf_size(numel, bs) == oracle.q8_buf_size(numel, bs)
+    np.testing.assert_array_equal(host_u32(got), want)
+    np.testing.assert_array_equal(host(ops.q8_dequantize(got, numel, bs)),
+                                  oracle.q8_dequantize(want, numel, bs))
+
+
+def test_q8_rejects_bad_block_size(ops):
+    say("q8 bad block size")
+    with pytest.raises(ops.RumusError):
+        ops.q8_quantize(dev(np.zeros(16, np.float32)), 6)
+    with pytest.raises(ops.RumusError):
+        ops.q8_quantize(dev(np.zeros(16, np.float32)), 0)
+
+
+@pytest.mark.parametrize("m,k,n,bs", [(32, 512, 512, 512), (4, 64, 10, 64), (3, 96, 7, 32),
+                                      (2, 40, 5, 8), (70, 256, 130, 128), (5, 100, 9, 20)])
+def test_matmul_q8_vs_oracle(ops, m, k, n, bs):
+    say(f"matmul_q8 m={m} k={k} n={n} bs={bs}")
+    from rumus_amd import nn
+    rng = np.random.default_rng(m + k + n)
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    a = rng.normal(0, 1, (m, k)).astype(np.float32)
+    b = rng.normal(0, 0.01, n).astype(np.float32)
+    words = oracle.tensor_quantize(w, bs)
+    wq = nn.quantize(dev(w), bs)                       # transpose + quantize on the GPU
+    np.testing.assert_array_equal(host_u32(wq.buffer), words)
+    want = oracle.add_bias(oracle.matmul_q8(a, words, k, n, bs, threads=8), b)
+    got = host(nn.linear_forward(nn.Linear(dev(w), dev(b)), dev(a), wq))
+    assert_close(got, want)
+    # Tensor::dequantize returns the buffer order ([N,K]) under the [K,N] shape
+    deq = host(nn.dequantize(wq))
+    np.testing.assert_array_equal(deq.reshape(-1), oracle.q8_dequantize(words, k * n, bs))
+
+
+def test_matmul_q8_naive_kernel_is_bit_exact(ops):
+    # block_size % 16 != 0 routes to the one-thread-per-output kernel (the reference's loop)
+    say("matmul_q8 naive kernel bit-exact")
+    rng = np.random.default_rng(5)
+    m, k, n, bs = 5, 100, 9, 20
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    a = rng.normal(0, 1, (m, k)).astype(np.float32)
+    words = oracle.tensor_quantize(w, bs)
+    got = host(ops.matmul_q8(dev(a), dev(words), k, n, bs))
+    np.testing.assert_array_equal(got, oracle.matmul_q8(a, words, k, n, bs))
+
+
+def test_api_errors_mirror_reference_asserts(ops):
+    say("module-level asserts")
+    from rumus_amd import nn
+    w = dev(np.zeros((8, 8), np.float32))
+    q = nn.quantize(w, 8)
+    with pytest.raises(ValueError):
+        nn.quantize(q, 8)                       # already quantized (ops.rs:2292)
+    with pytest.raises(ValueError):
+        nn.quantize(w, 6)                       # block_size % 4 (ops.rs:2291)
+    with pytest.raises(ValueError):
+        nn.matmul(q, q)                         # Q8 lhs (ops.rs:519)
+    with pytest.raises(ValueError):
+        nn.matmul(dev(np.zeros((2, 4), np.float32)), q)   # inner dim (ops.rs:523)
+
+
+# ---- W8A8 extension -------------------------------------------------------------
+
+@pytest.mark.parametrize("rows,cols", [(32, 512), (7, 100), (3, 4096), (1, 5), (130, 1024)])
+def test_i8_quantize_rows_bit_exact(ops, rows, cols):
+    say(f"i8_quantize_rows {rows}x{cols}")
+    rng = np.random.default_rng(rows * cols)
+    x = rng.normal(0, 1, (rows, cols)).astype(np.float32)
+    if rows > 2:
+        x[1] = 0.0
+    wq, ws = oracle.i8_quantize_rows(x)
+    xq, s = ops.i8_quantize_rows(dev(x))
+    np.testing.assert_array_equal(host(xq), wq)
+    np.testing.assert_array_equal(host(s), ws)
+
+
+@pytest.mark.parametrize("k,n", [(512, 512), (100, 37), (4096, 200), (64, 1)])
+def test_i8_quantize_cols_t_bit_exact(ops, k, n):
+    say(f"i8_quantize_cols_t k={k} n={n}")
+    rng = np.random.default_rng(k + n)
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    if n > 3:
+        w[:, 2] = 0.0
+    want_q, want_s = oracle.i8_quantize_rows(np.ascontiguousarray(w.T))
+    wq, sw = ops.i8_quantize_cols_t(dev(w))
+    np.testing.assert_array_equal(host(wq), want_q)
+    np.testing.assert_array_equal(host(sw), want_s)
+
+
+@pytest.mark.parametrize("m,k,n", [(32, 512, 512), (1, 16, 1), (77, 208, 133), (256, 1024, 384),
+                                   (300, 4096, 260), (2048, 256, 2304)])
+def test_i8_gemm_accumulators_bit_exact(ops, m, k, n):
+    say(f"i8_gemm m={m} k={k} n={n}")
+    rng = np.random.default_rng(m + k + n)
+    xq = rng.integers(-127, 128, (m, k)).astype(np.int8)
+    wq = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    sx = rng.uniform(0.001, 0.05, m).astype(np.float32)
+    sw = rng.uniform(0.0001, 0.001, n).astype(np.float32)
+    b = rng.normal(0, 0.01, n).astype(np.float32)
+    want_acc = oracle.i8_gemm_i32(xq, wq, threads=8)
+    y, acc = ops.i8_gemm(dev(xq), dev(wq), dev(sx), dev(sw), dev(b), want_acc=True)
+    np.testing.assert_array_equal(host(acc), want_acc)
+    # the epilogue uses the oracle's association, so it is bit-exact too
+    np.testing.assert_array_equal(host(y), oracle.i8_rescale_bias(want_acc, sx, sw, b))
+    y2, _ = ops.i8_gemm(dev(xq), dev(wq), dev(sx), dev(sw), None)
+    np.testing.assert_array_equal(host(y2), oracle.i8_rescale_bias(want_acc, sx, sw, None))
+    _, acc_only = ops.i8_gemm(dev(xq), dev(wq), want_acc=True, want_y=False)
+    np.testing.assert_array_equal(host(acc_only), want_acc)
+
+
+def test_i8_gemm_extreme_values(ops):
+    say("i8_gemm extremes")
+    m, k, n = 64, 4096, 64
+    xq = np.full((m, k), 127, np.int8)
+    wq = np.full((n, k), -128, np.int8)
+    wq[::2] = 127
+    _, acc = ops.i8_gemm(dev(xq), dev(wq), want_acc=True, want_y=False)
+    want = xq.astype(np.int64) @ wq.astype(np.int64).T
+    np.testing.assert_array_equal(host(acc), want)
+
+
+def test_int8_quantlinear_config(ops):
+    # BASELINE config 0: W [512,512] N(0,0.02), X [32,512] N(0,1), b N(0,0.01), seed 0
+    say("Int8Linear 32x512x512 seed 0")
+    from rumus_amd import nn
+    w, x, b = workloads.int8_linear(0)
+    want_y, want_acc, (xq, sx, wq, sw) = oracle.i8_linear(x, w, b)
+    layer = nn.Int8Linear.from_linear(nn.Linear(dev(w), dev(b)))
+    np.testing.assert_array_equal(host(layer.wq), wq)
+    np.testing.assert_array_equal(host(layer.sw), sw)
+    y, acc = layer.forward(dev(x), want_acc=True)
+    np.testing.assert_array_equal(host(acc), want_acc)
+    assert_close(host(y), want_y)
+
+
+def test_i8_gemm_prefill_shape_properties(ops):
+    # BASELINE config 3 at full size: 2048 x 4096 x 11008.  The oracle checks a
+    # sample of rows exactly; the rest is pinned by a row/column checksum
+    # identity computed in int64 on the host.
+    say("i8_gemm 2048x4096x11008")
+    x, w = workloads.int8_gemm(0)
+    xq_t, sx_t = ops.i8_quantize_rows(dev(x))
+    wq_t, sw_t = ops.i8_quantize_cols_t(dev(w))
+    xq, wq = host(xq_t), host(wq_t)
+    rows = [0, 1, 777, 2047]
+    wq_o, sw_o = oracle.i8_quantize_rows(np.ascontiguousarray(w.T[:64]))
+    np.testing.assert_array_equal(wq[:64], wq_o)
+    xq_o, sx_o = oracle.i8_quantize_rows(x[rows])
+    np.testing.assert_array_equal(xq[rows], xq_o)
+    y, acc = ops.i8_gemm(xq_t, wq_t, sx_t, sw_t, None, want_acc=True)
+    acc = host(acc)
+    np.testing.assert_array_equal(acc[rows], oracle.i8_gemm_i32(xq[rows], wq, threads=8))
+    # checksum of checksums: sum_m acc[m,:] == (sum_m xq[m,:]) @ wq^T, and the same by columns
+    np.testing.assert_array_equal(acc.sum(0, dtype=np.int64),
+                                  xq.sum(0, dtype=np.int64) @ wq.astype(np.int64).T)
+    np.testing.assert_array_equal(acc.sum(1, dtype=np.int64),
+                                  xq.astype(np.int64) @ wq.sum(0, dtype=np.int64))
+    yh = host(y)
+    np.testing.assert_array_equal(yh[rows], oracle.i8_rescale_bias(acc[rows], host(sx_t)[rows], host(sw_t), None))

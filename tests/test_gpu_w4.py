@@ -1,0 +1,210 @@
+"""GPU parity for the INT4 engine, through the C ABI (rumus_amd.ops -> librumus_hip.so)."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from rumus_amd import workloads
+
+from gpu_util import assert_close, dev, host, host_u32, say
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(__file__), "golden", "w4_kat.json")
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from rumus_amd import ops as o
+    return o
+
+
+def test_quantize_pack_known_answers(ops):
+    for case in json.load(open(GOLD))["cases"]:
+        say(f"w4_quantize_pack KAT {case['name']}")
+        w = np.array(case["w"], np.float32).reshape(case["k"], case["n"])
+        packed, scales, zp = ops.w4_quantize_pack(dev(w), case["group_size"])
+        assert [f"{v:08x}" for v in host_u32(packed).reshape(-1)] == case["packed_hex"]
+        np.testing.assert_array_equal(host(scales).reshape(-1), np.array(case["scales"], np.float32))
+        np.testing.assert_array_equal(host(zp).reshape(-1), np.array(case["zp"], np.float32))
+
+
+@pytest.mark.parametrize("k,n,g,sym", [(256, 48, 64, False), (200, 17, 64, False), (4096, 512, 128, False),
+                                       (512, 300, 128, True), (72, 5, 8, True)])
+def test_quantize_pack_bit_exact(ops, k, n, g, sym):
+    say(f"w4_quantize_pack k={k} n={n} g={g} sym={sym}")
+    rng = np.random.default_rng(k * 7 + n)
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    w[:: max(k // 5, 1), :: max(n // 3, 1)] = 0.0
+    if not sym and k >= 128:
+        w[64:128, 0] = 0.02   # a constant group: range <= 1e-10 branch
+    pw, sw_, zw = oracle.w4_from_f32(w, g, symmetric=sym)
+    packed, scales, zp = ops.w4_quantize_pack(dev(w), g, symmetric=sym)
+    np.testing.assert_array_equal(host_u32(packed), pw)
+    np.testing.assert_array_equal(host(scales), sw_)
+    np.testing.assert_array_equal(host(zp), zw)
+
+
+def test_quantize_pack_rejects_bad_group(ops):
+    say("w4_quantize_pack group_size=12")
+    with pytest.raises(ops.RumusError):
+        ops.w4_quantize_pack(dev(np.zeros((24, 4), np.float32)), 12)
+
+
+SHAPES = [
+    # m, k, n, g, bias
+    (1, 256, 64, 128, False),     # gemv, one pass
+    (1, 4096, 4096, 128, True),   # the headline decode shape
+    (3, 1000, 52, 64, True),      # K tail (1000 -> 1024), n % 16 != 0
+    (8, 512, 20, 8, False),       # smallest group, ragged columns
+    (1, 128, 10, 32, True),       # n % 4 != 0 -> reference-order kernel
+    (5, 72, 7, 8, False),         # reference-order kernel, odd everything
+    (16, 512, 256, 128, True),    # m > 8
+    (33, 384, 96, 64, False),
+]
+
+
+@pytest.mark.parametrize("m,k,n,g,with_bias", SHAPES)
+def test_qmatmul_int4_vs_oracle(ops, m, k, n, g, with_bias):
+    say(f"qmatmul_int4 m={m} k={k} n={n} g={g} bias={with_bias}")
+    rng = np.random.default_rng(m * 131 + k + n)
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    x = rng.normal(0, 1, (m, k)).astype(np.float32)
+    b = rng.normal(0, 0.01, n).astype(np.float32) if with_bias else None
+    packed, scales, zp = oracle.w4_from_f32(w, g)
+    want = oracle.qmatmul_int4(x, packed, scales, zp, k, g, bias=b, threads=8)
+    got = host(ops.qmatmul_int4(dev(x), dev(packed), dev(scales), dev(zp), k, g,
+                                bias=None if b is None else dev(b)))
+    assert_close(got, want)
+
+
+def test_reference_order_kernel_is_bit_exact(ops):
+    # n % 4 != 0 routes to the one-thread-per-column kernel, which performs the oracle's
+    # operations in the oracle's order: equality, not tolerance.
+    say("qmatmul_int4 reference-order kernel bit-exact")
+    rng = np.random.default_rng(17)
+    m, k, n, g = 6, 200, 37, 8
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    x = rng.normal(0, 1, (m, k)).astype(np.float32)
+    b = rng.normal(0, 0.01, n).astype(np.float32)
+    packed, scales, zp = oracle.w4_from_f32(w, g)
+    want = oracle.qmatmul_int4(x, packed, scales, zp, k, g, bias=b)
+    got = host(ops.qmatmul_int4(dev(x), dev(packed), dev(scales), dev(zp), k, g, bias=dev(b)))
+    np.testing.assert_array_equal(got, want)
+
+
+def test_qmatmul_int4_exact_integer_case(ops):
+    say("qmatmul_int4 integer special case")
+    rng = np.random.default_rng(3)
+    for m, k, n, g in [(1, 256, 64, 32), (16, 256, 64, 32)]:
+        q = rng.integers(0, 16, (k, n)).astype(np.uint32)
+        packed = np.zeros((k // 8, n), np.uint32)
+        for r in range(k):
+            packed[r // 8] |= q[r] << np.uint32(4 * (r % 8))
+        scales = np.ones((k // g, n), np.float32)
+        zp = np.zeros((k // g, n), np.float32)
+        x = rng.integers(-8, 9, (m, k)).astype(np.float32)
+        got = host(ops.qmatmul_int4(dev(x), dev(packed), dev(scales), dev(zp), k, g))
+        np.testing.assert_array_equal(got.astype(np.int64), x.astype(np.int64) @ q.astype(np.int64))
+
+
+def test_gemv_rows_match_gemm_rows_and_linearity(ops):
+    say("qmatmul_int4 row independence / linearity")
+    w, x = workloads.w4_gemv(1, m=4, k=1024, n=256)
+    packed, scales, zp = oracle.w4_from_f32(w, 128)
+    d = [dev(a) for a in (packed, scales, zp)]
+    y4 = host(ops.qmatmul_int4(dev(x), *d, 1024, 128))
+    y1 = host(ops.qmatmul_int4(dev(x[2:3]), *d, 1024, 128))
+    assert_close(y1[0], y4[2])
+    ysum = host(ops.qmatmul_int4(dev((x[0:1] + 2 * x[1:2]).astype(np.float32)), *d, 1024, 128))
+    assert_close(ysum[0], y4[0] + 2 * y4[1])
+
+
+@pytest.mark.parametrize("m", [1, 4, 16])
+def test_act_order(ops, m):
+    say(f"act-order m={m}")
+    k, n, g = 512, 128, 128
+    w, g_idx, x = workloads.w4_gemm_actorder(2, m=m, k=k, n=n, group_size=g)
+    # symmetric zp=8 quantization of the rows as grouped by g_idx
+    order = np.argsort(g_idx, kind="stable")
+    ps, ss, zs = oracle.w4_from_f32(w[order], g, symmetric=True)     # sorted layout
+    q_sorted = oracle.w4_unpack(ps, k)
+    q = np.empty_like(q_sorted)
+    q[order] = q_sorted                                             # original row order
+    packed = np.zeros((k // 8, n), np.uint32)
+    for r in range(k):
+        packed[r // 8] |= q[r].astype(np.uint32) << np.uint32(4 * (r % 8))
+    want = oracle.qmatmul_int4(x, packed, ss, zs, k, g, g_idx=g_idx, threads=8)
+    # (a) g_idx passed straight to the reference-order kernel: bit-exact
+    got_direct = host(ops.qmatmul_int4(dev(x), dev(packed), dev(ss), dev(zs), k, g, g_idx=dev(g_idx)))
+    np.testing.assert_array_equal(got_direct, want)
+    # (b) prepared once, then the fast kernels with a permuted activation gather
+    p_sorted, perm = ops.w4_actorder_prepare(dev(packed), dev(g_idx), g)
+    np.testing.assert_array_equal(host(perm), order.astype(np.int32))
+    np.testing.assert_array_equal(host_u32(p_sorted), ps)
+    got = host(ops.qmatmul_int4_perm(dev(x), p_sorted, dev(ss), dev(zs), k, g, perm=perm))
+    assert_close(got, want)
+    # (c) the trivial map reproduces the plain kernel bit for bit
+    trivial = (np.arange(k) // g).astype(np.int32)
+    pt, permt = ops.w4_actorder_prepare(dev(ps), dev(trivial), g)
+    np.testing.assert_array_equal(host(permt), np.arange(k, dtype=np.int32))
+    a = host(ops.qmatmul_int4_perm(dev(x), pt, dev(ss), dev(zs), k, g, perm=permt))
+    b = host(ops.qmatmul_int4(dev(x), dev(ps), dev(ss), dev(zs), k, g))
+    np.testing.assert_array_equal(a, b)
+
+
+def test_act_order_rejects_unbalanced_groups(ops):
+    say("act-order unbalanced g_idx")
+    k, n, g = 64, 8, 32
+    bad = np.zeros(k, np.int32)
+    with pytest.raises(ops.RumusError):
+        ops.w4_actorder_prepare(dev(np.zeros((k // 8, n), np.uint32)), dev(bad), g)
+
+
+@pytest.mark.parametrize("m,k,n,g", [(3, 72, 20, 8), (16, 512, 300, 128), (1, 1000, 64, 64)])
+def test_qmatmul_int4_transpose(ops, m, k, n, g):
+    say(f"qmatmul_int4_t m={m} k={k} n={n} g={g}")
+    rng = np.random.default_rng(k + n)
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    gy = rng.normal(0, 1, (m, n)).astype(np.float32)
+    packed, scales, zp = oracle.w4_from_f32(w, g)
+    want = oracle.qmatmul_int4_t(gy, packed, scales, zp, k, g, threads=8)
+    got = host(ops.qmatmul_int4_t(dev(gy), dev(packed), dev(scales), dev(zp), k, g))
+    assert got.shape == (m, k)
+    assert_close(got, want)
+
+
+def test_qlinear_module_mirror(ops):
+    say("QLinear.from_linear / forward")
+    from rumus_amd import nn
+    rng = np.random.default_rng(21)
+    k, n, m, g = 512, 256, 4, 128
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    b = rng.normal(0, 0.01, n).astype(np.float32)
+    x = rng.normal(0, 1, (m, k)).astype(np.float32)
+    ql = nn.QLinear.from_linear(nn.Linear(dev(w), dev(b)), g)
+    assert (ql.in_features, ql.out_features) == (k, n)
+    assert (ql.weight.padded_k, ql.weight.num_groups) == (512, 4)
+    packed, scales, zp = oracle.w4_from_f32(w, g)
+    np.testing.assert_array_equal(host_u32(ql.weight.packed_tensor), packed)
+    assert_close(host(ql.forward(dev(x))), oracle.qmatmul_int4(x, packed, scales, zp, k, g, bias=b))
+    gy = rng.normal(0, 1, (m, n)).astype(np.float32)
+    assert_close(host(ql.backward_input(dev(gy))), oracle.qmatmul_int4_t(gy, packed, scales, zp, k, g))
+    with pytest.raises(ValueError):
+        nn.QuantizedTensor.from_f32(dev(w), k, n, 12)
+
+
+def test_headline_shape_properties(ops):
+    # full BASELINE size: compare with the oracle (all host cores) and check linearity
+    say("w4 gemv 1x4096x4096 g128 full size")
+    w, x = workloads.w4_gemv(0)
+    pw, sw_, zw = oracle.w4_from_f32(w, 128)
+    packed, scales, zp = ops.w4_quantize_pack(dev(w), 128)
+    np.testing.assert_array_equal(host_u32(packed), pw)
+    np.testing.assert_array_equal(host(scales), sw_)
+    np.testing.assert_array_equal(host(zp), zw)
+    y = host(ops.qmatmul_int4(dev(x), packed, scales, zp, 4096, 128))
+    assert_close(y, oracle.qmatmul_int4(x, pw, sw_, zw, 4096, 128, threads=8))
+    y2 = host(ops.qmatmul_int4(dev((-0.5 * x).astype(np.float32)), packed, scales, zp, 4096, 128))
+    assert_close(y2, -0.5 * y)
