@@ -28,6 +28,11 @@ int w4_launch_generic(const W4Args& a, hipStream_t s);
 bool w4_gemv_supported(const W4Args& a);
 int w4_launch_gemv(const W4Args& a, hipStream_t s);
 
+// Decode kernel on v_dot8_u32_u4 (m <= 8, group_size % 64 == 0, n % 4 == 0,
+// 16-byte aligned buffers, no g_idx); preferred over the f32 bandwidth kernel.
+bool w4_gemv_dot8_supported(const W4Args& a);
+int w4_launch_gemv_dot8(const W4Args& a, hipStream_t s);
+
 // f16 MFMA kernel for larger m (needs group_size % 32 == 0, n % 4 == 0,
 // 16-byte aligned buffers, no g_idx).
 bool w4_gemm_supported(const W4Args& a);

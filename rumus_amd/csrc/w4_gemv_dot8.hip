@@ -1,0 +1,304 @@
+// INT4 engine: the decode-shape kernel (m <= 8, group_size % (8*OCT) == 0).
+//
+// At 1 x 4096 x 4096 the whole problem is 9.4 MB: the launch lasts a few
+// microseconds and is bound by latencies (dispatch, first byte from HBM) as
+// much as by bandwidth.  Everything below is arranged to put all weight loads
+// in flight at once, as early as possible, and to keep the dependent chain
+// that follows their arrival short: no LDS staging and no barrier before the
+// arithmetic.
+//
+// Data movement.  A workgroup owns 16 adjacent columns over the whole of K (no
+// partial sums cross workgroups: no atomics, no zero-fill, deterministic).
+// The four lanes of a quad cover the 16 columns with one 128-bit load each
+// (4 words = 4 columns x 8 rows); each quad is one "row lane" and owns OCT
+// consecutive packed word rows (a chunk of 8*OCT rows) per sweep.  A word row
+// is a 64-byte segment per workgroup; the XCD-contiguous workgroup order puts
+// the reader of the other half of each 128-byte line on the same L2.
+//
+// Arithmetic.  A packed word is 8 unsigned nibbles: exactly one operand of
+// v_dot8_u32_u4.  The activations of a chunk are turned into 20-bit fixed
+// point, X' = rint(x * f) + 2^19 (f a power of two from the chunk's abs-max),
+// and split into five nibble planes laid out like the weights, so that
+//   sum_j X'_j q_j = sum_i 16^i * dot8(word, plane_i)
+// is exact integer arithmetic with no unpacking at all; the 2^19 offset is
+// removed with dot8(word, 0x11111111) = sum_j q_j.  One conversion to f32 per
+// (chunk, column) follows, then  y += scale * (part - zp * sum_j x_j).
+// The planes never touch memory: the four lanes of a quad each build the
+// planes of OCT/4 word rows of their own chunk and exchange them with DPP
+// quad broadcasts.  Quantizing x to 20 bits relative to the abs-max of its
+// chunk costs < 2^-19 relative error per activation, two orders below the f32
+// tolerance of this path (rel 1e-3 / abs 1e-4).
+#include "w4.h"
+
+namespace rumus {
+
+constexpr int kD8Cols = 16;  // columns per workgroup
+
+__device__ __forceinline__ uint32_t udot8(uint32_t a, uint32_t b, uint32_t c) {
+    return __builtin_amdgcn_udot8(a, b, c, false);
+}
+
+// DPP lane exchanges (one VALU op each, no LDS round trip).
+#define RUMUS_DPP_F(v, ctrl) \
+    __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, (v)), (ctrl), 0xF, 0xF, true))
+#define RUMUS_DPP_I(v, ctrl) __builtin_amdgcn_update_dpp(0, (int)(v), (ctrl), 0xF, 0xF, true)
+constexpr int kDppXor1 = 0xB1;   // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;   // quad_perm [2,3,0,1]
+constexpr int kDppRowShr4 = 0x114, kDppRowShr8 = 0x118;
+
+// value of quad lane Q in all four lanes of the quad
+template <int Q> __device__ __forceinline__ uint32_t quad_bcast(uint32_t v) {
+    return (uint32_t)RUMUS_DPP_I(v, Q * 0x55);
+}
+
+// Sum across the 16 quads of a wave (lanes that share lane & 3).
+// Valid in lanes 12..15 afterwards.
+__device__ __forceinline__ float reduce_row_lanes(float v) {
+    v += RUMUS_DPP_F(v, kDppRowShr4);   // out-of-row reads give 0
+    v += RUMUS_DPP_F(v, kDppRowShr8);
+    v += __shfl_xor(v, 16);
+    v += __shfl_xor(v, 32);
+    return v;
+}
+
+// Kernel arguments are passed flat, hottest first: the first 16 dwords are
+// preloaded into SGPRs by the command processor (see the build flags), which
+// takes the kernel-argument fetch off the critical path.
+//
+// T threads = T/4 quads; a quad owns OCT consecutive word rows per sweep and
+// each of its lanes prepares OPL = OCT/4 of them.  FASTX: activations are
+// read with 128-bit loads (no perm, k % 8 == 0, 16-byte aligned x).
+template <int M, int T, int OCT, bool FASTX>
+__global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
+    const uint32_t* __restrict__ packed, const float* __restrict__ scales,
+    const float* __restrict__ zps, const float* __restrict__ xin, float* __restrict__ yout,
+    uint32_t n, uint32_t k, uint32_t padded_k, uint32_t group_size,
+    const float* __restrict__ bias, const int32_t* __restrict__ perm) {
+    static_assert(OCT == 4 || OCT == 8, "a quad shares 4 or 8 word rows");
+    constexpr int RL = T / 4;      // quads per workgroup
+    constexpr int WAVES = T / 64;
+    constexpr int OPL = OCT / 4;   // word rows prepared per lane
+    __shared__ float red[WAVES][M][kD8Cols];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t nchunks = padded_k / (8 * OCT);
+
+    // the grid size is recomputed from n: reading gridDim would cost a kernel-argument fetch
+    const uint32_t cchunk = xcd_contiguous(blockIdx.x, (n + kD8Cols - 1) / kD8Cols);
+    const uint32_t cq = tid & 3, rs = tid >> 2;
+    const uint32_t col = cchunk * kD8Cols + 4 * cq;
+    const bool col_ok = col < n;  // n % 4 == 0: a lane's four columns are all in or all out
+    const uint32_t col_c = col_ok ? col : 0;
+
+    float acc[M][4];
+#pragma unroll
+    for (int m = 0; m < M; m++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) acc[m][c] = 0.0f;
+
+    // every quad runs the same number of sweeps; a dead quad carries scale 0
+    for (uint32_t base = 0; base < nchunks; base += RL) {
+        const uint32_t chunk = base + rs;
+        const bool live = chunk < nchunks;
+        const uint32_t ch = live ? chunk : 0;
+
+        // ---- 1. loads, in the order their data is needed -----------------------
+        // The memory counter retires in order, so the activation loads go first:
+        // the nibble planes are then built while the weight loads are in flight.
+        // Branch-free (clamped addresses, values zeroed by select) so that the
+        // wait before the plane build covers x only.
+        float xv[M][OPL][8];
+        const uint32_t k0 = (ch * OCT + cq * OPL) * 8;   // first row this lane prepares
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+#pragma unroll
+            for (int t = 0; t < OPL; t++) {
+                const uint32_t kt = k0 + 8 * t;
+                if (FASTX) {
+                    const bool in = kt < k;              // k % 8 == 0: all 8 in or out
+                    const uint32_t kc = in ? kt : 0;
+                    const float4 lo = *reinterpret_cast<const float4*>(xin + (uint64_t)m * k + kc);
+                    const float4 hi = *reinterpret_cast<const float4*>(xin + (uint64_t)m * k + kc + 4);
+                    xv[m][t][0] = in ? lo.x : 0.0f; xv[m][t][1] = in ? lo.y : 0.0f;
+                    xv[m][t][2] = in ? lo.z : 0.0f; xv[m][t][3] = in ? lo.w : 0.0f;
+                    xv[m][t][4] = in ? hi.x : 0.0f; xv[m][t][5] = in ? hi.y : 0.0f;
+                    xv[m][t][6] = in ? hi.z : 0.0f; xv[m][t][7] = in ? hi.w : 0.0f;
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 8; j++) {
+                        const bool in = kt + j < k;
+                        const uint32_t kk = in ? kt + j : 0;
+                        const uint32_t src = perm ? (uint32_t)perm[kk] : kk;
+                        const float v = xin[(uint64_t)m * k + src];
+                        xv[m][t][j] = in ? v : 0.0f;
+                    }
+                }
+            }
+        }
+        uint4 w[OCT];
+        const uint32_t* p = packed + (uint64_t)ch * OCT * n + col_c;
+#pragma unroll
+        for (int u = 0; u < OCT; u++) w[u] = *reinterpret_cast<const uint4*>(p + (uint64_t)u * n);
+        const uint32_t g = (ch * 8 * OCT) / group_size;
+        float4 sc = *reinterpret_cast<const float4*>(scales + (uint64_t)g * n + col_c);
+        const float4 zp = *reinterpret_cast<const float4*>(zps + (uint64_t)g * n + col_c);
+        if (!(live && col_ok)) sc = make_float4(0, 0, 0, 0);
+
+        uint32_t wv[OCT][4];
+#pragma unroll
+        for (int u = 0; u < OCT; u++) { wv[u][0] = w[u].x; wv[u][1] = w[u].y; wv[u][2] = w[u].z; wv[u][3] = w[u].w; }
+        const float scv[4] = {sc.x, sc.y, sc.z, sc.w};
+        const float zv[4] = {zp.x, zp.y, zp.z, zp.w};
+
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            // ---- 2. activations of the chunk -> nibble planes (registers) -----
+            float amax = 0.0f;
+#pragma unroll
+            for (int t = 0; t < OPL; t++)
+#pragma unroll
+                for (int j = 0; j < 8; j++) amax = fmaxf(amax, fabsf(xv[m][t][j]));
+            amax = fmaxf(amax, RUMUS_DPP_F(amax, kDppXor1));
+            amax = fmaxf(amax, RUMUS_DPP_F(amax, kDppXor2));
+            // amax = a * 2^E (1 <= a < 2): scale by just under 2^(18-E) so that |x * f| < 2^19 - 1/2
+            const uint32_t ebits = __float_as_uint(amax) >> 23;   // biased exponent (amax >= 0)
+            // the factor 1 - 2^-20 keeps rint(amax * f) at 2^19 - 1 or below
+            float f = __uint_as_float((272u - ebits) << 23) * 0.99999905f;
+            float finv = __uint_as_float((ebits - 18u) << 23) * 1.00000095f;
+            if (ebits < 19) {              // zero or below 2^-108: contributes nothing
+                f = 0.0f;
+                finv = 0.0f;
+            }
+            if (ebits == 255) {            // inf / nan in the chunk: poison the result
+                f = 0.0f;
+                finv = __uint_as_float(0x7FC00000u);
+            }
+            uint32_t own[OPL][5];
+            int xsum = 0;
+#pragma unroll
+            for (int t = 0; t < OPL; t++) {
+                // adding 1.5*2^23 + 2^19 leaves rint(x*f) + 2^19 in the low 20 mantissa bits
+                uint32_t X[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) X[j] = __float_as_uint(fmaf(xv[m][t][j], f, 13107200.0f));
+                // plane i, nibble j = digit i of X[j]
+                uint32_t ze[4], zo[4];
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const uint32_t A = X[2 * q], B = X[2 * q + 1];
+                    ze[q] = (A & 0x0F0F0Fu) | ((B & 0x0F0F0Fu) << 4);   // bytes: digits 0,2,4 of (B,A)
+                    zo[q] = ((A >> 4) & 0x0F0Fu) | (B & 0xF0F0u);       // bytes: digits 1,3 of (B,A)
+                }
+#pragma unroll
+                for (int i = 0; i < 5; i++) {
+                    const uint32_t* z = (i & 1) ? zo : ze;
+                    const int sh = 8 * (i >> 1);
+                    own[t][i] = ((z[0] >> sh) & 0xFFu) | (((z[1] >> sh) & 0xFFu) << 8) |
+                                (((z[2] >> sh) & 0xFFu) << 16) | (((z[3] >> sh) & 0xFFu) << 24);
+                }
+                // sum_j X'_j from the planes, offsets removed: exact integer
+                uint32_t s = 0;
+#pragma unroll
+                for (int i = 4; i >= 0; i--) s = s * 16u + udot8(own[t][i], 0x11111111u, 0u);
+                xsum += (int)s - 8 * (1 << 19);
+            }
+            xsum += RUMUS_DPP_I(xsum, kDppXor1);
+            xsum += RUMUS_DPP_I(xsum, kDppXor2);
+            const float xs = (float)xsum * finv;
+            // planes of the whole chunk: word row u was prepared by quad lane u / OPL
+            uint32_t pl[OCT][5];
+#pragma unroll
+            for (int t = 0; t < OPL; t++)
+#pragma unroll
+                for (int i = 0; i < 5; i++) {
+                    pl[0 * OPL + t][i] = quad_bcast<0>(own[t][i]);
+                    pl[1 * OPL + t][i] = quad_bcast<1>(own[t][i]);
+                    pl[2 * OPL + t][i] = quad_bcast<2>(own[t][i]);
+                    pl[3 * OPL + t][i] = quad_bcast<3>(own[t][i]);
+                }
+
+            // ---- 3. dot products -------------------------------------------------
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                uint32_t d[5] = {0, 0, 0, 0, 0};
+                uint32_t qsum = 0;
+#pragma unroll
+                for (int u = 0; u < OCT; u++) {
+                    qsum = udot8(wv[u][c], 0x11111111u, qsum);
+#pragma unroll
+                    for (int i = 0; i < 5; i++) d[i] = udot8(wv[u][c], pl[u][i], d[i]);
+                }
+                // D < 2^31: 8*OCT*225 * (16^5 - 1) / 15
+                const uint32_t D = d[0] + 16u * (d[1] + 16u * (d[2] + 16u * (d[3] + 16u * d[4])));
+                const int I = (int)D - (int)(qsum << 19);
+                const float part = (float)I * finv;
+                acc[m][c] = fmaf(scv[c], fmaf(-zv[c], xs, part), acc[m][c]);
+            }
+        }
+    }
+
+    // ---- 4. reduce over the quads of a wave, then over the waves -----------------
+    const uint32_t lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+    for (int m = 0; m < M; m++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) acc[m][c] = reduce_row_lanes(acc[m][c]);
+    if (lane >= 12 && lane < 16) {
+#pragma unroll
+        for (int m = 0; m < M; m++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) red[wave][m][(lane - 12) * 4 + c] = acc[m][c];
+    }
+    __syncthreads();
+    if (tid < M * kD8Cols) {
+        const uint32_t m = tid / kD8Cols, c = tid % kD8Cols;
+        const uint32_t oc = cchunk * kD8Cols + c;
+        if (oc < n) {
+            float v = 0.0f;
+#pragma unroll
+            for (int wi = 0; wi < WAVES; wi++) v += red[wi][m][c];
+            if (bias) v += bias[oc];
+            yout[(uint64_t)m * n + oc] = v;
+        }
+    }
+}
+
+// Launch geometry: threads per workgroup and word rows per quad.
+constexpr int kD8Threads = 512, kD8Oct = 4;
+
+bool w4_gemv_dot8_supported(const W4Args& a) {
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(a.packed) | reinterpret_cast<uintptr_t>(a.scales) |
+                           reinterpret_cast<uintptr_t>(a.zp);
+    return a.m >= 1 && a.m <= 8 && a.n % 4 == 0 && (bits & 15) == 0 && !a.g_idx &&
+           a.group_size % (8 * kD8Oct) == 0;
+}
+
+template <int M>
+static int launch_m(const W4Args& a, hipStream_t s) {
+    const uint32_t ncolchunks = ceil_div(a.n, kD8Cols);
+    const bool fast_x = !a.perm && (a.k % 8 == 0) && ((reinterpret_cast<uintptr_t>(a.x) & 15) == 0);
+    if (fast_x)
+        hipLaunchKernelGGL((w4_gemv_dot8_kernel<M, kD8Threads, kD8Oct, true>), dim3(ncolchunks),
+                           dim3(kD8Threads), 0, s, a.packed, a.scales, a.zp, a.x, a.y, a.n, a.k,
+                           a.padded_k, a.group_size, a.bias, a.perm);
+    else
+        hipLaunchKernelGGL((w4_gemv_dot8_kernel<M, kD8Threads, kD8Oct, false>), dim3(ncolchunks),
+                           dim3(kD8Threads), 0, s, a.packed, a.scales, a.zp, a.x, a.y, a.n, a.k,
+                           a.padded_k, a.group_size, a.bias, a.perm);
+    return check_launch("w4_gemv_dot8_kernel");
+}
+
+int w4_launch_gemv_dot8(const W4Args& a, hipStream_t s) {
+    switch (a.m) {
+        case 1: return launch_m<1>(a, s);
+        case 2: return launch_m<2>(a, s);
+        case 3: return launch_m<3>(a, s);
+        case 4: return launch_m<4>(a, s);
+        case 5: return launch_m<5>(a, s);
+        case 6: return launch_m<6>(a, s);
+        case 7: return launch_m<7>(a, s);
+        case 8: return launch_m<8>(a, s);
+    }
+    return set_error(RUMUS_HIP_EINVAL, "w4 gemv: m = %u out of range", a.m);
+}
+
+}  // namespace rumus
