@@ -1,0 +1,87 @@
+// Pieces shared by the INT8 GEMM kernels: operand types, the LDS row swizzle
+// and the rescale/bias epilogue.
+#pragma once
+
+#include "common.h"
+
+namespace rumus {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+constexpr int kBK = 64;  // K bytes per LDS stage
+
+// chunk swizzle of an LDS row: bit0 = b1 ^ b3, bit1 = b2 of the row index
+__device__ __forceinline__ uint32_t row_swizzle(uint32_t row) {
+    return (((row >> 1) ^ (row >> 3)) & 1u) | ((row >> 1) & 2u);
+}
+
+// Epilogue shared by both kernels.  Accumulator register r of lane l is row
+// 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32x32 tile, so a store
+// instruction writes two full 128-byte row segments.  Interior tiles take a
+// branch-free path: the row scales of the lane are fetched up front as float4
+// (four consecutive rows per register quad) and y is written with
+// non-temporal stores (it is not read again by this kernel).
+template <int TM, int TN, int BM, int BN>
+__device__ __forceinline__ void i8_epilogue(const v16i (&acc)[TM][TN], const float* __restrict__ sx,
+                                            const float* __restrict__ sw,
+                                            const float* __restrict__ bias,
+                                            int32_t* __restrict__ acc_out, float* __restrict__ y,
+                                            uint32_t M, uint32_t N, uint32_t m0, uint32_t n0,
+                                            uint32_t wm, uint32_t wn, uint32_t lane) {
+    const uint32_t col_l = lane & 31, row_l = (lane >> 5) * 4;
+    const bool interior = m0 + BM <= M && n0 + BN <= N &&
+                          ((reinterpret_cast<uintptr_t>(sx) & 15) == 0);
+    if (interior && y && !acc_out) {
+        float4 sxv[TM][4];
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+                sxv[i][q] = *reinterpret_cast<const float4*>(sx + m0 + (wm * TM + i) * 32 + 8 * q + row_l);
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const uint32_t col = n0 + (wn * TN + j) * 32 + col_l;
+            const float swc = sw[col];
+            const float bc = bias ? bias[col] : 0.0f;
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const uint32_t row = m0 + (wm * TM + i) * 32 + 8 * (r / 4) + row_l + (r % 4);
+                    const float4 s4 = sxv[i][r / 4];
+                    const float sr = (r % 4) == 0 ? s4.x : (r % 4) == 1 ? s4.y : (r % 4) == 2 ? s4.z : s4.w;
+                    float v = __fmul_rn(__fmul_rn((float)acc[i][j][r], sr), swc);
+                    if (bias) v = __fadd_rn(v, bc);
+                    __builtin_nontemporal_store(v, y + (uint64_t)row * N + col);
+                }
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const uint32_t col = n0 + (wn * TN + j) * 32 + col_l;
+        if (col >= N) continue;
+        const float swc = y ? sw[col] : 0.0f;
+        const float bc = (y && bias) ? bias[col] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const uint32_t row = m0 + (wm * TM + i) * 32 + 8 * (r / 4) + row_l + (r % 4);
+                if (row >= M) continue;
+                const int32_t a = acc[i][j][r];
+                const uint64_t o = (uint64_t)row * N + col;
+                if (acc_out) acc_out[o] = a;
+                if (y) {
+                    float v = __fmul_rn(__fmul_rn((float)a, sx[row]), swc);
+                    if (bias) v = __fadd_rn(v, bc);
+                    y[o] = v;
+                }
+            }
+        }
+    }
+}
+
+}  // namespace rumus

@@ -12,16 +12,14 @@
 // Workgroup = 4 waves (2x2), block tile (64*TM) x (64*TN), K step 64 bytes,
 // two LDS stages: global -> registers -> LDS for step t+1 overlaps the MFMAs of
 // step t; one barrier per step.  LDS rows are 64 bytes with the 16-byte chunk
-// index XOR-swizzled by (row>>1)&3 so that both the 128-bit writes and the
-// 128-bit fragment reads are bank-conflict free.
-#include "common.h"
+// index XOR-swizzled by a function of row bits 1..3, chosen so that the
+// 128-bit fragment reads (consecutive lanes = consecutive rows, same chunk) hit
+// distinct 16-byte bank groups whether the LDS serves them 8 lanes per 128
+// bytes or 16 lanes per 256 bytes; the 128-bit writes cover whole rows and are
+// conflict-free under any per-row permutation.
+#include "i8_gemm.h"
 
 namespace rumus {
-
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
-
-constexpr int kBK = 64;  // K bytes per LDS stage
 
 template <int TM, int TN, int OCC>
 __global__ __launch_bounds__(256, OCC) void i8_gemm_kernel(
@@ -43,7 +41,7 @@ __global__ __launch_bounds__(256, OCC) void i8_gemm_kernel(
 
     // ---- global -> LDS staging assignment --------------------------------
     const uint32_t ld_row = tid >> 2, ld_c = tid & 3;
-    const uint32_t ld_lds = ld_row * kBK + ((ld_c ^ (ld_row >> 1)) & 3) * 16;
+    const uint32_t ld_lds = ld_row * kBK + ((ld_c ^ row_swizzle(ld_row)) & 3) * 16;
     const int8_t* pa[A_LOADS];
     const int8_t* pb[B_LOADS];
 #pragma unroll
@@ -78,7 +76,7 @@ __global__ __launch_bounds__(256, OCC) void i8_gemm_kernel(
     };
 
     // ---- fragment read addressing ------------------------------------------
-    const uint32_t fr = lane & 31, fh = lane >> 5, fsw = (fr >> 1) & 3;
+    const uint32_t fr = lane & 31, fh = lane >> 5, fsw = row_swizzle(fr);
     uint32_t a_off[2], b_off[2];
 #pragma unroll
     for (int s = 0; s < 2; s++) {
@@ -124,34 +122,203 @@ __global__ __launch_bounds__(256, OCC) void i8_gemm_kernel(
         __syncthreads();
     }
 
-    // ---- epilogue -----------------------------------------------------------
-    // Accumulator register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column
-    // l%32 of its 32x32 tile: a store instruction writes two 128-byte row
-    // segments.
-    const uint32_t col_l = lane & 31, row_l = (lane >> 5) * 4;
+    i8_epilogue<TM, TN, BM, BN>(acc, sx, sw, bias, acc_out, y, M, N, m0, n0, wm, wn, lane);
+}
+
+// ---------------------------------------------------------------------------
+// Large shapes (K % 64 == 0): 8 waves (4 x 2) per workgroup, one workgroup per
+// CU, block tile 256 x 128, five LDS stages fed by direct-to-LDS loads.
+//
+// global_load_lds_dwordx4 moves 16 bytes per lane from global memory straight
+// into LDS (lane l of a wave lands at base + 16*l), so a K step needs no
+// staging registers and several steps can be in flight, which is what hides the
+// L2/HBM latency (a step is only ~0.25 us of MFMA work).  The swizzled LDS
+// layout is produced on the global side: lane l of a 16-row block fetches row
+// l/4, logical chunk (l%4) ^ swizzle(row), and therefore lands in physical
+// chunk l%4.  Synchronisation is explicit: s_waitcnt vmcnt(n) leaves the
+// younger steps in flight, then one s_barrier per step.
+//
+// Measured on MI355X (2.2 GHz under MFMA load), per K step of one workgroup:
+// 512 cycles of MFMA per SIMD; fragment reads cost nothing extra once they are
+// interleaved with the MFMAs (571 cycles per step with the loads removed); the
+// LDS *write* side is the scarce resource: ds_write_b128 saturates at ~80 B/clk
+// per CU and the LDS-DMA path at less, so the 24 KB that a step brings in cost
+// ~350 cycles that do not hide under the MFMAs (~910 cycles per step in all).
+// ---------------------------------------------------------------------------
+typedef const void __attribute__((address_space(1)))* gptr_t;
+typedef void __attribute__((address_space(3)))* lptr_t;
+
+// s_waitcnt with only vmcnt set (gfx9 encoding: vmcnt[3:0] | expcnt 7 | lgkmcnt 15 | vmcnt[5:4] << 14)
+#define RUMUS_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | 0x70 | 0xF00)
+
+// WM x WN waves, each owning a (32*TM) x (32*TN) part of the block tile.
+template <int TM, int TN, int WM, int WN, int NS>
+__global__ __launch_bounds__(64 * WM * WN) void i8_gemm_dma_kernel(
+    const int8_t* __restrict__ A, const int8_t* __restrict__ B, const float* __restrict__ sx,
+    const float* __restrict__ sw, const float* __restrict__ bias, int32_t* __restrict__ acc_out,
+    float* __restrict__ y, uint32_t M, uint32_t K, uint32_t N, uint32_t tiles_m, uint32_t tiles_n) {
+    constexpr int WAVES = WM * WN;
+    constexpr int BM = 32 * TM * WM, BN = 32 * TN * WN;
+    constexpr int A_BYTES = BM * kBK, B_BYTES = BN * kBK, STAGE = A_BYTES + B_BYTES;
+    constexpr int A_LOADS = BM / 16 / WAVES, B_LOADS = BN / 16 / WAVES;   // 16-row blocks per wave per step
+    static_assert(A_LOADS * 16 * WAVES == BM && B_LOADS * 16 * WAVES == BN, "blocks must divide evenly");
+    constexpr int LOADS = A_LOADS + B_LOADS;
+    extern __shared__ __attribute__((aligned(16))) int8_t lds[];   // [NS][STAGE]
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    // the wave index is made scalar: LDS-DMA destinations then cost SALU work only
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t wm = wave / WN, wn = wave % WN;
+    const uint32_t tile = xcd_contiguous(blockIdx.x, tiles_m * tiles_n);
+    const uint32_t m0 = (tile % tiles_m) * BM, n0 = (tile / tiles_m) * BN;
+
+    // ---- global side of the LDS-DMA loads ------------------------------------
+    // block b = i*WAVES + wave holds rows 16b .. 16b+15 of the operand tile
+    const uint32_t lr = lane >> 2, lp = lane & 3;
+    const int8_t* pa[A_LOADS];
+    const int8_t* pb[B_LOADS];
 #pragma unroll
-    for (int j = 0; j < TN; j++) {
-        const uint32_t col = n0 + (wn * TN + j) * 32 + col_l;
-        if (col >= N) continue;
-        const float swc = y ? sw[col] : 0.0f;
-        const float bc = (y && bias) ? bias[col] : 0.0f;
-#pragma unroll
-        for (int i = 0; i < TM; i++) {
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const uint32_t row = m0 + (wm * TM + i) * 32 + 8 * (r / 4) + row_l + (r % 4);
-                if (row >= M) continue;
-                const int32_t a = acc[i][j][r];
-                const uint64_t o = (uint64_t)row * N + col;
-                if (acc_out) acc_out[o] = a;
-                if (y) {
-                    float v = __fmul_rn(__fmul_rn((float)a, sx[row]), swc);
-                    if (bias) v = __fadd_rn(v, bc);
-                    y[o] = v;
-                }
-            }
-        }
+    for (int i = 0; i < A_LOADS; i++) {
+        const uint32_t row = (i * WAVES + wave) * 16 + lr;
+        const uint32_t c = (lp ^ row_swizzle(row)) & 3;
+        pa[i] = A + (uint64_t)min(m0 + row, M - 1) * K + c * 16;
     }
+#pragma unroll
+    for (int i = 0; i < B_LOADS; i++) {
+        const uint32_t row = (i * WAVES + wave) * 16 + lr;
+        const uint32_t c = (lp ^ row_swizzle(row)) & 3;
+        pb[i] = B + (uint64_t)min(n0 + row, N - 1) * K + c * 16;
+    }
+    // loads [first, first + count) of a step: A blocks, then B blocks
+    auto issue_part = [&](uint32_t kt, uint32_t stage, int first, int count) {
+        int8_t* base = lds + stage * STAGE + wave * 1024;
+        const uint32_t k0 = kt * kBK;
+#pragma unroll
+        for (int q = 0; q < LOADS; q++) {
+            if (q < first || q >= first + count) continue;
+            if (q < A_LOADS)
+                __builtin_amdgcn_global_load_lds((gptr_t)(pa[q] + k0), (lptr_t)(base + q * WAVES * 1024), 16, 0, 0);
+            else
+                __builtin_amdgcn_global_load_lds((gptr_t)(pb[q - A_LOADS] + k0),
+                                                 (lptr_t)(base + A_BYTES + (q - A_LOADS) * WAVES * 1024), 16, 0, 0);
+        }
+    };
+    auto issue = [&](uint32_t kt, uint32_t stage) { issue_part(kt, stage, 0, LOADS); };
+
+    // ---- fragment read addressing ----------------------------------------------
+    const uint32_t fr = lane & 31, fh = lane >> 5, fsw = row_swizzle(fr);
+    uint32_t a_off[2], b_off[2];
+#pragma unroll
+    for (int s = 0; s < 2; s++) {
+        uint32_t chunk = ((2 * s + fh) ^ fsw) & 3;
+        a_off[s] = (wm * 32 * TM + fr) * kBK + chunk * 16;
+        b_off[s] = A_BYTES + (wn * 32 * TN + fr) * kBK + chunk * 16;
+    }
+
+    v16i acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+
+    // ---- software pipeline -----------------------------------------------------
+    // A wave sustains only one 128-bit LDS read per ~28 cycles, so fragment reads
+    // are never waited for in bulk: the reads of K half 1 of step kt are
+    // interleaved one-for-one with the MFMAs of half 0, and the reads of half 0 of
+    // step kt+1 with the MFMAs of half 1.  For that, the barrier of step kt
+    // publishes step kt+1 (one step ahead of its use), which leaves NS-2 steps of
+    // flight time to the LDS-DMA loads.
+    // Every step issues exactly LOADS loads, also past the end of K (the last
+    // step is then fetched again into a stage nobody reads any more): the memory
+    // counter arithmetic below needs no tail cases and the loop stays branch-free.
+    const uint32_t ksteps = K / kBK;
+#pragma unroll
+    for (int s = 0; s < NS - 1; s++) issue(min((uint32_t)s, ksteps - 1), s);
+
+    v4i af[2][TM], bf[2][TN];
+    auto read_half = [&](int h, uint32_t stage) {
+        const int8_t* base = lds + stage * STAGE;
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+            bf[h][j] = *reinterpret_cast<const v4i*>(base + b_off[h] + j * 32 * kBK);
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+            af[h][i] = *reinterpret_cast<const v4i*>(base + a_off[h] + i * 32 * kBK);
+    };
+    auto mfma_half = [&](int h) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[h][i], bf[h][j], acc[i][j], 0, 0, 0);
+    };
+    // (MFMA, read) pairs, then the MFMAs that are left; `dma` LDS-DMA loads are
+    // spread over the first pairs, one each, and split evenly over the two halves
+    // instead of being issued in a burst.
+    constexpr int DMA0 = LOADS / 2, DMA1 = LOADS - DMA0;
+    auto interleave = [&](int dma) {
+#pragma unroll
+        for (int q = 0; q < TM + TN; q++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (q < dma) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
+    };
+
+    // step 0 is visible once only the NS-2 younger steps are outstanding
+    RUMUS_WAIT_VMCNT((NS - 2) * LOADS);
+    __builtin_amdgcn_s_barrier();
+    read_half(0, 0);
+
+    uint32_t cur = 0;            // stage of step kt
+    for (uint32_t kt = 0; kt + 1 < ksteps; kt++) {
+        const uint32_t nxt = cur + 1 == NS ? 0 : cur + 1;        // stage of step kt+1
+        const uint32_t prv = cur == 0 ? NS - 1 : cur - 1;        // stage of step kt-1 (free)
+        // step kt+1 has landed once only the NS-3 younger steps are outstanding
+        RUMUS_WAIT_VMCNT((NS - 3) * LOADS);
+        __builtin_amdgcn_s_barrier();
+        // the refill of the stage freed by the barrier rides along with the MFMAs
+        const uint32_t kf = min(kt + (NS - 1), ksteps - 1);
+        issue_part(kf, prv, 0, DMA0);
+        read_half(1, cur);
+        mfma_half(0);
+        interleave(DMA0);
+        issue_part(kf, prv, DMA0, DMA1);
+        read_half(0, nxt);
+        mfma_half(1);
+        interleave(DMA1);
+        cur = nxt;
+    }
+    read_half(1, cur);
+    mfma_half(0);
+    interleave(0);
+    mfma_half(1);
+    RUMUS_WAIT_VMCNT(0);         // no LDS-DMA write may outlive the workgroup
+
+    i8_epilogue<TM, TN, BM, BN>(acc, sx, sw, bias, acc_out, y, M, N, m0, n0, wm, wn, lane);
+}
+
+template <int TM, int TN, int WM, int WN, int NS>
+static int launch_dma(const int8_t* A, const int8_t* B, const float* sx, const float* sw,
+                      const float* bias, int32_t* acc, float* y, uint32_t M, uint32_t K, uint32_t N,
+                      hipStream_t s) {
+    constexpr int BM = 32 * TM * WM, BN = 32 * TN * WN;
+    constexpr size_t lds_bytes = (size_t)NS * (BM + BN) * kBK;
+    static bool attr_set = false;   // benign race: setting the attribute is idempotent
+    if (!attr_set && lds_bytes > 64 * 1024) {
+        if (int rc = check_hip(hipFuncSetAttribute(
+                reinterpret_cast<const void*>(&i8_gemm_dma_kernel<TM, TN, WM, WN, NS>),
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes), "hipFuncSetAttribute"))
+            return rc;
+        attr_set = true;
+    }
+    uint32_t tm = ceil_div(M, BM), tn = ceil_div(N, BN);
+    hipLaunchKernelGGL((i8_gemm_dma_kernel<TM, TN, WM, WN, NS>), dim3(tm * tn), dim3(64 * WM * WN),
+                       lds_bytes, s, A, B, sx, sw, bias, acc, y, M, K, N, tm, tn);
+    return check_launch("i8_gemm_dma_kernel");
 }
 
 template <int TM, int TN, int OCC>
@@ -182,6 +349,7 @@ extern "C" int rumus_hip_i8_gemm(const int8_t* xq, const int8_t* wq, const float
     // Largest tile that still gives every CU a workgroup.
     const uint64_t big = (uint64_t)ceil_div(m, 256) * ceil_div(n, 128);
     const uint64_t mid = (uint64_t)ceil_div(m, 128) * ceil_div(n, 128);
+    if (big >= 256 && k % kBK == 0) return launch_dma<2, 2, 4, 2, 5>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
     if (big >= 256) return launch<4, 2, 2>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
     if (mid >= 256) return launch<2, 2, 2>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
     return launch<1, 1, 2>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
