@@ -60,8 +60,13 @@ SHAPES = [
     (8, 512, 20, 8, False),       # smallest group, ragged columns
     (1, 128, 10, 32, True),       # n % 4 != 0 -> reference-order kernel
     (5, 72, 7, 8, False),         # reference-order kernel, odd everything
-    (16, 512, 256, 128, True),    # m > 8
-    (33, 384, 96, 64, False),
+    (16, 512, 256, 128, True),    # m > 8: f16 MFMA kernel, one row tile
+    (33, 384, 96, 64, False),     # 64-row tile with dead rows, group 64, ragged strip
+    (9, 160, 40, 32, True),       # group 32, padded_k not a multiple of the 128-row stage
+    (64, 1024, 1024, 128, True),
+    (100, 2048, 520, 256, False), # group spans two stages
+    (20, 1000, 64, 64, True),     # K tail
+    (12, 256, 36, 8, False),      # group 8: not an MFMA case -> reference-order kernel
 ]
 
 
@@ -173,6 +178,26 @@ def test_qmatmul_int4_transpose(ops, m, k, n, g):
     got = host(ops.qmatmul_int4_t(dev(gy), dev(packed), dev(scales), dev(zp), k, g))
     assert got.shape == (m, k)
     assert_close(got, want)
+
+
+def test_gptq_actorder_config_full_size(ops):
+    # BASELINE config 2: M=16 and M=128, K=4096, N=11008, g128, symmetric zp=8, act-order g_idx
+    for m in (16, 128):
+        say(f"w4 gemm act-order {m}x4096x11008")
+        k, n, g = 4096, 11008, 128
+        w, g_idx, x = workloads.w4_gemm_actorder(0, m=m, k=k, n=n, group_size=g)
+        order = np.argsort(g_idx, kind="stable")
+        ps, ss, zs = oracle.w4_from_f32(w[order], g, symmetric=True)         # groups contiguous
+        rows = slice(0, m) if m == 16 else [0, 1, 63, 64, 127]               # oracle rows (CPU time)
+        xs = x[rows]
+        want = oracle.qmatmul_int4(np.ascontiguousarray(xs[:, order]), ps, ss, zs, k, g, threads=8)
+        got = host(ops.qmatmul_int4_perm(dev(x), dev(ps), dev(ss), dev(zs), k, g,
+                                         perm=dev(order.astype(np.int32))))
+        assert_close(got[rows], want)
+        # every row through a size-independent property: linearity, y(2x) == 2 y(x)
+        got2 = host(ops.qmatmul_int4_perm(dev((2 * x).astype(np.float32)), dev(ps), dev(ss), dev(zs), k, g,
+                                          perm=dev(order.astype(np.int32))))
+        assert_close(got2, 2 * got)
 
 
 def test_qlinear_module_mirror(ops):
