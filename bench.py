@@ -36,6 +36,9 @@ GROUPS = K // G
 BYTES_F32_ZP = K * N // 2 + 2 * GROUPS * N * 4 + K * 4 + N * 4           # 9,469,952 (layout executed)
 BYTES_U4_ZP = K * N // 2 + GROUPS * N * 4 + GROUPS * N // 2 + K * 4 + N * 4  # 9,011,200 (u4 zero-points)
 WEIGHT_SETS = 64
+# HBM bytes per GEMV launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by a 256 MiB copy
+# (profiles/w4_gemv_dot8_1x4096x4096_hbm_traffic.txt); a counter result, not measured by this script
+GEMV_TRAFFIC_BYTES = 9649213
 
 
 def log(msg):
@@ -214,6 +217,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=640)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-gemv", action="store_true", help="skip the secondary workloads")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run plain 256 MiB device copies (reference kernel of known traffic for "
+                         "scaling FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build targets one GPU; --gpus above 1 is not supported "
@@ -247,12 +253,20 @@ def main():
         "config": {"workload": "w4_gemv_1x4096x4096_g128_awq_f32zp", "weight_sets_rotated": WEIGHT_SETS,
                    "hip_graph": r["graph"], "bytes_per_step": BYTES_F32_ZP},
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": gbs / HBM_PEAK_GBS, "traffic": None},
+                     "frac": gbs / HBM_PEAK_GBS, "traffic": GEMV_TRAFFIC_BYTES},
         "gbs_at_u4_zero_point_bytes": BYTES_U4_ZP / per_launch / 1e9,
         "cache_resident": {"gbs": BYTES_F32_ZP / per_launch_res / 1e9,
                            "ms_per_step": per_launch_res * 1e3,
                            "note": "single weight set, served by Infinity Cache / L2; not HBM"},
     }
+
+    if args.calibrate_copy:
+        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device="cuda:0").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)              # reads 256 MiB, writes 256 MiB per launch
+        torch.cuda.synchronize()
+        del src, dst
 
     if not args.only_gemv:
         out["secondary"] = bench_i8_gemm(torch, ops)

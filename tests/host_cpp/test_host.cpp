@@ -1,0 +1,136 @@
+// GPU parity test of the C++ host mirror (include/rumus_hip.hpp) against the CPU
+// oracle: reads like a RUMUS integration test (build a Linear, quantize it, run
+// forward, compare).  Exit status 0 = every check passed.
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <random>
+#include <vector>
+
+#include "rumus_hip.hpp"
+#include "rumus_oracle.h"
+
+using namespace rumus_hip;
+
+static int g_fail = 0;
+#define CHECK(cond, ...)                                   \
+    do {                                                   \
+        if (!(cond)) { g_fail++; printf("FAIL %s:%d: ", __FILE__, __LINE__); printf(__VA_ARGS__); printf("\n"); } \
+    } while (0)
+
+static std::vector<float> normal(size_t n, float sigma, uint32_t seed) {
+    std::mt19937 gen(seed);
+    std::normal_distribution<float> d(0.0f, sigma);
+    std::vector<float> v(n);
+    for (auto& x : v) x = d(gen);
+    return v;
+}
+
+static bool close(const std::vector<float>& got, const std::vector<float>& want, const char* what) {
+    size_t bad = 0;
+    double worst = 0;
+    for (size_t i = 0; i < got.size(); i++) {
+        double err = std::fabs((double)got[i] - want[i]), tol = 1e-4 + 1e-3 * std::fabs(want[i]);
+        if (!(err <= tol)) bad++;
+        worst = std::fmax(worst, err);
+    }
+    printf("  %-34s max abs err %.3g, %zu of %zu outside rel 1e-3 / abs 1e-4\n", what, worst, bad, got.size());
+    return bad == 0;
+}
+
+static void test_qlinear(uint32_t m, uint32_t k, uint32_t n, uint32_t g) {
+    printf("[host-cpp] QLinear m=%u k=%u n=%u g=%u\n", m, k, n, g);
+    fflush(stdout);
+    auto w = normal((size_t)k * n, 0.02f, 1), b = normal(n, 0.01f, 2), x = normal((size_t)m * k, 1.0f, 3);
+    Linear linear(w, k, n, b);
+    QLinear q = QLinear::from_linear(linear, g);
+    CHECK(q.in_features == k && q.out_features == n, "feature sizes");
+    // oracle: QuantizedTensor::from_f32 then the WGSL kernel's loop
+    const uint32_t padded_k = ((k + g - 1) / g) * g, groups = padded_k / g;
+    std::vector<uint32_t> packed((size_t)(padded_k / 8) * n);
+    std::vector<float> scales((size_t)groups * n), zp((size_t)groups * n), want((size_t)m * n);
+    CHECK(orc_w4_from_f32(w.data(), k, n, g, packed.data(), scales.data(), zp.data()) == 0, "oracle from_f32");
+    CHECK(q.weight.padded_k == padded_k && q.weight.num_groups == groups, "padding metadata");
+    CHECK(q.weight.packed.download() == packed, "nibble pack is not bit-exact");
+    CHECK(q.weight.scales.download() == scales, "scales are not bit-exact");
+    CHECK(q.weight.zp.download() == zp, "zero-points are not bit-exact");
+    orc_qmatmul_int4(x.data(), packed.data(), scales.data(), zp.data(), b.data(), nullptr, want.data(), m, k, n,
+                     padded_k, g, groups, 8);
+    DeviceBuffer<float> dx(x);
+    CHECK(close(q.forward(dx).download(), want, "forward"), "QLinear::forward");
+    // grad_x
+    auto gy = normal((size_t)m * n, 1.0f, 4);
+    std::vector<float> want_gx((size_t)m * k);
+    orc_qmatmul_int4_t(gy.data(), packed.data(), scales.data(), zp.data(), want_gx.data(), m, k, n, padded_k, g,
+                       groups, 8);
+    CHECK(close(q.backward_input(DeviceBuffer<float>(gy)).download(), want_gx, "backward_input"), "grad_x");
+}
+
+static void test_q8(uint32_t m, uint32_t k, uint32_t n, uint32_t bs) {
+    printf("[host-cpp] Q8 quantize/matmul m=%u k=%u n=%u bs=%u\n", m, k, n, bs);
+    fflush(stdout);
+    auto w = normal((size_t)k * n, 0.02f, 5), a = normal((size_t)m * k, 1.0f, 6);
+    DeviceBuffer<float> dw(w), da(a);
+    Q8Tensor q = quantize(dw.data(), k, n, bs);
+    std::vector<float> wt((size_t)k * n);
+    orc_transpose(w.data(), wt.data(), k, n);
+    std::vector<uint32_t> words(orc_q8_buf_size((uint64_t)k * n, bs) / 4);
+    CHECK(orc_q8_quantize(wt.data(), words.data(), k * n, bs) == 0, "oracle quantize");
+    CHECK(q.buffer.download() == words, "Q8 buffer is not bit-exact");
+    std::vector<float> want((size_t)m * n), deq((size_t)k * n);
+    orc_matmul_q8(a.data(), words.data(), want.data(), m, k, n, bs, 8);
+    CHECK(close(matmul(da, m, q).download(), want, "matmul (Q8 rhs)"), "matmul_q8");
+    orc_q8_dequantize(words.data(), deq.data(), k * n, bs);
+    CHECK(dequantize(q).download() == deq, "dequantize is not bit-exact");
+}
+
+static void test_int8_linear(uint32_t m, uint32_t k, uint32_t n) {
+    printf("[host-cpp] Int8Linear m=%u k=%u n=%u\n", m, k, n);
+    fflush(stdout);
+    auto w = normal((size_t)k * n, 0.02f, 7), b = normal(n, 0.01f, 8), x = normal((size_t)m * k, 1.0f, 9);
+    Linear linear(w, k, n, b);
+    Int8Linear l = Int8Linear::from_linear(linear);
+    std::vector<float> wt((size_t)k * n), sw(n), sx(m), want((size_t)m * n);
+    std::vector<int8_t> wq((size_t)k * n), xq((size_t)m * k);
+    std::vector<int32_t> acc((size_t)m * n);
+    orc_transpose(w.data(), wt.data(), k, n);
+    orc_i8_quantize_rows(wt.data(), wq.data(), sw.data(), n, k);
+    orc_i8_quantize_rows(x.data(), xq.data(), sx.data(), m, k);
+    orc_i8_gemm_i32(xq.data(), wq.data(), acc.data(), m, k, n, 8);
+    orc_i8_rescale_bias(acc.data(), sx.data(), sw.data(), b.data(), want.data(), m, n);
+    CHECK(l.wq.download() == wq, "int8 weights are not bit-exact");
+    CHECK(l.sw.download() == sw, "weight scales are not bit-exact");
+    DeviceBuffer<int32_t> dacc;
+    auto y = l.forward(DeviceBuffer<float>(x), &dacc).download();
+    CHECK(dacc.download() == acc, "i32 accumulators are not bit-exact");
+    CHECK(close(y, want, "forward"), "Int8Linear::forward");
+}
+
+static void test_errors() {
+    printf("[host-cpp] preconditions\n");
+    fflush(stdout);
+    DeviceBuffer<float> w(std::vector<float>(64, 0.0f));
+    bool threw = false;
+    try { QuantizedTensor::from_f32(w.data(), 64, 8, 8, 12); } catch (const Error& e) { threw = e.code == RUMUS_HIP_EINVAL; }
+    CHECK(threw, "group_size 12 must be rejected");
+    threw = false;
+    try { quantize(w.data(), 8, 8, 6); } catch (const Error& e) { threw = e.code == RUMUS_HIP_EINVAL; }
+    CHECK(threw, "block_size 6 must be rejected");
+    threw = false;
+    try { QuantizedTensor::from_f32(w.data(), 60, 8, 8, 8); } catch (const Error&) { threw = true; }
+    CHECK(threw, "length mismatch must be rejected");
+}
+
+int main() {
+    check(rumus_hip_init(0));
+    test_qlinear(1, 1024, 512, 128);
+    test_qlinear(4, 200, 52, 8);
+    test_qlinear(16, 512, 256, 128);
+    test_q8(32, 512, 512, 512);
+    test_q8(3, 96, 7, 32);
+    test_int8_linear(32, 512, 512);
+    test_int8_linear(300, 1024, 260);
+    test_errors();
+    printf(g_fail ? "host-cpp: %d FAILED\n" : "host-cpp: all passed\n", g_fail);
+    return g_fail ? 1 : 0;
+}
