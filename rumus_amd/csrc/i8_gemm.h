@@ -11,6 +11,19 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 constexpr int kBK = 64;  // K bytes per LDS stage
 
+typedef const void __attribute__((address_space(1)))* gptr_t;
+typedef void __attribute__((address_space(3)))* lptr_t;
+
+// s_waitcnt with only vmcnt set (gfx9 encoding: vmcnt[3:0] | expcnt 7 | lgkmcnt 15 | vmcnt[5:4] << 14)
+#define RUMUS_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | 0x70 | 0xF00)
+
+// Wide-tile kernel (i8_gemm_wide.hip): tile width in 32-column units that deals the
+// problem to `cus` compute units in whole rounds with little padding, 0 if none does.
+int i8_gemm_wide_width(uint32_t M, uint32_t N, uint32_t cus);
+int i8_gemm_launch_wide(int tn, const int8_t* A, const int8_t* B, const float* sx, const float* sw,
+                        const float* bias, int32_t* acc, float* y, uint32_t M, uint32_t K, uint32_t N,
+                        hipStream_t s);
+
 // chunk swizzle of an LDS row: bit0 = b1 ^ b3, bit1 = b2 of the row index
 __device__ __forceinline__ uint32_t row_swizzle(uint32_t row) {
     return (((row >> 1) ^ (row >> 3)) & 1u) | ((row >> 1) & 2u);
@@ -30,8 +43,9 @@ __device__ __forceinline__ void i8_epilogue(const v16i (&acc)[TM][TN], const flo
                                             uint32_t M, uint32_t N, uint32_t m0, uint32_t n0,
                                             uint32_t wm, uint32_t wn, uint32_t lane) {
     const uint32_t col_l = lane & 31, row_l = (lane >> 5) * 4;
-    const bool interior = m0 + BM <= M && n0 + BN <= N &&
-                          ((reinterpret_cast<uintptr_t>(sx) & 15) == 0);
+    // whole 32-column MFMA tiles are in or out when N % 32 == 0, so the fast path
+    // only needs all rows of the block inside M
+    const bool interior = m0 + BM <= M && N % 32 == 0 && ((reinterpret_cast<uintptr_t>(sx) & 15) == 0);
     if (interior && y && !acc_out) {
         float4 sxv[TM][4];
 #pragma unroll
@@ -42,6 +56,7 @@ __device__ __forceinline__ void i8_epilogue(const v16i (&acc)[TM][TN], const flo
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             const uint32_t col = n0 + (wn * TN + j) * 32 + col_l;
+            if (n0 + (wn * TN + j) * 32 >= N) continue;    // uniform: this column tile lies past N
             const float swc = sw[col];
             const float bc = bias ? bias[col] : 0.0f;
 #pragma unroll

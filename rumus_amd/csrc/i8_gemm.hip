@@ -145,12 +145,6 @@ __global__ __launch_bounds__(256, OCC) void i8_gemm_kernel(
 // per CU and the LDS-DMA path at less, so the 24 KB that a step brings in cost
 // ~350 cycles that do not hide under the MFMAs (~910 cycles per step in all).
 // ---------------------------------------------------------------------------
-typedef const void __attribute__((address_space(1)))* gptr_t;
-typedef void __attribute__((address_space(3)))* lptr_t;
-
-// s_waitcnt with only vmcnt set (gfx9 encoding: vmcnt[3:0] | expcnt 7 | lgkmcnt 15 | vmcnt[5:4] << 14)
-#define RUMUS_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | 0x70 | 0xF00)
-
 // WM x WN waves, each owning a (32*TM) x (32*TN) part of the block tile.
 template <int TM, int TN, int WM, int WN, int NS>
 __global__ __launch_bounds__(64 * WM * WN) void i8_gemm_dma_kernel(
@@ -160,8 +154,11 @@ __global__ __launch_bounds__(64 * WM * WN) void i8_gemm_dma_kernel(
     constexpr int WAVES = WM * WN;
     constexpr int BM = 32 * TM * WM, BN = 32 * TN * WN;
     constexpr int A_BYTES = BM * kBK, B_BYTES = BN * kBK, STAGE = A_BYTES + B_BYTES;
-    constexpr int A_LOADS = BM / 16 / WAVES, B_LOADS = BN / 16 / WAVES;   // 16-row blocks per wave per step
-    static_assert(A_LOADS * 16 * WAVES == BM && B_LOADS * 16 * WAVES == BN, "blocks must divide evenly");
+    // 16-row blocks per wave and step; when the blocks do not divide evenly the
+    // last block is fetched twice (same bytes to the same place), so that every
+    // wave issues the same number of loads per step
+    constexpr int A_BLOCKS = BM / 16, B_BLOCKS = BN / 16;
+    constexpr int A_LOADS = (A_BLOCKS + WAVES - 1) / WAVES, B_LOADS = (B_BLOCKS + WAVES - 1) / WAVES;
     constexpr int LOADS = A_LOADS + B_LOADS;
     extern __shared__ __attribute__((aligned(16))) int8_t lds[];   // [NS][STAGE]
 
@@ -177,30 +174,33 @@ __global__ __launch_bounds__(64 * WM * WN) void i8_gemm_dma_kernel(
     const uint32_t lr = lane >> 2, lp = lane & 3;
     const int8_t* pa[A_LOADS];
     const int8_t* pb[B_LOADS];
+    uint32_t blk_a[A_LOADS], blk_b[B_LOADS];
 #pragma unroll
     for (int i = 0; i < A_LOADS; i++) {
-        const uint32_t row = (i * WAVES + wave) * 16 + lr;
+        blk_a[i] = min(i * WAVES + wave, (uint32_t)A_BLOCKS - 1);
+        const uint32_t row = blk_a[i] * 16 + lr;
         const uint32_t c = (lp ^ row_swizzle(row)) & 3;
         pa[i] = A + (uint64_t)min(m0 + row, M - 1) * K + c * 16;
     }
 #pragma unroll
     for (int i = 0; i < B_LOADS; i++) {
-        const uint32_t row = (i * WAVES + wave) * 16 + lr;
+        blk_b[i] = min(i * WAVES + wave, (uint32_t)B_BLOCKS - 1);
+        const uint32_t row = blk_b[i] * 16 + lr;
         const uint32_t c = (lp ^ row_swizzle(row)) & 3;
         pb[i] = B + (uint64_t)min(n0 + row, N - 1) * K + c * 16;
     }
     // loads [first, first + count) of a step: A blocks, then B blocks
     auto issue_part = [&](uint32_t kt, uint32_t stage, int first, int count) {
-        int8_t* base = lds + stage * STAGE + wave * 1024;
+        int8_t* base = lds + stage * STAGE;
         const uint32_t k0 = kt * kBK;
 #pragma unroll
         for (int q = 0; q < LOADS; q++) {
             if (q < first || q >= first + count) continue;
             if (q < A_LOADS)
-                __builtin_amdgcn_global_load_lds((gptr_t)(pa[q] + k0), (lptr_t)(base + q * WAVES * 1024), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((gptr_t)(pa[q] + k0), (lptr_t)(base + blk_a[q] * 1024), 16, 0, 0);
             else
                 __builtin_amdgcn_global_load_lds((gptr_t)(pb[q - A_LOADS] + k0),
-                                                 (lptr_t)(base + A_BYTES + (q - A_LOADS) * WAVES * 1024), 16, 0, 0);
+                                                 (lptr_t)(base + A_BYTES + blk_b[q - A_LOADS] * 1024), 16, 0, 0);
         }
     };
     auto issue = [&](uint32_t kt, uint32_t stage) { issue_part(kt, stage, 0, LOADS); };
@@ -349,7 +349,12 @@ extern "C" int rumus_hip_i8_gemm(const int8_t* xq, const int8_t* wq, const float
     // Largest tile that still gives every CU a workgroup.
     const uint64_t big = (uint64_t)ceil_div(m, 256) * ceil_div(n, 128);
     const uint64_t mid = (uint64_t)ceil_div(m, 128) * ceil_div(n, 128);
-    if (big >= 256 && k % kBK == 0) return launch_dma<2, 2, 4, 2, 5>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
+    if (big >= 256 && k % kBK == 0) {
+        // one round of 256 x (256..352) tiles when the shape divides that way
+        if (const int tn = i8_gemm_wide_width(m, n, 256))
+            return i8_gemm_launch_wide(tn, xq, wq, sx, sw, bias, acc, y, m, k, n, s);
+        return launch_dma<2, 2, 4, 2, 5>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
+    }
     if (big >= 256) return launch<4, 2, 2>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
     if (mid >= 256) return launch<2, 2, 2>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
     return launch<1, 1, 2>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);

@@ -134,6 +134,20 @@ def test_i8_quantize_cols_t_bit_exact(ops, k, n):
 @pytest.mark.parametrize("m,k,n", [(32, 512, 512), (1, 16, 1), (77, 208, 133), (256, 1024, 384),
                                    (300, 4096, 260), (2048, 256, 2304)])
 def test_i8_gemm_accumulators_bit_exact(ops, m, k, n):
+    check_i8_gemm(ops, m, k, n)
+
+
+# Shapes that take the wide-block kernel (256 x 32*W blocks in whole rounds over 256 CUs),
+# one per block width W = 8..12, with K of 1, 2, 3 and 5 steps of 64 (fewer steps than
+# pipeline stages included), a ragged last row block and N that is not a multiple of 32.
+@pytest.mark.parametrize("m,k,n", [(4096, 192, 4096), (2048, 64, 9216), (2048, 128, 10240),
+                                   (2048, 320, 11008), (2000, 64, 10990), (2048, 64, 12288),
+                                   (1990, 128, 12281)])
+def test_i8_gemm_wide_blocks_bit_exact(ops, m, k, n):
+    check_i8_gemm(ops, m, k, n)
+
+
+def check_i8_gemm(ops, m, k, n):
     say(f"i8_gemm m={m} k={k} n={n}")
     rng = np.random.default_rng(m + k + n)
     xq = rng.integers(-127, 128, (m, k)).astype(np.int8)
