@@ -143,13 +143,51 @@ def bench_i8_gemm(torch, ops, steps=30, warmup=5):
     torch.cuda.synchronize()
     sec_q = start.elapsed_time(end) * 1e-3 / steps
     tops = ops_per / sec / 1e12
+    # Two yardsticks measured in the same run, on the same operands where it applies:
+    # the matrix cores alone (MFMA from registers, random operand bits, no memory traffic:
+    # what the board's power limit lets them sustain), and the vendor library's int8 GEMM
+    # (hipBLASLt through torch._int_mm: i32 output, no rescale) on the same xq, wq.
+    ceiling = probe_mfma_ceiling()
+    vendor = None
+    try:
+        wt = wq.t()
+        for _ in range(warmup):
+            torch._int_mm(xq, wt)
+        start.record()
+        for _ in range(steps):
+            torch._int_mm(xq, wt)
+        end.record()
+        torch.cuda.synchronize()
+        vendor = ops_per / (start.elapsed_time(end) * 1e-3 / steps) / 1e12
+    except Exception as exc:   # informational only
+        log(f"[bench] vendor int8 GEMM not timed: {exc}")
     return {
         "workload": "int8_gemm_2048x4096x11008", "ms_per_launch": sec * 1e3, "tops": tops,
         "roofline": {"bound": "mfma", "achieved": tops, "peak": I8_PEAK_TOPS, "unit": "TOP/s",
                      "frac": tops / I8_PEAK_TOPS, "traffic": None},
+        "mfma_only_random_operands": ceiling,
+        "frac_of_mfma_only": (tops / ceiling["tops"]) if ceiling else None,
+        "vendor_int_mm_tops": vendor,
         "act_quantize_rows_ms": sec_q * 1e3,
         "act_quantize_rows_gbs": (m * k * 5 + m * 4) / sec_q / 1e9,
     }
+
+
+def probe_mfma_ceiling():
+    """int8 TOP/s of v_mfma_i32_32x32x32_i8 issued back to back from registers with random
+    operand bits (rumus_amd/csrc/probe_mfma.hip, its own small library), or None."""
+    import ctypes
+    path = os.path.join(ROOT, "rumus_amd", "librumus_probe.so")
+    if not os.path.exists(path):
+        return None
+    lib = ctypes.CDLL(path)
+    lib.rumus_probe_i8_mfma.restype = ctypes.c_int
+    lib.rumus_probe_i8_mfma.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_double),
+                                        ctypes.POINTER(ctypes.c_double)]
+    tops, mhz = ctypes.c_double(), ctypes.c_double()
+    if lib.rumus_probe_i8_mfma(1, ctypes.byref(tops), ctypes.byref(mhz)) != 0:
+        return None
+    return {"tops": tops.value, "shader_mhz": mhz.value}
 
 
 def bench_w4_gemm(torch, ops, m, steps=50, warmup=5):
