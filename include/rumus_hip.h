@@ -53,6 +53,17 @@ const char* rumus_hip_version(void);
 /* device.poll(Wait) (context.rs:840-850): block until `stream` is idle. */
 int rumus_hip_sync(rumus_hip_stream_t stream);
 
+/* Workspace.  The reference takes every temporary from its BufferPool
+ * (rumus/src/backend/gpu/pool.rs:34-75) and returns it on drop; here the only
+ * temporaries are the partial sums of matmuls that split K over workgroups
+ * (qmatmul_int4 with 9 <= m and few output tiles).  They live in one device
+ * buffer per (device, stream), grown on demand inside the call that needs it.
+ * A caller that must not allocate later (graph capture, serving loop) reserves
+ * the size up front: for qmatmul_int4 at most 16 * m * n * 4 bytes.
+ * rumus_hip_shutdown frees every workspace (no launch may be in flight). */
+int rumus_hip_workspace_reserve(rumus_hip_stream_t stream, uint64_t bytes);
+int rumus_hip_shutdown(void);
+
 /* ---- INT8 engine, reference Q8 block format ----------------------------- */
 
 /* DType::Q8{block_size}.gpu_buf_size(numel) (rumus/src/tensor/core.rs:87-98):

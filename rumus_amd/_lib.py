@@ -41,6 +41,8 @@ PROTOTYPES = {
     "rumus_hip_last_error": (C.c_char_p, []),
     "rumus_hip_version": (C.c_char_p, []),
     "rumus_hip_sync": (_i32, [_vp]),
+    "rumus_hip_workspace_reserve": (_i32, [_vp, _u64]),
+    "rumus_hip_shutdown": (_i32, []),
     "rumus_hip_q8_buf_size": (_u64, [_u64, _u32]),
     "rumus_hip_q8_quantize": (_i32, [_vp, _vp, _u32, _u32, _vp]),
     "rumus_hip_q8_dequantize": (_i32, [_vp, _vp, _u32, _u32, _vp]),

@@ -14,6 +14,9 @@ int set_error(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3
 // Converts a HIP status into a return code (0 when hipSuccess).
 int check_hip(hipError_t e, const char* what);
 
+// Device workspace of at least `bytes` for work queued on `stream` (runtime.hip).
+int workspace_get(hipStream_t stream, size_t bytes, void** out);
+
 // hipGetLastError() after a kernel launch.
 inline int check_launch(const char* kernel) { return check_hip(hipGetLastError(), kernel); }
 

@@ -3,6 +3,9 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
+#include <unordered_map>
+
 #include "common.h"
 
 namespace rumus {
@@ -22,9 +25,81 @@ int check_hip(hipError_t e, const char* what) {
     return set_error(RUMUS_HIP_EHIP, "%s: %s", what, hipGetErrorString(e));
 }
 
+// ---- workspace: one device buffer per (device, stream), grown on demand -----------------
+// Kernels that split the reduction axis over workgroups park their partial sums here.
+// Calls on one stream run in order, so they can share a buffer; different streams get
+// different buffers.  Growing is the only time the library allocates: it waits for the
+// stream, frees the old buffer and allocates the new size.
+namespace {
+struct Arena {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+};
+struct ArenaKey {
+    int device;
+    hipStream_t stream;
+    bool operator==(const ArenaKey& o) const { return device == o.device && stream == o.stream; }
+};
+struct ArenaKeyHash {
+    size_t operator()(const ArenaKey& k) const {
+        return std::hash<const void*>()(k.stream) ^ (std::hash<int>()(k.device) * 0x9e3779b97f4a7c15ull);
+    }
+};
+std::mutex g_arena_mutex;
+std::unordered_map<ArenaKey, Arena, ArenaKeyHash> g_arenas;
+}  // namespace
+
+int workspace_get(hipStream_t stream, size_t bytes, void** out) {
+    int device = 0;
+    if (int rc = check_hip(hipGetDevice(&device), "hipGetDevice")) return rc;
+    std::lock_guard<std::mutex> lock(g_arena_mutex);
+    Arena& a = g_arenas[ArenaKey{device, stream}];
+    if (a.bytes < bytes) {
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (stream && hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
+            return set_error(RUMUS_HIP_EINVAL,
+                             "workspace of %zu bytes needed while the stream is capturing: call "
+                             "rumus_hip_workspace_reserve before the capture", bytes);
+        if (a.ptr) {
+            if (int rc = check_hip(hipStreamSynchronize(stream), "hipStreamSynchronize")) return rc;
+            if (int rc = check_hip(hipFree(a.ptr), "hipFree(workspace)")) return rc;
+            a.ptr = nullptr;
+            a.bytes = 0;
+        }
+        const size_t want = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);   // whole MiB
+        if (int rc = check_hip(hipMalloc(&a.ptr, want), "hipMalloc(workspace)")) return rc;
+        a.bytes = want;
+    }
+    *out = a.ptr;
+    return RUMUS_HIP_OK;
+}
+
+static int workspace_release_all() {
+    std::lock_guard<std::mutex> lock(g_arena_mutex);
+    int rc = RUMUS_HIP_OK;
+    for (auto& kv : g_arenas) {
+        if (!kv.second.ptr) continue;
+        int cur = 0;
+        (void)hipGetDevice(&cur);
+        (void)hipSetDevice(kv.first.device);
+        if (int e = check_hip(hipFree(kv.second.ptr), "hipFree(workspace)")) rc = e;
+        (void)hipSetDevice(cur);
+    }
+    g_arenas.clear();
+    return rc;
+}
+
 }  // namespace rumus
 
 extern "C" {
+
+int rumus_hip_workspace_reserve(rumus_hip_stream_t stream, uint64_t bytes) {
+    void* p = nullptr;
+    if (bytes == 0) return RUMUS_HIP_OK;
+    return rumus::workspace_get(rumus::as_stream(stream), (size_t)bytes, &p);
+}
+
+int rumus_hip_shutdown(void) { return rumus::workspace_release_all(); }
 
 int rumus_hip_init(int device) {
     int count = 0;

@@ -33,8 +33,8 @@ int w4_launch_gemv(const W4Args& a, hipStream_t s);
 bool w4_gemv_dot8_supported(const W4Args& a);
 int w4_launch_gemv_dot8(const W4Args& a, hipStream_t s);
 
-// f16 MFMA kernel for larger m (needs group_size % 32 == 0, n % 4 == 0,
-// 16-byte aligned buffers, no g_idx).
+// f16 MFMA kernel for larger m (needs group_size 32, 64 or a multiple of 128,
+// n % 4 == 0, 16-byte aligned buffers, no g_idx).
 bool w4_gemm_supported(const W4Args& a);
 int w4_launch_gemm(const W4Args& a, hipStream_t s);
 

@@ -1,0 +1,355 @@
+// INT4 engine: dequant-fused GEMM on the f16 matrix cores, for m > 8.
+//
+//   y[m,n] = sum_g scales[g,n] * ( sum_{k in g} x[m,k] * q[k,n] - zp[g,n] * sum_{k in g} x[m,k] ) (+ bias[n])
+//
+// which equals sum_k x[m,k] * (q[k,n] - zp) * scale with the scale applied once
+// per group in f32.  Inside a group only x and the raw nibbles meet in the MFMA:
+//   - q is 0..15, exact in f16;
+//   - x is split as hi + lo with hi = f16(x), lo = f16(x - hi) (gfx950 MFMAs keep
+//     f16 subnormals), two MFMAs per tile, f32 accumulate.  x keeps ~21
+//     significant bits, so the f32 tolerance of this path (rel 1e-3 / abs 1e-4)
+//     holds; a single f16 x, or scale folded into f16 weights, would not hold it
+//     for outputs near zero.
+//
+// One accumulator set serves all groups: it is kept in units of the current
+// group's scale.  When a group ends, the zero-point term is subtracted
+// (zp * sum of x over the group, the sums come with the staged activations) and
+// the accumulator is multiplied by scale_cur / scale_next; the last unit is
+// multiplied out in the epilogue.  That is ~2 extra f32 roundings per group,
+// far inside the tolerance, and it halves the accumulator registers compared
+// with a second "finished groups" set.  A zero scale is replaced by 1e-30 (its
+// group then contributes ~0, as it should).
+//
+// Weights never pass through LDS.  v_mfma_f32_32x32x16_f16 wants, per lane, 8
+// consecutive k of one column: exactly one packed u32 word
+// (rumus-vision/src/quant.rs:98-100).  Lane l of a wave loads the two words of
+// columns 2*(l%32), +1 at word row 2*step + l/32 with one 64-bit load (a wave
+// covers 64 columns x 16 rows of K per step, 256-byte segments) and converts
+// each word to a B fragment in registers (magic-number nibble -> f16, packed f16
+// math).  The conversion yields k in the order 0,4,1,5,2,6,3,7; the A fragments
+// are stored in the same order, and a dot product does not care.  MFMA j of a
+// lane works on columns 2*(l%32)+j, so the two results of a row are adjacent
+// and leave as one float2.  The eight loads of a stage sit in eight registers
+// pairs that are refilled for the next stage as soon as they are consumed, so
+// one stage of weights (4 KB per wave, 32 KB per workgroup) is always in flight.
+//
+// A workgroup is 8 waves side by side = 512 columns (two waves per SIMD, so one
+// converts or rescales while the other multiplies), BM = 32 or 64 rows.  Per
+// stage of 128 rows of K the activations of the BM rows are converted once (hi/lo
+// f16, fragment layout, sums per 16 k for the zero-point term) into one of two
+// LDS buffers while the previous stage is multiplied; one barrier per stage.
+// `perm` (act-order) gathers x columns at this point.
+//
+// The zero-point term of a group, -zp[n] * X[m] with X the sum of x over the
+// group, is a rank-1 update: it is added by one v_mfma_f32_32x32x2_f32 per tile
+// (f32 operands, so nothing is lost), not by the vector ALU.
+//
+// Few output tiles (small m): K is split over gridDim.z workgroups, each
+// writes its partial tile to the workspace, and a second kernel adds the
+// partials in a fixed order (deterministic, no atomics) and the bias.
+#include <type_traits>
+
+#include "w4.h"
+
+namespace rumus {
+
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int kTileCols = 512;   // columns per workgroup (8 waves x 64)
+constexpr int kTileThreads = 512;
+constexpr int kStageK = 128;     // rows of K staged per barrier (8 MFMA steps of 16)
+constexpr int kMaxSplits = 16;
+
+// one packed word -> B fragment, k order 0,4,1,5,2,6,3,7
+__device__ __forceinline__ v8h nibbles_to_f16(uint32_t w) {
+    const v2h k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+    const v2h k64 = {(_Float16)-64.0f, (_Float16)-64.0f};
+    const v2h k16th = {(_Float16)0.0625f, (_Float16)0.0625f};
+    const uint32_t t0 = (w & 0x000F000Fu) | 0x64006400u;          // 1024 + n0, 1024 + n4
+    const uint32_t t1 = (w & 0x00F000F0u) | 0x64006400u;          // 1024 + 16 n1, 1024 + 16 n5
+    const uint32_t w8 = w >> 8;
+    const uint32_t t2 = (w8 & 0x000F000Fu) | 0x64006400u;         // n2, n6
+    const uint32_t t3 = (w8 & 0x00F000F0u) | 0x64006400u;         // 16 n3, 16 n7
+    const v2h h0 = __builtin_bit_cast(v2h, t0) - k1024;
+    const v2h h1 = __builtin_elementwise_fma(__builtin_bit_cast(v2h, t1), k16th, k64);   // exact: (1024+16n)/16 - 64
+    const v2h h2 = __builtin_bit_cast(v2h, t2) - k1024;
+    const v2h h3 = __builtin_elementwise_fma(__builtin_bit_cast(v2h, t3), k16th, k64);
+    return v8h{h0[0], h0[1], h1[0], h1[1], h2[0], h2[1], h3[0], h3[1]};
+}
+
+__device__ __forceinline__ float2 nonzero2(float2 s) {
+    return make_float2(s.x == 0.0f ? 1e-30f : s.x, s.y == 0.0f ? 1e-30f : s.y);
+}
+
+// RT = 32-row tiles per workgroup (BM = 32 * RT).  out = y when gridDim.z == 1,
+// else the partial tiles [split][m][n].
+template <int RT>
+__global__ __launch_bounds__(kTileThreads, 2) void w4_gemm_tile_kernel(W4Args a, float* __restrict__ out,
+                                                                      uint32_t stages_per_split) {
+    constexpr int BM = 32 * RT;
+    constexpr int STEP = RT * 1024;              // bytes of one k16 step of one plane: [row tile][k block][row] x 16
+    constexpr int PLANE = 8 * STEP;
+    __shared__ __attribute__((aligned(16))) uint8_t lds_a[2][2][PLANE];   // [buffer][hi, lo]
+    __shared__ __attribute__((aligned(16))) float lds_xs[2][8][BM];       // [buffer][k16 step][row]: sum of x
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t l32 = lane & 31, kb = lane >> 5;
+    const uint32_t m0 = blockIdx.y * BM;
+    const uint32_t colbase = blockIdx.x * kTileCols + wave * 64 + 2 * l32;   // this lane's 2 columns
+    const bool col_ok = colbase < a.n;                   // n % 4 == 0
+    const uint32_t col_c = col_ok ? colbase : 0;
+    const uint32_t nstages = (a.padded_k + kStageK - 1) / kStageK;
+    const uint32_t st_begin = blockIdx.z * stages_per_split;
+    const uint32_t st_end = min(nstages, st_begin + stages_per_split);
+    const uint32_t word_rows = a.padded_k / 8;
+    const uint32_t k_end = min(a.padded_k, st_end * kStageK);
+
+    // ---- staging role: thread t converts 16 consecutive k (MFMA step t%8) of row t/8 -----
+    const uint32_t s_row = tid >> 3, s_step = tid & 7;
+    const bool s_active = s_row < BM;
+    const bool x_vec = !a.perm && (a.k % 4 == 0) && ((reinterpret_cast<uintptr_t>(a.x) & 15) == 0);
+    float xv[16];
+    auto stage_load = [&](uint32_t st) __attribute__((always_inline)) {
+        if (!s_active) return;
+        const uint32_t k0 = st * kStageK + s_step * 16;
+        const uint32_t row = m0 + s_row;
+        const bool row_ok = row < a.m;
+        const float* xrow = a.x + (uint64_t)min(row, a.m - 1) * a.k;
+        if (x_vec) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t kk = k0 + 4 * i;
+                const bool in = row_ok && kk < a.k;       // k % 4 == 0: all four in or out
+                const float4 v = *reinterpret_cast<const float4*>(xrow + (in ? kk : 0));
+                xv[4 * i] = in ? v.x : 0.0f; xv[4 * i + 1] = in ? v.y : 0.0f;
+                xv[4 * i + 2] = in ? v.z : 0.0f; xv[4 * i + 3] = in ? v.w : 0.0f;
+            }
+        } else {
+            // act-order: the 16 source columns first (contiguous), then the gather
+            uint32_t src[16];
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const uint32_t kk = min(k0 + i, a.k - 1);
+                src[i] = a.perm ? (uint32_t)a.perm[kk] : kk;
+            }
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const float v = xrow[src[i]];
+                xv[i] = (row_ok && k0 + i < a.k) ? v : 0.0f;
+            }
+        }
+    };
+    auto stage_store = [&](uint32_t buf) __attribute__((always_inline)) {
+        if (!s_active) return;
+        float sum = 0.0f;
+        const uint32_t rt = s_row >> 5, r32 = s_row & 31;
+#pragma unroll
+        for (int b = 0; b < 2; b++) {                     // the two 8-k blocks of this thread's step
+            v8h hi, lo;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const int j = (e >> 1) + 4 * (e & 1);     // fragment element e holds k offset j
+                const float x = xv[8 * b + j];
+                const _Float16 h = (_Float16)x;
+                const float back = (float)h;
+                const _Float16 l = (_Float16)(x - back);
+                hi[e] = h;
+                lo[e] = l;
+                sum += back + (float)l;                   // the value the MFMAs see, summed
+            }
+            const uint32_t off = s_step * STEP + (rt * 2 + b) * 512 + r32 * 16;
+            *reinterpret_cast<v8h*>(lds_a[buf][0] + off) = hi;
+            *reinterpret_cast<v8h*>(lds_a[buf][1] + off) = lo;
+        }
+        lds_xs[buf][s_step][s_row] = sum;
+    };
+
+    // ---- weights: one 64-bit load per MFMA step; register s is refilled for the next
+    // stage right after step s has been converted ------------------------------------------
+    uint2 wq[8];
+    auto weight_load = [&](uint32_t st, int s) __attribute__((always_inline)) {
+        const uint32_t kr = min(st * 16 + s * 2 + kb, word_rows - 1);
+        wq[s] = *reinterpret_cast<const uint2*>(a.packed + (uint64_t)kr * a.n + col_c);
+    };
+
+    v16f acc[RT][2];
+#pragma unroll
+    for (int i = 0; i < RT; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    // scale / zero-point of the current group and of the next one (fetched a group ahead)
+    auto meta_load = [&](uint32_t g, float2& sc, float2& zp) __attribute__((always_inline)) {
+        g = min(g, a.num_groups - 1);
+        sc = nonzero2(*reinterpret_cast<const float2*>(a.scales + (uint64_t)g * a.n + col_c));
+        zp = *reinterpret_cast<const float2*>(a.zp + (uint64_t)g * a.n + col_c);
+    };
+    uint32_t g_cur = st_begin * kStageK / a.group_size;
+    float2 sc_cur, zp_cur, sc_next, zp_next;
+    meta_load(g_cur, sc_cur, zp_cur);
+    meta_load(g_cur + 1, sc_next, zp_next);
+    // the zero-point term is settled every `fold_steps` MFMA steps: at group ends, and at
+    // stage ends for groups longer than a stage
+    const uint32_t fold_steps = min(a.group_size, (uint32_t)kStageK) / 16;
+
+    auto fold = [&](uint32_t buf, uint32_t s_last, uint32_t kend) __attribute__((always_inline)) {
+        // rank-1 update acc[i][j] += X[i] (x) (-zp[j]) on the f32 matrix core: operand slot k=0
+        // carries the values (lanes 0..31), slot k=1 (lanes 32..63) is zero
+        const float zb[2] = {kb == 0 ? -zp_cur.x : 0.0f, kb == 0 ? -zp_cur.y : 0.0f};
+#pragma unroll
+        for (int i = 0; i < RT; i++) {
+            float xs = 0.0f;
+            for (uint32_t cc = 0; cc < fold_steps; cc++) xs += lds_xs[buf][s_last - cc][i * 32 + l32];
+            xs = kb == 0 ? xs : 0.0f;
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(xs, zb[j], acc[i][j], 0, 0, 0);
+        }
+        const uint32_t g_after = kend / a.group_size;
+        if (kend < k_end && g_after != g_cur) {           // uniform: a new group starts
+            const float rv[2] = {sc_cur.x / sc_next.x, sc_cur.y / sc_next.y};
+#pragma unroll
+            for (int i = 0; i < RT; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) acc[i][j][r] *= rv[j];
+            g_cur = g_after;
+            sc_cur = sc_next;
+            zp_cur = zp_next;
+            meta_load(g_cur + 1, sc_next, zp_next);
+        }
+    };
+
+    // Multiply stage `st` from LDS buffer `buf`; refill the weight registers for stage st+1.
+    auto compute = [&](uint32_t st, uint32_t buf) __attribute__((always_inline)) {
+        const bool more = st + 1 < st_end;
+#pragma unroll
+        for (int s = 0; s < 8; s++) {
+            v8h bfr[2], ah[RT], al[RT];
+            bfr[0] = nibbles_to_f16(wq[s].x);
+            bfr[1] = nibbles_to_f16(wq[s].y);
+            if (more) weight_load(st + 1, s);
+#pragma unroll
+            for (int i = 0; i < RT; i++) {
+                const uint32_t off = s * STEP + i * 1024 + lane * 16;
+                ah[i] = *reinterpret_cast<const v8h*>(lds_a[buf][0] + off);
+                al[i] = *reinterpret_cast<const v8h*>(lds_a[buf][1] + off);
+            }
+            // all hi products, then all lo products: dependent MFMAs are 2*RT apart
+#pragma unroll
+            for (int i = 0; i < RT; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[i], bfr[j], acc[i][j], 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < RT; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[i], bfr[j], acc[i][j], 0, 0, 0);
+            if ((s + 1) % fold_steps == 0) fold(buf, s, st * kStageK + (s + 1) * 16);
+        }
+    };
+
+    stage_load(st_begin);
+#pragma unroll
+    for (int s = 0; s < 8; s++) weight_load(st_begin, s);
+    stage_store(0);
+    uint32_t buf = 0;
+    for (uint32_t st = st_begin; st < st_end; st++) {
+        __syncthreads();                              // buffer `buf` staged; the other one is free
+        if (st + 1 < st_end) stage_load(st + 1);
+        compute(st, buf);
+        if (st + 1 < st_end) stage_store(buf ^ 1);
+        buf ^= 1;
+    }
+
+    // ---- store: for each row a lane holds 2 adjacent columns -----------------------------
+    if (!col_ok) return;
+    const bool final_out = gridDim.z == 1;
+    float* dst = out + (final_out ? 0 : (uint64_t)blockIdx.z * a.m * a.n);
+    float2 bv = make_float2(0, 0);
+    if (final_out && a.bias) bv = *reinterpret_cast<const float2*>(a.bias + colbase);
+#pragma unroll
+    for (int i = 0; i < RT; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const uint32_t row = m0 + i * 32 + 8 * (r / 4) + 4 * kb + (r % 4);
+            if (row >= a.m) continue;
+            const float2 o = make_float2(fmaf(acc[i][0][r], sc_cur.x, bv.x), fmaf(acc[i][1][r], sc_cur.y, bv.y));
+            *reinterpret_cast<float2*>(dst + (uint64_t)row * a.n + colbase) = o;
+        }
+}
+
+// y = part[0] + part[1] + ... (in that order) + bias; count4 = m*n/4
+__global__ __launch_bounds__(256) void w4_gemm_reduce_kernel(const float4* __restrict__ part,
+                                                             const float* __restrict__ bias,
+                                                             float4* __restrict__ y, uint32_t count4,
+                                                             uint32_t n4, uint32_t splits) {
+    const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= count4) return;
+    float4 s = part[idx];
+    for (uint32_t p = 1; p < splits; p++) {
+        const float4 v = part[(uint64_t)p * count4 + idx];
+        s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+    if (bias) {
+        const float4 b = *reinterpret_cast<const float4*>(bias + 4 * (idx % n4));
+        s.x += b.x; s.y += b.y; s.z += b.z; s.w += b.w;
+    }
+    y[idx] = s;
+}
+
+bool w4_gemm_supported(const W4Args& a) {
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(a.packed) | reinterpret_cast<uintptr_t>(a.scales) |
+                           reinterpret_cast<uintptr_t>(a.zp) | reinterpret_cast<uintptr_t>(a.y) |
+                           (a.bias ? reinterpret_cast<uintptr_t>(a.bias) : 0);
+    // zero-point terms are settled every 32, 64 or 128 rows of K: groups must end there
+    const bool group_ok = a.group_size == 32 || a.group_size == 64 || a.group_size % kStageK == 0;
+    return a.m >= 1 && a.n % 4 == 0 && (bits & 15) == 0 && !a.g_idx && group_ok;
+}
+
+// K splits for `tiles` output tiles on a 256-CU device: enough workgroups to cover the
+// chip while every split keeps at least one stage; capped, since partial tiles cost traffic.
+static uint32_t pick_splits(uint32_t tiles, uint32_t nstages, uint32_t* stages_per_split) {
+    uint32_t want = tiles >= 192 ? 1 : min(min((uint32_t)kMaxSplits, nstages), max(1u, 256 / tiles));
+    const uint32_t sps = ceil_div(nstages, want);
+    *stages_per_split = sps;
+    return ceil_div(nstages, sps);                       // no empty split
+}
+
+template <int RT>
+static int launch_tile(const W4Args& a, hipStream_t s) {
+    const uint32_t tn = ceil_div(a.n, kTileCols), tm = ceil_div(a.m, 32 * RT);
+    const uint32_t nstages = ceil_div(a.padded_k, kStageK);
+    uint32_t sps = nstages;
+    const uint32_t splits = pick_splits(tn * tm, nstages, &sps);
+    float* out = a.y;
+    if (splits > 1) {
+        void* ws = nullptr;
+        if (int rc = workspace_get(s, (size_t)splits * a.m * a.n * sizeof(float), &ws)) return rc;
+        out = static_cast<float*>(ws);
+    }
+    hipLaunchKernelGGL(w4_gemm_tile_kernel<RT>, dim3(tn, tm, splits), dim3(kTileThreads), 0, s, a, out, sps);
+    if (int rc = check_launch("w4_gemm_tile_kernel")) return rc;
+    if (splits > 1) {
+        const uint32_t count4 = (uint32_t)((uint64_t)a.m * a.n / 4);
+        hipLaunchKernelGGL(w4_gemm_reduce_kernel, dim3(ceil_div(count4, 256)), dim3(256), 0, s,
+                           reinterpret_cast<const float4*>(out), a.bias, reinterpret_cast<float4*>(a.y), count4,
+                           a.n / 4, splits);
+        return check_launch("w4_gemm_reduce_kernel");
+    }
+    return RUMUS_HIP_OK;
+}
+
+int w4_launch_gemm(const W4Args& a, hipStream_t s) {
+    RUMUS_REQUIRE((uint64_t)a.m * a.n < (1ull << 32), "qmatmul_int4: m * n must fit 32 bits");
+    if (a.m <= 32) return launch_tile<1>(a, s);
+    return launch_tile<2>(a, s);
+}
+
+}  // namespace rumus
