@@ -55,11 +55,12 @@ int rumus_hip_sync(rumus_hip_stream_t stream);
 
 /* Workspace.  The reference takes every temporary from its BufferPool
  * (rumus/src/backend/gpu/pool.rs:34-75) and returns it on drop; here the only
- * temporaries are the partial sums of matmuls that split K over workgroups
- * (qmatmul_int4 with 9 <= m and few output tiles).  They live in one device
- * buffer per (device, stream), grown on demand inside the call that needs it.
- * A caller that must not allocate later (graph capture, serving loop) reserves
- * the size up front: for qmatmul_int4 at most 16 * m * n * 4 bytes.
+ * temporaries are those of qmatmul_int4 / qmatmul_int4_perm with m > 8: the
+ * partial sums when K is split over workgroups (few output tiles) and the
+ * act-order copy of x.  They live in one device buffer per (device, stream),
+ * grown on demand inside the call that needs it.  A caller that must not
+ * allocate later (graph capture, serving loop) reserves the size up front:
+ * at most (m * k + 16 * m * n) * 4 + 256 bytes per call.
  * rumus_hip_shutdown frees every workspace (no launch may be in flight). */
 int rumus_hip_workspace_reserve(rumus_hip_stream_t stream, uint64_t bytes);
 int rumus_hip_shutdown(void);

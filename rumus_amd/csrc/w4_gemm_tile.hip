@@ -322,17 +322,43 @@ static uint32_t pick_splits(uint32_t tiles, uint32_t nstages, uint32_t* stages_p
     return ceil_div(nstages, sps);                       // no empty split
 }
 
+// xp[r][j] = x[r][perm[j]]: the act-order column gather, done once per call instead of once
+// per workgroup column.  One thread per 4 consecutive j (k % 4 == 0).
+__global__ __launch_bounds__(256) void w4_gather_columns_kernel(const float* __restrict__ x,
+                                                                const int32_t* __restrict__ perm,
+                                                                float* __restrict__ xp, uint32_t m, uint32_t k) {
+    const uint32_t q = blockIdx.x * 256 + threadIdx.x, row = blockIdx.y;
+    if (q * 4 >= k) return;
+    const int4 p = *reinterpret_cast<const int4*>(perm + 4 * q);
+    const float* xr = x + (uint64_t)row * k;
+    const float4 v = make_float4(xr[p.x], xr[p.y], xr[p.z], xr[p.w]);
+    *reinterpret_cast<float4*>(xp + (uint64_t)row * k + 4 * q) = v;
+}
+
 template <int RT>
-static int launch_tile(const W4Args& a, hipStream_t s) {
+static int launch_tile(const W4Args& a_in, hipStream_t s) {
+    W4Args a = a_in;
     const uint32_t tn = ceil_div(a.n, kTileCols), tm = ceil_div(a.m, 32 * RT);
     const uint32_t nstages = ceil_div(a.padded_k, kStageK);
     uint32_t sps = nstages;
     const uint32_t splits = pick_splits(tn * tm, nstages, &sps);
+    // workspace: [gathered activations][partial tiles]
+    const bool gather = a.perm && a.m <= 65535 && a.k % 4 == 0 && ((reinterpret_cast<uintptr_t>(a.perm) & 15) == 0);
+    const size_t x_bytes = gather ? (((size_t)a.m * a.k * sizeof(float) + 255) & ~size_t(255)) : 0;
+    const size_t part_bytes = splits > 1 ? (size_t)splits * a.m * a.n * sizeof(float) : 0;
     float* out = a.y;
-    if (splits > 1) {
+    if (x_bytes + part_bytes) {
         void* ws = nullptr;
-        if (int rc = workspace_get(s, (size_t)splits * a.m * a.n * sizeof(float), &ws)) return rc;
-        out = static_cast<float*>(ws);
+        if (int rc = workspace_get(s, x_bytes + part_bytes, &ws)) return rc;
+        if (gather) {
+            float* xp = static_cast<float*>(ws);
+            hipLaunchKernelGGL(w4_gather_columns_kernel, dim3(ceil_div(a.k / 4, 256), a.m), dim3(256), 0, s, a.x,
+                               a.perm, xp, a.m, a.k);
+            if (int rc = check_launch("w4_gather_columns_kernel")) return rc;
+            a.x = xp;
+            a.perm = nullptr;
+        }
+        if (splits > 1) out = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + x_bytes);
     }
     hipLaunchKernelGGL(w4_gemm_tile_kernel<RT>, dim3(tn, tm, splits), dim3(kTileThreads), 0, s, a, out, sps);
     if (int rc = check_launch("w4_gemm_tile_kernel")) return rc;
