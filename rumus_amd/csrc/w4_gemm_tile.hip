@@ -89,7 +89,10 @@ template <int RT>
 __global__ __launch_bounds__(kTileThreads, 2) void w4_gemm_tile_kernel(W4Args a, float* __restrict__ out,
                                                                       uint32_t stages_per_split) {
     constexpr int BM = 32 * RT;
-    constexpr int STEP = RT * 1024;              // bytes of one k16 step of one plane: [row tile][k block][row] x 16
+    // bytes of one k16 step of one plane: [row tile][k block][row] x 16, plus 128 bytes of skew so
+    // that the eight staging lanes of a row (one step each) do not write to the same banks
+    constexpr int STEP = RT * 1024 + 128;
+    constexpr int NI = RT > 2 ? RT / 2 : 1;      // (row, step) pairs staged per thread
     constexpr int PLANE = 8 * STEP;
     __shared__ __attribute__((aligned(16))) uint8_t lds_a[2][2][PLANE];   // [buffer][hi, lo]
     __shared__ __attribute__((aligned(16))) float lds_xs[2][8][BM];       // [buffer][k16 step][row]: sum of x
@@ -108,62 +111,67 @@ __global__ __launch_bounds__(kTileThreads, 2) void w4_gemm_tile_kernel(W4Args a,
 
     // ---- staging role: thread t converts 16 consecutive k (MFMA step t%8) of row t/8 -----
     const uint32_t s_row = tid >> 3, s_step = tid & 7;
-    const bool s_active = s_row < BM;
+    const bool s_active = s_row < BM;            // BM = 32: half of the threads stage
     const bool x_vec = !a.perm && (a.k % 4 == 0) && ((reinterpret_cast<uintptr_t>(a.x) & 15) == 0);
-    float xv[16];
+    float xv[NI][16];
     auto stage_load = [&](uint32_t st) __attribute__((always_inline)) {
         if (!s_active) return;
         const uint32_t k0 = st * kStageK + s_step * 16;
-        const uint32_t row = m0 + s_row;
-        const bool row_ok = row < a.m;
-        const float* xrow = a.x + (uint64_t)min(row, a.m - 1) * a.k;
-        if (x_vec) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const uint32_t kk = k0 + 4 * i;
-                const bool in = row_ok && kk < a.k;       // k % 4 == 0: all four in or out
-                const float4 v = *reinterpret_cast<const float4*>(xrow + (in ? kk : 0));
-                xv[4 * i] = in ? v.x : 0.0f; xv[4 * i + 1] = in ? v.y : 0.0f;
-                xv[4 * i + 2] = in ? v.z : 0.0f; xv[4 * i + 3] = in ? v.w : 0.0f;
-            }
-        } else {
-            // act-order: the 16 source columns first (contiguous), then the gather
-            uint32_t src[16];
+        for (int it = 0; it < NI; it++) {
+            const uint32_t row = m0 + s_row + 64 * it;
+            const bool row_ok = row < a.m;
+            const float* xrow = a.x + (uint64_t)min(row, a.m - 1) * a.k;
+            if (x_vec) {
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const uint32_t kk = min(k0 + i, a.k - 1);
-                src[i] = a.perm ? (uint32_t)a.perm[kk] : kk;
-            }
+                for (int i = 0; i < 4; i++) {
+                    const uint32_t kk = k0 + 4 * i;
+                    const bool in = row_ok && kk < a.k;   // k % 4 == 0: all four in or out
+                    const float4 v = *reinterpret_cast<const float4*>(xrow + (in ? kk : 0));
+                    xv[it][4 * i] = in ? v.x : 0.0f; xv[it][4 * i + 1] = in ? v.y : 0.0f;
+                    xv[it][4 * i + 2] = in ? v.z : 0.0f; xv[it][4 * i + 3] = in ? v.w : 0.0f;
+                }
+            } else {
+                // act-order: the 16 source columns first (contiguous), then the gather
+                uint32_t src[16];
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const float v = xrow[src[i]];
-                xv[i] = (row_ok && k0 + i < a.k) ? v : 0.0f;
+                for (int i = 0; i < 16; i++) {
+                    const uint32_t kk = min(k0 + i, a.k - 1);
+                    src[i] = a.perm ? (uint32_t)a.perm[kk] : kk;
+                }
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const float v = xrow[src[i]];
+                    xv[it][i] = (row_ok && k0 + i < a.k) ? v : 0.0f;
+                }
             }
         }
     };
-    auto stage_store = [&](uint32_t buf) __attribute__((always_inline)) {
+    // Conversion of the loaded values, in 2*NI pieces of 8 values so that it can be spread
+    // over the MFMA steps of the stage being multiplied.
+    constexpr int PIECES = 2 * NI;
+    float xsum[NI];
+    auto stage_store_piece = [&](uint32_t buf, int piece) __attribute__((always_inline)) {
         if (!s_active) return;
-        float sum = 0.0f;
-        const uint32_t rt = s_row >> 5, r32 = s_row & 31;
+        const int it = piece >> 1, b = piece & 1;         // b: which 8-k block of this thread's step
+        const uint32_t row = s_row + 64 * it;
+        const uint32_t rt = row >> 5, r32 = row & 31;
+        v8h hi, lo;
+        float sum = b ? xsum[it] : 0.0f;
 #pragma unroll
-        for (int b = 0; b < 2; b++) {                     // the two 8-k blocks of this thread's step
-            v8h hi, lo;
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const int j = (e >> 1) + 4 * (e & 1);     // fragment element e holds k offset j
-                const float x = xv[8 * b + j];
-                const _Float16 h = (_Float16)x;
-                const float back = (float)h;
-                const _Float16 l = (_Float16)(x - back);
-                hi[e] = h;
-                lo[e] = l;
-                sum += back + (float)l;                   // the value the MFMAs see, summed
-            }
-            const uint32_t off = s_step * STEP + (rt * 2 + b) * 512 + r32 * 16;
-            *reinterpret_cast<v8h*>(lds_a[buf][0] + off) = hi;
-            *reinterpret_cast<v8h*>(lds_a[buf][1] + off) = lo;
+        for (int e = 0; e < 8; e++) {
+            const int j = (e >> 1) + 4 * (e & 1);         // fragment element e holds k offset j
+            const float x = xv[it][8 * b + j];
+            const _Float16 h = (_Float16)x;
+            hi[e] = h;
+            lo[e] = (_Float16)(x - (float)h);
+            sum += x;                                     // hi + lo equals x to 2^-22 |x|
         }
-        lds_xs[buf][s_step][s_row] = sum;
+        const uint32_t off = s_step * STEP + (rt * 2 + b) * 512 + r32 * 16;
+        *reinterpret_cast<v8h*>(lds_a[buf][0] + off) = hi;
+        *reinterpret_cast<v8h*>(lds_a[buf][1] + off) = lo;
+        xsum[it] = sum;
+        if (b) lds_xs[buf][s_step][row] = sum;
     };
 
     // ---- weights: one 64-bit load per MFMA step; register s is refilled for the next
@@ -252,19 +260,21 @@ __global__ __launch_bounds__(kTileThreads, 2) void w4_gemm_tile_kernel(W4Args a,
                 for (int j = 0; j < 2; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[i], bfr[j], acc[i][j], 0, 0, 0);
             if ((s + 1) % fold_steps == 0) fold(buf, s, st * kStageK + (s + 1) * 16);
+            // the activations of the next stage are converted in the shadow of the last steps
+            if (more && s >= 8 - PIECES) stage_store_piece(buf ^ 1, s - (8 - PIECES));
         }
     };
 
     stage_load(st_begin);
 #pragma unroll
     for (int s = 0; s < 8; s++) weight_load(st_begin, s);
-    stage_store(0);
+#pragma unroll
+    for (int piece = 0; piece < PIECES; piece++) stage_store_piece(0, piece);
     uint32_t buf = 0;
     for (uint32_t st = st_begin; st < st_end; st++) {
         __syncthreads();                              // buffer `buf` staged; the other one is free
         if (st + 1 < st_end) stage_load(st + 1);
         compute(st, buf);
-        if (st + 1 < st_end) stage_store(buf ^ 1);
         buf ^= 1;
     }
 
@@ -375,7 +385,11 @@ static int launch_tile(const W4Args& a_in, hipStream_t s) {
 int w4_launch_gemm(const W4Args& a, hipStream_t s) {
     RUMUS_REQUIRE((uint64_t)a.m * a.n < (1ull << 32), "qmatmul_int4: m * n must fit 32 bits");
     if (a.m <= 32) return launch_tile<1>(a, s);
-    return launch_tile<2>(a, s);
+    // 128-row tiles convert each weight word once per 16 MFMAs instead of 8; worth it once
+    // there are enough of them to fill the chip
+    const uint64_t big_tiles = (uint64_t)ceil_div(a.m, 128) * ceil_div(a.n, kTileCols);
+    if (a.m <= 64 || big_tiles < 192) return launch_tile<2>(a, s);
+    return launch_tile<4>(a, s);
 }
 
 }  // namespace rumus
