@@ -79,15 +79,30 @@ __device__ __forceinline__ v8h nibbles_to_f16(uint32_t w) {
     return v8h{h0[0], h0[1], h1[0], h1[1], h2[0], h2[1], h3[0], h3[1]};
 }
 
+// Workgroup barrier that waits for this wave's LDS traffic only.  __syncthreads() also waits
+// for every global load in flight (vmcnt(0)), which would drain the weight prefetch at each
+// stage; nothing here communicates through global memory inside a workgroup.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_s_waitcnt(0xC07F);          // lgkmcnt(0); vmcnt and expcnt untouched
+    __builtin_amdgcn_s_barrier();
+}
+
 __device__ __forceinline__ float2 nonzero2(float2 s) {
     return make_float2(s.x == 0.0f ? 1e-30f : s.x, s.y == 0.0f ? 1e-30f : s.y);
 }
 
-// RT = 32-row tiles per workgroup (BM = 32 * RT).  out = y when gridDim.z == 1,
-// else the partial tiles [split][m][n].
-template <int RT>
+// RT = 32-row tiles per workgroup (BM = 32 * RT); DEPTH = stages of weights in flight;
+// FOLD = MFMA steps between settlements of the zero-point term (group_size / 16, at most a
+// stage).  out = y when gridDim.z == 1, else the partial tiles [split][m][n].
+//
+// The stage body is straight-line code: loads past the end of the work are clamped to valid
+// addresses and their results never used, instead of being skipped, and nothing is consumed
+// right after it was loaded, so that the memory counter never has to drain.
+template <int RT, int DEPTH, int FOLD>
 __global__ __launch_bounds__(kTileThreads, 2) void w4_gemm_tile_kernel(W4Args a, float* __restrict__ out,
                                                                       uint32_t stages_per_split) {
+    // a.x: rows of a.k floats, a.k % 4 == 0, 16-byte aligned, columns already in weight order
+    // (the launcher copies x into that form when the caller's x is not)
     constexpr int BM = 32 * RT;
     // bytes of one k16 step of one plane: [row tile][k block][row] x 16, plus 128 bytes of skew so
     // that the eight staging lanes of a row (one step each) do not write to the same banks
@@ -112,56 +127,39 @@ __global__ __launch_bounds__(kTileThreads, 2) void w4_gemm_tile_kernel(W4Args a,
     // ---- staging role: thread t converts 16 consecutive k (MFMA step t%8) of row t/8 -----
     const uint32_t s_row = tid >> 3, s_step = tid & 7;
     const bool s_active = s_row < BM;            // BM = 32: half of the threads stage
-    const bool x_vec = !a.perm && (a.k % 4 == 0) && ((reinterpret_cast<uintptr_t>(a.x) & 15) == 0);
-    float xv[NI][16];
-    auto stage_load = [&](uint32_t st) __attribute__((always_inline)) {
+    float4 xraw[DEPTH][NI][4];                   // DEPTH stages of activations in flight, too
+    auto stage_load = [&](uint32_t st, int slot) __attribute__((always_inline)) {
         if (!s_active) return;
         const uint32_t k0 = st * kStageK + s_step * 16;
 #pragma unroll
         for (int it = 0; it < NI; it++) {
-            const uint32_t row = m0 + s_row + 64 * it;
-            const bool row_ok = row < a.m;
-            const float* xrow = a.x + (uint64_t)min(row, a.m - 1) * a.k;
-            if (x_vec) {
+            const float* xrow = a.x + (uint64_t)min(m0 + s_row + 64 * it, a.m - 1) * a.k;
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const uint32_t kk = k0 + 4 * i;
-                    const bool in = row_ok && kk < a.k;   // k % 4 == 0: all four in or out
-                    const float4 v = *reinterpret_cast<const float4*>(xrow + (in ? kk : 0));
-                    xv[it][4 * i] = in ? v.x : 0.0f; xv[it][4 * i + 1] = in ? v.y : 0.0f;
-                    xv[it][4 * i + 2] = in ? v.z : 0.0f; xv[it][4 * i + 3] = in ? v.w : 0.0f;
-                }
-            } else {
-                // act-order: the 16 source columns first (contiguous), then the gather
-                uint32_t src[16];
-#pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    const uint32_t kk = min(k0 + i, a.k - 1);
-                    src[i] = a.perm ? (uint32_t)a.perm[kk] : kk;
-                }
-#pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    const float v = xrow[src[i]];
-                    xv[it][i] = (row_ok && k0 + i < a.k) ? v : 0.0f;
-                }
-            }
+            for (int i = 0; i < 4; i++)
+                xraw[slot][it][i] = *reinterpret_cast<const float4*>(xrow + min(k0 + 4 * i, a.k - 4));
         }
     };
-    // Conversion of the loaded values, in 2*NI pieces of 8 values so that it can be spread
-    // over the MFMA steps of the stage being multiplied.
+    // Conversion of the values loaded for stage `st`, in 2*NI pieces of 8 values so that it can
+    // be spread over the MFMA steps of the stage being multiplied.
     constexpr int PIECES = 2 * NI;
     float xsum[NI];
-    auto stage_store_piece = [&](uint32_t buf, int piece) __attribute__((always_inline)) {
+    auto stage_store_piece = [&](uint32_t st, uint32_t buf, int piece, int slot) __attribute__((always_inline)) {
         if (!s_active) return;
         const int it = piece >> 1, b = piece & 1;         // b: which 8-k block of this thread's step
         const uint32_t row = s_row + 64 * it;
         const uint32_t rt = row >> 5, r32 = row & 31;
+        const uint32_t kk = st * kStageK + s_step * 16 + 8 * b;
+        const bool row_ok = m0 + row < a.m;
+        const float4 q0 = xraw[slot][it][2 * b], q1 = xraw[slot][it][2 * b + 1];
+        const bool in0 = row_ok && kk < a.k, in1 = row_ok && kk + 4 < a.k;   // k % 4 == 0
+        const float xv[8] = {in0 ? q0.x : 0.0f, in0 ? q0.y : 0.0f, in0 ? q0.z : 0.0f, in0 ? q0.w : 0.0f,
+                             in1 ? q1.x : 0.0f, in1 ? q1.y : 0.0f, in1 ? q1.z : 0.0f, in1 ? q1.w : 0.0f};
         v8h hi, lo;
         float sum = b ? xsum[it] : 0.0f;
 #pragma unroll
         for (int e = 0; e < 8; e++) {
             const int j = (e >> 1) + 4 * (e & 1);         // fragment element e holds k offset j
-            const float x = xv[it][8 * b + j];
+            const float x = xv[j];
             const _Float16 h = (_Float16)x;
             hi[e] = h;
             lo[e] = (_Float16)(x - (float)h);
@@ -174,12 +172,12 @@ __global__ __launch_bounds__(kTileThreads, 2) void w4_gemm_tile_kernel(W4Args a,
         if (b) lds_xs[buf][s_step][row] = sum;
     };
 
-    // ---- weights: one 64-bit load per MFMA step; register s is refilled for the next
-    // stage right after step s has been converted ------------------------------------------
-    uint2 wq[8];
-    auto weight_load = [&](uint32_t st, int s) __attribute__((always_inline)) {
+    // ---- weights: one 64-bit load per MFMA step; a register is refilled for DEPTH stages
+    // later right after its step has been converted -----------------------------------------
+    uint2 wq[DEPTH][8];
+    auto weight_load = [&](uint32_t st, int set, int s) __attribute__((always_inline)) {
         const uint32_t kr = min(st * 16 + s * 2 + kb, word_rows - 1);
-        wq[s] = *reinterpret_cast<const uint2*>(a.packed + (uint64_t)kr * a.n + col_c);
+        wq[set][s] = *reinterpret_cast<const uint2*>(a.packed + (uint64_t)kr * a.n + col_c);
     };
 
     v16f acc[RT][2];
@@ -190,28 +188,35 @@ __global__ __launch_bounds__(kTileThreads, 2) void w4_gemm_tile_kernel(W4Args a,
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-    // scale / zero-point of the current group and of the next one (fetched a group ahead)
+    // scale / zero-point: of the current group, and (requested DEPTH stages ahead, like the
+    // weights) of the group that follows each settlement point of a stage
+    constexpr int NF = 8 / FOLD;                 // settlements per stage
     auto meta_load = [&](uint32_t g, float2& sc, float2& zp) __attribute__((always_inline)) {
         g = min(g, a.num_groups - 1);
-        sc = nonzero2(*reinterpret_cast<const float2*>(a.scales + (uint64_t)g * a.n + col_c));
+        sc = *reinterpret_cast<const float2*>(a.scales + (uint64_t)g * a.n + col_c);
         zp = *reinterpret_cast<const float2*>(a.zp + (uint64_t)g * a.n + col_c);
     };
     uint32_t g_cur = st_begin * kStageK / a.group_size;
-    float2 sc_cur, zp_cur, sc_next, zp_next;
+    float2 sc_cur, zp_cur, sc_after[DEPTH][NF], zp_after[DEPTH][NF];
     meta_load(g_cur, sc_cur, zp_cur);
-    meta_load(g_cur + 1, sc_next, zp_next);
-    // the zero-point term is settled every `fold_steps` MFMA steps: at group ends, and at
-    // stage ends for groups longer than a stage
-    const uint32_t fold_steps = min(a.group_size, (uint32_t)kStageK) / 16;
+    sc_cur = nonzero2(sc_cur);
 
-    auto fold = [&](uint32_t buf, uint32_t s_last, uint32_t kend) __attribute__((always_inline)) {
+    // metadata of the groups that follow the settlement points of stage `st`
+    auto stage_meta_load = [&](uint32_t st, int set) __attribute__((always_inline)) {
+#pragma unroll
+        for (int f = 0; f < NF; f++)
+            meta_load((st * kStageK + (f + 1) * FOLD * 16) / a.group_size, sc_after[set][f], zp_after[set][f]);
+    };
+
+    auto fold = [&](uint32_t buf, int s_last, uint32_t kend, int set, int f) __attribute__((always_inline)) {
         // rank-1 update acc[i][j] += X[i] (x) (-zp[j]) on the f32 matrix core: operand slot k=0
         // carries the values (lanes 0..31), slot k=1 (lanes 32..63) is zero
         const float zb[2] = {kb == 0 ? -zp_cur.x : 0.0f, kb == 0 ? -zp_cur.y : 0.0f};
 #pragma unroll
         for (int i = 0; i < RT; i++) {
             float xs = 0.0f;
-            for (uint32_t cc = 0; cc < fold_steps; cc++) xs += lds_xs[buf][s_last - cc][i * 32 + l32];
+#pragma unroll
+            for (int cc = 0; cc < FOLD; cc++) xs += lds_xs[buf][s_last - cc][i * 32 + l32];
             xs = kb == 0 ? xs : 0.0f;
 #pragma unroll
             for (int j = 0; j < 2; j++)
@@ -219,7 +224,8 @@ __global__ __launch_bounds__(kTileThreads, 2) void w4_gemm_tile_kernel(W4Args a,
         }
         const uint32_t g_after = kend / a.group_size;
         if (kend < k_end && g_after != g_cur) {           // uniform: a new group starts
-            const float rv[2] = {sc_cur.x / sc_next.x, sc_cur.y / sc_next.y};
+            const float2 sn = nonzero2(sc_after[set][f]);
+            const float rv[2] = {sc_cur.x / sn.x, sc_cur.y / sn.y};
 #pragma unroll
             for (int i = 0; i < RT; i++)
 #pragma unroll
@@ -227,21 +233,21 @@ __global__ __launch_bounds__(kTileThreads, 2) void w4_gemm_tile_kernel(W4Args a,
 #pragma unroll
                     for (int r = 0; r < 16; r++) acc[i][j][r] *= rv[j];
             g_cur = g_after;
-            sc_cur = sc_next;
-            zp_cur = zp_next;
-            meta_load(g_cur + 1, sc_next, zp_next);
+            sc_cur = sn;
+            zp_cur = zp_after[set][f];
         }
     };
 
-    // Multiply stage `st` from LDS buffer `buf`; refill the weight registers for stage st+1.
-    auto compute = [&](uint32_t st, uint32_t buf) __attribute__((always_inline)) {
-        const bool more = st + 1 < st_end;
+    // Multiply stage `st` from LDS buffer `buf`; refill the weight registers for stage
+    // st+DEPTH and convert the activations of stage st+1 into the other buffer.
+    auto compute = [&](uint32_t st, uint32_t buf, auto set_tag) __attribute__((always_inline)) {
+        constexpr int SET = decltype(set_tag)::value;
 #pragma unroll
         for (int s = 0; s < 8; s++) {
             v8h bfr[2], ah[RT], al[RT];
-            bfr[0] = nibbles_to_f16(wq[s].x);
-            bfr[1] = nibbles_to_f16(wq[s].y);
-            if (more) weight_load(st + 1, s);
+            bfr[0] = nibbles_to_f16(wq[SET][s].x);
+            bfr[1] = nibbles_to_f16(wq[SET][s].y);
+            weight_load(st + DEPTH, SET, s);
 #pragma unroll
             for (int i = 0; i < RT; i++) {
                 const uint32_t off = s * STEP + i * 1024 + lane * 16;
@@ -259,23 +265,37 @@ __global__ __launch_bounds__(kTileThreads, 2) void w4_gemm_tile_kernel(W4Args a,
 #pragma unroll
                 for (int j = 0; j < 2; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[i], bfr[j], acc[i][j], 0, 0, 0);
-            if ((s + 1) % fold_steps == 0) fold(buf, s, st * kStageK + (s + 1) * 16);
-            // the activations of the next stage are converted in the shadow of the last steps
-            if (more && s >= 8 - PIECES) stage_store_piece(buf ^ 1, s - (8 - PIECES));
+            if ((s + 1) % FOLD == 0) fold(buf, s, st * kStageK + (s + 1) * 16, SET, s / FOLD);
+            if (s >= 8 - PIECES) stage_store_piece(st + 1, buf ^ 1, s - (8 - PIECES), DEPTH - 1 - SET);
         }
+        stage_meta_load(st + DEPTH, SET);
     };
 
-    stage_load(st_begin);
+    // Stage st_begin + i lives in weight set and activation slot i % DEPTH.  While stage st is
+    // multiplied, the activations of st+1 (loaded a stage earlier when DEPTH is 2) are converted
+    // and those of st+DEPTH are requested.
+    stage_load(st_begin, 0);
 #pragma unroll
-    for (int s = 0; s < 8; s++) weight_load(st_begin, s);
+    for (int d = 0; d < DEPTH; d++)
 #pragma unroll
-    for (int piece = 0; piece < PIECES; piece++) stage_store_piece(0, piece);
+        for (int s = 0; s < 8; s++) weight_load(st_begin + d, d, s);
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) stage_meta_load(st_begin + d, d);
+    if (DEPTH == 2) stage_load(st_begin + 1, DEPTH - 1);
+#pragma unroll
+    for (int piece = 0; piece < PIECES; piece++) stage_store_piece(st_begin, 0, piece, 0);
     uint32_t buf = 0;
-    for (uint32_t st = st_begin; st < st_end; st++) {
-        __syncthreads();                              // buffer `buf` staged; the other one is free
-        if (st + 1 < st_end) stage_load(st + 1);
-        compute(st, buf);
+    for (uint32_t st = st_begin; st < st_end; st += DEPTH) {
+        lds_barrier();                                // buffer `buf` staged; the other one is free
+        stage_load(st + DEPTH, 0);
+        compute(st, buf, std::integral_constant<int, 0>{});
         buf ^= 1;
+        if (DEPTH == 2 && st + 1 < st_end) {
+            lds_barrier();
+            stage_load(st + 1 + DEPTH, DEPTH - 1);
+            compute(st + 1, buf, std::integral_constant<int, DEPTH - 1>{});
+            buf ^= 1;
+        }
     }
 
     // ---- store: for each row a lane holds 2 adjacent columns -----------------------------
@@ -332,45 +352,48 @@ static uint32_t pick_splits(uint32_t tiles, uint32_t nstages, uint32_t* stages_p
     return ceil_div(nstages, sps);                       // no empty split
 }
 
-// xp[r][j] = x[r][perm[j]]: the act-order column gather, done once per call instead of once
-// per workgroup column.  One thread per 4 consecutive j (k % 4 == 0).
-__global__ __launch_bounds__(256) void w4_gather_columns_kernel(const float* __restrict__ x,
-                                                                const int32_t* __restrict__ perm,
-                                                                float* __restrict__ xp, uint32_t m, uint32_t k) {
-    const uint32_t q = blockIdx.x * 256 + threadIdx.x, row = blockIdx.y;
-    if (q * 4 >= k) return;
-    const int4 p = *reinterpret_cast<const int4*>(perm + 4 * q);
-    const float* xr = x + (uint64_t)row * k;
-    const float4 v = make_float4(xr[p.x], xr[p.y], xr[p.z], xr[p.w]);
-    *reinterpret_cast<float4*>(xp + (uint64_t)row * k + 4 * q) = v;
+// xp[r][j] = x[r][perm[j]] (perm null: j) for j < k, 0 for k <= j < k4: the act-order column
+// gather done once per call instead of once per workgroup column, and the padding / alignment
+// of rows that the tile kernel's 128-bit loads need.
+__global__ __launch_bounds__(256) void w4_prepare_x_kernel(const float* __restrict__ x,
+                                                           const int32_t* __restrict__ perm,
+                                                           float* __restrict__ xp, uint32_t k, uint32_t k4) {
+    const uint32_t j = blockIdx.x * 256 + threadIdx.x, row = blockIdx.y;
+    if (j >= k4) return;
+    float v = 0.0f;
+    if (j < k) v = x[(uint64_t)row * k + (perm ? (uint32_t)perm[j] : j)];
+    xp[(uint64_t)row * k4 + j] = v;
 }
 
-template <int RT>
+template <int RT, int DEPTH, int FOLD>
 static int launch_tile(const W4Args& a_in, hipStream_t s) {
     W4Args a = a_in;
     const uint32_t tn = ceil_div(a.n, kTileCols), tm = ceil_div(a.m, 32 * RT);
     const uint32_t nstages = ceil_div(a.padded_k, kStageK);
     uint32_t sps = nstages;
     const uint32_t splits = pick_splits(tn * tm, nstages, &sps);
-    // workspace: [gathered activations][partial tiles]
-    const bool gather = a.perm && a.m <= 65535 && a.k % 4 == 0 && ((reinterpret_cast<uintptr_t>(a.perm) & 15) == 0);
-    const size_t x_bytes = gather ? (((size_t)a.m * a.k * sizeof(float) + 255) & ~size_t(255)) : 0;
+    // workspace: [activations in the form the kernel reads][partial tiles]
+    const bool prepare = a.perm || a.k % 4 != 0 || (reinterpret_cast<uintptr_t>(a.x) & 15) != 0;
+    const uint32_t k4 = (a.k + 3) & ~3u;
+    RUMUS_REQUIRE(!prepare || a.m <= 65535, "qmatmul_int4: m %u is beyond the grid limit of the activation copy", a.m);
+    const size_t x_bytes = prepare ? (((size_t)a.m * k4 * sizeof(float) + 255) & ~size_t(255)) : 0;
     const size_t part_bytes = splits > 1 ? (size_t)splits * a.m * a.n * sizeof(float) : 0;
     float* out = a.y;
     if (x_bytes + part_bytes) {
         void* ws = nullptr;
         if (int rc = workspace_get(s, x_bytes + part_bytes, &ws)) return rc;
-        if (gather) {
+        if (prepare) {
             float* xp = static_cast<float*>(ws);
-            hipLaunchKernelGGL(w4_gather_columns_kernel, dim3(ceil_div(a.k / 4, 256), a.m), dim3(256), 0, s, a.x,
-                               a.perm, xp, a.m, a.k);
-            if (int rc = check_launch("w4_gather_columns_kernel")) return rc;
+            hipLaunchKernelGGL(w4_prepare_x_kernel, dim3(ceil_div(k4, 256), a.m), dim3(256), 0, s, a.x, a.perm, xp,
+                               a.k, k4);
+            if (int rc = check_launch("w4_prepare_x_kernel")) return rc;
             a.x = xp;
             a.perm = nullptr;
+            a.k = k4;                                     // the added columns are zero
         }
         if (splits > 1) out = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + x_bytes);
     }
-    hipLaunchKernelGGL(w4_gemm_tile_kernel<RT>, dim3(tn, tm, splits), dim3(kTileThreads), 0, s, a, out, sps);
+    hipLaunchKernelGGL((w4_gemm_tile_kernel<RT, DEPTH, FOLD>), dim3(tn, tm, splits), dim3(kTileThreads), 0, s, a, out, sps);
     if (int rc = check_launch("w4_gemm_tile_kernel")) return rc;
     if (splits > 1) {
         const uint32_t count4 = (uint32_t)((uint64_t)a.m * a.n / 4);
@@ -382,14 +405,24 @@ static int launch_tile(const W4Args& a_in, hipStream_t s) {
     return RUMUS_HIP_OK;
 }
 
+template <int RT, int DEPTH>
+static int launch_fold(const W4Args& a, hipStream_t s) {
+    switch (a.group_size) {                              // MFMA steps of 16 per zero-point settlement
+        case 32: return launch_tile<RT, DEPTH, 2>(a, s);
+        case 64: return launch_tile<RT, DEPTH, 4>(a, s);
+        default: return launch_tile<RT, DEPTH, 8>(a, s);  // a multiple of 128: once per stage
+    }
+}
+
 int w4_launch_gemm(const W4Args& a, hipStream_t s) {
     RUMUS_REQUIRE((uint64_t)a.m * a.n < (1ull << 32), "qmatmul_int4: m * n must fit 32 bits");
-    if (a.m <= 32) return launch_tile<1>(a, s);
+    RUMUS_REQUIRE(a.m <= 65535 * 32, "qmatmul_int4: m %u is beyond the grid limit", a.m);
+    if (a.m <= 32) return launch_fold<1, 2>(a, s);
     // 128-row tiles convert each weight word once per 16 MFMAs instead of 8; worth it once
     // there are enough of them to fill the chip
     const uint64_t big_tiles = (uint64_t)ceil_div(a.m, 128) * ceil_div(a.n, kTileCols);
-    if (a.m <= 64 || big_tiles < 192) return launch_tile<2>(a, s);
-    return launch_tile<4>(a, s);
+    if (a.m <= 64 || big_tiles < 192) return launch_fold<2, 2>(a, s);
+    return launch_fold<4, 1>(a, s);
 }
 
 }  // namespace rumus

@@ -300,8 +300,11 @@ static int validate(const W4Args& a, const char* who) {
 static int dispatch(const W4Args& a, hipStream_t s) {
     if (a.m == 0 || a.n == 0) return RUMUS_HIP_OK;
     RUMUS_REQUIRE(a.k > 0, "qmatmul_int4: k must be > 0");
-    if (w4_gemv_dot8_supported(a)) return w4_launch_gemv_dot8(a, s);
-    if (w4_gemv_supported(a)) return w4_launch_gemv(a, s);
+    // The decode kernels cost a fixed amount per row of x; from 6 rows on the matrix-core
+    // kernel (whose cost barely depends on m up to 32) is the faster one.
+    const bool few_rows = a.m <= 5 || !w4_gemm_supported(a);
+    if (few_rows && w4_gemv_dot8_supported(a)) return w4_launch_gemv_dot8(a, s);
+    if (few_rows && w4_gemv_supported(a)) return w4_launch_gemv(a, s);
     if (w4_gemm_supported(a)) return w4_launch_gemm(a, s);
     return w4_launch_generic(a, s);
 }

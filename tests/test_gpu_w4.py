@@ -67,6 +67,13 @@ SHAPES = [
     (100, 2048, 520, 256, False), # group spans two stages
     (20, 1000, 64, 64, True),     # K tail
     (12, 256, 36, 8, False),      # group 8: not an MFMA case -> reference-order kernel
+    (7, 512, 128, 128, True),     # 6..8 rows already take the MFMA kernel
+    (16, 4096, 4096, 128, True),  # few tiles: K split 16 ways over workgroups, ordered reduction
+    (40, 1001, 64, 64, False),    # k % 4 != 0: activations are copied into padded rows first
+    (100, 160, 520, 32, True),    # group 32: four settlements per stage, two row tiles
+    (24, 192, 48, 96, False),     # group 96 does not divide a stage -> reference-order kernel
+    (1536, 256, 8192, 128, True), # enough tiles for the 128-row variant
+    (1500, 128, 8200, 64, False), # 128-row variant, group 64, ragged rows and columns
 ]
 
 
@@ -81,6 +88,23 @@ def test_qmatmul_int4_vs_oracle(ops, m, k, n, g, with_bias):
     want = oracle.qmatmul_int4(x, packed, scales, zp, k, g, bias=b, threads=8)
     got = host(ops.qmatmul_int4(dev(x), dev(packed), dev(scales), dev(zp), k, g,
                                 bias=None if b is None else dev(b)))
+    assert_close(got, want)
+
+
+def test_zero_scale_group_contributes_nothing(ops):
+    # the MFMA kernel keeps its accumulator in units of the current group's scale; a zero scale
+    # must not poison the groups around it
+    say("qmatmul_int4 zero scale")
+    rng = np.random.default_rng(5)
+    m, k, n, g = 16, 512, 64, 128
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    x = rng.normal(0, 1, (m, k)).astype(np.float32)
+    packed, scales, zp = oracle.w4_from_f32(w, g)
+    scales[1, ::2] = 0.0
+    scales[3, 5] = 0.0
+    want = oracle.qmatmul_int4(x, packed, scales, zp, k, g, threads=8)
+    got = host(ops.qmatmul_int4(dev(x), dev(packed), dev(scales), dev(zp), k, g))
+    assert np.isfinite(got).all()
     assert_close(got, want)
 
 
