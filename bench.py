@@ -173,6 +173,27 @@ def bench_i8_gemm(torch, ops, steps=30, warmup=5):
     }
 
 
+def probe_launch_floor():
+    """What a single launch of the GEMV's size can reach on this GPU: an empty kernel, and a
+    kernel that only reads 8 MiB (the packed weights) from 64 rotating buffers, both replayed
+    from a HIP graph (rumus_amd/csrc/probe_mfma.hip).  None when the probe library is absent."""
+    import ctypes
+    path = os.path.join(ROOT, "rumus_amd", "librumus_probe.so")
+    if not os.path.exists(path):
+        return None
+    lib = ctypes.CDLL(path)
+    lib.rumus_probe_read_launch.restype = ctypes.c_int
+    lib.rumus_probe_read_launch.argtypes = [ctypes.c_uint64, ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
+    empty, read = ctypes.c_double(), ctypes.c_double()
+    nbytes = K * N // 2
+    if lib.rumus_probe_read_launch(0, 1, ctypes.byref(empty)) != 0:
+        return None
+    if lib.rumus_probe_read_launch(nbytes, WEIGHT_SETS, ctypes.byref(read)) != 0:
+        return None
+    return {"empty_kernel_us": empty.value, "read_only_us": read.value, "read_only_bytes": nbytes,
+            "read_only_gbs": nbytes / read.value / 1e3}
+
+
 def probe_mfma_ceiling():
     """int8 TOP/s of v_mfma_i32_32x32x32_i8 issued back to back from registers with random
     operand bits (rumus_amd/csrc/probe_mfma.hip, its own small library), or None."""
@@ -297,6 +318,11 @@ def main():
                            "ms_per_step": per_launch_res * 1e3,
                            "note": "single weight set, served by Infinity Cache / L2; not HBM"},
     }
+
+    floor = probe_launch_floor()
+    if floor:
+        out["single_launch_floor"] = floor
+        out["frac_of_read_only_launch"] = floor["read_only_us"] * 1e-6 / per_launch
 
     if args.calibrate_copy:
         src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device="cuda:0").normal_()

@@ -8,6 +8,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <vector>
+
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
@@ -76,4 +78,74 @@ extern "C" int rumus_probe_i8_mfma(int random_bits, double* tops, double* mhz) {
     *tops = ops / (best_ms * 1e-3) / 1e12;
     *mhz = (double)h[0] / (double)h[1] * 100.0;
     return 0;
+}
+
+// ---- what one small memory-bound launch can reach -----------------------------------------
+// A kernel that only reads `bytes` (64 bytes per thread, four 128-bit loads issued at once,
+// one XCD-contiguous slab per workgroup) and folds them into a value it never stores, launched
+// back to back from a graph over `buffers` distinct buffers so that no cache can serve it.
+// bytes = 0 times an empty kernel.  This is the floor for any single launch that must read
+// that many bytes (a decode GEMV reads 9.4 MB): dispatch, first-byte latency and drain included.
+__global__ __launch_bounds__(512) void probe_read_kernel(const uint4* __restrict__ p, uint32_t* sink, uint32_t wgs) {
+    if (!p) {
+        if (threadIdx.x == 9999) sink[0] = 1;
+        return;
+    }
+    const uint32_t b = blockIdx.x, slab = (b % 8) * (wgs / 8) + b / 8;     // one contiguous range per XCD
+    const uint4* q = p + (size_t)slab * 2048 + threadIdx.x;
+    const uint4 a = q[0], c = q[512], d = q[1024], e = q[1536];
+    const uint32_t v = (a.x ^ c.x ^ d.x ^ e.x) | (a.y ^ c.y ^ d.y ^ e.y) | (a.z ^ c.z ^ d.z ^ e.z) | (a.w ^ c.w ^ d.w ^ e.w);
+    if (v == 0x12345678u) sink[threadIdx.x] = v;
+}
+
+extern "C" int rumus_probe_read_launch(uint64_t bytes, int buffers, double* us_per_launch) {
+    const uint32_t wgs = (uint32_t)(bytes / (512 * 64)) / 8 * 8;
+    if (bytes && wgs == 0) return 1;
+    if (buffers < 1 || buffers > 256) return 1;
+    std::vector<uint4*> bufs(bytes ? buffers : 0, nullptr);
+    uint32_t* sink = nullptr;
+    int rc = 1;
+    hipStream_t stream = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    do {
+        if (hipMalloc(&sink, 4096) != hipSuccess) break;
+        bool ok = true;
+        for (auto& b : bufs) {
+            if (hipMalloc(&b, (size_t)wgs * 512 * 64) != hipSuccess) { ok = false; break; }
+            (void)hipMemset(b, 1, (size_t)wgs * 512 * 64);
+        }
+        if (!ok) break;
+        if (hipStreamCreate(&stream) != hipSuccess) break;
+        if (hipDeviceSynchronize() != hipSuccess) break;
+        const int launches = bytes ? buffers : 64;
+        if (hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal) != hipSuccess) break;
+        for (int i = 0; i < launches; i++)
+            hipLaunchKernelGGL(probe_read_kernel, dim3(bytes ? wgs : 256), dim3(512), 0, stream,
+                               bytes ? bufs[i] : nullptr, sink, wgs);
+        if (hipStreamEndCapture(stream, &graph) != hipSuccess) break;
+        if (hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0) != hipSuccess) break;
+        (void)hipEventCreate(&e0);
+        (void)hipEventCreate(&e1);
+        const int replays = 20;
+        for (int w = 0; w < 3; w++) (void)hipGraphLaunch(exec, stream);
+        (void)hipEventRecord(e0, stream);
+        for (int r = 0; r < replays; r++) (void)hipGraphLaunch(exec, stream);
+        (void)hipEventRecord(e1, stream);
+        if (hipEventSynchronize(e1) != hipSuccess) break;
+        float ms = 0;
+        (void)hipEventElapsedTime(&ms, e0, e1);
+        *us_per_launch = (double)ms * 1e3 / ((double)replays * launches);
+        rc = 0;
+    } while (0);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (exec) (void)hipGraphExecDestroy(exec);
+    if (graph) (void)hipGraphDestroy(graph);
+    if (stream) (void)hipStreamDestroy(stream);
+    for (auto b : bufs)
+        if (b) (void)hipFree(b);
+    if (sink) (void)hipFree(sink);
+    return rc;
 }
