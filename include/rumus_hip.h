@@ -55,7 +55,7 @@ int rumus_hip_sync(rumus_hip_stream_t stream);
 
 /* Workspace.  The reference takes every temporary from its BufferPool
  * (rumus/src/backend/gpu/pool.rs:34-75) and returns it on drop; here the only
- * temporaries are those of qmatmul_int4 / qmatmul_int4_perm with m > 8: the
+ * temporaries are those of qmatmul_int4 / qmatmul_int4_perm with m > 5: the
  * partial sums when K is split over workgroups (few output tiles) and the
  * act-order copy of x.  They live in one device buffer per (device, stream),
  * grown on demand inside the call that needs it.  A caller that must not
