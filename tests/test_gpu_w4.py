@@ -257,3 +257,45 @@ def test_headline_shape_properties(ops):
     assert_close(y, oracle.qmatmul_int4(x, pw, sw_, zw, 4096, 128, threads=8))
     y2 = host(ops.qmatmul_int4(dev((-0.5 * x).astype(np.float32)), packed, scales, zp, 4096, 128))
     assert_close(y2, -0.5 * y)
+
+
+def test_workspace_reserved_then_captured_in_a_graph(ops):
+    # K-split GEMM inside a HIP graph: the workspace is reserved on the capture stream first
+    # (the library must not allocate while capturing); every replay, with eager work in
+    # between, must reproduce the eager result bit for bit (fixed-order reduction).
+    say("qmatmul_int4 workspace + graph replay")
+    import torch
+    from rumus_amd import _lib
+    rng = np.random.default_rng(11)
+    m, k, n, g = 16, 1024, 512, 128
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    packed, scales, zp = oracle.w4_from_f32(w, g)
+    d = [dev(a) for a in (packed, scales, zp)]
+    g_idx = (rng.permutation(k) // g).astype(np.int32)
+    ps, perm = ops.w4_actorder_prepare(d[0], dev(g_idx), g)
+    xs = [dev(rng.normal(0, 1, (m, k)).astype(np.float32)) for _ in range(3)]
+    x = torch.empty_like(xs[0])
+    y = torch.empty((m, n), dtype=torch.float32, device="cuda")
+    eager = []
+    for xi in xs:
+        eager.append(host(ops.qmatmul_int4_perm(xi, ps, d[1], d[2], k, g, perm=perm)))
+    side = torch.cuda.Stream()
+    _lib.call("rumus_hip_workspace_reserve", side.cuda_stream, (m * k + 16 * m * n) * 4 + 256)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        ops.qmatmul_int4_perm(x, ps, d[1], d[2], k, g, perm=perm, out=y)
+    for xi, want in zip(xs, eager):
+        x.copy_(xi)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(host(y), want)
+        # eager work between replays, on the default stream
+        np.testing.assert_array_equal(host(ops.qmatmul_int4_perm(xi, ps, d[1], d[2], k, g, perm=perm)), want)
+    # without a reservation a capture on a fresh stream is refused with a clear error
+    fresh = torch.cuda.Stream()
+    g2 = torch.cuda.CUDAGraph()
+    with pytest.raises(Exception, match="workspace"):
+        with torch.cuda.graph(g2, stream=fresh):
+            ops.qmatmul_int4_perm(x, ps, d[1], d[2], k, g, perm=perm, out=y)
