@@ -83,7 +83,7 @@ def bench_gemv(torch, ops, steps, warmup):
     dev = torch.device("cuda:0")
     w0, x0 = workloads.w4_gemv(0)
     x = torch.from_numpy(x0).to(dev)
-    sets = []
+    sets, sets_awq = [], []       # reference storage (f32 zero-points); AWQ storage (u4 zero-points)
     gen = torch.Generator(device=dev).manual_seed(0)
     for i in range(WEIGHT_SETS):
         if i == 0:
@@ -91,6 +91,7 @@ def bench_gemv(torch, ops, steps, warmup):
         else:
             w = torch.randn((K, N), generator=gen, device=dev, dtype=torch.float32) * 0.02
         sets.append(ops.w4_quantize_pack(w, G))
+        sets_awq.append(ops.w4_quantize_pack_awq(w, G))
         del w
     ys = [torch.empty((M, N), dtype=torch.float32, device=dev) for _ in range(WEIGHT_SETS)]
     torch.cuda.synchronize()
@@ -104,13 +105,20 @@ def bench_gemv(torch, ops, steps, warmup):
         for y in ys:
             ops.qmatmul_int4(x, p, s, z, K, G, out=y)
 
+    def burst_rotating_awq():
+        for (p, s, qz), y in zip(sets_awq, ys):
+            ops.qmatmul_int4_zp4(x, p, s, qz, K, G, out=y)
+
     # the timed region of record: EXACTLY `steps` launches, bracketed by device syncs
     sec, launches, used_graph = time_graph(torch, burst_rotating, WEIGHT_SETS, steps, warmup)
     sec_res, launches_res, _ = time_graph(torch, burst_resident, WEIGHT_SETS, steps, warmup)
+    y0 = ys[0].cpu().numpy()
+    sec_awq, launches_awq, _ = time_graph(torch, burst_rotating_awq, WEIGHT_SETS, steps, warmup)
     return {
+        "sec_awq": sec_awq, "launches_awq": launches_awq,
         "sec": sec, "launches": launches, "graph": used_graph,
         "sec_resident": sec_res, "launches_resident": launches_res,
-        "x": x0, "w": w0, "y0": ys[0].cpu().numpy(),
+        "x": x0, "w": w0, "y0": y0,
     }
 
 
@@ -314,6 +322,10 @@ def main():
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": gbs / HBM_PEAK_GBS, "traffic": GEMV_TRAFFIC_BYTES},
         "gbs_at_u4_zero_point_bytes": BYTES_U4_ZP / per_launch / 1e9,
+        "awq_storage_u4_zero_points": {
+            "ms_per_step": r["sec_awq"] / r["launches_awq"] * 1e3, "bytes_per_step": BYTES_U4_ZP,
+            "gbs": BYTES_U4_ZP / (r["sec_awq"] / r["launches_awq"]) / 1e9,
+            "note": "same shape with integer zero-points packed eight per word (rumus_hip_qmatmul_int4_zp4)"},
         "cache_resident": {"gbs": BYTES_F32_ZP / per_launch_res / 1e9,
                            "ms_per_step": per_launch_res * 1e3,
                            "note": "single weight set, served by Infinity Cache / L2; not HBM"},

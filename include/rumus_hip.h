@@ -145,6 +145,19 @@ int rumus_hip_w4_quantize_pack_sym(const float* w, uint32_t k, uint32_t n,
                                    float* scales, float* zero_points,
                                    rumus_hip_stream_t stream);
 
+/* EXTENSION: AWQ storage, integer zero-points packed eight per u32 along n
+ * (the reference keeps an unrounded f32 zero-point per group and column,
+ * quant.rs:77-79, which a u4 cannot hold, so this is a second format, not a
+ * re-encoding):  scale = max(max-min, 1e-5)/15,
+ *   z = clamp(-rint(min/scale), 0, 15),  q = clamp(rint(w/scale) + z, 0, 15),
+ * rint = half to even (AutoAWQ's pseudo-quantizer).  packed and scales as
+ * above; qzeros u32 [num_groups, n/8], column col in bits 4*(col%8) of word
+ * col/8.  EINVAL unless group_size % 8 == 0 and n % 8 == 0. */
+int rumus_hip_w4_quantize_pack_awq(const float* w, uint32_t k, uint32_t n,
+                                   uint32_t group_size, uint32_t* packed,
+                                   float* scales, uint32_t* qzeros,
+                                   rumus_hip_stream_t stream);
+
 /* custom_forward(&QMatMulINT4FwdOp, [x, packed, scales, zp]) followed by
  * add_bias (rumus-vision/src/quant.rs:191-221,228-256; kernel
  * shaders/qmatmul_int4.wgsl:40-87).  The six scalars are the op's uniform
@@ -188,6 +201,16 @@ int rumus_hip_qmatmul_int4_perm(const float* x, const uint32_t* packed_sorted,
                                 uint32_t m, uint32_t k, uint32_t n, uint32_t padded_k,
                                 uint32_t group_size, uint32_t num_groups,
                                 rumus_hip_stream_t stream);
+
+/* EXTENSION: qmatmul_int4_perm on AWQ storage: zero-points come as qzeros
+ * (layout above) instead of f32.  perm may be NULL (plain k order).
+ * EINVAL also unless n % 8 == 0. */
+int rumus_hip_qmatmul_int4_zp4(const float* x, const uint32_t* packed,
+                               const float* scales, const uint32_t* qzeros,
+                               const float* bias, const int32_t* perm, float* y,
+                               uint32_t m, uint32_t k, uint32_t n, uint32_t padded_k,
+                               uint32_t group_size, uint32_t num_groups,
+                               rumus_hip_stream_t stream);
 
 #ifdef __cplusplus
 }

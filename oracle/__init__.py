@@ -81,6 +81,30 @@ def w4_from_f32(w, group_size: int, symmetric: bool = False):
     return packed, scales, zp
 
 
+def w4_awq_from_f32(w, group_size: int):
+    """AWQ storage: w [K,N] -> (packed u32 [padded_k/8, N], scales f32 [G, N], qzeros u32 [G, N/8])."""
+    w = _f32(w)
+    k, n = w.shape
+    if group_size <= 0 or group_size % 8 or n % 8:
+        raise ValueError("group_size and n must be multiples of 8")
+    padded_k, g = w4_geometry(k, group_size)
+    packed = np.zeros((padded_k // 8, n), np.uint32)
+    scales = np.zeros((g, n), np.float32)
+    qzeros = np.zeros((g, n // 8), np.uint32)
+    rc = lib().orc_w4_awq_from_f32(_p(w), C.c_size_t(k), C.c_size_t(n), C.c_size_t(group_size),
+                                   _p(packed), _p(scales), _p(qzeros))
+    if rc != 0:
+        raise RuntimeError(f"oracle w4_awq_from_f32 failed: {rc}")
+    return packed, scales, qzeros
+
+
+def w4_qzeros_unpack(qzeros, n: int):
+    """qzeros u32 [G, N/8] -> zero-points f32 [G, N] (column col in bits 4*(col%8) of word col/8)."""
+    qzeros = np.ascontiguousarray(qzeros, np.uint32)
+    cols = np.arange(n)
+    return ((qzeros[:, cols // 8] >> (4 * (cols % 8)).astype(np.uint32)) & 0xF).astype(np.float32)
+
+
 def qmatmul_int4(x, packed, scales, zp, k: int, group_size: int, bias=None,
                  g_idx=None, threads: int = 1):
     x = _f32(x)

@@ -184,6 +184,42 @@ int orc_w4_sym_from_f32(const float* data, size_t k, size_t n, size_t group_size
     return 0;
 }
 
+/* EXTENSION: AWQ storage.  Integer zero-points, eight per u32 along N.
+ *   scale = max(max - min, 1e-5) / 15;  z = clamp(-rint(min / scale), 0, 15)
+ *   q = clamp(rint(w / scale) + z, 0, 15)          (rint: half to even)
+ * which is AutoAWQ's pseudo_quantize_tensor with zero_point=True on w.view(-1, group).
+ * qzeros[g * (n/8) + col/8] holds z of column col in bits 4*(col%8) .. +3. */
+int orc_w4_awq_from_f32(const float* data, size_t k, size_t n, size_t group_size,
+                        uint32_t* packed, float* scales, uint32_t* qzeros) {
+    if (group_size == 0 || group_size % 8 != 0 || n % 8 != 0) return -1;
+    size_t padded_k = ((k + group_size - 1) / group_size) * group_size;
+    size_t num_groups = padded_k / group_size;
+    memset(packed, 0, (padded_k / 8) * n * sizeof(uint32_t));
+    memset(qzeros, 0, num_groups * (n / 8) * sizeof(uint32_t));
+    for (size_t col = 0; col < n; col++) {
+        for (size_t g = 0; g < num_groups; g++) {
+            float mn = FLT_MAX, mx = -FLT_MAX;
+            for (size_t row = g * group_size; row < (g + 1) * group_size; row++) {
+                float v = row < k ? data[row * n + col] : 0.0f;
+                if (v < mn) mn = v;
+                if (v > mx) mx = v;
+            }
+            float range = mx - mn;
+            if (!(range > 1e-5f)) range = 1e-5f;
+            float scale = range / 15.0f;
+            int32_t z = clamp_i32(-f32_as_i32_sat(rintf(mn / scale)), 0, 15);
+            scales[g * n + col] = scale;
+            qzeros[g * (n / 8) + col / 8] |= (uint32_t)z << ((col % 8) * 4u);
+            for (size_t row = g * group_size; row < (g + 1) * group_size; row++) {
+                float v = row < k ? data[row * n + col] : 0.0f;
+                int32_t q = clamp_i32(f32_as_i32_sat(rintf(v / scale)) + z, 0, 15);
+                packed[(row / 8) * n + col] |= (uint32_t)q << ((row % 8) * 4u);
+            }
+        }
+    }
+    return 0;
+}
+
 /* qmatmul_int4.wgsl:40-87 */
 void orc_qmatmul_int4(const float* x, const uint32_t* packed, const float* scales,
                       const float* zp, const float* bias, const int32_t* g_idx,

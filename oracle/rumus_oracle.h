@@ -24,6 +24,9 @@
  *   orc_i8_gemm_i32         EXTENSION: numpy int32/int64 matmul, bit-exact
  *   orc_i8_rescale_bias     EXTENSION: float64 closed form
  *   orc_w4_sym_from_f32     EXTENSION: known answers (zp=8, scale=max|w|/7)
+ *   orc_w4_awq_from_f32     EXTENSION: known answers (exact power-of-two scale,
+ *                           half-even ties, nibble order of qzeros) + numpy
+ *                           restatement of the published AutoAWQ formula
  * The reference ships no test, fixture or golden vector for this path and its
  * Rust/WGSL sources cannot be built in this environment, so none of the above
  * is pinned by running the reference; f32 matmul outputs of the reference
@@ -52,6 +55,13 @@ int orc_w4_from_f32(const float* data, size_t k, size_t n, size_t group_size,
  * zero_points (may be NULL) is filled with 8.0f. */
 int orc_w4_sym_from_f32(const float* data, size_t k, size_t n, size_t group_size,
                         uint32_t* packed, float* scales, float* zero_points);
+
+/* EXTENSION: AWQ storage (integer zero-points, eight per u32 along N):
+ * scale = max(max-min, 1e-5)/15, z = clamp(-rint(min/scale), 0, 15),
+ * q = clamp(rint(w/scale) + z, 0, 15), rint = half to even.
+ * qzeros [num_groups, n/8], column col in bits 4*(col%8).  -1 unless n % 8 == 0. */
+int orc_w4_awq_from_f32(const float* data, size_t k, size_t n, size_t group_size,
+                        uint32_t* packed, float* scales, uint32_t* qzeros);
 
 /* rumus-vision/src/shaders/qmatmul_int4.wgsl:40-87 (one invocation per
  * (row, col); strictly ascending k; w=(f32(q)-zp)*scale, then sum += a*w).

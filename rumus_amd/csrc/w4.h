@@ -18,7 +18,23 @@ struct W4Args {
     const int32_t* perm;
     float* y;
     uint32_t m, k, n, padded_k, group_size, num_groups;
+    // AWQ storage (or null): integer zero-points, eight per word along n, column col in bits
+    // 4*(col%8) of word g*(n/8) + col/8; `zp` is null then and n % 8 == 0
+    const uint32_t* zp4;
 };
+
+// zero-points of 4 (col % 4 == 0) or 2 (col % 2 == 0) adjacent columns from the packed form
+__device__ __forceinline__ float4 w4_zp4_load4(const uint32_t* zp4, uint32_t g, uint32_t n, uint32_t col) {
+    const uint32_t v = zp4[(uint64_t)g * (n / 8) + col / 8] >> ((col & 4u) * 4u);
+    return make_float4((float)(v & 15u), (float)((v >> 4) & 15u), (float)((v >> 8) & 15u), (float)((v >> 12) & 15u));
+}
+__device__ __forceinline__ float2 w4_zp4_load2(const uint32_t* zp4, uint32_t g, uint32_t n, uint32_t col) {
+    const uint32_t v = zp4[(uint64_t)g * (n / 8) + col / 8] >> ((col & 6u) * 4u);
+    return make_float2((float)(v & 15u), (float)((v >> 4) & 15u));
+}
+__device__ __forceinline__ float w4_zp4_load1(const uint32_t* zp4, uint64_t g, uint32_t n, uint32_t col) {
+    return (float)((zp4[g * (n / 8) + col / 8] >> ((col & 7u) * 4u)) & 15u);
+}
 
 // Reference-order kernel: any shape, g_idx and perm; one thread per column.
 int w4_launch_generic(const W4Args& a, hipStream_t s);

@@ -93,12 +93,12 @@ __device__ __forceinline__ float2 nonzero2(float2 s) {
 
 // RT = 32-row tiles per workgroup (BM = 32 * RT); DEPTH = stages of weights in flight;
 // FOLD = MFMA steps between settlements of the zero-point term (group_size / 16, at most a
-// stage).  out = y when gridDim.z == 1, else the partial tiles [split][m][n].
+// stage); ZP4: zero-points come packed, eight integers per word along n.  out = y when gridDim.z == 1, else the partial tiles [split][m][n].
 //
 // The stage body is straight-line code: loads past the end of the work are clamped to valid
 // addresses and their results never used, instead of being skipped, and nothing is consumed
 // right after it was loaded, so that the memory counter never has to drain.
-template <int RT, int DEPTH, int FOLD>
+template <int RT, int DEPTH, int FOLD, bool ZP4>
 __global__ __launch_bounds__(kTileThreads, 2) void w4_gemm_tile_kernel(W4Args a, float* __restrict__ out,
                                                                       uint32_t stages_per_split) {
     // a.x: rows of a.k floats, a.k % 4 == 0, 16-byte aligned, columns already in weight order
@@ -194,7 +194,8 @@ __global__ __launch_bounds__(kTileThreads, 2) void w4_gemm_tile_kernel(W4Args a,
     auto meta_load = [&](uint32_t g, float2& sc, float2& zp) __attribute__((always_inline)) {
         g = min(g, a.num_groups - 1);
         sc = *reinterpret_cast<const float2*>(a.scales + (uint64_t)g * a.n + col_c);
-        zp = *reinterpret_cast<const float2*>(a.zp + (uint64_t)g * a.n + col_c);
+        zp = ZP4 ? w4_zp4_load2(a.zp4, g, a.n, col_c)
+                 : *reinterpret_cast<const float2*>(a.zp + (uint64_t)g * a.n + col_c);
     };
     uint32_t g_cur = st_begin * kStageK / a.group_size;
     float2 sc_cur, zp_cur, sc_after[DEPTH][NF], zp_after[DEPTH][NF];
@@ -393,7 +394,12 @@ static int launch_tile(const W4Args& a_in, hipStream_t s) {
         }
         if (splits > 1) out = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + x_bytes);
     }
-    hipLaunchKernelGGL((w4_gemm_tile_kernel<RT, DEPTH, FOLD>), dim3(tn, tm, splits), dim3(kTileThreads), 0, s, a, out, sps);
+    if (a.zp4)
+        hipLaunchKernelGGL((w4_gemm_tile_kernel<RT, DEPTH, FOLD, true>), dim3(tn, tm, splits), dim3(kTileThreads), 0,
+                           s, a, out, sps);
+    else
+        hipLaunchKernelGGL((w4_gemm_tile_kernel<RT, DEPTH, FOLD, false>), dim3(tn, tm, splits), dim3(kTileThreads), 0,
+                           s, a, out, sps);
     if (int rc = check_launch("w4_gemm_tile_kernel")) return rc;
     if (splits > 1) {
         const uint32_t count4 = (uint32_t)((uint64_t)a.m * a.n / 4);

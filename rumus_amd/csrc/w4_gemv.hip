@@ -26,7 +26,7 @@ __global__ __launch_bounds__(64) void w4_generic_kernel(W4Args a) {
     const uint32_t wpg = a.group_size / 8;
     for (uint32_t g = 0; g < a.num_groups; g++) {
         float scale = a.scales[(uint64_t)g * a.n + col];
-        float z = a.zp[(uint64_t)g * a.n + col];
+        float z = a.zp4 ? w4_zp4_load1(a.zp4, g, a.n, col) : a.zp[(uint64_t)g * a.n + col];
         for (uint32_t w = 0; w < wpg; w++) {
             const uint32_t k_base = g * a.group_size + w * 8;
             if (k_base >= a.k) break;
@@ -36,9 +36,9 @@ __global__ __launch_bounds__(64) void w4_generic_kernel(W4Args a) {
                 if (kk >= a.k) break;  // padding rows (qmatmul_int4.wgsl:71)
                 const float q = (float)((word >> (4 * j)) & 0xFu);
                 if (a.g_idx) {
-                    const uint64_t mi = (uint64_t)a.g_idx[kk] * a.n + col;
+                    const uint64_t gi = (uint64_t)a.g_idx[kk], mi = gi * a.n + col;
                     scale = a.scales[mi];
-                    z = a.zp[mi];
+                    z = a.zp4 ? w4_zp4_load1(a.zp4, gi, a.n, col) : a.zp[mi];
                 }
                 const float wv = __fmul_rn(__fsub_rn(q, z), scale);
                 const uint32_t xk = a.perm ? (uint32_t)a.perm[kk] : kk;
@@ -207,7 +207,7 @@ static size_t gemv_lds_bytes(const W4Args& a) {
 bool w4_gemv_supported(const W4Args& a) {
     const uintptr_t bits = reinterpret_cast<uintptr_t>(a.packed) | reinterpret_cast<uintptr_t>(a.scales) |
                            reinterpret_cast<uintptr_t>(a.zp);
-    return a.m >= 1 && a.m <= 8 && a.n % 4 == 0 && (bits & 15) == 0 && !a.g_idx &&
+    return a.m >= 1 && a.m <= 8 && a.n % 4 == 0 && (bits & 15) == 0 && !a.g_idx && !a.zp4 &&
            gemv_lds_bytes(a) <= 64 * 1024;
 }
 
@@ -293,7 +293,8 @@ static int validate(const W4Args& a, const char* who) {
     RUMUS_REQUIRE(a.k <= a.padded_k && a.padded_k < a.k + a.group_size,
                   "%s: padded_k %u does not pad k %u to group_size %u", who, a.padded_k, a.k,
                   a.group_size);
-    RUMUS_REQUIRE(a.x && a.packed && a.scales && a.zp && a.y, "%s: null buffer", who);
+    RUMUS_REQUIRE(a.x && a.packed && a.scales && (a.zp || a.zp4) && a.y, "%s: null buffer", who);
+    RUMUS_REQUIRE(!a.zp4 || a.n % 8 == 0, "%s: packed zero-points need n %% 8 == 0 (got %u)", who, a.n);
     return RUMUS_HIP_OK;
 }
 
@@ -332,6 +333,16 @@ int rumus_hip_qmatmul_int4_perm(const float* x, const uint32_t* packed_sorted, c
     if (int rc = validate(a, "qmatmul_int4_perm")) return rc;
     RUMUS_REQUIRE(!perm || k == padded_k, "qmatmul_int4_perm: perm needs k == padded_k (%u vs %u)", k,
                   padded_k);
+    return dispatch(a, as_stream(stream));
+}
+
+int rumus_hip_qmatmul_int4_zp4(const float* x, const uint32_t* packed, const float* scales,
+                               const uint32_t* qzeros, const float* bias, const int32_t* perm, float* y,
+                               uint32_t m, uint32_t k, uint32_t n, uint32_t padded_k, uint32_t group_size,
+                               uint32_t num_groups, rumus_hip_stream_t stream) {
+    W4Args a{x, packed, scales, nullptr, bias, nullptr, perm, y, m, k, n, padded_k, group_size, num_groups, qzeros};
+    if (int rc = validate(a, "qmatmul_int4_zp4")) return rc;
+    RUMUS_REQUIRE(!perm || k == padded_k, "qmatmul_int4_zp4: perm needs k == padded_k (%u vs %u)", k, padded_k);
     return dispatch(a, as_stream(stream));
 }
 

@@ -68,7 +68,8 @@ __device__ __forceinline__ float reduce_row_lanes(float v) {
 // T threads = T/4 quads; a quad owns OCT consecutive word rows per sweep and
 // each of its lanes prepares OPL = OCT/4 of them.  FASTX: activations are
 // read with 128-bit loads (no perm, k % 8 == 0, 16-byte aligned x).
-template <int M, int T, int OCT, bool FASTX>
+// ZP4: `zps` points at packed integer zero-points (eight per word along n) instead of floats.
+template <int M, int T, int OCT, bool FASTX, bool ZP4>
 __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
     const uint32_t* __restrict__ packed, const float* __restrict__ scales,
     const float* __restrict__ zps, const float* __restrict__ xin, float* __restrict__ yout,
@@ -140,7 +141,8 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
         for (int u = 0; u < OCT; u++) w[u] = *reinterpret_cast<const uint4*>(p + (uint64_t)u * n);
         const uint32_t g = (ch * 8 * OCT) / group_size;
         float4 sc = *reinterpret_cast<const float4*>(scales + (uint64_t)g * n + col_c);
-        const float4 zp = *reinterpret_cast<const float4*>(zps + (uint64_t)g * n + col_c);
+        const float4 zp = ZP4 ? w4_zp4_load4(reinterpret_cast<const uint32_t*>(zps), g, n, col_c)
+                              : *reinterpret_cast<const float4*>(zps + (uint64_t)g * n + col_c);
         if (!(live && col_ok)) sc = make_float4(0, 0, 0, 0);
 
         uint32_t wv[OCT][4];
@@ -272,18 +274,24 @@ bool w4_gemv_dot8_supported(const W4Args& a) {
            a.group_size % (8 * kD8Oct) == 0;
 }
 
+template <int M, bool FASTX, bool ZP4>
+static void launch_variant(const W4Args& a, hipStream_t s) {
+    const float* zps = ZP4 ? reinterpret_cast<const float*>(a.zp4) : a.zp;
+    hipLaunchKernelGGL((w4_gemv_dot8_kernel<M, kD8Threads, kD8Oct, FASTX, ZP4>), dim3(ceil_div(a.n, kD8Cols)),
+                       dim3(kD8Threads), 0, s, a.packed, a.scales, zps, a.x, a.y, a.n, a.k, a.padded_k,
+                       a.group_size, a.bias, a.perm);
+}
+
 template <int M>
 static int launch_m(const W4Args& a, hipStream_t s) {
-    const uint32_t ncolchunks = ceil_div(a.n, kD8Cols);
     const bool fast_x = !a.perm && (a.k % 8 == 0) && ((reinterpret_cast<uintptr_t>(a.x) & 15) == 0);
-    if (fast_x)
-        hipLaunchKernelGGL((w4_gemv_dot8_kernel<M, kD8Threads, kD8Oct, true>), dim3(ncolchunks),
-                           dim3(kD8Threads), 0, s, a.packed, a.scales, a.zp, a.x, a.y, a.n, a.k,
-                           a.padded_k, a.group_size, a.bias, a.perm);
-    else
-        hipLaunchKernelGGL((w4_gemv_dot8_kernel<M, kD8Threads, kD8Oct, false>), dim3(ncolchunks),
-                           dim3(kD8Threads), 0, s, a.packed, a.scales, a.zp, a.x, a.y, a.n, a.k,
-                           a.padded_k, a.group_size, a.bias, a.perm);
+    if (a.zp4) {
+        if (fast_x) launch_variant<M, true, true>(a, s);
+        else launch_variant<M, false, true>(a, s);
+    } else {
+        if (fast_x) launch_variant<M, true, false>(a, s);
+        else launch_variant<M, false, false>(a, s);
+    }
     return check_launch("w4_gemv_dot8_kernel");
 }
 

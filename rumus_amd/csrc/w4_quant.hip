@@ -65,6 +65,48 @@ __global__ __launch_bounds__(256) void w4_quantize_pack_kernel(
     }
 }
 
+// AWQ storage: integer zero-points packed eight per word along n.
+//   scale = max(max - min, 1e-5) / 15;  z = clamp(-rint(min / scale), 0, 15);
+//   q = clamp(rint(w / scale) + z, 0, 15)        (rint: half to even)
+// Same thread layout as above; the eight lanes that share a zero-point word combine their
+// nibbles with lane exchanges (n % 8 == 0, so the eight are all inside or all outside).
+__global__ __launch_bounds__(256) void w4_quantize_pack_awq_kernel(
+    const float* __restrict__ w, uint32_t k, uint32_t n, uint32_t gs,
+    uint32_t* __restrict__ packed, float* __restrict__ scales, uint32_t* __restrict__ qzeros) {
+    const uint32_t col = blockIdx.x * 256 + threadIdx.x;
+    const uint32_t g = blockIdx.y;
+    if (col >= n) return;
+    const uint32_t r0 = g * gs;
+    float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
+    for (uint32_t r = r0; r < r0 + gs; r++) {
+        const float v = r < k ? w[(uint64_t)r * n + col] : 0.0f;
+        if (v < mn) mn = v;
+        if (v > mx) mx = v;
+    }
+    float range = __fsub_rn(mx, mn);
+    if (!(range > 1e-5f)) range = 1e-5f;
+    const float scale = __fdiv_rn(range, 15.0f);
+    const float zf = fminf(fmaxf(-rintf(__fdiv_rn(mn, scale)), 0.0f), 15.0f);   // NaN -> 0
+    scales[(uint64_t)g * n + col] = scale;
+    uint32_t zw = (uint32_t)zf << (4 * (col & 7));
+    zw |= __shfl_xor(zw, 1);
+    zw |= __shfl_xor(zw, 2);
+    zw |= __shfl_xor(zw, 4);
+    if ((col & 7) == 0) qzeros[(uint64_t)g * (n / 8) + col / 8] = zw;
+    for (uint32_t wr = 0; wr < gs / 8; wr++) {
+        uint32_t word = 0;
+#pragma unroll
+        for (uint32_t j = 0; j < 8; j++) {
+            const uint32_t r = r0 + wr * 8 + j;
+            const float v = r < k ? w[(uint64_t)r * n + col] : 0.0f;
+            float t = __fadd_rn(rintf(__fdiv_rn(v, scale)), zf);
+            t = fminf(fmaxf(t, 0.0f), 15.0f);
+            word |= (uint32_t)t << (4 * j);
+        }
+        packed[(uint64_t)(r0 / 8 + wr) * n + col] = word;
+    }
+}
+
 // packed_sorted word (jr, col) gathers the nibbles of original rows
 // perm[8*jr .. 8*jr+7].
 __global__ __launch_bounds__(256) void w4_gather_rows_kernel(const uint32_t* __restrict__ packed,
@@ -106,6 +148,20 @@ int rumus_hip_w4_quantize_pack(const float* w, uint32_t k, uint32_t n, uint32_t 
                                uint32_t* packed, float* scales, float* zero_points,
                                rumus_hip_stream_t stream) {
     return quantize_pack<false>(w, k, n, group_size, packed, scales, zero_points, as_stream(stream));
+}
+
+int rumus_hip_w4_quantize_pack_awq(const float* w, uint32_t k, uint32_t n, uint32_t group_size,
+                                   uint32_t* packed, float* scales, uint32_t* qzeros,
+                                   rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE(group_size > 0 && group_size % 8 == 0,
+                  "w4_quantize_pack_awq: group_size must be a multiple of 8 (got %u)", group_size);
+    RUMUS_REQUIRE(n % 8 == 0, "w4_quantize_pack_awq: n must be a multiple of 8 (got %u)", n);
+    RUMUS_REQUIRE(w && packed && scales && qzeros, "w4_quantize_pack_awq: null buffer");
+    if (k == 0 || n == 0) return RUMUS_HIP_OK;
+    const uint32_t groups = ceil_div(k, group_size);
+    hipLaunchKernelGGL(w4_quantize_pack_awq_kernel, dim3(ceil_div(n, 256), groups), dim3(256), 0,
+                       as_stream(stream), w, k, n, group_size, packed, scales, qzeros);
+    return check_launch("w4_quantize_pack_awq_kernel");
 }
 
 int rumus_hip_w4_quantize_pack_sym(const float* w, uint32_t k, uint32_t n, uint32_t group_size,

@@ -144,6 +144,32 @@ def w4_quantize_pack(w: torch.Tensor, group_size: int, symmetric: bool = False):
     return packed, scales, zp
 
 
+def w4_quantize_pack_awq(w: torch.Tensor, group_size: int):
+    """AWQ storage: (packed int32 [padded_k/8, n], scales f32 [groups, n], qzeros int32 [groups, n/8])."""
+    k, n = w.shape
+    padded_k, groups = w4_geometry(k, max(group_size, 1))
+    packed = torch.empty((max(padded_k // 8, 1), n), dtype=torch.int32, device=w.device)
+    scales = torch.empty((groups, n), dtype=torch.float32, device=w.device)
+    qzeros = torch.empty((groups, max(n // 8, 1)), dtype=torch.int32, device=w.device)
+    call("rumus_hip_w4_quantize_pack_awq", _dev(w, torch.float32, "w"), k, n, group_size, packed.data_ptr(),
+         scales.data_ptr(), qzeros.data_ptr(), _stream())
+    return packed, scales, qzeros
+
+
+def qmatmul_int4_zp4(x, packed, scales, qzeros, k, group_size, bias=None, perm=None, out=None):
+    m = x.shape[0]
+    n = packed.shape[1]
+    if x.dim() != 2 or x.shape[1] != k:
+        raise ValueError("qmatmul_int4_zp4: x must be [m, k]")
+    padded_k, groups = w4_geometry(k, group_size) if group_size > 0 else (k, 0)
+    y = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=x.device)
+    call("rumus_hip_qmatmul_int4_zp4", _dev(x, torch.float32, "x"), _dev(packed, torch.int32, "packed"),
+         _dev(scales, torch.float32, "scales"), _dev(qzeros, torch.int32, "qzeros"),
+         _opt(bias, torch.float32, "bias"), _opt(perm, torch.int32, "perm"),
+         _dev(y, torch.float32, "y"), m, k, n, padded_k, group_size, groups, _stream())
+    return y
+
+
 def _w4_call(name, x, packed, scales, zp, bias, extra, k, group_size, out=None):
     m = x.shape[0]
     n = packed.shape[1]

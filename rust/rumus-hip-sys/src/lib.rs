@@ -40,6 +40,11 @@ extern "C" {
                                       scales: *mut f32, zero_points: *mut f32, s: Stream) -> c_int;
     pub fn rumus_hip_w4_quantize_pack_sym(w: *const f32, k: u32, n: u32, group_size: u32, packed: *mut u32,
                                           scales: *mut f32, zero_points: *mut f32, s: Stream) -> c_int;
+    pub fn rumus_hip_w4_quantize_pack_awq(w: *const f32, k: u32, n: u32, group_size: u32, packed: *mut u32,
+                                          scales: *mut f32, qzeros: *mut u32, s: Stream) -> c_int;
+    pub fn rumus_hip_qmatmul_int4_zp4(x: *const f32, packed: *const u32, scales: *const f32, qzeros: *const u32,
+                                      bias: *const f32, perm: *const i32, y: *mut f32, m: u32, k: u32, n: u32,
+                                      padded_k: u32, group_size: u32, num_groups: u32, s: Stream) -> c_int;
     pub fn rumus_hip_qmatmul_int4(x: *const f32, packed: *const u32, scales: *const f32, zp: *const f32,
                                   bias: *const f32, g_idx: *const i32, y: *mut f32, m: u32, k: u32, n: u32,
                                   padded_k: u32, group_size: u32, num_groups: u32, s: Stream) -> c_int;

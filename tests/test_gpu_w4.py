@@ -299,3 +299,72 @@ def test_workspace_reserved_then_captured_in_a_graph(ops):
     with pytest.raises(Exception, match="workspace"):
         with torch.cuda.graph(g2, stream=fresh):
             ops.qmatmul_int4_perm(x, ps, d[1], d[2], k, g, perm=perm, out=y)
+
+
+# ---- AWQ storage: integer zero-points, eight per word along n -------------------------------
+
+@pytest.mark.parametrize("k,n,g", [(16, 8, 16), (200, 24, 64), (4096, 4096, 128), (1000, 264, 8)])
+def test_awq_quantize_pack_bit_exact(ops, k, n, g):
+    say(f"w4_quantize_pack_awq k={k} n={n} g={g}")
+    rng = np.random.default_rng(k + n + g)
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    w[:, 3] = np.abs(w[:, 3])        # zero-point clamps to 0
+    w[:, 5] = 0.02                   # constant column: range clamps to 1e-5
+    want = oracle.w4_awq_from_f32(w, g)
+    got = ops.w4_quantize_pack_awq(dev(w), g)
+    np.testing.assert_array_equal(host_u32(got[0]), want[0])
+    np.testing.assert_array_equal(host(got[1]), want[1])
+    np.testing.assert_array_equal(host_u32(got[2]), want[2])
+
+
+def test_awq_rejects_bad_shapes(ops):
+    from rumus_amd._lib import RumusError
+    with pytest.raises(RumusError):
+        ops.w4_quantize_pack_awq(dev(np.zeros((16, 12), np.float32)), 8)      # n % 8 != 0
+    with pytest.raises(RumusError):
+        ops.w4_quantize_pack_awq(dev(np.zeros((24, 8), np.float32)), 12)      # group % 8 != 0
+
+
+@pytest.mark.parametrize("m,k,n,g,with_bias", [
+    (1, 4096, 4096, 128, True),     # decode kernel, the BASELINE config 2 storage to the letter
+    (4, 1024, 264, 64, False),      # decode kernel, n % 16 != 0
+    (3, 200, 24, 8, True),          # group 8 -> reference-order kernel
+    (16, 4096, 4096, 128, True),    # MFMA kernel, K split
+    (70, 512, 520, 32, False),      # MFMA kernel, group 32
+    (300, 256, 8192, 128, True),    # MFMA kernel, 128-row tiles
+])
+def test_qmatmul_int4_zp4_vs_oracle(ops, m, k, n, g, with_bias):
+    say(f"qmatmul_int4_zp4 m={m} k={k} n={n} g={g}")
+    rng = np.random.default_rng(m * 7 + k + n)
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    x = rng.normal(0, 1, (m, k)).astype(np.float32)
+    b = rng.normal(0, 0.01, n).astype(np.float32) if with_bias else None
+    packed, scales, qzeros = oracle.w4_awq_from_f32(w, g)
+    zp = oracle.w4_qzeros_unpack(qzeros, n)
+    want = oracle.qmatmul_int4(x, packed, scales, zp, k, g, bias=b, threads=8)
+    got = host(ops.qmatmul_int4_zp4(dev(x), dev(packed), dev(scales), dev(qzeros), k, g,
+                                    bias=None if b is None else dev(b)))
+    assert_close(got, want)
+    # the packed zero-points and their f32 expansion are the same numbers: the two entry points
+    # must agree bit for bit (same kernels, same arithmetic)
+    same = host(ops.qmatmul_int4(dev(x), dev(packed), dev(scales), dev(zp), k, g,
+                                 bias=None if b is None else dev(b)))
+    if g % 32 == 0:
+        np.testing.assert_array_equal(got, same)
+    else:
+        assert_close(got, same)
+
+
+def test_zp4_act_order(ops):
+    say("qmatmul_int4_zp4 with perm")
+    rng = np.random.default_rng(33)
+    m, k, n, g = 16, 512, 64, 128
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    x = rng.normal(0, 1, (m, k)).astype(np.float32)
+    perm = rng.permutation(k).astype(np.int32)
+    # a weight whose rows are already in act-order: sorted row j multiplies x[:, perm[j]]
+    packed, scales, qzeros = oracle.w4_awq_from_f32(w, g)
+    zp = oracle.w4_qzeros_unpack(qzeros, n)
+    want = oracle.qmatmul_int4(x[:, perm], packed, scales, zp, k, g, threads=8)
+    got = host(ops.qmatmul_int4_zp4(dev(x), dev(packed), dev(scales), dev(qzeros), k, g, perm=dev(perm)))
+    assert_close(got, want)

@@ -156,3 +156,51 @@ def test_qmatmul_transpose_matches_float64():
     ref = gy.astype(np.float64) @ _dequant64(packed, scales, zp, k, g).T
     np.testing.assert_allclose(gx, ref, rtol=1e-3, atol=1e-4)
     assert gx.shape == (m, k)
+
+
+def test_awq_known_answers():
+    # Column c holds (k - c) * 2^-6 for k = 0..15: min = -c*s, max = (15-c)*s, so scale = s exactly,
+    # zero-point = c, q[k] = k.  qzeros packs column c in bits 4*c.
+    s = np.float32(2.0 ** -6)
+    w = np.stack([(np.arange(16) - c) * s for c in range(8)], axis=1).astype(np.float32)
+    packed, scales, qzeros = oracle.w4_awq_from_f32(w, 16)
+    np.testing.assert_array_equal(scales, np.full((1, 8), s, np.float32))
+    np.testing.assert_array_equal(qzeros, np.array([[0x76543210]], np.uint32))
+    np.testing.assert_array_equal(packed, np.tile(np.array([[0x76543210], [0xFEDCBA98]], np.uint32), (1, 8)))
+    np.testing.assert_array_equal(oracle.w4_qzeros_unpack(qzeros, 8), np.arange(8, dtype=np.float32)[None, :])
+    # ties go to even (AutoAWQ rounds with torch.round): 0, 15s, 2.5s, 0.5s, 3.5s -> 2, 0, 4
+    w = np.zeros((8, 8), np.float32)
+    w[:5, 0] = np.array([0, 15, 2.5, 0.5, 3.5], np.float32) * s
+    packed, scales, qzeros = oracle.w4_awq_from_f32(w, 8)
+    assert scales[0, 0] == s and (qzeros[0, 0] & 0xF) == 0
+    assert [(int(packed[0, 0]) >> (4 * j)) & 0xF for j in range(5)] == [0, 15, 2, 0, 4]
+    # a constant group: range clamps to 1e-5, zero-point 0, everything saturates at 15
+    w = np.full((8, 8), 0.02, np.float32)
+    packed, scales, qzeros = oracle.w4_awq_from_f32(w, 8)
+    assert scales[0, 0] == np.float32(1e-5) / np.float32(15) and qzeros[0, 0] == 0 and packed[0, 0] == 0xFFFFFFFF
+    with pytest.raises(ValueError):
+        oracle.w4_awq_from_f32(np.zeros((8, 4), np.float32), 8)       # n % 8 != 0
+
+
+def test_awq_matches_vectorised_formula_and_bounds():
+    rng = np.random.default_rng(21)
+    k, n, g = 200, 24, 64
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    w[:, 3] = np.abs(w[:, 3])                       # all positive: zero-point clamps to 0
+    packed, scales, qzeros = oracle.w4_awq_from_f32(w, g)
+    pk, G = oracle.w4_geometry(k, g)
+    wp = np.zeros((pk, n), np.float32)
+    wp[:k] = w
+    wg = wp.reshape(G, g, n)
+    mn, mx = wg.min(1), wg.max(1)
+    sc = (np.maximum(mx - mn, np.float32(1e-5)) / np.float32(15)).astype(np.float32)
+    z = np.clip(-np.rint(mn / sc), 0, 15)
+    q = np.clip(np.rint(wg / sc[:, None, :]) + z[:, None, :], 0, 15).astype(np.uint32).reshape(pk, n)
+    np.testing.assert_array_equal(scales, sc)
+    np.testing.assert_array_equal(oracle.w4_qzeros_unpack(qzeros, n), z.astype(np.float32))
+    np.testing.assert_array_equal(oracle.w4_unpack(packed, pk), q.astype(np.uint8))
+    # dequantised error is at most half a step wherever the zero-point did not clamp
+    deq = (q.astype(np.float32).reshape(G, g, n) - z[:, None, :]) * sc[:, None, :]
+    free = (mn <= 0) & (mx >= 0)
+    err = np.abs(deq - wg).max(1)
+    assert (err[free] <= sc[free] * 0.5001).all()
