@@ -212,6 +212,38 @@ int rumus_hip_qmatmul_int4_zp4(const float* x, const uint32_t* packed,
                                uint32_t group_size, uint32_t num_groups,
                                rumus_hip_stream_t stream);
 
+/* ---- f32 operators between the projections of a decoder block (EXTENSION) --
+ * None of these is on the reference's quantized path; they exist so that a
+ * block built from the matmuls above needs no other library.  Reference
+ * analogue of the attention: flash_attention (rumus/src/tensor/ops.rs:2685-2743,
+ * shaders/flash_attn.wgsl): same online-softmax result, f32, head_dim 128. */
+
+/* y[r,:] = x[r,:] * rsqrt(mean(x[r,:]^2) + eps) * weight[:] */
+int rumus_hip_rmsnorm(const float* x, const float* weight, float* y, uint32_t rows,
+                      uint32_t dim, float eps, rumus_hip_stream_t stream);
+
+/* out = silu(gate) * up, silu(t) = t / (1 + exp(-t)); out may alias gate or up */
+int rumus_hip_swiglu(const float* gate, const float* up, float* out, uint64_t numel,
+                     rumus_hip_stream_t stream);
+
+/* out = a + b; out may alias a or b */
+int rumus_hip_add(const float* a, const float* b, float* out, uint64_t numel,
+                  rumus_hip_stream_t stream);
+
+/* out = softmax(q k^T / sqrt(head_dim)) v per (batch, head).
+ * strides: HOST array of 12 element strides (in floats, multiples of 4):
+ * {q_batch, q_head, q_row, k_batch, k_head, k_row, v_batch, v_head, v_row,
+ *  o_batch, o_head, o_row}; head_dim is contiguous.  A projection output
+ * [batch*rows, heads*128] is {rows*heads*128, 128, heads*128}; the reference's
+ * [B,H,N,d] is {H*N*128, N*128, 128}.
+ * causal != 0: query row i is token kv_len - q_len + i and sees keys up to
+ * itself.  q_len == 1 (decode) splits the keys over workgroups and uses the
+ * workspace.  EINVAL unless head_dim == 128, q_len <= kv_len, 16-byte aligned. */
+int rumus_hip_attention(const float* q, const float* k, const float* v, float* out,
+                        uint32_t batch, uint32_t heads, uint32_t q_len, uint32_t kv_len,
+                        uint32_t head_dim, const uint64_t* strides, int causal,
+                        rumus_hip_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

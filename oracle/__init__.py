@@ -247,3 +247,66 @@ def i8_linear(x, w, bias=None, threads: int = 1):
     xq, sx = i8_quantize_rows(x)
     acc = i8_gemm_i32(xq, wq, threads)
     return i8_rescale_bias(acc, sx, sw, bias), acc, (xq, sx, wq, sw)
+
+
+# --------------------------------------------------------------------------
+# EXTENSION: the f32 operators around the projections of a decoder block, in
+# float64 numpy.  Closed forms, no reference code behind them (the reference's
+# flash_attention computes the same softmax(q k^T / sqrt(d)) v).
+# --------------------------------------------------------------------------
+
+def w4_dequant(packed, scales, zp, k: int, group_size: int):
+    """float64 [k, n] matrix (q - zp) * scale of an INT4 weight."""
+    q = w4_unpack(packed, k).astype(np.float64)
+    g = np.arange(k) // group_size
+    return (q - np.asarray(zp, np.float64)[g]) * np.asarray(scales, np.float64)[g]
+
+
+def rmsnorm(x, weight, eps: float = 1e-6):
+    x = np.asarray(x, np.float64)
+    return x / np.sqrt((x * x).mean(-1, keepdims=True) + eps) * np.asarray(weight, np.float64)
+
+
+def swiglu(gate, up):
+    gate = np.asarray(gate, np.float64)
+    return gate / (1.0 + np.exp(-gate)) * np.asarray(up, np.float64)
+
+
+def attention(q, k, v, causal: bool):
+    """q [B, Nq, H, d], k, v [B, Nkv, H, d] -> [B, Nq, H, d]; query i is token Nkv - Nq + i."""
+    q, k, v = (np.asarray(t, np.float64) for t in (q, k, v))
+    nq, nkv, d = q.shape[1], k.shape[1], q.shape[3]
+    s = np.einsum("bqhd,bkhd->bhqk", q, k) / np.sqrt(d)
+    if causal:
+        pos = np.arange(nq)[:, None] + (nkv - nq)
+        s = np.where(np.arange(nkv)[None, :] <= pos, s, -np.inf)
+    s = s - s.max(-1, keepdims=True)
+    p = np.exp(s)
+    p /= p.sum(-1, keepdims=True)
+    return np.einsum("bhqk,bkhd->bqhd", p, v)
+
+
+def decoder_block(x, wd: dict, heads: int, k_cache=None, v_cache=None, pos: int = 0, eps: float = 1e-6):
+    """Pre-norm Llama-shaped block on dequantized float64 weights ``wd[name]`` ([in, out]), RMSNorm
+    weights 1.  Returns (y, k, v); with caches the new key/value are placed at ``pos`` first."""
+    x = np.asarray(x, np.float64)
+    b, n, d = x.shape
+    ones = np.ones(d)
+    x2 = x.reshape(b * n, d)
+    hn = rmsnorm(x2, ones, eps)
+    q = (hn @ wd["q"]).reshape(b, n, heads, -1)
+    k = (hn @ wd["k"]).reshape(b, n, heads, -1)
+    v = (hn @ wd["v"]).reshape(b, n, heads, -1)
+    if k_cache is None:
+        att = attention(q, k, v, True)
+    else:
+        k_cache = np.array(k_cache, np.float64)
+        v_cache = np.array(v_cache, np.float64)
+        k_cache[:, pos] = k[:, 0]
+        v_cache[:, pos] = v[:, 0]
+        att = attention(q, k_cache[:, :pos + 1], v_cache[:, :pos + 1], False)
+        k, v = k_cache, v_cache
+    x1 = x2 + att.reshape(b * n, d) @ wd["o"]
+    h2 = rmsnorm(x1, ones, eps)
+    y = x1 + swiglu(h2 @ wd["gate"], h2 @ wd["up"]) @ wd["down"]
+    return y.reshape(b, n, d), k, v

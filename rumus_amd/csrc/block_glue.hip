@@ -1,0 +1,287 @@
+// The f32 operators that sit between the quantized projections of a decoder
+// block: RMSNorm, SwiGLU, residual add and scaled-dot-product attention
+// (reference analogue for attention: flash_attention, rumus/src/tensor/ops.rs:
+// 2685-2743 with shaders/flash_attn.wgsl; the others have no counterpart in the
+// reference).  All of them are bandwidth- or latency-bound helpers around the
+// INT4 / INT8 matmuls, written so that no permute or copy is needed between a
+// projection's [tokens, heads*dim] output and the attention operands: every
+// attention operand carries its own (batch, head, row) strides.
+#include "common.h"
+
+namespace rumus {
+
+// ---- RMSNorm: y[r,:] = x[r,:] * rsqrt(mean(x[r,:]^2) + eps) * weight ---------------------
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                      float* __restrict__ y, uint32_t dim, float eps) {
+    __shared__ float red[4];
+    const float* xr = x + (uint64_t)blockIdx.x * dim;
+    float* yr = y + (uint64_t)blockIdx.x * dim;
+    float ss = 0.0f;
+    for (uint32_t i = threadIdx.x; i < dim; i += 256) ss = fmaf(xr[i], xr[i], ss);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float total = (red[0] + red[1]) + (red[2] + red[3]);
+    const float inv = 1.0f / sqrtf(total / (float)dim + eps);
+    for (uint32_t i = threadIdx.x; i < dim; i += 256) yr[i] = xr[i] * inv * w[i];
+}
+
+// ---- SwiGLU: out = silu(gate) * up, silu(t) = t / (1 + exp(-t)) ----------------------------
+__global__ __launch_bounds__(256) void swiglu_kernel(const float* __restrict__ gate, const float* __restrict__ up,
+                                                     float* __restrict__ out, uint64_t numel) {
+    const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= numel) return;
+    const float g = gate[i];
+    out[i] = g / (1.0f + expf(-g)) * up[i];
+}
+
+__global__ __launch_bounds__(256) void add_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                  float* __restrict__ out, uint64_t numel) {
+    const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < numel) out[i] = a[i] + b[i];
+}
+
+// ---- attention -------------------------------------------------------------------------
+// Operand (b, h, row, :) lives at base + b*sb + h*sh + row*sr, head_dim contiguous.
+struct AttnArgs {
+    const float *q, *k, *v;
+    float* o;
+    uint64_t q_sb, q_sh, q_sr, k_sb, k_sh, k_sr, v_sb, v_sh, v_sr, o_sb, o_sh, o_sr;
+    uint32_t batch, heads, q_len, kv_len;
+    float scale;
+    int causal;
+};
+
+constexpr int kHeadDim = 128;
+
+// Prefill / general case.  Workgroup = 64 query rows of one (batch, head); 4 lanes per row,
+// each holding 32 of the 128 dims of q and of the output.  K/V tiles of 32 keys go through
+// LDS (every lane reads the same key, so the reads are broadcasts); online softmax per row.
+// Causal: query row i sits at position kv_len - q_len + i and sees keys up to its position.
+__global__ __launch_bounds__(256) void attention_rows_kernel(AttnArgs a) {
+    constexpr int BC = 32;
+    __shared__ __attribute__((aligned(16))) float ks[BC][kHeadDim];
+    __shared__ __attribute__((aligned(16))) float vs[BC][kHeadDim];
+    const uint32_t tid = threadIdx.x, part = tid & 3, r = tid >> 2;
+    const uint32_t bh = blockIdx.y, b = bh / a.heads, h = bh % a.heads;
+    const uint32_t row = blockIdx.x * 64 + r;
+    const bool row_ok = row < a.q_len;
+    const uint32_t shift = a.kv_len - a.q_len;                 // causal offset of the query rows
+    const float* qp = a.q + b * a.q_sb + h * a.q_sh + (uint64_t)min(row, a.q_len - 1) * a.q_sr + part * 32;
+    float q[32], acc[32];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const float4 t = *reinterpret_cast<const float4*>(qp + 4 * i);
+        q[4 * i] = t.x * a.scale; q[4 * i + 1] = t.y * a.scale; q[4 * i + 2] = t.z * a.scale; q[4 * i + 3] = t.w * a.scale;
+    }
+#pragma unroll
+    for (int i = 0; i < 32; i++) acc[i] = 0.0f;
+    float mrun = -INFINITY, lrun = 0.0f;
+    // keys this workgroup needs: all of them, or up to the position of its last row
+    const uint32_t last_row = min(blockIdx.x * 64 + 63, a.q_len - 1);
+    const uint32_t kv_end = a.causal ? min(a.kv_len, last_row + shift + 1) : a.kv_len;
+    const uint32_t my_end = a.causal ? min(a.kv_len, row + shift + 1) : a.kv_len;   // exclusive
+    const float* kb = a.k + b * a.k_sb + h * a.k_sh;
+    const float* vb = a.v + b * a.v_sb + h * a.v_sh;
+    for (uint32_t j0 = 0; j0 < kv_end; j0 += BC) {
+        __syncthreads();
+        // 32 keys x 128 floats = 1024 float4 per tile and operand: 4 per thread
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const uint32_t e = tid + 256 * t, kr = e >> 5, c4 = e & 31;
+            const uint32_t key = min(j0 + kr, a.kv_len - 1);
+            *reinterpret_cast<float4*>(&ks[kr][4 * c4]) = *reinterpret_cast<const float4*>(kb + (uint64_t)key * a.k_sr + 4 * c4);
+            *reinterpret_cast<float4*>(&vs[kr][4 * c4]) = *reinterpret_cast<const float4*>(vb + (uint64_t)key * a.v_sr + 4 * c4);
+        }
+        __syncthreads();
+        float s[BC];
+        float mtile = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < BC; j++) {
+            float d = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const float4 kk = *reinterpret_cast<const float4*>(&ks[j][part * 32 + 4 * i]);
+                d = fmaf(q[4 * i], kk.x, d); d = fmaf(q[4 * i + 1], kk.y, d);
+                d = fmaf(q[4 * i + 2], kk.z, d); d = fmaf(q[4 * i + 3], kk.w, d);
+            }
+            d += __shfl_xor(d, 1);
+            d += __shfl_xor(d, 2);
+            s[j] = (j0 + j < my_end) ? d : -INFINITY;
+            mtile = fmaxf(mtile, s[j]);
+        }
+        const float mnew = fmaxf(mrun, mtile);
+        if (mnew == -INFINITY) continue;                       // nothing visible yet (uniform per quad)
+        const float corr = expf(mrun - mnew);                  // exp(-inf) = 0 on the first visible tile
+        lrun *= corr;
+#pragma unroll
+        for (int i = 0; i < 32; i++) acc[i] *= corr;
+#pragma unroll
+        for (int j = 0; j < BC; j++) {
+            const float p = expf(s[j] - mnew);                 // masked keys: exp(-inf) = 0
+            lrun += p;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const float4 vv = *reinterpret_cast<const float4*>(&vs[j][part * 32 + 4 * i]);
+                acc[4 * i] = fmaf(p, vv.x, acc[4 * i]); acc[4 * i + 1] = fmaf(p, vv.y, acc[4 * i + 1]);
+                acc[4 * i + 2] = fmaf(p, vv.z, acc[4 * i + 2]); acc[4 * i + 3] = fmaf(p, vv.w, acc[4 * i + 3]);
+            }
+        }
+        mrun = mnew;
+    }
+    if (!row_ok) return;
+    const float inv = lrun > 0.0f ? 1.0f / lrun : 0.0f;
+    float* op = a.o + b * a.o_sb + h * a.o_sh + (uint64_t)row * a.o_sr + part * 32;
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+        *reinterpret_cast<float4*>(op + 4 * i) =
+            make_float4(acc[4 * i] * inv, acc[4 * i + 1] * inv, acc[4 * i + 2] * inv, acc[4 * i + 3] * inv);
+}
+
+// Decode case (q_len == 1): the keys of one (batch, head) are split over gridDim.x workgroups
+// so that the chip is covered; each writes (max, sum, unnormalised output) of its slice and
+// attention_merge_kernel combines the slices.  Within a workgroup: 4 lanes per key for the
+// scores (64 keys per sweep), then one thread per output dim and key half for p.V.
+constexpr int kDecodeSlice = 256;   // keys per workgroup
+
+__global__ __launch_bounds__(256) void attention_decode_kernel(AttnArgs a, float* __restrict__ part) {
+    __shared__ float sc[kDecodeSlice];
+    __shared__ float red[4], lsum[2];
+    __shared__ float osum[2][kHeadDim];
+    const uint32_t tid = threadIdx.x, lane4 = tid & 3, kq = tid >> 2;
+    const uint32_t bh = blockIdx.y, b = bh / a.heads, h = bh % a.heads;
+    const uint32_t j0 = blockIdx.x * kDecodeSlice, j1 = min(a.kv_len, j0 + kDecodeSlice);
+    const float* qp = a.q + b * a.q_sb + h * a.q_sh + lane4 * 32;
+    const float* kb = a.k + b * a.k_sb + h * a.k_sh;
+    const float* vb = a.v + b * a.v_sb + h * a.v_sh;
+    float q[32];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const float4 t = *reinterpret_cast<const float4*>(qp + 4 * i);
+        q[4 * i] = t.x * a.scale; q[4 * i + 1] = t.y * a.scale; q[4 * i + 2] = t.z * a.scale; q[4 * i + 3] = t.w * a.scale;
+    }
+    float mloc = -INFINITY;
+#pragma unroll
+    for (int sweep = 0; sweep < kDecodeSlice / 64; sweep++) {
+        const uint32_t jj = sweep * 64 + kq, key = j0 + jj;
+        const float* kp = kb + (uint64_t)min(key, a.kv_len - 1) * a.k_sr + lane4 * 32;
+        float d = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const float4 kk = *reinterpret_cast<const float4*>(kp + 4 * i);
+            d = fmaf(q[4 * i], kk.x, d); d = fmaf(q[4 * i + 1], kk.y, d);
+            d = fmaf(q[4 * i + 2], kk.z, d); d = fmaf(q[4 * i + 3], kk.w, d);
+        }
+        d += __shfl_xor(d, 1);
+        d += __shfl_xor(d, 2);
+        d = key < j1 ? d : -INFINITY;
+        if (lane4 == 0) sc[jj] = d;
+        mloc = fmaxf(mloc, d);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mloc = fmaxf(mloc, __shfl_xor(mloc, o));
+    if ((tid & 63) == 0) red[tid >> 6] = mloc;
+    __syncthreads();
+    const float m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));   // finite: the slice is not empty
+    // p.V: thread = (dim, key half); the probabilities are recomputed from the scores
+    const uint32_t dim = tid & 127, half = tid >> 7;
+    float o = 0.0f, l = 0.0f;
+    for (uint32_t jj = half * (kDecodeSlice / 2); jj < (half + 1) * (kDecodeSlice / 2); jj++) {
+        if (j0 + jj >= j1) break;
+        const float p = expf(sc[jj] - m);
+        l += p;
+        o = fmaf(p, vb[(uint64_t)(j0 + jj) * a.v_sr + dim], o);
+    }
+    osum[half][dim] = o;
+    if (dim == 0) lsum[half] = l;
+    __syncthreads();
+    if (tid < kHeadDim) {
+        float* dst = part + ((uint64_t)bh * gridDim.x + blockIdx.x) * (kHeadDim + 2);
+        dst[2 + tid] = osum[0][tid] + osum[1][tid];
+        if (tid == 0) {
+            dst[0] = m;
+            dst[1] = lsum[0] + lsum[1];
+        }
+    }
+}
+
+__global__ __launch_bounds__(kHeadDim) void attention_merge_kernel(AttnArgs a, const float* __restrict__ part,
+                                                                   uint32_t slices) {
+    const uint32_t bh = blockIdx.x, b = bh / a.heads, h = bh % a.heads, dim = threadIdx.x;
+    const float* src = part + (uint64_t)bh * slices * (kHeadDim + 2);
+    float m = -INFINITY;
+    for (uint32_t s = 0; s < slices; s++) m = fmaxf(m, src[s * (kHeadDim + 2)]);
+    float l = 0.0f, o = 0.0f;
+    for (uint32_t s = 0; s < slices; s++) {
+        const float w = expf(src[s * (kHeadDim + 2)] - m);
+        l = fmaf(w, src[s * (kHeadDim + 2) + 1], l);
+        o = fmaf(w, src[s * (kHeadDim + 2) + 2 + dim], o);
+    }
+    a.o[b * a.o_sb + h * a.o_sh + dim] = o / l;
+}
+
+}  // namespace rumus
+
+using namespace rumus;
+
+extern "C" {
+
+int rumus_hip_rmsnorm(const float* x, const float* weight, float* y, uint32_t rows, uint32_t dim, float eps,
+                      rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE(x && weight && y, "rmsnorm: null buffer");
+    RUMUS_REQUIRE(dim > 0, "rmsnorm: dim must be > 0");
+    if (rows == 0) return RUMUS_HIP_OK;
+    hipLaunchKernelGGL(rmsnorm_kernel, dim3(rows), dim3(256), 0, as_stream(stream), x, weight, y, dim, eps);
+    return check_launch("rmsnorm_kernel");
+}
+
+int rumus_hip_swiglu(const float* gate, const float* up, float* out, uint64_t numel, rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE(gate && up && out, "swiglu: null buffer");
+    if (numel == 0) return RUMUS_HIP_OK;
+    hipLaunchKernelGGL(swiglu_kernel, dim3((uint32_t)((numel + 255) / 256)), dim3(256), 0, as_stream(stream), gate,
+                       up, out, numel);
+    return check_launch("swiglu_kernel");
+}
+
+int rumus_hip_add(const float* a, const float* b, float* out, uint64_t numel, rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE(a && b && out, "add: null buffer");
+    if (numel == 0) return RUMUS_HIP_OK;
+    hipLaunchKernelGGL(add_kernel, dim3((uint32_t)((numel + 255) / 256)), dim3(256), 0, as_stream(stream), a, b, out,
+                       numel);
+    return check_launch("add_kernel");
+}
+
+int rumus_hip_attention(const float* q, const float* k, const float* v, float* out, uint32_t batch, uint32_t heads,
+                        uint32_t q_len, uint32_t kv_len, uint32_t head_dim, const uint64_t* strides, int causal,
+                        rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE(q && k && v && out && strides, "attention: null buffer");
+    RUMUS_REQUIRE(head_dim == kHeadDim, "attention: head_dim must be %d (got %u)", kHeadDim, head_dim);
+    RUMUS_REQUIRE(q_len <= kv_len, "attention: q_len %u exceeds kv_len %u", q_len, kv_len);
+    if (batch == 0 || heads == 0 || q_len == 0) return RUMUS_HIP_OK;
+    for (int i = 0; i < 12; i++)
+        RUMUS_REQUIRE(strides[i] % 4 == 0, "attention: stride %d (%llu) must be a multiple of 4 floats", i,
+                      (unsigned long long)strides[i]);
+    RUMUS_REQUIRE(((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
+                    reinterpret_cast<uintptr_t>(out)) & 15) == 0, "attention: operands must be 16-byte aligned");
+    RUMUS_REQUIRE((uint64_t)batch * heads <= 65535, "attention: batch * heads beyond the grid limit");
+    AttnArgs a{q, k, v, out, strides[0], strides[1], strides[2], strides[3], strides[4], strides[5],
+               strides[6], strides[7], strides[8], strides[9], strides[10], strides[11],
+               batch, heads, q_len, kv_len, 1.0f / sqrtf((float)head_dim), causal};
+    hipStream_t s = as_stream(stream);
+    if (q_len == 1) {
+        const uint32_t slices = ceil_div(kv_len, kDecodeSlice);
+        void* ws = nullptr;
+        if (int rc = workspace_get(s, (size_t)batch * heads * slices * (kHeadDim + 2) * sizeof(float), &ws)) return rc;
+        hipLaunchKernelGGL(attention_decode_kernel, dim3(slices, batch * heads), dim3(256), 0, s, a,
+                           static_cast<float*>(ws));
+        if (int rc = check_launch("attention_decode_kernel")) return rc;
+        hipLaunchKernelGGL(attention_merge_kernel, dim3(batch * heads), dim3(kHeadDim), 0, s, a,
+                           static_cast<const float*>(ws), slices);
+        return check_launch("attention_merge_kernel");
+    }
+    hipLaunchKernelGGL(attention_rows_kernel, dim3(ceil_div(q_len, 64), batch * heads), dim3(256), 0, s, a);
+    return check_launch("attention_rows_kernel");
+}
+
+}  // extern "C"

@@ -183,3 +183,67 @@ class Int8Linear:
         return (y, acc) if want_acc else y
 
     __call__ = forward
+
+
+# ---- a decoder block built from the INT4 projections ---------------------------------------
+
+class DecoderBlockW4:
+    """Llama-shaped pre-norm decoder block whose seven projections are INT4 ``QLinear`` layers:
+    RMSNorm -> q, k, v -> attention (f32, no rotary embedding) -> o -> residual ->
+    RMSNorm -> gate, up -> SwiGLU -> down -> residual.  Activations stay ``[tokens, features]``
+    between the layers; the attention reads the projection outputs through strides, so nothing
+    is permuted or copied.  The K/V cache is token-major: ``[batch, positions, heads, 128]``."""
+
+    NAMES = ("q", "k", "v", "o", "gate", "up", "down")
+
+    def __init__(self, proj: dict, norm1: torch.Tensor, norm2: torch.Tensor, heads: int, eps: float = 1e-6):
+        self.proj, self.norm1, self.norm2, self.heads, self.eps = proj, norm1, norm2, heads, eps
+        self.dim = proj["q"].in_features
+        if self.dim != heads * 128:
+            raise ValueError("DecoderBlockW4: head_dim must be 128")
+
+    @classmethod
+    def from_f32(cls, weights: dict, group_size: int, heads: int, eps: float = 1e-6) -> "DecoderBlockW4":
+        """``weights[name]`` is the f32 ``[in, out]`` matrix of projection ``name`` (on the device)."""
+        proj = {}
+        for name in cls.NAMES:
+            w = weights[name]
+            proj[name] = QLinear(QuantizedTensor.from_f32(w, w.shape[0], w.shape[1], group_size), None)
+        d = weights["q"].shape[0]
+        ones = torch.ones(d, dtype=torch.float32, device=weights["q"].device)
+        return cls(proj, weights.get("norm1", ones), weights.get("norm2", ones), heads, eps)
+
+    def forward(self, x: torch.Tensor, k_cache: Optional[torch.Tensor] = None,
+                v_cache: Optional[torch.Tensor] = None, pos: int = 0):
+        """``x`` is ``[batch, n, dim]``.  Without caches: causal self-attention over the n tokens
+        (prefill); returns ``(y, k, v)`` with k, v ``[batch, n, heads, 128]``.  With caches
+        (``[batch, T, heads, 128]``, valid below ``pos``): n must be 1; the new key/value are
+        written at ``pos`` and the token attends positions ``0..pos``; returns ``(y, k_cache, v_cache)``."""
+        b, n, d = x.shape
+        h = self.heads
+        x2 = x.reshape(b * n, d)
+        hn = ops.rmsnorm(x2, self.norm1, self.eps)
+        q = self.proj["q"](hn).view(b, n, h, 128)
+        k = self.proj["k"](hn).view(b, n, h, 128)
+        v = self.proj["v"](hn).view(b, n, h, 128)
+        if k_cache is None:
+            att = ops.attention(q, k, v, causal=True)
+            k_out, v_out = k, v
+        else:
+            if n != 1:
+                raise ValueError("DecoderBlockW4: decode takes one token per sequence")
+            k_cache[:, pos].copy_(k[:, 0])
+            v_cache[:, pos].copy_(v[:, 0])
+            att = ops.attention(q, k_cache[:, :pos + 1], v_cache[:, :pos + 1], causal=False)
+            k_out, v_out = k_cache, v_cache
+        o = self.proj["o"](att.view(b * n, d))
+        x1 = ops.add(x2, o, out=o)
+        h2 = ops.rmsnorm(x1, self.norm2, self.eps, out=hn)
+        gate = self.proj["gate"](h2)
+        up = self.proj["up"](h2)
+        act = ops.swiglu(gate, up, out=gate)
+        down = self.proj["down"](act)
+        y = ops.add(x1, down, out=down)
+        return y.view(b, n, d), k_out, v_out
+
+    __call__ = forward

@@ -214,3 +214,43 @@ def w4_actorder_prepare(packed, g_idx, group_size):
          _dev(g_idx, torch.int32, "g_idx"), padded_k, n, group_size, out.data_ptr(), perm.data_ptr(),
          _stream())
     return out, perm
+
+
+# ---- f32 operators between the projections of a decoder block ---------------------------------
+
+def rmsnorm(x, weight, eps: float = 1e-6, out=None):
+    rows, dim = x.shape
+    y = out if out is not None else torch.empty_like(x)
+    call("rumus_hip_rmsnorm", _dev(x, torch.float32, "x"), _dev(weight, torch.float32, "weight"),
+         _dev(y, torch.float32, "y"), rows, dim, float(eps), _stream())
+    return y
+
+
+def swiglu(gate, up, out=None):
+    y = out if out is not None else torch.empty_like(gate)
+    call("rumus_hip_swiglu", _dev(gate, torch.float32, "gate"), _dev(up, torch.float32, "up"),
+         _dev(y, torch.float32, "out"), gate.numel(), _stream())
+    return y
+
+
+def add(a, b, out=None):
+    y = out if out is not None else torch.empty_like(a)
+    call("rumus_hip_add", _dev(a, torch.float32, "a"), _dev(b, torch.float32, "b"), _dev(y, torch.float32, "out"),
+         a.numel(), _stream())
+    return y
+
+
+def attention(q, k, v, causal: bool, out=None):
+    """q [B, Nq, H, 128], k and v [B, Nkv, H, 128] (any strides with the last dim contiguous) ->
+    [B, Nq, H, 128]: softmax(q k^T / sqrt(128)) v per batch and head."""
+    import ctypes
+    b, nq, h, d = q.shape
+    nkv = k.shape[1]
+    o = out if out is not None else torch.empty((b, nq, h, d), dtype=torch.float32, device=q.device)
+    for t, name in ((q, "q"), (k, "k"), (v, "v"), (o, "out")):
+        if t.dtype != torch.float32 or not t.is_cuda or t.stride(3) != 1:
+            raise ValueError(f"attention: {name} must be a float32 device tensor with a contiguous last dim")
+    strides = (ctypes.c_uint64 * 12)(*[s for t in (q, k, v, o) for s in (t.stride(0), t.stride(2), t.stride(1))])
+    call("rumus_hip_attention", q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), b, h, nq, nkv, d,
+         strides, 1 if causal else 0, _stream())
+    return o
