@@ -248,6 +248,66 @@ def bench_w4_gemm(torch, ops, m, steps=50, warmup=5):
             "tflops": flops / sec / 1e12, "f16_mfma_frac": flops / sec / 1e12 / F16_PEAK_TFLOPS}
 
 
+def bench_decoder_block(torch, ops):
+    """Llama-7B-shaped block, all seven projections INT4 g128 with the reference's f32 zero-points:
+    one decode step (batch 1, position 2047 of a 2048-entry cache) and one prefill of 8 x 512
+    tokens.  Times include every kernel of the block (norms, projections, attention, SwiGLU,
+    residuals) and the Python launch path."""
+    from rumus_amd import nn, workloads
+    dev = torch.device("cuda:0")
+    dim, heads = 4096, 32
+    w = workloads.decoder_block()
+    blk = nn.DecoderBlockW4.from_f32({k: torch.from_numpy(v).to(dev) for k, v in w.items()}, G, heads)
+    del w
+    x, kc, vc = workloads.decoder_block_inputs(1, 1, dim, cache_len=2048, heads=heads)
+    x, kc, vc = (torch.from_numpy(t).to(dev) for t in (x, kc, vc))
+    xp = torch.from_numpy(workloads.decoder_block_inputs(8, 512, dim, seed=9)[0]).to(dev)
+
+    def timed(fn, steps, warmup):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(steps):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(end) * 1e-3 / steps
+
+    t_dec = timed(lambda: blk(x, kc, vc, pos=2047), 50, 5)
+    t_pre = timed(lambda: blk(xp), 5, 2)
+    # the same decode step replayed from a HIP graph (what a serving loop would do): the capture
+    # stream's workspace is reserved first, the library does not allocate while capturing
+    t_dec_graph = None
+    try:
+        from rumus_amd import _lib
+        side = torch.cuda.Stream()
+        _lib.call("rumus_hip_workspace_reserve", side.cuda_stream, 1 << 22)
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            blk(x, kc, vc, pos=2047)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(10):
+                blk(x, kc, vc, pos=2047)
+        t_dec_graph = timed(graph.replay, 20, 3) / 10
+    except Exception as exc:
+        log(f"[bench] decoder-block graph capture unavailable: {exc!r}")
+    weight_bytes = 4 * (dim * dim // 2 + 2 * (dim // G) * dim * 4) + \
+        2 * (dim * 11008 // 2 + 2 * (dim // G) * 11008 * 4) + (11008 * dim // 2 + 2 * (11008 // G) * dim * 4)
+    kv_bytes = 2 * 2048 * dim * 4
+    flops = 2.0 * 8 * 512 * (4 * dim * dim + 3 * dim * 11008)
+    t_best = t_dec_graph if t_dec_graph else t_dec
+    return {"workload": "llama7b_block_w4_g128", "decode_ms": t_dec * 1e3,
+            "decode_hip_graph_ms": None if t_dec_graph is None else t_dec_graph * 1e3,
+            "decode_weight_and_cache_gbs": (weight_bytes + kv_bytes) / t_best / 1e9,
+            "prefill_8x512_ms": t_pre * 1e3, "prefill_tokens_per_s": 8 * 512 / t_pre,
+            "prefill_projection_tflops": flops / t_pre / 1e12}
+
+
 def cpu_baseline(x, w, budget_s=12.0):
     """The CPU restatement of the reference kernels on the host cores: single thread (the
     reference CpuBackend's contract) for `value`, all cores as an extra figure."""
@@ -347,6 +407,7 @@ def main():
     if not args.only_gemv:
         out["secondary"] = bench_i8_gemm(torch, ops)
         out["w4_gemm"] = [bench_w4_gemm(torch, ops, 16), bench_w4_gemm(torch, ops, 128)]
+        out["decoder_block"] = bench_decoder_block(torch, ops)
 
     if not args.no_cpu:
         cb, y_cpu = cpu_baseline(r["x"], r["w"])

@@ -142,13 +142,13 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(AttnArgs a) {
 // Decode case (q_len == 1): the keys of one (batch, head) are split over gridDim.x workgroups
 // so that the chip is covered; each writes (max, sum, unnormalised output) of its slice and
 // attention_merge_kernel combines the slices.  Within a workgroup: 4 lanes per key for the
-// scores (64 keys per sweep), then one thread per output dim and key half for p.V.
+// scores (64 keys per sweep), then one thread per 4 output dims and key group for p.V.
 constexpr int kDecodeSlice = 256;   // keys per workgroup
 
 __global__ __launch_bounds__(256) void attention_decode_kernel(AttnArgs a, float* __restrict__ part) {
     __shared__ float sc[kDecodeSlice];
-    __shared__ float red[4], lsum[2];
-    __shared__ float osum[2][kHeadDim];
+    __shared__ float red[4], lsum[8];
+    __shared__ __attribute__((aligned(16))) float osum[8][kHeadDim];
     const uint32_t tid = threadIdx.x, lane4 = tid & 3, kq = tid >> 2;
     const uint32_t bh = blockIdx.y, b = bh / a.heads, h = bh % a.heads;
     const uint32_t j0 = blockIdx.x * kDecodeSlice, j1 = min(a.kv_len, j0 + kDecodeSlice);
@@ -184,24 +184,41 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttnArgs a, float
     if ((tid & 63) == 0) red[tid >> 6] = mloc;
     __syncthreads();
     const float m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));   // finite: the slice is not empty
-    // p.V: thread = (dim, key half); the probabilities are recomputed from the scores
-    const uint32_t dim = tid & 127, half = tid >> 7;
-    float o = 0.0f, l = 0.0f;
-    for (uint32_t jj = half * (kDecodeSlice / 2); jj < (half + 1) * (kDecodeSlice / 2); jj++) {
-        if (j0 + jj >= j1) break;
-        const float p = expf(sc[jj] - m);
-        l += p;
-        o = fmaf(p, vb[(uint64_t)(j0 + jj) * a.v_sr + dim], o);
+    // p.V: thread = (4 output dims, 1 of 8 key groups), eight 128-bit loads of V in flight
+    const uint32_t c4 = tid & 31, kg = tid >> 5;
+    float4 o = make_float4(0, 0, 0, 0);
+    float l = 0.0f;
+    for (uint32_t jj = kg; jj < kDecodeSlice; jj += 64) {
+        float p[8];
+        float4 vv[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const uint32_t key = j0 + jj + 8 * u;
+            vv[u] = *reinterpret_cast<const float4*>(vb + (uint64_t)min(key, a.kv_len - 1) * a.v_sr + 4 * c4);
+            p[u] = key < j1 ? expf(sc[jj + 8 * u] - m) : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            l += p[u];
+            o.x = fmaf(p[u], vv[u].x, o.x); o.y = fmaf(p[u], vv[u].y, o.y);
+            o.z = fmaf(p[u], vv[u].z, o.z); o.w = fmaf(p[u], vv[u].w, o.w);
+        }
     }
-    osum[half][dim] = o;
-    if (dim == 0) lsum[half] = l;
+    *reinterpret_cast<float4*>(&osum[kg][4 * c4]) = o;
+    if (c4 == 0) lsum[kg] = l;
     __syncthreads();
     if (tid < kHeadDim) {
         float* dst = part + ((uint64_t)bh * gridDim.x + blockIdx.x) * (kHeadDim + 2);
-        dst[2 + tid] = osum[0][tid] + osum[1][tid];
+        float t = 0.0f;
+#pragma unroll
+        for (int g = 0; g < 8; g++) t += osum[g][tid];
+        dst[2 + tid] = t;
         if (tid == 0) {
+            float ls = 0.0f;
+#pragma unroll
+            for (int g = 0; g < 8; g++) ls += lsum[g];
             dst[0] = m;
-            dst[1] = lsum[0] + lsum[1];
+            dst[1] = ls;
         }
     }
 }
