@@ -226,6 +226,11 @@ int rumus_hip_rmsnorm(const float* x, const float* weight, float* y, uint32_t ro
 int rumus_hip_swiglu(const float* gate, const float* up, float* out, uint64_t numel,
                      rumus_hip_stream_t stream);
 
+/* out[r, c] = silu(gate_up[r, c]) * gate_up[r, n + c] for gate_up [rows, 2n]: the two
+ * halves of a fused gate|up projection.  out [rows, n] must not alias gate_up. */
+int rumus_hip_swiglu_rows(const float* gate_up, float* out, uint32_t rows, uint32_t n,
+                          rumus_hip_stream_t stream);
+
 /* out = a + b; out may alias a or b */
 int rumus_hip_add(const float* a, const float* b, float* out, uint64_t numel,
                   rumus_hip_stream_t stream);

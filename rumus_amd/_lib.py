@@ -62,6 +62,7 @@ PROTOTYPES = {
     "rumus_hip_qmatmul_int4_perm": (_i32, [_vp] * 7 + [_u32] * 6 + [_vp]),
     "rumus_hip_rmsnorm": (_i32, [_vp, _vp, _vp, _u32, _u32, C.c_float, _vp]),
     "rumus_hip_swiglu": (_i32, [_vp, _vp, _vp, _u64, _vp]),
+    "rumus_hip_swiglu_rows": (_i32, [_vp, _vp, _u32, _u32, _vp]),
     "rumus_hip_add": (_i32, [_vp, _vp, _vp, _u64, _vp]),
     "rumus_hip_attention": (_i32, [_vp] * 4 + [_u32] * 5 + [C.POINTER(C.c_uint64), _i32, _vp]),
 }

@@ -36,6 +36,16 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const float* __restrict__ g
     out[i] = g / (1.0f + expf(-g)) * up[i];
 }
 
+// gate and up as the two halves of one [rows, 2n] matrix (the output of a fused gate|up projection)
+__global__ __launch_bounds__(256) void swiglu_rows_kernel(const float* __restrict__ gate_up, float* __restrict__ out,
+                                                          uint32_t n) {
+    const uint32_t c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= n) return;
+    const float* row = gate_up + (uint64_t)blockIdx.y * 2 * n;
+    const float g = row[c];
+    out[(uint64_t)blockIdx.y * n + c] = g / (1.0f + expf(-g)) * row[n + c];
+}
+
 __global__ __launch_bounds__(256) void add_kernel(const float* __restrict__ a, const float* __restrict__ b,
                                                   float* __restrict__ out, uint64_t numel) {
     const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
@@ -259,6 +269,15 @@ int rumus_hip_swiglu(const float* gate, const float* up, float* out, uint64_t nu
     hipLaunchKernelGGL(swiglu_kernel, dim3((uint32_t)((numel + 255) / 256)), dim3(256), 0, as_stream(stream), gate,
                        up, out, numel);
     return check_launch("swiglu_kernel");
+}
+
+int rumus_hip_swiglu_rows(const float* gate_up, float* out, uint32_t rows, uint32_t n, rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE(gate_up && out, "swiglu_rows: null buffer");
+    RUMUS_REQUIRE(rows <= 65535, "swiglu_rows: rows %u beyond the grid limit", rows);
+    if (rows == 0 || n == 0) return RUMUS_HIP_OK;
+    hipLaunchKernelGGL(swiglu_rows_kernel, dim3(ceil_div(n, 256), rows), dim3(256), 0, as_stream(stream), gate_up, out,
+                       n);
+    return check_launch("swiglu_rows_kernel");
 }
 
 int rumus_hip_add(const float* a, const float* b, float* out, uint64_t numel, rumus_hip_stream_t stream) {

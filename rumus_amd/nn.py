@@ -201,6 +201,24 @@ class DecoderBlockW4:
         self.dim = proj["q"].in_features
         if self.dim != heads * 128:
             raise ValueError("DecoderBlockW4: head_dim must be 128")
+        # q|k|v and gate|up read the same activations: one launch each over the column-wise
+        # concatenation of their weights (packed words, scales and zero-points are all [rows, n])
+        self.qkv = self._concat([proj["q"], proj["k"], proj["v"]])
+        self.gate_up = self._concat([proj["gate"], proj["up"]])
+
+    @staticmethod
+    def _concat(layers) -> QLinear:
+        w0 = layers[0].weight
+        for lin in layers:
+            w = lin.weight
+            if (w.k, w.group_size) != (w0.k, w0.group_size) or w.perm is not None or lin.bias is not None:
+                raise ValueError("DecoderBlockW4: fused projections need equal k / group_size, no act-order, no bias")
+        cat = lambda ts: torch.cat(ts, dim=1).contiguous()
+        n = sum(lin.weight.n for lin in layers)
+        return QLinear(QuantizedTensor(w0.k, n, w0.padded_k, w0.group_size, w0.num_groups,
+                                       cat([lin.weight.packed_tensor for lin in layers]),
+                                       cat([lin.weight.scales_tensor for lin in layers]),
+                                       cat([lin.weight.zp_tensor for lin in layers])), None)
 
     @classmethod
     def from_f32(cls, weights: dict, group_size: int, heads: int, eps: float = 1e-6) -> "DecoderBlockW4":
@@ -216,16 +234,16 @@ class DecoderBlockW4:
     def forward(self, x: torch.Tensor, k_cache: Optional[torch.Tensor] = None,
                 v_cache: Optional[torch.Tensor] = None, pos: int = 0):
         """``x`` is ``[batch, n, dim]``.  Without caches: causal self-attention over the n tokens
-        (prefill); returns ``(y, k, v)`` with k, v ``[batch, n, heads, 128]``.  With caches
-        (``[batch, T, heads, 128]``, valid below ``pos``): n must be 1; the new key/value are
-        written at ``pos`` and the token attends positions ``0..pos``; returns ``(y, k_cache, v_cache)``."""
+        (prefill); returns ``(y, k, v)`` with k, v ``[batch, n, heads, 128]`` (views of the fused
+        q|k|v output).  With caches (``[batch, T, heads, 128]``, valid below ``pos``): n must be 1;
+        the new key/value are written at ``pos`` and the token attends positions ``0..pos``;
+        returns ``(y, k_cache, v_cache)``."""
         b, n, d = x.shape
         h = self.heads
         x2 = x.reshape(b * n, d)
         hn = ops.rmsnorm(x2, self.norm1, self.eps)
-        q = self.proj["q"](hn).view(b, n, h, 128)
-        k = self.proj["k"](hn).view(b, n, h, 128)
-        v = self.proj["v"](hn).view(b, n, h, 128)
+        qkv = self.qkv(hn).view(b, n, 3, h, 128)
+        q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
         if k_cache is None:
             att = ops.attention(q, k, v, causal=True)
             k_out, v_out = k, v
@@ -239,9 +257,7 @@ class DecoderBlockW4:
         o = self.proj["o"](att.view(b * n, d))
         x1 = ops.add(x2, o, out=o)
         h2 = ops.rmsnorm(x1, self.norm2, self.eps, out=hn)
-        gate = self.proj["gate"](h2)
-        up = self.proj["up"](h2)
-        act = ops.swiglu(gate, up, out=gate)
+        act = ops.swiglu_rows(self.gate_up(h2))
         down = self.proj["down"](act)
         y = ops.add(x1, down, out=down)
         return y.view(b, n, d), k_out, v_out

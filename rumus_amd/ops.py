@@ -233,6 +233,15 @@ def swiglu(gate, up, out=None):
     return y
 
 
+def swiglu_rows(gate_up, out=None):
+    """gate_up [rows, 2n] (gate | up side by side) -> silu(gate) * up, [rows, n]."""
+    rows, n2 = gate_up.shape
+    y = out if out is not None else torch.empty((rows, n2 // 2), dtype=torch.float32, device=gate_up.device)
+    call("rumus_hip_swiglu_rows", _dev(gate_up, torch.float32, "gate_up"), _dev(y, torch.float32, "out"), rows,
+         n2 // 2, _stream())
+    return y
+
+
 def add(a, b, out=None):
     y = out if out is not None else torch.empty_like(a)
     call("rumus_hip_add", _dev(a, torch.float32, "a"), _dev(b, torch.float32, "b"), _dev(y, torch.float32, "out"),

@@ -36,6 +36,7 @@ def test_swiglu_and_add(ops):
     u = rng.normal(0, 1, (5, 1001)).astype(np.float32)
     g[0, :4] = [-100.0, 100.0, 0.0, -20.0]
     close(host(ops.swiglu(dev(g), dev(u))), oracle.swiglu(g, u), atol=1e-6)
+    close(host(ops.swiglu_rows(dev(np.concatenate([g, u], axis=1)))), oracle.swiglu(g, u), atol=1e-6)
     np.testing.assert_array_equal(host(ops.add(dev(g), dev(u))), g + u)
 
 
