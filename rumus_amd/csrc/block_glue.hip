@@ -11,20 +11,49 @@
 namespace rumus {
 
 // ---- RMSNorm: y[r,:] = x[r,:] * rsqrt(mean(x[r,:]^2) + eps) * weight ---------------------
+// One workgroup per row.  VEC: dim % 4 == 0, dim <= 8192 and 16-byte aligned rows: the row is
+// read once with up to eight 128-bit loads per thread, all issued before the first use (a
+// single decode row is pure latency otherwise: sixteen dependent 4-byte loads per thread).
+template <bool VEC>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                       float* __restrict__ y, uint32_t dim, float eps) {
     __shared__ float red[4];
     const float* xr = x + (uint64_t)blockIdx.x * dim;
     float* yr = y + (uint64_t)blockIdx.x * dim;
+    float4 v[8], wv[8];
     float ss = 0.0f;
-    for (uint32_t i = threadIdx.x; i < dim; i += 256) ss = fmaf(xr[i], xr[i], ss);
+    if (VEC) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t i = (j * 256 + threadIdx.x) * 4;
+            const bool in = i < dim;
+            v[j] = *reinterpret_cast<const float4*>(xr + (in ? i : 0));
+            wv[j] = *reinterpret_cast<const float4*>(w + (in ? i : 0));
+            if (!in) v[j] = make_float4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            ss = fmaf(v[j].x, v[j].x, fmaf(v[j].y, v[j].y, fmaf(v[j].z, v[j].z, fmaf(v[j].w, v[j].w, ss))));
+    } else {
+        for (uint32_t i = threadIdx.x; i < dim; i += 256) ss = fmaf(xr[i], xr[i], ss);
+    }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
     __syncthreads();
     const float total = (red[0] + red[1]) + (red[2] + red[3]);
     const float inv = 1.0f / sqrtf(total / (float)dim + eps);
-    for (uint32_t i = threadIdx.x; i < dim; i += 256) yr[i] = xr[i] * inv * w[i];
+    if (VEC) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t i = (j * 256 + threadIdx.x) * 4;
+            if (i < dim)
+                *reinterpret_cast<float4*>(yr + i) = make_float4(v[j].x * inv * wv[j].x, v[j].y * inv * wv[j].y,
+                                                                 v[j].z * inv * wv[j].z, v[j].w * inv * wv[j].w);
+        }
+    } else {
+        for (uint32_t i = threadIdx.x; i < dim; i += 256) yr[i] = xr[i] * inv * w[i];
+    }
 }
 
 // ---- SwiGLU: out = silu(gate) * up, silu(t) = t / (1 + exp(-t)) ----------------------------
@@ -237,13 +266,17 @@ __global__ __launch_bounds__(kHeadDim) void attention_merge_kernel(AttnArgs a, c
                                                                    uint32_t slices) {
     const uint32_t bh = blockIdx.x, b = bh / a.heads, h = bh % a.heads, dim = threadIdx.x;
     const float* src = part + (uint64_t)bh * slices * (kHeadDim + 2);
+    // slices is small (kv_len / 256); the loads of a pass do not depend on each other
     float m = -INFINITY;
+#pragma unroll 8
     for (uint32_t s = 0; s < slices; s++) m = fmaxf(m, src[s * (kHeadDim + 2)]);
     float l = 0.0f, o = 0.0f;
+#pragma unroll 8
     for (uint32_t s = 0; s < slices; s++) {
-        const float w = expf(src[s * (kHeadDim + 2)] - m);
-        l = fmaf(w, src[s * (kHeadDim + 2) + 1], l);
-        o = fmaf(w, src[s * (kHeadDim + 2) + 2 + dim], o);
+        const float ms = src[s * (kHeadDim + 2)], ls = src[s * (kHeadDim + 2) + 1], os = src[s * (kHeadDim + 2) + 2 + dim];
+        const float w = expf(ms - m);
+        l = fmaf(w, ls, l);
+        o = fmaf(w, os, o);
     }
     a.o[b * a.o_sb + h * a.o_sh + dim] = o / l;
 }
@@ -259,7 +292,11 @@ int rumus_hip_rmsnorm(const float* x, const float* weight, float* y, uint32_t ro
     RUMUS_REQUIRE(x && weight && y, "rmsnorm: null buffer");
     RUMUS_REQUIRE(dim > 0, "rmsnorm: dim must be > 0");
     if (rows == 0) return RUMUS_HIP_OK;
-    hipLaunchKernelGGL(rmsnorm_kernel, dim3(rows), dim3(256), 0, as_stream(stream), x, weight, y, dim, eps);
+    const bool vec = dim % 4 == 0 && dim <= 8192 &&
+                     ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(weight) |
+                       reinterpret_cast<uintptr_t>(y)) & 15) == 0;
+    if (vec) hipLaunchKernelGGL(rmsnorm_kernel<true>, dim3(rows), dim3(256), 0, as_stream(stream), x, weight, y, dim, eps);
+    else hipLaunchKernelGGL(rmsnorm_kernel<false>, dim3(rows), dim3(256), 0, as_stream(stream), x, weight, y, dim, eps);
     return check_launch("rmsnorm_kernel");
 }
 
