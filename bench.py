@@ -83,7 +83,8 @@ def bench_gemv(torch, ops, steps, warmup):
     dev = torch.device("cuda:0")
     w0, x0 = workloads.w4_gemv(0)
     x = torch.from_numpy(x0).to(dev)
-    sets, sets_awq = [], []       # reference storage (f32 zero-points); AWQ storage (u4 zero-points)
+    # reference storage (f32 zero-points); its tile-major decode layout; AWQ storage (u4 zero-points)
+    sets, sets_dl, sets_awq = [], [], []
     gen = torch.Generator(device=dev).manual_seed(0)
     for i in range(WEIGHT_SETS):
         if i == 0:
@@ -91,18 +92,25 @@ def bench_gemv(torch, ops, steps, warmup):
         else:
             w = torch.randn((K, N), generator=gen, device=dev, dtype=torch.float32) * 0.02
         sets.append(ops.w4_quantize_pack(w, G))
+        sets_dl.append(ops.w4_decode_layout(*sets[-1], G))
         sets_awq.append(ops.w4_quantize_pack_awq(w, G))
         del w
     ys = [torch.empty((M, N), dtype=torch.float32, device=dev) for _ in range(WEIGHT_SETS)]
     torch.cuda.synchronize()
 
+    # what QLinear.forward launches for a decode row: the decode-layout entry point
     def burst_rotating():
-        for (p, s, z), y in zip(sets, ys):
-            ops.qmatmul_int4(x, p, s, z, K, G, out=y)
+        for (p, s, z), y in zip(sets_dl, ys):
+            ops.qmatmul_int4_decode(x, p, s, z, K, G, out=y)
 
     def burst_resident():
-        p, s, z = sets[0]
+        p, s, z = sets_dl[0]
         for y in ys:
+            ops.qmatmul_int4_decode(x, p, s, z, K, G, out=y)
+
+    # the same GEMV through the reference-layout entry point (64-byte segments 16 KB apart)
+    def burst_rotating_ref():
+        for (p, s, z), y in zip(sets, ys):
             ops.qmatmul_int4(x, p, s, z, K, G, out=y)
 
     def burst_rotating_awq():
@@ -114,7 +122,9 @@ def bench_gemv(torch, ops, steps, warmup):
     sec_res, launches_res, _ = time_graph(torch, burst_resident, WEIGHT_SETS, steps, warmup)
     y0 = ys[0].cpu().numpy()
     sec_awq, launches_awq, _ = time_graph(torch, burst_rotating_awq, WEIGHT_SETS, steps, warmup)
+    sec_ref, launches_ref, _ = time_graph(torch, burst_rotating_ref, WEIGHT_SETS, steps, warmup)
     return {
+        "sec_ref": sec_ref, "launches_ref": launches_ref,
         "sec_awq": sec_awq, "launches_awq": launches_awq,
         "sec": sec, "launches": launches, "graph": used_graph,
         "sec_resident": sec_res, "launches_resident": launches_res,
@@ -377,11 +387,16 @@ def main():
         "value": gbs, "unit": "GB/s", "n_gpus": 1, "steps": r["launches"], "warmup": warmup,
         "ms_per_step": per_launch * 1e3, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "w4_gemv_1x4096x4096_g128_awq_f32zp", "weight_sets_rotated": WEIGHT_SETS,
+        "config": {"workload": "w4_gemv_1x4096x4096_g128_awq_f32zp", "weight_layout": "tile-major copy (16 columns)", "weight_sets_rotated": WEIGHT_SETS,
                    "hip_graph": r["graph"], "bytes_per_step": BYTES_F32_ZP},
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": gbs / HBM_PEAK_GBS, "traffic": GEMV_TRAFFIC_BYTES},
         "gbs_at_u4_zero_point_bytes": BYTES_U4_ZP / per_launch / 1e9,
+        "reference_layout_entry": {
+            "ms_per_step": r["sec_ref"] / r["launches_ref"] * 1e3,
+            "gbs": BYTES_F32_ZP / (r["sec_ref"] / r["launches_ref"]) / 1e9,
+            "note": "rumus_hip_qmatmul_int4 on the reference's row-major arrays; the headline uses the "
+                    "tile-major copy QuantizedTensor builds once (same words, same bytes)"},
         "awq_storage_u4_zero_points": {
             "ms_per_step": r["sec_awq"] / r["launches_awq"] * 1e3, "bytes_per_step": BYTES_U4_ZP,
             "gbs": BYTES_U4_ZP / (r["sec_awq"] / r["launches_awq"]) / 1e9,

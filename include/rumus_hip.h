@@ -202,6 +202,27 @@ int rumus_hip_qmatmul_int4_perm(const float* x, const uint32_t* packed_sorted,
                                 uint32_t group_size, uint32_t num_groups,
                                 rumus_hip_stream_t stream);
 
+/* EXTENSION (decode layout, done once per weight): tile-major copies of the
+ * three arrays of a QuantizedTensor, tile = 16 columns over all rows:
+ *   packed_t[(c*(padded_k/8) + r)*16 + j] = packed[r*n + 16*c + j]
+ *   scales_t[(c*num_groups + g)*16 + j]   = scales[g*n + 16*c + j]   (zero_points alike)
+ * Same words, same sizes, another order: the decode kernel's workgroup (16
+ * columns, all of K) then reads one contiguous slab.  EINVAL unless n % 16 == 0. */
+int rumus_hip_w4_decode_layout(const uint32_t* packed, const float* scales,
+                               const float* zero_points, uint32_t padded_k, uint32_t n,
+                               uint32_t group_size, uint32_t* packed_t, float* scales_t,
+                               float* zero_points_t, rumus_hip_stream_t stream);
+
+/* EXTENSION: QLinear::forward for m <= 8 on the decode layout; same arithmetic
+ * and results as rumus_hip_qmatmul_int4_perm (bit for bit).  perm may be NULL.
+ * EINVAL unless m <= 8, n % 16 == 0, group_size % 32 == 0. */
+int rumus_hip_qmatmul_int4_decode(const float* x, const uint32_t* packed_t,
+                                  const float* scales_t, const float* zero_points_t,
+                                  const float* bias, const int32_t* perm, float* y,
+                                  uint32_t m, uint32_t k, uint32_t n, uint32_t padded_k,
+                                  uint32_t group_size, uint32_t num_groups,
+                                  rumus_hip_stream_t stream);
+
 /* EXTENSION: qmatmul_int4_perm on AWQ storage: zero-points come as qzeros
  * (layout above) instead of f32.  perm may be NULL (plain k order).
  * EINVAL also unless n % 8 == 0. */

@@ -21,6 +21,9 @@ struct W4Args {
     // AWQ storage (or null): integer zero-points, eight per word along n, column col in bits
     // 4*(col%8) of word g*(n/8) + col/8; `zp` is null then and n % 8 == 0
     const uint32_t* zp4;
+    // decode layout (w4_gemv_dot8 only): packed, scales and zp are tile-major copies, tile = 16
+    // columns: packed_t[(c*word_rows + r)*16 + j] = packed[r*n + 16*c + j], likewise the metadata
+    bool tiled;
 };
 
 // zero-points of 4 (col % 4 == 0) or 2 (col % 2 == 0) adjacent columns from the packed form

@@ -107,6 +107,15 @@ __global__ __launch_bounds__(256) void w4_quantize_pack_awq_kernel(
     }
 }
 
+// Decode layout: tile-major copy of a [rows, n] array of 32-bit words, tile = 16 columns:
+// out[(c*rows + r)*16 + j] = in[r*n + 16*c + j].  One thread per 4 words.
+__global__ __launch_bounds__(256) void w4_tile16_kernel(const uint4* __restrict__ in, uint4* __restrict__ out,
+                                                        uint32_t rows, uint32_t n) {
+    const uint32_t q = blockIdx.x * 256 + threadIdx.x, r = blockIdx.y;     // q: which group of 4 columns
+    if (q * 4 >= n) return;
+    out[((uint64_t)(q >> 2) * rows + r) * 4 + (q & 3)] = in[(uint64_t)r * (n / 4) + q];
+}
+
 // packed_sorted word (jr, col) gathers the nibbles of original rows
 // perm[8*jr .. 8*jr+7].
 __global__ __launch_bounds__(256) void w4_gather_rows_kernel(const uint32_t* __restrict__ packed,
@@ -148,6 +157,32 @@ int rumus_hip_w4_quantize_pack(const float* w, uint32_t k, uint32_t n, uint32_t 
                                uint32_t* packed, float* scales, float* zero_points,
                                rumus_hip_stream_t stream) {
     return quantize_pack<false>(w, k, n, group_size, packed, scales, zero_points, as_stream(stream));
+}
+
+int rumus_hip_w4_decode_layout(const uint32_t* packed, const float* scales, const float* zero_points,
+                               uint32_t padded_k, uint32_t n, uint32_t group_size, uint32_t* packed_t,
+                               float* scales_t, float* zero_points_t, rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE(packed && scales && zero_points && packed_t && scales_t && zero_points_t,
+                  "w4_decode_layout: null buffer");
+    RUMUS_REQUIRE(n % 16 == 0, "w4_decode_layout: n must be a multiple of 16 (got %u)", n);
+    RUMUS_REQUIRE(group_size > 0 && padded_k % group_size == 0 && group_size % 8 == 0,
+                  "w4_decode_layout: padded_k %u is not a whole number of groups of %u", padded_k, group_size);
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(packed) | reinterpret_cast<uintptr_t>(scales) |
+                           reinterpret_cast<uintptr_t>(zero_points) | reinterpret_cast<uintptr_t>(packed_t) |
+                           reinterpret_cast<uintptr_t>(scales_t) | reinterpret_cast<uintptr_t>(zero_points_t);
+    RUMUS_REQUIRE((bits & 15) == 0, "w4_decode_layout: buffers must be 16-byte aligned");
+    if (padded_k == 0 || n == 0) return RUMUS_HIP_OK;
+    const uint32_t word_rows = padded_k / 8, groups = padded_k / group_size;
+    RUMUS_REQUIRE(word_rows <= 65535, "w4_decode_layout: padded_k %u beyond the grid limit", padded_k);
+    hipStream_t s = as_stream(stream);
+    const dim3 gx(ceil_div(n / 4, 256));
+    hipLaunchKernelGGL(w4_tile16_kernel, dim3(gx.x, word_rows), dim3(256), 0, s,
+                       reinterpret_cast<const uint4*>(packed), reinterpret_cast<uint4*>(packed_t), word_rows, n);
+    hipLaunchKernelGGL(w4_tile16_kernel, dim3(gx.x, groups), dim3(256), 0, s,
+                       reinterpret_cast<const uint4*>(scales), reinterpret_cast<uint4*>(scales_t), groups, n);
+    hipLaunchKernelGGL(w4_tile16_kernel, dim3(gx.x, groups), dim3(256), 0, s,
+                       reinterpret_cast<const uint4*>(zero_points), reinterpret_cast<uint4*>(zero_points_t), groups, n);
+    return check_launch("w4_tile16_kernel");
 }
 
 int rumus_hip_w4_quantize_pack_awq(const float* w, uint32_t k, uint32_t n, uint32_t group_size,

@@ -52,6 +52,11 @@ class QuantizedTensor:
         self.group_size, self.num_groups = group_size, num_groups
         self.packed_tensor, self.scales_tensor, self.zp_tensor = packed, scales, zp
         self.perm = perm  # act-order: original row held at each sorted position
+        # tile-major copies for the decode kernel (same words in the order one workgroup reads
+        # them); built once, costs a second copy of the weight in device memory
+        self.decode = None
+        if n % 16 == 0 and group_size % 32 == 0 and packed.is_cuda:
+            self.decode = ops.w4_decode_layout(packed, scales, zp, group_size)
 
     @classmethod
     def from_f32(cls, data: torch.Tensor, k: int, n: int, group_size: int,
@@ -82,6 +87,11 @@ class QuantizedTensor:
         return cls(k, packed.shape[1], padded_k, group_size, groups, packed, scales, zp, perm)
 
 
+# batches up to this many rows take the decode kernel (its cost grows with the rows; from 6 on
+# the matrix-core kernel is faster)
+DECODE_ROWS = 5
+
+
 class QLinear:
     """Linear layer with frozen INT4 weights and optional bias (quant.rs:165-222)."""
 
@@ -99,6 +109,8 @@ class QLinear:
     def forward(self, x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``y = x @ dequant(W) + bias`` in one launch (the reference runs a second add_bias pass)."""
         w = self.weight
+        if w.decode is not None and x.shape[0] <= DECODE_ROWS:
+            return ops.qmatmul_int4_decode(x, *w.decode, w.k, w.group_size, bias=self.bias, perm=w.perm, out=out)
         return ops.qmatmul_int4_perm(x, w.packed_tensor, w.scales_tensor, w.zp_tensor, w.k,
                                      w.group_size, bias=self.bias, perm=w.perm, out=out)
 

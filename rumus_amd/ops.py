@@ -156,6 +156,20 @@ def w4_quantize_pack_awq(w: torch.Tensor, group_size: int):
     return packed, scales, qzeros
 
 
+def w4_decode_layout(packed, scales, zp, group_size):
+    """Tile-major copies (16 columns per tile) of the three arrays of an INT4 weight."""
+    rows, n = packed.shape
+    out = (torch.empty_like(packed), torch.empty_like(scales), torch.empty_like(zp))
+    call("rumus_hip_w4_decode_layout", _dev(packed, torch.int32, "packed"), _dev(scales, torch.float32, "scales"),
+         _dev(zp, torch.float32, "zero_points"), rows * 8, n, group_size, out[0].data_ptr(), out[1].data_ptr(),
+         out[2].data_ptr(), _stream())
+    return out
+
+
+def qmatmul_int4_decode(x, packed_t, scales_t, zp_t, k, group_size, bias=None, perm=None, out=None):
+    return _w4_call("rumus_hip_qmatmul_int4_decode", x, packed_t, scales_t, zp_t, bias, perm, k, group_size, out)
+
+
 def qmatmul_int4_zp4(x, packed, scales, qzeros, k, group_size, bias=None, perm=None, out=None):
     m = x.shape[0]
     n = packed.shape[1]

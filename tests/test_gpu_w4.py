@@ -368,3 +368,40 @@ def test_zp4_act_order(ops):
     want = oracle.qmatmul_int4(x[:, perm], packed, scales, zp, k, g, threads=8)
     got = host(ops.qmatmul_int4_zp4(dev(x), dev(packed), dev(scales), dev(qzeros), k, g, perm=dev(perm)))
     assert_close(got, want)
+
+
+# ---- decode layout: tile-major copies of the weight arrays -----------------------------------
+
+@pytest.mark.parametrize("m,k,n,g", [(1, 4096, 4096, 128), (3, 1000, 48, 64), (8, 512, 11008, 32), (5, 256, 16, 256)])
+def test_decode_layout_is_bit_identical(ops, m, k, n, g):
+    say(f"qmatmul_int4_decode m={m} k={k} n={n} g={g}")
+    rng = np.random.default_rng(m + k + n)
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    x = rng.normal(0, 1, (m, k)).astype(np.float32)
+    b = rng.normal(0, 0.01, n).astype(np.float32)
+    packed, scales, zp = oracle.w4_from_f32(w, g)
+    d = [dev(a) for a in (packed, scales, zp)]
+    pt, st, zt = ops.w4_decode_layout(*d, g)
+    # the layout itself: tile c holds columns 16c .. 16c+15 of every row, row-major
+    want_pt = packed.reshape(packed.shape[0], n // 16, 16).transpose(1, 0, 2).reshape(-1)
+    np.testing.assert_array_equal(host_u32(pt).reshape(-1), want_pt)
+    want_st = scales.reshape(scales.shape[0], n // 16, 16).transpose(1, 0, 2).reshape(-1)
+    np.testing.assert_array_equal(host(st).reshape(-1), want_st)
+    got = host(ops.qmatmul_int4_decode(dev(x), pt, st, zt, k, g, bias=dev(b)))
+    assert_close(got, oracle.qmatmul_int4(x, packed, scales, zp, k, g, bias=b, threads=8))
+    if m <= 5:   # the reference-layout entry point runs the same kernel on these shapes
+        np.testing.assert_array_equal(got, host(ops.qmatmul_int4(dev(x), *d, k, g, bias=dev(b))))
+
+
+def test_decode_layout_rejects_bad_arguments(ops):
+    from rumus_amd._lib import RumusError
+    import torch
+    p = torch.zeros((16, 24), dtype=torch.int32, device="cuda")
+    s = torch.zeros((1, 24), dtype=torch.float32, device="cuda")
+    with pytest.raises(RumusError):
+        ops.w4_decode_layout(p, s, s, 128)                       # n % 16 != 0
+    p = torch.zeros((16, 32), dtype=torch.int32, device="cuda")
+    s = torch.zeros((1, 32), dtype=torch.float32, device="cuda")
+    x = torch.zeros((9, 128), dtype=torch.float32, device="cuda")
+    with pytest.raises(RumusError):
+        ops.qmatmul_int4_decode(x, p, s, s, 128, 128)            # more than 8 rows
