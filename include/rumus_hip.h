@@ -55,12 +55,14 @@ int rumus_hip_sync(rumus_hip_stream_t stream);
 
 /* Workspace.  The reference takes every temporary from its BufferPool
  * (rumus/src/backend/gpu/pool.rs:34-75) and returns it on drop; here the only
- * temporaries are those of qmatmul_int4 / qmatmul_int4_perm with m > 5: the
- * partial sums when K is split over workgroups (few output tiles) and the
- * act-order copy of x.  They live in one device buffer per (device, stream),
+ * temporaries are those of qmatmul_int4 / _perm / _zp4 with m > 5 (the partial
+ * sums when K is split over workgroups, and a copy of x when it has to be
+ * gathered or padded) and of attention with q_len == 1 (partial results per
+ * slice of 256 keys).  They live in one device buffer per (device, stream),
  * grown on demand inside the call that needs it.  A caller that must not
  * allocate later (graph capture, serving loop) reserves the size up front:
- * at most (m * k + 16 * m * n) * 4 + 256 bytes per call.
+ * at most (m * k + 16 * m * n) * 4 + 256 bytes per matmul call and
+ * batch * heads * ceil(kv_len / 256) * 520 bytes per attention call.
  * rumus_hip_shutdown frees every workspace (no launch may be in flight). */
 int rumus_hip_workspace_reserve(rumus_hip_stream_t stream, uint64_t bytes);
 int rumus_hip_shutdown(void);
