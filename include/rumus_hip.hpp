@@ -96,6 +96,11 @@ struct QuantizedTensor {
     uint32_t k = 0, n = 0, padded_k = 0, group_size = 0, num_groups = 0;
     DeviceBuffer<uint32_t> packed;    // [(padded_k/8), n]
     DeviceBuffer<float> scales, zp;   // [num_groups, n]
+    // Tile-major copies of the three arrays for the decode kernel (16 columns per tile), built
+    // when the shape allows (n % 16 == 0, group_size % 32 == 0); empty otherwise.
+    DeviceBuffer<uint32_t> packed_t;
+    DeviceBuffer<float> scales_t, zp_t;
+    bool has_decode_layout() const { return packed_t.size() != 0; }
 
     // quant.rs:42-102 on the device; `data` is a device pointer to [k, n] f32.
     static QuantizedTensor from_f32(const float* data, size_t len, uint32_t k, uint32_t n, uint32_t group_size,
@@ -111,6 +116,13 @@ struct QuantizedTensor {
         q.zp = DeviceBuffer<float>((size_t)q.num_groups * n);
         check(rumus_hip_w4_quantize_pack(data, k, n, group_size, q.packed.data(), q.scales.data(), q.zp.data(),
                                          stream));
+        if (n % 16 == 0 && group_size % 32 == 0) {
+            q.packed_t = DeviceBuffer<uint32_t>(q.packed.size());
+            q.scales_t = DeviceBuffer<float>(q.scales.size());
+            q.zp_t = DeviceBuffer<float>(q.zp.size());
+            check(rumus_hip_w4_decode_layout(q.packed.data(), q.scales.data(), q.zp.data(), q.padded_k, n, group_size,
+                                             q.packed_t.data(), q.scales_t.data(), q.zp_t.data(), stream));
+        }
         return q;
     }
 };
@@ -136,7 +148,15 @@ struct QLinear {
     }
 
     // y[m, out] = x[m, in] . dequant(W) + bias; x and y are device pointers.
+    // Up to 5 rows take the decode kernel on the tile-major copy (same result bit for bit).
     void forward(const float* x, uint32_t m, float* y, hipStream_t stream = nullptr) const {
+        if (m <= 5 && weight.has_decode_layout()) {
+            check(rumus_hip_qmatmul_int4_decode(x, weight.packed_t.data(), weight.scales_t.data(), weight.zp_t.data(),
+                                                bias.size() ? bias.data() : nullptr, nullptr, y, m, weight.k,
+                                                weight.n, weight.padded_k, weight.group_size, weight.num_groups,
+                                                stream));
+            return;
+        }
         check(rumus_hip_qmatmul_int4(x, weight.packed.data(), weight.scales.data(), weight.zp.data(),
                                      bias.size() ? bias.data() : nullptr, nullptr, y, m, weight.k, weight.n,
                                      weight.padded_k, weight.group_size, weight.num_groups, stream));
