@@ -91,31 +91,61 @@ __device__ __forceinline__ float2 nonzero2(float2 s) {
     return make_float2(s.x == 0.0f ? 1e-30f : s.x, s.y == 0.0f ? 1e-30f : s.y);
 }
 
-// RT = 32-row tiles per workgroup (BM = 32 * RT); DEPTH = stages of weights in flight;
-// FOLD = MFMA steps between settlements of the zero-point term (group_size / 16, at most a
-// stage); ZP4: zero-points come packed, eight integers per word along n.  out = y when gridDim.z == 1, else the partial tiles [split][m][n].
+// Words and metadata of TN adjacent columns, TN = 2 or 4.
+template <int TN> struct WVec;
+template <> struct WVec<2> { typedef uint2 words; typedef float2 floats; };
+template <> struct WVec<4> { typedef uint4 words; typedef float4 floats; };
+__device__ __forceinline__ uint32_t word_of(const uint2& v, int j) { return j == 0 ? v.x : v.y; }
+__device__ __forceinline__ uint32_t word_of(const uint4& v, int j) { return j == 0 ? v.x : j == 1 ? v.y : j == 2 ? v.z : v.w; }
+__device__ __forceinline__ float flt_of(const float2& v, int j) { return j == 0 ? v.x : v.y; }
+__device__ __forceinline__ float flt_of(const float4& v, int j) { return j == 0 ? v.x : j == 1 ? v.y : j == 2 ? v.z : v.w; }
+__device__ __forceinline__ float2 nonzero(float2 s) { return make_float2(s.x == 0.0f ? 1e-30f : s.x, s.y == 0.0f ? 1e-30f : s.y); }
+__device__ __forceinline__ float4 nonzero(float4 s) {
+    return make_float4(s.x == 0.0f ? 1e-30f : s.x, s.y == 0.0f ? 1e-30f : s.y, s.z == 0.0f ? 1e-30f : s.z,
+                       s.w == 0.0f ? 1e-30f : s.w);
+}
+__device__ __forceinline__ float2 zp4_load(const uint32_t* zp4, uint32_t g, uint32_t n, uint32_t col, float2) {
+    return w4_zp4_load2(zp4, g, n, col);
+}
+__device__ __forceinline__ float4 zp4_load(const uint32_t* zp4, uint32_t g, uint32_t n, uint32_t col, float4) {
+    return w4_zp4_load4(zp4, g, n, col);
+}
+
+// The 8 waves of a workgroup form a WM x (8/WM) grid; a wave owns RT row tiles of 32 and TN
+// column tiles (its lanes hold TN adjacent columns each), so the workgroup covers
+// BM = 32*RT*WM rows and 512 columns.  Wide wave tiles matter: every wave reads the A fragments
+// of its rows from LDS at every step, and with 64-column waves (TN = 2) side by side those
+// reads, not the MFMAs, bound the 128-row tile.
+// DEPTH = stages of weights in flight; FOLD = MFMA steps between settlements of the zero-point
+// term (group_size / 16, at most a stage); ZP4: zero-points come packed, eight integers per
+// word along n.  out = y when gridDim.z == 1, else the partial tiles [split][m][n].
 //
 // The stage body is straight-line code: loads past the end of the work are clamped to valid
 // addresses and their results never used, instead of being skipped, and nothing is consumed
 // right after it was loaded, so that the memory counter never has to drain.
-template <int RT, int DEPTH, int FOLD, bool ZP4>
+template <int RT, int WM, int TN, int DEPTH, int FOLD, bool ZP4>
 __global__ __launch_bounds__(kTileThreads, 2) void w4_gemm_tile_kernel(W4Args a, float* __restrict__ out,
                                                                       uint32_t stages_per_split) {
     // a.x: rows of a.k floats, a.k % 4 == 0, 16-byte aligned, columns already in weight order
     // (the launcher copies x into that form when the caller's x is not)
-    constexpr int BM = 32 * RT;
+    typedef typename WVec<TN>::words words_t;
+    typedef typename WVec<TN>::floats floats_t;
+    constexpr int WN = 8 / WM;
+    static_assert(WN * 32 * TN == kTileCols, "a workgroup covers 512 columns");
+    constexpr int BM = 32 * RT * WM;
     // bytes of one k16 step of one plane: [row tile][k block][row] x 16, plus 128 bytes of skew so
     // that the eight staging lanes of a row (one step each) do not write to the same banks
-    constexpr int STEP = RT * 1024 + 128;
-    constexpr int NI = RT > 2 ? RT / 2 : 1;      // (row, step) pairs staged per thread
+    constexpr int STEP = (BM / 32) * 1024 + 128;
+    constexpr int NI = BM > 64 ? BM / 64 : 1;    // (row, step) pairs staged per thread
     constexpr int PLANE = 8 * STEP;
     __shared__ __attribute__((aligned(16))) uint8_t lds_a[2][2][PLANE];   // [buffer][hi, lo]
     __shared__ __attribute__((aligned(16))) float lds_xs[2][8][BM];       // [buffer][k16 step][row]: sum of x
 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t wm = wave / WN, wn = wave % WN;
     const uint32_t l32 = lane & 31, kb = lane >> 5;
     const uint32_t m0 = blockIdx.y * BM;
-    const uint32_t colbase = blockIdx.x * kTileCols + wave * 64 + 2 * l32;   // this lane's 2 columns
+    const uint32_t colbase = blockIdx.x * kTileCols + wn * (32 * TN) + TN * l32;   // this lane's TN columns
     const bool col_ok = colbase < a.n;                   // n % 4 == 0
     const uint32_t col_c = col_ok ? colbase : 0;
     const uint32_t nstages = (a.padded_k + kStageK - 1) / kStageK;
@@ -172,35 +202,35 @@ __global__ __launch_bounds__(kTileThreads, 2) void w4_gemm_tile_kernel(W4Args a,
         if (b) lds_xs[buf][s_step][row] = sum;
     };
 
-    // ---- weights: one 64-bit load per MFMA step; a register is refilled for DEPTH stages
+    // ---- weights: one load of TN words per MFMA step; a register is refilled for DEPTH stages
     // later right after its step has been converted -----------------------------------------
-    uint2 wq[DEPTH][8];
+    words_t wq[DEPTH][8];
     auto weight_load = [&](uint32_t st, int set, int s) __attribute__((always_inline)) {
         const uint32_t kr = min(st * 16 + s * 2 + kb, word_rows - 1);
-        wq[set][s] = *reinterpret_cast<const uint2*>(a.packed + (uint64_t)kr * a.n + col_c);
+        wq[set][s] = *reinterpret_cast<const words_t*>(a.packed + (uint64_t)kr * a.n + col_c);
     };
 
-    v16f acc[RT][2];
+    v16f acc[RT][TN];
 #pragma unroll
     for (int i = 0; i < RT; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < TN; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
     // scale / zero-point: of the current group, and (requested DEPTH stages ahead, like the
     // weights) of the group that follows each settlement point of a stage
     constexpr int NF = 8 / FOLD;                 // settlements per stage
-    auto meta_load = [&](uint32_t g, float2& sc, float2& zp) __attribute__((always_inline)) {
+    auto meta_load = [&](uint32_t g, floats_t& sc, floats_t& zp) __attribute__((always_inline)) {
         g = min(g, a.num_groups - 1);
-        sc = *reinterpret_cast<const float2*>(a.scales + (uint64_t)g * a.n + col_c);
-        zp = ZP4 ? w4_zp4_load2(a.zp4, g, a.n, col_c)
-                 : *reinterpret_cast<const float2*>(a.zp + (uint64_t)g * a.n + col_c);
+        sc = *reinterpret_cast<const floats_t*>(a.scales + (uint64_t)g * a.n + col_c);
+        zp = ZP4 ? zp4_load(a.zp4, g, a.n, col_c, floats_t{})
+                 : *reinterpret_cast<const floats_t*>(a.zp + (uint64_t)g * a.n + col_c);
     };
     uint32_t g_cur = st_begin * kStageK / a.group_size;
-    float2 sc_cur, zp_cur, sc_after[DEPTH][NF], zp_after[DEPTH][NF];
+    floats_t sc_cur, zp_cur, sc_after[DEPTH][NF], zp_after[DEPTH][NF];
     meta_load(g_cur, sc_cur, zp_cur);
-    sc_cur = nonzero2(sc_cur);
+    sc_cur = nonzero(sc_cur);
 
     // metadata of the groups that follow the settlement points of stage `st`
     auto stage_meta_load = [&](uint32_t st, int set) __attribute__((always_inline)) {
@@ -212,25 +242,29 @@ __global__ __launch_bounds__(kTileThreads, 2) void w4_gemm_tile_kernel(W4Args a,
     auto fold = [&](uint32_t buf, int s_last, uint32_t kend, int set, int f) __attribute__((always_inline)) {
         // rank-1 update acc[i][j] += X[i] (x) (-zp[j]) on the f32 matrix core: operand slot k=0
         // carries the values (lanes 0..31), slot k=1 (lanes 32..63) is zero
-        const float zb[2] = {kb == 0 ? -zp_cur.x : 0.0f, kb == 0 ? -zp_cur.y : 0.0f};
+        float zb[TN];
+#pragma unroll
+        for (int j = 0; j < TN; j++) zb[j] = kb == 0 ? -flt_of(zp_cur, j) : 0.0f;
 #pragma unroll
         for (int i = 0; i < RT; i++) {
             float xs = 0.0f;
 #pragma unroll
-            for (int cc = 0; cc < FOLD; cc++) xs += lds_xs[buf][s_last - cc][i * 32 + l32];
+            for (int cc = 0; cc < FOLD; cc++) xs += lds_xs[buf][s_last - cc][(wm * RT + i) * 32 + l32];
             xs = kb == 0 ? xs : 0.0f;
 #pragma unroll
-            for (int j = 0; j < 2; j++)
+            for (int j = 0; j < TN; j++)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(xs, zb[j], acc[i][j], 0, 0, 0);
         }
         const uint32_t g_after = kend / a.group_size;
         if (kend < k_end && g_after != g_cur) {           // uniform: a new group starts
-            const float2 sn = nonzero2(sc_after[set][f]);
-            const float rv[2] = {sc_cur.x / sn.x, sc_cur.y / sn.y};
+            const floats_t sn = nonzero(sc_after[set][f]);
+            float rv[TN];
+#pragma unroll
+            for (int j = 0; j < TN; j++) rv[j] = flt_of(sc_cur, j) / flt_of(sn, j);
 #pragma unroll
             for (int i = 0; i < RT; i++)
 #pragma unroll
-                for (int j = 0; j < 2; j++)
+                for (int j = 0; j < TN; j++)
 #pragma unroll
                     for (int r = 0; r < 16; r++) acc[i][j][r] *= rv[j];
             g_cur = g_after;
@@ -239,33 +273,50 @@ __global__ __launch_bounds__(kTileThreads, 2) void w4_gemm_tile_kernel(W4Args a,
         }
     };
 
+    // A fragments of MFMA step s; with PREFETCH they are read one step ahead of their use, into
+    // the slot of the step's parity (not for the largest tile: it has no registers to spare and
+    // sixteen MFMAs per step to hide the read behind).
+    constexpr bool PREFETCH = RT * TN <= 4;
+    v8h ah[PREFETCH ? 2 : 1][RT], al[PREFETCH ? 2 : 1][RT];
+    auto read_frags = [&](uint32_t buf, int s, int slot) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < RT; i++) {
+            const uint32_t off = s * STEP + (wm * RT + i) * 1024 + lane * 16;
+            ah[slot][i] = *reinterpret_cast<const v8h*>(lds_a[buf][0] + off);
+            al[slot][i] = *reinterpret_cast<const v8h*>(lds_a[buf][1] + off);
+        }
+    };
+
     // Multiply stage `st` from LDS buffer `buf`; refill the weight registers for stage
     // st+DEPTH and convert the activations of stage st+1 into the other buffer.
     auto compute = [&](uint32_t st, uint32_t buf, auto set_tag) __attribute__((always_inline)) {
         constexpr int SET = decltype(set_tag)::value;
+        if (PREFETCH) read_frags(buf, 0, 0);
 #pragma unroll
         for (int s = 0; s < 8; s++) {
-            v8h bfr[2], ah[RT], al[RT];
-            bfr[0] = nibbles_to_f16(wq[SET][s].x);
-            bfr[1] = nibbles_to_f16(wq[SET][s].y);
-            weight_load(st + DEPTH, SET, s);
-#pragma unroll
-            for (int i = 0; i < RT; i++) {
-                const uint32_t off = s * STEP + i * 1024 + lane * 16;
-                ah[i] = *reinterpret_cast<const v8h*>(lds_a[buf][0] + off);
-                al[i] = *reinterpret_cast<const v8h*>(lds_a[buf][1] + off);
+            constexpr int kOne = 1;
+            const int cur = PREFETCH ? (s & kOne) : 0;
+            if (PREFETCH) {
+                if (s + 1 < 8) read_frags(buf, s + 1, (s + 1) & 1);
+                __builtin_amdgcn_sched_barrier(0);    // keep the reads above this step's arithmetic
+            } else {
+                read_frags(buf, s, 0);
             }
-            // all hi products, then all lo products: dependent MFMAs are 2*RT apart
+            v8h bfr[TN];
+#pragma unroll
+            for (int j = 0; j < TN; j++) bfr[j] = nibbles_to_f16(word_of(wq[SET][s], j));
+            weight_load(st + DEPTH, SET, s);
+            // all hi products, then all lo products: dependent MFMAs are TN*RT apart
 #pragma unroll
             for (int i = 0; i < RT; i++)
 #pragma unroll
-                for (int j = 0; j < 2; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[i], bfr[j], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[cur][i], bfr[j], acc[i][j], 0, 0, 0);
 #pragma unroll
             for (int i = 0; i < RT; i++)
 #pragma unroll
-                for (int j = 0; j < 2; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[i], bfr[j], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[cur][i], bfr[j], acc[i][j], 0, 0, 0);
             if ((s + 1) % FOLD == 0) fold(buf, s, st * kStageK + (s + 1) * 16, SET, s / FOLD);
             if (s >= 8 - PIECES) stage_store_piece(st + 1, buf ^ 1, s - (8 - PIECES), DEPTH - 1 - SET);
         }
@@ -299,20 +350,30 @@ __global__ __launch_bounds__(kTileThreads, 2) void w4_gemm_tile_kernel(W4Args a,
         }
     }
 
-    // ---- store: for each row a lane holds 2 adjacent columns -----------------------------
+    // ---- store: for each row a lane holds TN adjacent columns ----------------------------
     if (!col_ok) return;
     const bool final_out = gridDim.z == 1;
     float* dst = out + (final_out ? 0 : (uint64_t)blockIdx.z * a.m * a.n);
-    float2 bv = make_float2(0, 0);
-    if (final_out && a.bias) bv = *reinterpret_cast<const float2*>(a.bias + colbase);
+    float bv[TN];
+#pragma unroll
+    for (int j = 0; j < TN; j++) bv[j] = 0.0f;
+    if (final_out && a.bias) {
+        const floats_t b = *reinterpret_cast<const floats_t*>(a.bias + colbase);
+#pragma unroll
+        for (int j = 0; j < TN; j++) bv[j] = flt_of(b, j);
+    }
 #pragma unroll
     for (int i = 0; i < RT; i++)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            const uint32_t row = m0 + i * 32 + 8 * (r / 4) + 4 * kb + (r % 4);
+            const uint32_t row = m0 + (wm * RT + i) * 32 + 8 * (r / 4) + 4 * kb + (r % 4);
             if (row >= a.m) continue;
-            const float2 o = make_float2(fmaf(acc[i][0][r], sc_cur.x, bv.x), fmaf(acc[i][1][r], sc_cur.y, bv.y));
-            *reinterpret_cast<float2*>(dst + (uint64_t)row * a.n + colbase) = o;
+            float o[TN];
+#pragma unroll
+            for (int j = 0; j < TN; j++) o[j] = fmaf(acc[i][j][r], flt_of(sc_cur, j), bv[j]);
+            float* p = dst + (uint64_t)row * a.n + colbase;
+            if (TN == 4) *reinterpret_cast<float4*>(p) = make_float4(o[0], o[1], o[2], o[TN - 1]);
+            else *reinterpret_cast<float2*>(p) = make_float2(o[0], o[1]);
         }
 }
 
@@ -366,10 +427,10 @@ __global__ __launch_bounds__(256) void w4_prepare_x_kernel(const float* __restri
     xp[(uint64_t)row * k4 + j] = v;
 }
 
-template <int RT, int DEPTH, int FOLD>
+template <int RT, int WM, int TN, int DEPTH, int FOLD>
 static int launch_tile(const W4Args& a_in, hipStream_t s) {
     W4Args a = a_in;
-    const uint32_t tn = ceil_div(a.n, kTileCols), tm = ceil_div(a.m, 32 * RT);
+    const uint32_t tn = ceil_div(a.n, kTileCols), tm = ceil_div(a.m, 32 * RT * WM);
     const uint32_t nstages = ceil_div(a.padded_k, kStageK);
     uint32_t sps = nstages;
     const uint32_t splits = pick_splits(tn * tm, nstages, &sps);
@@ -395,10 +456,10 @@ static int launch_tile(const W4Args& a_in, hipStream_t s) {
         if (splits > 1) out = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + x_bytes);
     }
     if (a.zp4)
-        hipLaunchKernelGGL((w4_gemm_tile_kernel<RT, DEPTH, FOLD, true>), dim3(tn, tm, splits), dim3(kTileThreads), 0,
+        hipLaunchKernelGGL((w4_gemm_tile_kernel<RT, WM, TN, DEPTH, FOLD, true>), dim3(tn, tm, splits), dim3(kTileThreads), 0,
                            s, a, out, sps);
     else
-        hipLaunchKernelGGL((w4_gemm_tile_kernel<RT, DEPTH, FOLD, false>), dim3(tn, tm, splits), dim3(kTileThreads), 0,
+        hipLaunchKernelGGL((w4_gemm_tile_kernel<RT, WM, TN, DEPTH, FOLD, false>), dim3(tn, tm, splits), dim3(kTileThreads), 0,
                            s, a, out, sps);
     if (int rc = check_launch("w4_gemm_tile_kernel")) return rc;
     if (splits > 1) {
@@ -411,24 +472,24 @@ static int launch_tile(const W4Args& a_in, hipStream_t s) {
     return RUMUS_HIP_OK;
 }
 
-template <int RT, int DEPTH>
+template <int RT, int WM, int TN, int DEPTH>
 static int launch_fold(const W4Args& a, hipStream_t s) {
     switch (a.group_size) {                              // MFMA steps of 16 per zero-point settlement
-        case 32: return launch_tile<RT, DEPTH, 2>(a, s);
-        case 64: return launch_tile<RT, DEPTH, 4>(a, s);
-        default: return launch_tile<RT, DEPTH, 8>(a, s);  // a multiple of 128: once per stage
+        case 32: return launch_tile<RT, WM, TN, DEPTH, 2>(a, s);
+        case 64: return launch_tile<RT, WM, TN, DEPTH, 4>(a, s);
+        default: return launch_tile<RT, WM, TN, DEPTH, 8>(a, s);  // a multiple of 128: once per stage
     }
 }
 
 int w4_launch_gemm(const W4Args& a, hipStream_t s) {
     RUMUS_REQUIRE((uint64_t)a.m * a.n < (1ull << 32), "qmatmul_int4: m * n must fit 32 bits");
     RUMUS_REQUIRE(a.m <= 65535 * 32, "qmatmul_int4: m %u is beyond the grid limit", a.m);
-    if (a.m <= 32) return launch_fold<1, 2>(a, s);
-    // 128-row tiles convert each weight word once per 16 MFMAs instead of 8; worth it once
-    // there are enough of them to fill the chip
+    // 32 rows: eight waves side by side, 64 columns each.  64 and 128 rows: a 2 x 4 grid of
+    // waves with 128 columns each (32 or 64 rows per wave).
+    if (a.m <= 32) return launch_fold<1, 1, 2, 2>(a, s);
     const uint64_t big_tiles = (uint64_t)ceil_div(a.m, 128) * ceil_div(a.n, kTileCols);
-    if (a.m <= 64 || big_tiles < 192) return launch_fold<2, 2>(a, s);
-    return launch_fold<4, 1>(a, s);
+    if (a.m <= 64 || big_tiles < 192) return launch_fold<1, 2, 4, 2>(a, s);
+    return launch_fold<2, 2, 4, 1>(a, s);
 }
 
 }  // namespace rumus
