@@ -33,8 +33,8 @@
 // pairs that are refilled for the next stage as soon as they are consumed, so
 // one stage of weights (4 KB per wave, 32 KB per workgroup) is always in flight.
 //
-// A workgroup is 8 waves side by side = 512 columns (two waves per SIMD, so one
-// converts or rescales while the other multiplies), BM = 32 or 64 rows.  Per
+// A workgroup covers 512 columns and 32 or 64 rows with 8 or 4 waves (see the kernel's
+// comment for the wave grids).  Per
 // stage of 128 rows of K the activations of the BM rows are converted once (hi/lo
 // f16, fragment layout, sums per 16 k for the zero-point term) into one of two
 // LDS buffers while the previous stage is multiplied; one barrier per stage.
@@ -123,20 +123,21 @@ __device__ __forceinline__ float4 zp4_load(const uint32_t* zp4, uint32_t g, uint
 // The stage body is straight-line code: loads past the end of the work are clamped to valid
 // addresses and their results never used, instead of being skipped, and nothing is consumed
 // right after it was loaded, so that the memory counter never has to drain.
-template <int RT, int WM, int TN, int DEPTH, int FOLD, bool ZP4>
-__global__ __launch_bounds__(kTileThreads, 2) void w4_gemm_tile_kernel(W4Args a, float* __restrict__ out,
+template <int RT, int WM, int TN, int WAVES, int DEPTH, int FOLD, bool ZP4>
+__global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, float* __restrict__ out,
                                                                       uint32_t stages_per_split) {
     // a.x: rows of a.k floats, a.k % 4 == 0, 16-byte aligned, columns already in weight order
     // (the launcher copies x into that form when the caller's x is not)
     typedef typename WVec<TN>::words words_t;
     typedef typename WVec<TN>::floats floats_t;
-    constexpr int WN = 8 / WM;
+    constexpr int WN = WAVES / WM;
+    constexpr int RPP = 8 * WAVES;               // rows staged per pass: 8 threads per row
     static_assert(WN * 32 * TN == kTileCols, "a workgroup covers 512 columns");
     constexpr int BM = 32 * RT * WM;
     // bytes of one k16 step of one plane: [row tile][k block][row] x 16, plus 128 bytes of skew so
     // that the eight staging lanes of a row (one step each) do not write to the same banks
     constexpr int STEP = (BM / 32) * 1024 + 128;
-    constexpr int NI = BM > 64 ? BM / 64 : 1;    // (row, step) pairs staged per thread
+    constexpr int NI = BM > RPP ? BM / RPP : 1;  // (row, step) pairs staged per thread
     constexpr int PLANE = 8 * STEP;
     __shared__ __attribute__((aligned(16))) uint8_t lds_a[2][2][PLANE];   // [buffer][hi, lo]
     __shared__ __attribute__((aligned(16))) float lds_xs[2][8][BM];       // [buffer][k16 step][row]: sum of x
@@ -156,14 +157,14 @@ __global__ __launch_bounds__(kTileThreads, 2) void w4_gemm_tile_kernel(W4Args a,
 
     // ---- staging role: thread t converts 16 consecutive k (MFMA step t%8) of row t/8 -----
     const uint32_t s_row = tid >> 3, s_step = tid & 7;
-    const bool s_active = s_row < BM;            // BM = 32: half of the threads stage
+    const bool s_active = s_row < BM;            // 32 rows, 8 waves: half of the threads stage
     float4 xraw[DEPTH][NI][4];                   // DEPTH stages of activations in flight, too
     auto stage_load = [&](uint32_t st, int slot) __attribute__((always_inline)) {
         if (!s_active) return;
         const uint32_t k0 = st * kStageK + s_step * 16;
 #pragma unroll
         for (int it = 0; it < NI; it++) {
-            const float* xrow = a.x + (uint64_t)min(m0 + s_row + 64 * it, a.m - 1) * a.k;
+            const float* xrow = a.x + (uint64_t)min(m0 + s_row + RPP * it, a.m - 1) * a.k;
 #pragma unroll
             for (int i = 0; i < 4; i++)
                 xraw[slot][it][i] = *reinterpret_cast<const float4*>(xrow + min(k0 + 4 * i, a.k - 4));
@@ -176,7 +177,7 @@ __global__ __launch_bounds__(kTileThreads, 2) void w4_gemm_tile_kernel(W4Args a,
     auto stage_store_piece = [&](uint32_t st, uint32_t buf, int piece, int slot) __attribute__((always_inline)) {
         if (!s_active) return;
         const int it = piece >> 1, b = piece & 1;         // b: which 8-k block of this thread's step
-        const uint32_t row = s_row + 64 * it;
+        const uint32_t row = s_row + RPP * it;
         const uint32_t rt = row >> 5, r32 = row & 31;
         const uint32_t kk = st * kStageK + s_step * 16 + 8 * b;
         const bool row_ok = m0 + row < a.m;
@@ -427,7 +428,7 @@ __global__ __launch_bounds__(256) void w4_prepare_x_kernel(const float* __restri
     xp[(uint64_t)row * k4 + j] = v;
 }
 
-template <int RT, int WM, int TN, int DEPTH, int FOLD>
+template <int RT, int WM, int TN, int WAVES, int DEPTH, int FOLD>
 static int launch_tile(const W4Args& a_in, hipStream_t s) {
     W4Args a = a_in;
     const uint32_t tn = ceil_div(a.n, kTileCols), tm = ceil_div(a.m, 32 * RT * WM);
@@ -456,10 +457,10 @@ static int launch_tile(const W4Args& a_in, hipStream_t s) {
         if (splits > 1) out = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + x_bytes);
     }
     if (a.zp4)
-        hipLaunchKernelGGL((w4_gemm_tile_kernel<RT, WM, TN, DEPTH, FOLD, true>), dim3(tn, tm, splits), dim3(kTileThreads), 0,
+        hipLaunchKernelGGL((w4_gemm_tile_kernel<RT, WM, TN, WAVES, DEPTH, FOLD, true>), dim3(tn, tm, splits), dim3(64 * WAVES), 0,
                            s, a, out, sps);
     else
-        hipLaunchKernelGGL((w4_gemm_tile_kernel<RT, WM, TN, DEPTH, FOLD, false>), dim3(tn, tm, splits), dim3(kTileThreads), 0,
+        hipLaunchKernelGGL((w4_gemm_tile_kernel<RT, WM, TN, WAVES, DEPTH, FOLD, false>), dim3(tn, tm, splits), dim3(64 * WAVES), 0,
                            s, a, out, sps);
     if (int rc = check_launch("w4_gemm_tile_kernel")) return rc;
     if (splits > 1) {
@@ -472,24 +473,26 @@ static int launch_tile(const W4Args& a_in, hipStream_t s) {
     return RUMUS_HIP_OK;
 }
 
-template <int RT, int WM, int TN, int DEPTH>
+template <int RT, int WM, int TN, int WAVES, int DEPTH>
 static int launch_fold(const W4Args& a, hipStream_t s) {
     switch (a.group_size) {                              // MFMA steps of 16 per zero-point settlement
-        case 32: return launch_tile<RT, WM, TN, DEPTH, 2>(a, s);
-        case 64: return launch_tile<RT, WM, TN, DEPTH, 4>(a, s);
-        default: return launch_tile<RT, WM, TN, DEPTH, 8>(a, s);  // a multiple of 128: once per stage
+        case 32: return launch_tile<RT, WM, TN, WAVES, DEPTH, 2>(a, s);
+        case 64: return launch_tile<RT, WM, TN, WAVES, DEPTH, 4>(a, s);
+        default: return launch_tile<RT, WM, TN, WAVES, DEPTH, 8>(a, s);  // a multiple of 128: once per stage
     }
 }
 
 int w4_launch_gemm(const W4Args& a, hipStream_t s) {
     RUMUS_REQUIRE((uint64_t)a.m * a.n < (1ull << 32), "qmatmul_int4: m * n must fit 32 bits");
     RUMUS_REQUIRE(a.m <= 65535 * 32, "qmatmul_int4: m %u is beyond the grid limit", a.m);
-    // 32 rows: eight waves side by side, 64 columns each.  64 and 128 rows: a 2 x 4 grid of
-    // waves with 128 columns each (32 or 64 rows per wave).
-    if (a.m <= 32) return launch_fold<1, 1, 2, 2>(a, s);
+    // 32 rows: eight waves side by side, 64 columns each.  64 rows, few tiles: a 2 x 4 grid of
+    // waves (32 rows x 128 columns each).  Many tiles: four waves side by side (64 rows x 128
+    // columns each), two such workgroups per CU: the same work per wave as a 128-row tile of
+    // eight waves, finer-grained rounds (25 % faster at m = 2048, n = 11008).
+    if (a.m <= 32) return launch_fold<1, 1, 2, 8, 2>(a, s);
     const uint64_t big_tiles = (uint64_t)ceil_div(a.m, 128) * ceil_div(a.n, kTileCols);
-    if (a.m <= 64 || big_tiles < 192) return launch_fold<1, 2, 4, 2>(a, s);
-    return launch_fold<2, 2, 4, 1>(a, s);
+    if (a.m <= 64 || big_tiles < 128) return launch_fold<1, 2, 4, 8, 2>(a, s);
+    return launch_fold<2, 1, 4, 4, 1>(a, s);
 }
 
 }  // namespace rumus
