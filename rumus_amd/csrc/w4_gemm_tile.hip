@@ -57,8 +57,7 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-constexpr int kTileCols = 512;   // columns per workgroup (8 waves x 64)
-constexpr int kTileThreads = 512;
+constexpr int kTileCols = 512;   // columns per workgroup (every wave-grid shape covers 512)
 constexpr int kStageK = 128;     // rows of K staged per barrier (8 MFMA steps of 16)
 constexpr int kMaxSplits = 16;
 
@@ -85,10 +84,6 @@ __device__ __forceinline__ v8h nibbles_to_f16(uint32_t w) {
 __device__ __forceinline__ void lds_barrier() {
     __builtin_amdgcn_s_waitcnt(0xC07F);          // lgkmcnt(0); vmcnt and expcnt untouched
     __builtin_amdgcn_s_barrier();
-}
-
-__device__ __forceinline__ float2 nonzero2(float2 s) {
-    return make_float2(s.x == 0.0f ? 1e-30f : s.x, s.y == 0.0f ? 1e-30f : s.y);
 }
 
 // Words and metadata of TN adjacent columns, TN = 2 or 4.
@@ -485,13 +480,17 @@ static int launch_fold(const W4Args& a, hipStream_t s) {
 int w4_launch_gemm(const W4Args& a, hipStream_t s) {
     RUMUS_REQUIRE((uint64_t)a.m * a.n < (1ull << 32), "qmatmul_int4: m * n must fit 32 bits");
     RUMUS_REQUIRE(a.m <= 65535 * 32, "qmatmul_int4: m %u is beyond the grid limit", a.m);
-    // 32 rows: eight waves side by side, 64 columns each.  64 rows, few tiles: a 2 x 4 grid of
-    // waves (32 rows x 128 columns each).  Many tiles: four waves side by side (64 rows x 128
-    // columns each), two such workgroups per CU: the same work per wave as a 128-row tile of
-    // eight waves, finer-grained rounds (25 % faster at m = 2048, n = 11008).
-    if (a.m <= 32) return launch_fold<1, 1, 2, 8, 2>(a, s);
-    const uint64_t big_tiles = (uint64_t)ceil_div(a.m, 128) * ceil_div(a.n, kTileCols);
-    if (a.m <= 64 || big_tiles < 128) return launch_fold<1, 2, 4, 8, 2>(a, s);
+    // Three shapes of workgroup, chosen by how many tiles the problem makes (measured on
+    // n = 4096 and n = 11008, m = 16 .. 4096):
+    //   up to 72 tiles of 32 rows: eight waves side by side, 32 rows x 64 columns each; the small
+    //       tile keeps more workgroups in flight when there are fewer tiles than CUs;
+    //   up to 255 tiles of 128 rows: the same eight waves with 64 rows each, so a converted weight
+    //       fragment serves two row tiles;
+    //   beyond: four waves side by side, 64 rows x 128 columns each, two such workgroups per CU
+    //       (fewer LDS fragment reads per MFMA, finer-grained rounds).
+    const uint64_t col_tiles = ceil_div(a.n, kTileCols);
+    if (ceil_div(a.m, 32) * col_tiles <= 72) return launch_fold<1, 1, 2, 8, 1>(a, s);
+    if (ceil_div(a.m, 128) * col_tiles < 256) return launch_fold<2, 1, 2, 8, 1>(a, s);
     return launch_fold<2, 1, 4, 4, 1>(a, s);
 }
 

@@ -72,8 +72,12 @@ SHAPES = [
     (40, 1001, 64, 64, False),    # k % 4 != 0: activations are copied into padded rows first
     (100, 160, 520, 32, True),    # group 32: four settlements per stage, two row tiles
     (24, 192, 48, 96, False),     # group 96 does not divide a stage -> reference-order kernel
-    (1536, 256, 8192, 128, True), # enough tiles for the 128-row variant
-    (1500, 128, 8200, 64, False), # 128-row variant, group 64, ragged rows and columns
+    (1536, 256, 8192, 128, True), # more than 72 tiles: eight waves of 64 rows each
+    (1500, 128, 8200, 64, False), # the same, group 64, ragged rows and columns
+    (300, 160, 4100, 32, True),   # the same, group 32, K tail inside a stage
+    (2048, 256, 8192, 128, True), # 256 tiles of 128 rows: four-wave workgroups, 64 x 128 per wave
+    (1990, 192, 8200, 64, False), # four-wave workgroups, group 64, ragged rows and columns
+    (2100, 96, 8192, 32, True),   # four-wave workgroups, group 32, K shorter than a stage
 ]
 
 
