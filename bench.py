@@ -229,6 +229,51 @@ def probe_mfma_ceiling():
     return {"tops": tops.value, "shader_mhz": mhz.value}
 
 
+def bench_gemv_shapes(torch, ops, steps=400, warmup=40):
+    """The same decode kernel on the wider projections of a Llama-7B block (q|k|v, gate|up, down),
+    each rotating over enough weight sets (> 600 MB) to defeat the Infinity Cache.  The longer a
+    launch, the smaller the share of its fixed start-up and drain."""
+    import ctypes
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev).manual_seed(5)
+    probe = None
+    path = os.path.join(ROOT, "rumus_amd", "librumus_probe.so")
+    if os.path.exists(path):
+        probe = ctypes.CDLL(path)
+        probe.rumus_probe_read_launch.restype = ctypes.c_int
+        probe.rumus_probe_read_launch.argtypes = [ctypes.c_uint64, ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
+    rows = []
+    for k, n in ((4096, 12288), (4096, 22016), (11008, 4096)):
+        nbytes = k * n // 2 + 2 * (k // G) * n * 4 + k * 4 + n * 4
+        nsets = -(-640_000_000 // nbytes)
+        sets = []
+        for _ in range(nsets):
+            w = torch.randn((k, n), generator=gen, device=dev, dtype=torch.float32) * 0.02
+            q = ops.w4_quantize_pack(w, G)
+            sets.append(ops.w4_decode_layout(*q, G))
+            del w, q
+        x = torch.randn((1, k), generator=gen, device=dev)
+        y = torch.empty((1, n), dtype=torch.float32, device=dev)
+
+        def burst():
+            for p, s, z in sets:
+                ops.qmatmul_int4_decode(x, p, s, z, k, G, out=y)
+
+        launches = max(nsets, (steps // nsets) * nsets)
+        sec, timed, _ = time_graph(torch, burst, nsets, launches, warmup)
+        per = sec / timed
+        row = {"workload": f"w4_gemv_1x{k}x{n}_g128", "weight_sets_rotated": nsets, "bytes_per_step": nbytes,
+               "ms_per_step": per * 1e3, "gbs": nbytes / per / 1e9, "hbm_frac": nbytes / per / 1e9 / HBM_PEAK_GBS}
+        if probe is not None:
+            us = ctypes.c_double()
+            if probe.rumus_probe_read_launch(k * n // 2, nsets, ctypes.byref(us)) == 0:
+                row["read_only_launch_us"] = us.value
+                row["frac_of_read_only_launch"] = us.value * 1e-6 * (nbytes / (k * n // 2)) / per
+        rows.append(row)
+        del sets
+    return rows
+
+
 def bench_w4_gemm(torch, ops, m, steps=50, warmup=5):
     """W4 GEMM with act-order (GPTQ style), K=4096, N=11008, g128, symmetric zp=8."""
     k, n = 4096, 11008
@@ -421,6 +466,7 @@ def main():
 
     if not args.only_gemv:
         out["secondary"] = bench_i8_gemm(torch, ops)
+        out["w4_gemv_wider"] = bench_gemv_shapes(torch, ops)
         out["w4_gemm"] = [bench_w4_gemm(torch, ops, 16), bench_w4_gemm(torch, ops, 128)]
         out["decoder_block"] = bench_decoder_block(torch, ops)
 
