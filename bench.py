@@ -351,6 +351,29 @@ def bench_decoder_block(torch, ops):
         t_dec_graph = timed(graph.replay, 20, 3) / 10
     except Exception as exc:
         log(f"[bench] decoder-block graph capture unavailable: {exc!r}")
+    # the block's seven layers through the on-disk form: written once, then loaded (file -> pinned
+    # staging -> device, tile-major copies rebuilt); the file sits in the page cache
+    ckpt = None
+    try:
+        import tempfile
+        import time
+        from rumus_amd import checkpoint
+        with tempfile.TemporaryDirectory() as tmp:
+            path = os.path.join(tmp, "block.safetensors")
+            checkpoint.save_w4(path, {f"blk.{name}": lin for name, lin in blk.proj.items()})
+            size = os.path.getsize(path)
+            checkpoint.load_w4(path, dev)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            loaded = checkpoint.load_w4(path, dev)
+            torch.cuda.synchronize()
+            t_load = time.perf_counter() - t0
+            same = all(torch.equal(loaded[f"blk.{n}"].weight.packed_tensor, blk.proj[n].weight.packed_tensor)
+                       for n in blk.proj)
+            del loaded
+        ckpt = {"file_bytes": size, "load_ms": t_load * 1e3, "gbs": size / t_load / 1e9, "bits_identical": same}
+    except Exception as exc:
+        log(f"[bench] checkpoint leg failed: {exc!r}")
     weight_bytes = 4 * (dim * dim // 2 + 2 * (dim // G) * dim * 4) + \
         2 * (dim * 11008 // 2 + 2 * (dim // G) * 11008 * 4) + (11008 * dim // 2 + 2 * (11008 // G) * dim * 4)
     kv_bytes = 2 * 2048 * dim * 4
@@ -360,7 +383,7 @@ def bench_decoder_block(torch, ops):
             "decode_hip_graph_ms": None if t_dec_graph is None else t_dec_graph * 1e3,
             "decode_weight_and_cache_gbs": (weight_bytes + kv_bytes) / t_best / 1e9,
             "prefill_8x512_ms": t_pre * 1e3, "prefill_tokens_per_s": 8 * 512 / t_pre,
-            "prefill_projection_tflops": flops / t_pre / 1e12}
+            "prefill_projection_tflops": flops / t_pre / 1e12, "checkpoint_load": ckpt}
 
 
 def cpu_baseline(x, w, budget_s=12.0):

@@ -160,6 +160,14 @@ int rumus_hip_w4_quantize_pack_awq(const float* w, uint32_t k, uint32_t n,
                                    float* scales, uint32_t* qzeros,
                                    rumus_hip_stream_t stream);
 
+/* EXTENSION: u4 zero-points of a stored checkpoint (qzeros u32 [num_groups,
+ * n/8], column col in bits 4*(col%8) of word col/8) -> the f32 zero-point
+ * array of the reference's QuantizedTensor (quant.rs:29-31,77-79), exactly.
+ * EINVAL unless n % 8 == 0 and zero_points is 16-byte aligned. */
+int rumus_hip_w4_qzeros_unpack(const uint32_t* qzeros, uint32_t num_groups,
+                               uint32_t n, float* zero_points,
+                               rumus_hip_stream_t stream);
+
 /* custom_forward(&QMatMulINT4FwdOp, [x, packed, scales, zp]) followed by
  * add_bias (rumus-vision/src/quant.rs:191-221,228-256; kernel
  * shaders/qmatmul_int4.wgsl:40-87).  The six scalars are the op's uniform

@@ -135,6 +135,22 @@ __global__ __launch_bounds__(256) void w4_gather_rows_kernel(const uint32_t* __r
     out[(uint64_t)jr * n + col] = word;
 }
 
+// u4 zero-points, eight per word (nibble of column c at bits 4 * (c % 8) of word c / 8) -> one f32 each.
+__global__ __launch_bounds__(256) void w4_qzeros_unpack_kernel(const uint32_t* __restrict__ qzeros,
+                                                               float* __restrict__ zps, uint32_t n) {
+    const uint32_t word = blockIdx.x * 256 + threadIdx.x, g = blockIdx.y;
+    if (word >= n / 8) return;
+    const uint32_t q = qzeros[(uint64_t)g * (n / 8) + word];
+    float4 lo, hi;
+    lo.x = (float)(q & 15u);         lo.y = (float)((q >> 4) & 15u);
+    lo.z = (float)((q >> 8) & 15u);  lo.w = (float)((q >> 12) & 15u);
+    hi.x = (float)((q >> 16) & 15u); hi.y = (float)((q >> 20) & 15u);
+    hi.z = (float)((q >> 24) & 15u); hi.w = (float)(q >> 28);
+    float4* dst = reinterpret_cast<float4*>(zps + (uint64_t)g * n + 8 * word);
+    dst[0] = lo;
+    dst[1] = hi;
+}
+
 template <bool SYM>
 static int quantize_pack(const float* w, uint32_t k, uint32_t n, uint32_t gs, uint32_t* packed,
                          float* scales, float* zps, hipStream_t s) {
@@ -183,6 +199,19 @@ int rumus_hip_w4_decode_layout(const uint32_t* packed, const float* scales, cons
     hipLaunchKernelGGL(w4_tile16_kernel, dim3(gx.x, groups), dim3(256), 0, s,
                        reinterpret_cast<const uint4*>(zero_points), reinterpret_cast<uint4*>(zero_points_t), groups, n);
     return check_launch("w4_tile16_kernel");
+}
+
+int rumus_hip_w4_qzeros_unpack(const uint32_t* qzeros, uint32_t num_groups, uint32_t n, float* zero_points,
+                               rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE(qzeros && zero_points, "w4_qzeros_unpack: null buffer");
+    RUMUS_REQUIRE(n % 8 == 0, "w4_qzeros_unpack: n must be a multiple of 8 (got %u)", n);
+    RUMUS_REQUIRE((reinterpret_cast<uintptr_t>(zero_points) & 15) == 0,
+                  "w4_qzeros_unpack: zero_points must be 16-byte aligned");
+    RUMUS_REQUIRE(num_groups <= 65535, "w4_qzeros_unpack: %u groups are beyond the grid limit", num_groups);
+    if (num_groups == 0 || n == 0) return RUMUS_HIP_OK;
+    hipLaunchKernelGGL(w4_qzeros_unpack_kernel, dim3(ceil_div(n / 8, 256), num_groups), dim3(256), 0,
+                       as_stream(stream), qzeros, zero_points, n);
+    return check_launch("w4_qzeros_unpack_kernel");
 }
 
 int rumus_hip_w4_quantize_pack_awq(const float* w, uint32_t k, uint32_t n, uint32_t group_size,

@@ -156,6 +156,16 @@ def w4_quantize_pack_awq(w: torch.Tensor, group_size: int):
     return packed, scales, qzeros
 
 
+def w4_qzeros_unpack(qzeros, n):
+    """u4 zero-points ``[groups, n/8]`` (eight per word) -> f32 ``[groups, n]``."""
+    groups = qzeros.shape[0]
+    if n % 8 != 0 or qzeros.shape[1] != n // 8:
+        raise ValueError("w4_qzeros_unpack: qzeros must be [groups, n/8]")
+    zp = torch.empty((groups, n), dtype=torch.float32, device=qzeros.device)
+    call("rumus_hip_w4_qzeros_unpack", _dev(qzeros, torch.int32, "qzeros"), groups, n, zp.data_ptr(), _stream())
+    return zp
+
+
 def w4_decode_layout(packed, scales, zp, group_size):
     """Tile-major copies (16 columns per tile) of the three arrays of an INT4 weight."""
     rows, n = packed.shape
