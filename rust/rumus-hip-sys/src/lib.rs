@@ -42,6 +42,23 @@ extern "C" {
                                           scales: *mut f32, zero_points: *mut f32, s: Stream) -> c_int;
     pub fn rumus_hip_w4_quantize_pack_awq(w: *const f32, k: u32, n: u32, group_size: u32, packed: *mut u32,
                                           scales: *mut f32, qzeros: *mut u32, s: Stream) -> c_int;
+    pub fn rumus_hip_w4_qzeros_unpack(qzeros: *const u32, num_groups: u32, n: u32, zero_points: *mut f32,
+                                      s: Stream) -> c_int;
+    pub fn rumus_hip_w4_decode_layout(packed: *const u32, scales: *const f32, zero_points: *const f32,
+                                      padded_k: u32, n: u32, group_size: u32, packed_t: *mut u32,
+                                      scales_t: *mut f32, zero_points_t: *mut f32, s: Stream) -> c_int;
+    pub fn rumus_hip_qmatmul_int4_decode(x: *const f32, packed_t: *const u32, scales_t: *const f32,
+                                         zero_points_t: *const f32, bias: *const f32, perm: *const i32,
+                                         y: *mut f32, m: u32, k: u32, n: u32, padded_k: u32, group_size: u32,
+                                         num_groups: u32, s: Stream) -> c_int;
+    pub fn rumus_hip_rmsnorm(x: *const f32, weight: *const f32, y: *mut f32, rows: u32, dim: u32, eps: f32,
+                             s: Stream) -> c_int;
+    pub fn rumus_hip_swiglu(gate: *const f32, up: *const f32, out: *mut f32, numel: u64, s: Stream) -> c_int;
+    pub fn rumus_hip_swiglu_rows(gate_up: *const f32, out: *mut f32, rows: u32, n: u32, s: Stream) -> c_int;
+    pub fn rumus_hip_add(a: *const f32, b: *const f32, out: *mut f32, numel: u64, s: Stream) -> c_int;
+    pub fn rumus_hip_attention(q: *const f32, k: *const f32, v: *const f32, out: *mut f32, batch: u32,
+                               heads: u32, q_len: u32, kv_len: u32, head_dim: u32, strides: *const u64,
+                               causal: c_int, s: Stream) -> c_int;
     pub fn rumus_hip_qmatmul_int4_zp4(x: *const f32, packed: *const u32, scales: *const f32, qzeros: *const u32,
                                       bias: *const f32, perm: *const i32, y: *mut f32, m: u32, k: u32, n: u32,
                                       padded_k: u32, group_size: u32, num_groups: u32, s: Stream) -> c_int;
