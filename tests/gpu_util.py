@@ -4,7 +4,7 @@ import sys
 import numpy as np
 import torch
 
-RTOL, ATOL = 1e-3, 1e-4   # f32 outputs: north-star tolerance (reduction order differs)
+RTOL, ATOL = 1e-3, 1e-4   # f32 outputs: rel 1e-3, abs 1e-4 (the reduction order differs from the sequential restatement)
 
 
 def say(msg: str) -> None:

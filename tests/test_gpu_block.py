@@ -113,7 +113,7 @@ def test_decoder_block_small(ops):
 
 
 def test_decoder_block_llama7b_shape(ops):
-    # BASELINE's decoder-block configuration at full width: decode at position 2047 against a
+    # the benchmark's decoder-block configuration at full width: decode at position 2047 against a
     # 2047-entry cache, and a (shortened) prefill of 2 x 192 tokens.
     say("decoder block 4096/11008, decode at 2047 and prefill 2x192")
     import torch

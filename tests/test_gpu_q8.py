@@ -178,7 +178,7 @@ def test_i8_gemm_extreme_values(ops):
 
 
 def test_int8_quantlinear_config(ops):
-    # BASELINE config 0: W [512,512] N(0,0.02), X [32,512] N(0,1), b N(0,0.01), seed 0
+    # smallest benchmark configuration: W [512,512] N(0,0.02), X [32,512] N(0,1), b N(0,0.01), seed 0
     say("Int8Linear 32x512x512 seed 0")
     from rumus_amd import nn
     w, x, b = workloads.int8_linear(0)
@@ -192,7 +192,7 @@ def test_int8_quantlinear_config(ops):
 
 
 def test_i8_gemm_prefill_shape_properties(ops):
-    # BASELINE config 3 at full size: 2048 x 4096 x 11008.  The oracle checks a
+    # the INT8 benchmark shape at full size: 2048 x 4096 x 11008.  The oracle checks a
     # sample of rows exactly; the rest is pinned by a row/column checksum
     # identity computed in int64 on the host.
     say("i8_gemm 2048x4096x11008")

@@ -209,7 +209,7 @@ def test_qmatmul_int4_transpose(ops, m, k, n, g):
 
 
 def test_gptq_actorder_config_full_size(ops):
-    # BASELINE config 2: M=16 and M=128, K=4096, N=11008, g128, symmetric zp=8, act-order g_idx
+    # benchmark configuration: M=16 and M=128, K=4096, N=11008, g128, symmetric zp=8, act-order g_idx
     for m in (16, 128):
         say(f"w4 gemm act-order {m}x4096x11008")
         k, n, g = 4096, 11008, 128
@@ -249,7 +249,7 @@ def test_qlinear_module_mirror(ops):
 
 
 def test_headline_shape_properties(ops):
-    # full BASELINE size: compare with the oracle (all host cores) and check linearity
+    # full benchmark size: compare with the oracle (all host cores) and check linearity
     say("w4 gemv 1x4096x4096 g128 full size")
     w, x = workloads.w4_gemv(0)
     pw, sw_, zw = oracle.w4_from_f32(w, 128)
@@ -330,7 +330,7 @@ def test_awq_rejects_bad_shapes(ops):
 
 
 @pytest.mark.parametrize("m,k,n,g,with_bias", [
-    (1, 4096, 4096, 128, True),     # decode kernel, the BASELINE config 2 storage to the letter
+    (1, 4096, 4096, 128, True),     # decode kernel, the benchmark storage (u4 zero-points) to the letter
     (4, 1024, 264, 64, False),      # decode kernel, n % 16 != 0
     (3, 200, 24, 8, True),          # group 8 -> reference-order kernel
     (16, 4096, 4096, 128, True),    # MFMA kernel, K split
