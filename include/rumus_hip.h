@@ -168,6 +168,12 @@ int rumus_hip_w4_qzeros_unpack(const uint32_t* qzeros, uint32_t num_groups,
                                uint32_t n, float* zero_points,
                                rumus_hip_stream_t stream);
 
+/* EXTENSION: IEEE half -> f32, exact (scales of stored checkpoints kept in
+ * half precision; the reference's scales are f32, quant.rs:29).  No
+ * counterpart in the reference. */
+int rumus_hip_f16_to_f32(const uint16_t* in, float* out, uint64_t numel,
+                         rumus_hip_stream_t stream);
+
 /* custom_forward(&QMatMulINT4FwdOp, [x, packed, scales, zp]) followed by
  * add_bias (rumus-vision/src/quant.rs:191-221,228-256; kernel
  * shaders/qmatmul_int4.wgsl:40-87).  The six scalars are the op's uniform

@@ -102,28 +102,64 @@ struct QuantizedTensor {
     DeviceBuffer<float> scales_t, zp_t;
     bool has_decode_layout() const { return packed_t.size() != 0; }
 
+    // Act-order: original input feature held by each stored row (rows sorted by group); empty =
+    // rows in their natural order.
+    DeviceBuffer<int32_t> perm;
+
     // quant.rs:42-102 on the device; `data` is a device pointer to [k, n] f32.
     static QuantizedTensor from_f32(const float* data, size_t len, uint32_t k, uint32_t n, uint32_t group_size,
                                     hipStream_t stream = nullptr) {
         require(group_size > 0 && group_size % 8 == 0, "group_size must be a multiple of 8");
         require((size_t)k * n == len, "data length mismatch");
         QuantizedTensor q;
-        q.k = k; q.n = n; q.group_size = group_size;
-        q.padded_k = ((k + group_size - 1) / group_size) * group_size;
-        q.num_groups = q.padded_k / group_size;
+        q.set_geometry(k, n, group_size);
         q.packed = DeviceBuffer<uint32_t>((size_t)(q.padded_k / 8) * n);
         q.scales = DeviceBuffer<float>((size_t)q.num_groups * n);
         q.zp = DeviceBuffer<float>((size_t)q.num_groups * n);
         check(rumus_hip_w4_quantize_pack(data, k, n, group_size, q.packed.data(), q.scales.data(), q.zp.data(),
                                          stream));
-        if (n % 16 == 0 && group_size % 32 == 0) {
-            q.packed_t = DeviceBuffer<uint32_t>(q.packed.size());
-            q.scales_t = DeviceBuffer<float>(q.scales.size());
-            q.zp_t = DeviceBuffer<float>(q.zp.size());
-            check(rumus_hip_w4_decode_layout(q.packed.data(), q.scales.data(), q.zp.data(), q.padded_k, n, group_size,
-                                             q.packed_t.data(), q.scales_t.data(), q.zp_t.data(), stream));
-        }
+        q.build_decode_layout(stream);
         return q;
+    }
+
+    // Adopt pre-quantized device arrays (GPTQ/AWQ style).  With g_idx (group of each of the k
+    // rows, rows in their original order) the rows are sorted once so that groups are contiguous.
+    static QuantizedTensor from_packed(DeviceBuffer<uint32_t>&& packed, DeviceBuffer<float>&& scales,
+                                       DeviceBuffer<float>&& zp, uint32_t k, uint32_t n, uint32_t group_size,
+                                       const int32_t* g_idx = nullptr, hipStream_t stream = nullptr) {
+        require(group_size > 0 && group_size % 8 == 0, "group_size must be a multiple of 8");
+        QuantizedTensor q;
+        q.set_geometry(k, n, group_size);
+        require(packed.size() == (size_t)(q.padded_k / 8) * n && scales.size() == (size_t)q.num_groups * n &&
+                    zp.size() == scales.size(), "from_packed: array sizes do not match k / n / group_size");
+        q.scales = std::move(scales);
+        q.zp = std::move(zp);
+        if (g_idx) {
+            require(k == q.padded_k, "act-order needs k to be a multiple of group_size");
+            q.packed = DeviceBuffer<uint32_t>(packed.size());
+            q.perm = DeviceBuffer<int32_t>(k);
+            check(rumus_hip_w4_actorder_prepare(packed.data(), g_idx, q.padded_k, n, group_size, q.packed.data(),
+                                                q.perm.data(), stream));
+            check(rumus_hip_sync(stream));   // `packed` is released on return
+        } else {
+            q.packed = std::move(packed);
+        }
+        q.build_decode_layout(stream);
+        return q;
+    }
+
+    void set_geometry(uint32_t k_, uint32_t n_, uint32_t group_size_) {
+        k = k_; n = n_; group_size = group_size_;
+        padded_k = ((k + group_size - 1) / group_size) * group_size;
+        num_groups = padded_k / group_size;
+    }
+    void build_decode_layout(hipStream_t stream = nullptr) {
+        if (n % 16 != 0 || group_size % 32 != 0 || packed.size() == 0) return;
+        packed_t = DeviceBuffer<uint32_t>(packed.size());
+        scales_t = DeviceBuffer<float>(scales.size());
+        zp_t = DeviceBuffer<float>(zp.size());
+        check(rumus_hip_w4_decode_layout(packed.data(), scales.data(), zp.data(), padded_k, n, group_size,
+                                         packed_t.data(), scales_t.data(), zp_t.data(), stream));
     }
 };
 
@@ -150,16 +186,17 @@ struct QLinear {
     // y[m, out] = x[m, in] . dequant(W) + bias; x and y are device pointers.
     // Up to 5 rows take the decode kernel on the tile-major copy (same result bit for bit).
     void forward(const float* x, uint32_t m, float* y, hipStream_t stream = nullptr) const {
+        const int32_t* perm = weight.perm.size() ? weight.perm.data() : nullptr;
         if (m <= 5 && weight.has_decode_layout()) {
             check(rumus_hip_qmatmul_int4_decode(x, weight.packed_t.data(), weight.scales_t.data(), weight.zp_t.data(),
-                                                bias.size() ? bias.data() : nullptr, nullptr, y, m, weight.k,
+                                                bias.size() ? bias.data() : nullptr, perm, y, m, weight.k,
                                                 weight.n, weight.padded_k, weight.group_size, weight.num_groups,
                                                 stream));
             return;
         }
-        check(rumus_hip_qmatmul_int4(x, weight.packed.data(), weight.scales.data(), weight.zp.data(),
-                                     bias.size() ? bias.data() : nullptr, nullptr, y, m, weight.k, weight.n,
-                                     weight.padded_k, weight.group_size, weight.num_groups, stream));
+        check(rumus_hip_qmatmul_int4_perm(x, weight.packed.data(), weight.scales.data(), weight.zp.data(),
+                                          bias.size() ? bias.data() : nullptr, perm, y, m, weight.k, weight.n,
+                                          weight.padded_k, weight.group_size, weight.num_groups, stream));
     }
     DeviceBuffer<float> forward(const DeviceBuffer<float>& x, hipStream_t stream = nullptr) const {
         require(in_features && x.size() % in_features == 0, "QLinear::forward: x must be [m, in_features]");
@@ -171,6 +208,7 @@ struct QLinear {
     // grad_x[m, in] = grad_y[m, out] . dequant(W)^T (QLinearBackward, quant.rs:298-317)
     DeviceBuffer<float> backward_input(const DeviceBuffer<float>& grad_y, hipStream_t stream = nullptr) const {
         require(out_features && grad_y.size() % out_features == 0, "QLinear::backward: grad_y must be [m, out]");
+        require(weight.perm.size() == 0, "QLinear::backward: grad_x for act-order weights is not implemented");
         const uint32_t m = (uint32_t)(grad_y.size() / out_features);
         DeviceBuffer<float> gx((size_t)m * in_features);
         check(rumus_hip_qmatmul_int4_t(grad_y.data(), weight.packed.data(), weight.scales.data(), weight.zp.data(),

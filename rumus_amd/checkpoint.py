@@ -220,7 +220,8 @@ def load_w4(path: str, device="cuda:0") -> Dict[str, QLinear]:
             scales = get(f"{name}.scales", ("F32", "F16"), (groups, n))
             if scales is None:
                 raise ValueError(f"{path}: {name}.scales is missing")
-            scales = scales.float()
+            if scales.dtype == torch.float16:
+                scales = ops.f16_to_f32(scales)
             zp = get(f"{name}.zeros", ("F32",), (groups, n))
             if zp is None:
                 qz = get(f"{name}.qzeros", ("I32",), (groups, n // 8) if n % 8 == 0 else None)

@@ -151,6 +151,13 @@ __global__ __launch_bounds__(256) void w4_qzeros_unpack_kernel(const uint32_t* _
     dst[1] = hi;
 }
 
+// f16 -> f32 (exact): stored checkpoints often keep their scales in half precision.
+__global__ __launch_bounds__(256) void f16_to_f32_kernel(const _Float16* __restrict__ in, float* __restrict__ out,
+                                                         uint64_t numel) {
+    const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < numel) out[i] = (float)in[i];
+}
+
 template <bool SYM>
 static int quantize_pack(const float* w, uint32_t k, uint32_t n, uint32_t gs, uint32_t* packed,
                          float* scales, float* zps, hipStream_t s) {
@@ -199,6 +206,16 @@ int rumus_hip_w4_decode_layout(const uint32_t* packed, const float* scales, cons
     hipLaunchKernelGGL(w4_tile16_kernel, dim3(gx.x, groups), dim3(256), 0, s,
                        reinterpret_cast<const uint4*>(zero_points), reinterpret_cast<uint4*>(zero_points_t), groups, n);
     return check_launch("w4_tile16_kernel");
+}
+
+int rumus_hip_f16_to_f32(const uint16_t* in, float* out, uint64_t numel, rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE(numel == 0 || (in && out), "f16_to_f32: null buffer");
+    RUMUS_REQUIRE(numel < (1ull << 39), "f16_to_f32: %llu elements are beyond the grid limit",
+                  (unsigned long long)numel);
+    if (numel == 0) return RUMUS_HIP_OK;
+    hipLaunchKernelGGL(f16_to_f32_kernel, dim3((uint32_t)((numel + 255) / 256)), dim3(256), 0, as_stream(stream),
+                       reinterpret_cast<const _Float16*>(in), out, numel);
+    return check_launch("f16_to_f32_kernel");
 }
 
 int rumus_hip_w4_qzeros_unpack(const uint32_t* qzeros, uint32_t num_groups, uint32_t n, float* zero_points,

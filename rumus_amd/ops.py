@@ -156,6 +156,13 @@ def w4_quantize_pack_awq(w: torch.Tensor, group_size: int):
     return packed, scales, qzeros
 
 
+def f16_to_f32(t):
+    """Half -> f32 (exact), same shape."""
+    out = torch.empty(t.shape, dtype=torch.float32, device=t.device)
+    call("rumus_hip_f16_to_f32", _dev(t, torch.float16, "in"), out.data_ptr(), t.numel(), _stream())
+    return out
+
+
 def w4_qzeros_unpack(qzeros, n):
     """u4 zero-points ``[groups, n/8]`` (eight per word) -> f32 ``[groups, n]``."""
     groups = qzeros.shape[0]

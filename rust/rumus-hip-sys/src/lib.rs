@@ -42,6 +42,7 @@ extern "C" {
                                           scales: *mut f32, zero_points: *mut f32, s: Stream) -> c_int;
     pub fn rumus_hip_w4_quantize_pack_awq(w: *const f32, k: u32, n: u32, group_size: u32, packed: *mut u32,
                                           scales: *mut f32, qzeros: *mut u32, s: Stream) -> c_int;
+    pub fn rumus_hip_f16_to_f32(input: *const u16, out: *mut f32, numel: u64, s: Stream) -> c_int;
     pub fn rumus_hip_w4_qzeros_unpack(qzeros: *const u32, num_groups: u32, n: u32, zero_points: *mut f32,
                                       s: Stream) -> c_int;
     pub fn rumus_hip_w4_decode_layout(packed: *const u32, scales: *const f32, zero_points: *const f32,

@@ -4,10 +4,13 @@
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <algorithm>
 #include <random>
+#include <string>
 #include <vector>
 
 #include "rumus_hip.hpp"
+#include "rumus_hip_file.hpp"
 #include "rumus_oracle.h"
 
 using namespace rumus_hip;
@@ -106,6 +109,112 @@ static void test_int8_linear(uint32_t m, uint32_t k, uint32_t n) {
     CHECK(close(y, want, "forward"), "Int8Linear::forward");
 }
 
+
+static std::vector<char> slurp(const std::string& path) {
+    std::vector<char> out;
+    if (FILE* f = fopen(path.c_str(), "rb")) {
+        char buf[1 << 16];
+        size_t got;
+        while ((got = fread(buf, 1, sizeof buf, f)) > 0) out.insert(out.end(), buf, buf + got);
+        fclose(f);
+    }
+    return out;
+}
+
+static void spill(const std::string& path, const void* data, size_t nbytes) {
+    FILE* f = fopen(path.c_str(), "wb");
+    CHECK(f && fwrite(data, 1, nbytes, f) == nbytes, "cannot write %s", path.c_str());
+    if (f) fclose(f);
+}
+
+// Layers through the on-disk form and back: same bits, same outputs; an act-order layer built
+// from g_idx matches the oracle.  With a directory argument the file and one forward pass are
+// left there for the Python loader to check, and a file the Python writer left is loaded and run.
+static void test_file(const std::string& dir) {
+    printf("[host-cpp] save_w4 / load_w4 in %s\n", dir.c_str());
+    fflush(stdout);
+    const uint32_t k = 512, n = 272, g = 128, m = 3;
+    auto w = normal((size_t)k * n, 0.02f, 11), b = normal(n, 0.01f, 12), x = normal((size_t)m * k, 1.0f, 13);
+    Linear linear(w, k, n, b);
+    QLinear plain = QLinear::from_linear(linear, g);
+    // act-order: the same quantized rows, announced in a shuffled group order
+    std::vector<int32_t> g_idx(k);
+    {
+        std::vector<uint32_t> order(k);
+        for (uint32_t i = 0; i < k; i++) order[i] = i;
+        std::mt19937 gen(14);
+        std::shuffle(order.begin(), order.end(), gen);
+        for (uint32_t i = 0; i < k; i++) g_idx[order[i]] = (int32_t)(i / g);
+    }
+    auto hp = plain.weight.packed.download();
+    auto hs = plain.weight.scales.download(), hz = plain.weight.zp.download();
+    QLinear ao;
+    {
+        DeviceBuffer<int32_t> dg(g_idx);
+        ao.weight = QuantizedTensor::from_packed(DeviceBuffer<uint32_t>(hp), DeviceBuffer<float>(hs),
+                                                 DeviceBuffer<float>(hz), k, n, g, dg.data());
+        check(rumus_hip_sync(nullptr));
+    }
+    ao.in_features = k;
+    ao.out_features = n;
+    std::vector<float> want((size_t)m * n);
+    orc_qmatmul_int4(x.data(), hp.data(), hs.data(), hz.data(), nullptr, g_idx.data(), want.data(), m, k, n, k, g,
+                     k / g, 8);
+    DeviceBuffer<float> dx(x);
+    CHECK(close(ao.forward(dx).download(), want, "act-order forward (from g_idx)"), "from_packed with g_idx");
+
+    const std::string path = dir + "/cpp.safetensors";
+    save_w4(path, {{"blk.plain", &plain}, {"blk.act_order", &ao}});
+    auto back = load_w4(path, nullptr, 40000);             // odd chunk size: many pieces per tensor
+    CHECK(back.size() == 2 && back.count("blk.plain") && back.count("blk.act_order"), "layer names");
+    if (back.size() == 2) {
+        const QLinear& p2 = back.at("blk.plain");
+        const QLinear& a2 = back.at("blk.act_order");
+        CHECK(p2.weight.packed.download() == hp && p2.weight.scales.download() == hs && p2.weight.zp.download() == hz,
+              "plain layer arrays changed");
+        CHECK(p2.bias.download() == b, "bias changed");
+        CHECK(p2.weight.k == k && p2.weight.n == n && p2.weight.group_size == g && p2.in_features == k, "metadata");
+        CHECK(p2.forward(dx).download() == plain.forward(dx).download(), "plain forward differs after reload");
+        CHECK(a2.weight.perm.download() == ao.weight.perm.download(), "perm changed");
+        CHECK(a2.weight.packed.download() == ao.weight.packed.download(), "sorted rows changed");
+        CHECK(a2.forward(dx).download() == ao.forward(dx).download(), "act-order forward differs after reload");
+    }
+    // refusals: a cut file, a header that is not JSON
+    auto bytes = slurp(path);
+    spill(dir + "/cut.safetensors", bytes.data(), bytes.size() - 100);
+    bool threw = false;
+    try { load_w4(dir + "/cut.safetensors"); } catch (const Error& e) { threw = e.code == RUMUS_HIP_EINVAL; }
+    CHECK(threw, "a truncated file must be refused");
+    auto bad = bytes;
+    bad[8] = '[';
+    spill(dir + "/bad.safetensors", bad.data(), bad.size());
+    threw = false;
+    try { load_w4(dir + "/bad.safetensors"); } catch (const Error& e) { threw = e.code == RUMUS_HIP_EINVAL; }
+    CHECK(threw, "a malformed header must be refused");
+    remove((dir + "/cut.safetensors").c_str());
+    remove((dir + "/bad.safetensors").c_str());
+
+    // exchange with the Python side
+    spill(dir + "/cpp_x.bin", x.data(), x.size() * 4);
+    auto y = plain.forward(dx).download();
+    spill(dir + "/cpp_y.bin", y.data(), y.size() * 4);
+    const auto px = slurp(dir + "/py_x.bin");
+    if (!px.empty()) {
+        auto layers = load_w4(dir + "/py.safetensors");
+        CHECK(!layers.empty(), "py.safetensors holds no layer");
+        for (const auto& kv : layers) {
+            const QLinear& lin = kv.second;
+            const uint32_t rows = (uint32_t)(px.size() / 4 / lin.in_features);
+            std::vector<float> hx(px.size() / 4);
+            memcpy(hx.data(), px.data(), px.size());
+            auto out = lin.forward(DeviceBuffer<float>(hx)).download();
+            spill(dir + "/py_y_" + kv.first + ".bin", out.data(), out.size() * 4);
+            printf("  loaded %s: k=%u n=%u g=%u rows=%u perm=%zu\n", kv.first.c_str(), lin.weight.k, lin.weight.n,
+                   lin.weight.group_size, rows, lin.weight.perm.size());
+        }
+    }
+}
+
 static void test_errors() {
     printf("[host-cpp] preconditions\n");
     fflush(stdout);
@@ -121,7 +230,7 @@ static void test_errors() {
     CHECK(threw, "length mismatch must be rejected");
 }
 
-int main() {
+int main(int argc, char** argv) {
     check(rumus_hip_init(0));
     test_qlinear(1, 1024, 512, 128);
     test_qlinear(4, 200, 52, 8);
@@ -131,6 +240,7 @@ int main() {
     test_int8_linear(32, 512, 512);
     test_int8_linear(300, 1024, 260);
     test_errors();
+    test_file(argc > 1 ? argv[1] : "/tmp");
     printf(g_fail ? "host-cpp: %d FAILED\n" : "host-cpp: all passed\n", g_fail);
     return g_fail ? 1 : 0;
 }
