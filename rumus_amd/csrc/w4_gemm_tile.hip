@@ -373,22 +373,26 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
         }
 }
 
-// y = part[0] + part[1] + ... (in that order) + bias; count4 = m*n/4
+// y = part[0] + part[1] + ... (in that order) + bias; count4 = m*n/4.  All partials are requested
+// before the first is added (a split beyond the last re-reads the last one and is not added), so
+// the kernel costs one round trip to memory instead of one per split.
 __global__ __launch_bounds__(256) void w4_gemm_reduce_kernel(const float4* __restrict__ part,
                                                              const float* __restrict__ bias,
                                                              float4* __restrict__ y, uint32_t count4,
                                                              uint32_t n4, uint32_t splits) {
     const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
     if (idx >= count4) return;
-    float4 s = part[idx];
-    for (uint32_t p = 1; p < splits; p++) {
-        const float4 v = part[(uint64_t)p * count4 + idx];
-        s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    float4 v[kMaxSplits];
+#pragma unroll
+    for (uint32_t p = 0; p < kMaxSplits; p++) v[p] = part[(uint64_t)min(p, splits - 1) * count4 + idx];
+    float4 b = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (bias) b = *reinterpret_cast<const float4*>(bias + 4 * (idx % n4));
+    float4 s = v[0];
+#pragma unroll
+    for (uint32_t p = 1; p < kMaxSplits; p++) {
+        if (p < splits) { s.x += v[p].x; s.y += v[p].y; s.z += v[p].z; s.w += v[p].w; }
     }
-    if (bias) {
-        const float4 b = *reinterpret_cast<const float4*>(bias + 4 * (idx % n4));
-        s.x += b.x; s.y += b.y; s.z += b.z; s.w += b.w;
-    }
+    if (bias) { s.x += b.x; s.y += b.y; s.z += b.z; s.w += b.w; }
     y[idx] = s;
 }
 
