@@ -239,6 +239,19 @@ int rumus_hip_qmatmul_int4_decode(const float* x, const uint32_t* packed_t,
                                   uint32_t group_size, uint32_t num_groups,
                                   rumus_hip_stream_t stream);
 
+/* EXTENSION: rumus_hip_qmatmul_int4_decode whose input is the output of a
+ * fused gate|up projection: gate_up [m, 2k] (gate in columns 0..k-1, up in
+ * k..2k-1), x[m, j] = silu(gate[m, j]) * up[m, j] computed on the way in, so the
+ * SwiGLU of a decoder block costs no launch of its own.  Same bits as
+ * rumus_hip_swiglu_rows followed by rumus_hip_qmatmul_int4_decode.
+ * EINVAL unless m <= 8, n % 16 == 0, k % 8 == 0, group_size % 32 == 0 and
+ * 16-byte aligned buffers.  No counterpart in the reference. */
+int rumus_hip_qmatmul_int4_decode_swiglu(const float* gate_up, const uint32_t* packed_t,
+                                         const float* scales_t, const float* zero_points_t,
+                                         const float* bias, float* y, uint32_t m, uint32_t k,
+                                         uint32_t n, uint32_t padded_k, uint32_t group_size,
+                                         uint32_t num_groups, rumus_hip_stream_t stream);
+
 /* EXTENSION: qmatmul_int4_perm on AWQ storage: zero-points come as qzeros
  * (layout above) instead of f32.  perm may be NULL (plain k order).
  * EINVAL also unless n % 8 == 0. */
@@ -258,6 +271,14 @@ int rumus_hip_qmatmul_int4_zp4(const float* x, const uint32_t* packed,
 /* y[r,:] = x[r,:] * rsqrt(mean(x[r,:]^2) + eps) * weight[:] */
 int rumus_hip_rmsnorm(const float* x, const float* weight, float* y, uint32_t rows,
                       uint32_t dim, float eps, rumus_hip_stream_t stream);
+
+/* sum = x + delta; y = rmsnorm(sum) with the formula above, in one launch (the
+ * residual update and the norm that follows it in a pre-norm block).  sum may
+ * alias x or delta; y must not alias any of them.  Same bits as rumus_hip_add
+ * followed by rumus_hip_rmsnorm. */
+int rumus_hip_add_rmsnorm(const float* x, const float* delta, const float* weight,
+                          float* sum, float* y, uint32_t rows, uint32_t dim, float eps,
+                          rumus_hip_stream_t stream);
 
 /* out = silu(gate) * up, silu(t) = t / (1 + exp(-t)); out may alias gate or up */
 int rumus_hip_swiglu(const float* gate, const float* up, float* out, uint64_t numel,

@@ -14,12 +14,20 @@ namespace rumus {
 // One workgroup per row.  VEC: dim % 4 == 0, dim <= 8192 and 16-byte aligned rows: the row is
 // read once with up to eight 128-bit loads per thread, all issued before the first use (a
 // single decode row is pure latency otherwise: sixteen dependent 4-byte loads per thread).
-template <bool VEC>
-__global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+// ADD: the row normalised is x + delta (the residual stream after a projection); the sum is
+// written to `sum` as well, so that the separate addition and its launch disappear.
+template <bool VEC, bool ADD>
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float* x, const float* delta,
+                                                      const float* __restrict__ w, float* sum,
                                                       float* __restrict__ y, uint32_t dim, float eps) {
+    // `sum` may be x or delta (the residual stream updated in place): every thread reads its own
+    // elements before it writes them
     __shared__ float red[4];
-    const float* xr = x + (uint64_t)blockIdx.x * dim;
-    float* yr = y + (uint64_t)blockIdx.x * dim;
+    const uint64_t base = (uint64_t)blockIdx.x * dim;
+    const float* xr = x + base;
+    const float* dr = ADD ? delta + base : nullptr;
+    float* sr = ADD ? sum + base : nullptr;
+    float* yr = y + base;
     float4 v[8], wv[8];
     float ss = 0.0f;
     if (VEC) {
@@ -29,13 +37,24 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
             const bool in = i < dim;
             v[j] = *reinterpret_cast<const float4*>(xr + (in ? i : 0));
             wv[j] = *reinterpret_cast<const float4*>(w + (in ? i : 0));
+            if (ADD) {
+                const float4 d = *reinterpret_cast<const float4*>(dr + (in ? i : 0));
+                v[j] = make_float4(v[j].x + d.x, v[j].y + d.y, v[j].z + d.z, v[j].w + d.w);
+            }
             if (!in) v[j] = make_float4(0, 0, 0, 0);
         }
 #pragma unroll
-        for (int j = 0; j < 8; j++)
+        for (int j = 0; j < 8; j++) {
             ss = fmaf(v[j].x, v[j].x, fmaf(v[j].y, v[j].y, fmaf(v[j].z, v[j].z, fmaf(v[j].w, v[j].w, ss))));
+            const uint32_t i = (j * 256 + threadIdx.x) * 4;
+            if (ADD && i < dim) *reinterpret_cast<float4*>(sr + i) = v[j];
+        }
     } else {
-        for (uint32_t i = threadIdx.x; i < dim; i += 256) ss = fmaf(xr[i], xr[i], ss);
+        for (uint32_t i = threadIdx.x; i < dim; i += 256) {
+            float t = xr[i];
+            if (ADD) { t += dr[i]; sr[i] = t; }
+            ss = fmaf(t, t, ss);
+        }
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
@@ -52,7 +71,8 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
                                                                  v[j].z * inv * wv[j].z, v[j].w * inv * wv[j].w);
         }
     } else {
-        for (uint32_t i = threadIdx.x; i < dim; i += 256) yr[i] = xr[i] * inv * w[i];
+        const float* src = ADD ? sr : xr;  // each thread re-reads the elements it wrote itself
+        for (uint32_t i = threadIdx.x; i < dim; i += 256) yr[i] = src[i] * inv * w[i];
     }
 }
 
@@ -295,8 +315,27 @@ int rumus_hip_rmsnorm(const float* x, const float* weight, float* y, uint32_t ro
     const bool vec = dim % 4 == 0 && dim <= 8192 &&
                      ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(weight) |
                        reinterpret_cast<uintptr_t>(y)) & 15) == 0;
-    if (vec) hipLaunchKernelGGL(rmsnorm_kernel<true>, dim3(rows), dim3(256), 0, as_stream(stream), x, weight, y, dim, eps);
-    else hipLaunchKernelGGL(rmsnorm_kernel<false>, dim3(rows), dim3(256), 0, as_stream(stream), x, weight, y, dim, eps);
+    if (vec) hipLaunchKernelGGL((rmsnorm_kernel<true, false>), dim3(rows), dim3(256), 0, as_stream(stream), x, nullptr,
+                                weight, nullptr, y, dim, eps);
+    else hipLaunchKernelGGL((rmsnorm_kernel<false, false>), dim3(rows), dim3(256), 0, as_stream(stream), x, nullptr,
+                            weight, nullptr, y, dim, eps);
+    return check_launch("rmsnorm_kernel");
+}
+
+int rumus_hip_add_rmsnorm(const float* x, const float* delta, const float* weight, float* sum, float* y,
+                          uint32_t rows, uint32_t dim, float eps, rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE(x && delta && weight && sum && y, "add_rmsnorm: null buffer");
+    RUMUS_REQUIRE(dim > 0, "add_rmsnorm: dim must be positive");
+    RUMUS_REQUIRE(y != x && y != delta && y != sum, "add_rmsnorm: y must not alias x, delta or sum");
+    if (rows == 0) return RUMUS_HIP_OK;
+    const bool vec = dim % 4 == 0 && dim <= 8192 &&
+                     ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(delta) |
+                       reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(sum) |
+                       reinterpret_cast<uintptr_t>(y)) & 15) == 0;
+    if (vec) hipLaunchKernelGGL((rmsnorm_kernel<true, true>), dim3(rows), dim3(256), 0, as_stream(stream), x, delta,
+                                weight, sum, y, dim, eps);
+    else hipLaunchKernelGGL((rmsnorm_kernel<false, true>), dim3(rows), dim3(256), 0, as_stream(stream), x, delta,
+                            weight, sum, y, dim, eps);
     return check_launch("rmsnorm_kernel");
 }
 

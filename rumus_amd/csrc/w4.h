@@ -24,6 +24,8 @@ struct W4Args {
     // decode layout (w4_gemv_dot8 only): packed, scales and zp are tile-major copies, tile = 16
     // columns: packed_t[(c*word_rows + r)*16 + j] = packed[r*n + 16*c + j], likewise the metadata
     bool tiled;
+    // w4_gemv_dot8 only: x holds rows of 2k floats, gate | up; the activations are silu(gate) * up
+    bool glu;
 };
 
 // zero-points of 4 (col % 4 == 0) or 2 (col % 2 == 0) adjacent columns from the packed form

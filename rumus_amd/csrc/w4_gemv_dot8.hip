@@ -46,6 +46,10 @@ constexpr int kDppXor1 = 0xB1;   // quad_perm [1,0,3,2]
 constexpr int kDppXor2 = 0x4E;   // quad_perm [2,3,0,1]
 constexpr int kDppRowShr4 = 0x114, kDppRowShr8 = 0x118;
 
+// silu(g) * u, the expression of swiglu_kernel (block_glue.hip), so that the fused and the
+// separate path give the same bits
+__device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+
 // value of quad lane Q in all four lanes of the quad
 template <int Q> __device__ __forceinline__ uint32_t quad_bcast(uint32_t v) {
     return (uint32_t)RUMUS_DPP_I(v, Q * 0x55);
@@ -72,7 +76,10 @@ __device__ __forceinline__ float reduce_row_lanes(float v) {
 // TILED: packed / scales / zps are tile-major copies (a tile = this workgroup's 16 columns, all
 // rows), so the workgroup reads one contiguous 32 KB slab and each load instruction of a wave
 // a contiguous 1 KB, instead of 64-byte segments 4*n bytes apart (10 % faster at 4096 x 4096).
-template <int M, int T, int OCT, bool FASTX, bool ZP4, bool TILED>
+// GLU (with FASTX): `xin` holds rows of 2k floats, gate | up, and the activations are
+// silu(gate) * up computed on the way in: the SwiGLU between a fused gate|up projection and the
+// down projection costs no launch and no round trip of its own.
+template <int M, int T, int OCT, bool FASTX, bool ZP4, bool TILED, bool GLU = false>
 __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
     const uint32_t* __restrict__ packed, const float* __restrict__ scales,
     const float* __restrict__ zps, const float* __restrict__ xin, float* __restrict__ yout,
@@ -120,8 +127,17 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
                 if (FASTX) {
                     const bool in = kt < k;              // k % 8 == 0: all 8 in or out
                     const uint32_t kc = in ? kt : 0;
-                    const float4 lo = *reinterpret_cast<const float4*>(xin + (uint64_t)m * k + kc);
-                    const float4 hi = *reinterpret_cast<const float4*>(xin + (uint64_t)m * k + kc + 4);
+                    const float* xrow = xin + (uint64_t)m * (GLU ? 2 * k : k) + kc;
+                    float4 lo = *reinterpret_cast<const float4*>(xrow);
+                    float4 hi = *reinterpret_cast<const float4*>(xrow + 4);
+                    if (GLU) {
+                        const float4 ul = *reinterpret_cast<const float4*>(xrow + k);
+                        const float4 uh = *reinterpret_cast<const float4*>(xrow + k + 4);
+                        lo = make_float4(silu_mul(lo.x, ul.x), silu_mul(lo.y, ul.y), silu_mul(lo.z, ul.z),
+                                         silu_mul(lo.w, ul.w));
+                        hi = make_float4(silu_mul(hi.x, uh.x), silu_mul(hi.y, uh.y), silu_mul(hi.z, uh.z),
+                                         silu_mul(hi.w, uh.w));
+                    }
                     xv[m][t][0] = in ? lo.x : 0.0f; xv[m][t][1] = in ? lo.y : 0.0f;
                     xv[m][t][2] = in ? lo.z : 0.0f; xv[m][t][3] = in ? lo.w : 0.0f;
                     xv[m][t][4] = in ? hi.x : 0.0f; xv[m][t][5] = in ? hi.y : 0.0f;
@@ -281,10 +297,10 @@ bool w4_gemv_dot8_supported(const W4Args& a) {
            a.group_size % (8 * kD8Oct) == 0;
 }
 
-template <int M, bool FASTX, bool ZP4, bool TILED>
+template <int M, bool FASTX, bool ZP4, bool TILED, bool GLU = false>
 static void launch_variant(const W4Args& a, hipStream_t s) {
     const float* zps = ZP4 ? reinterpret_cast<const float*>(a.zp4) : a.zp;
-    hipLaunchKernelGGL((w4_gemv_dot8_kernel<M, kD8Threads, kD8Oct, FASTX, ZP4, TILED>), dim3(ceil_div(a.n, kD8Cols)),
+    hipLaunchKernelGGL((w4_gemv_dot8_kernel<M, kD8Threads, kD8Oct, FASTX, ZP4, TILED, GLU>), dim3(ceil_div(a.n, kD8Cols)),
                        dim3(kD8Threads), 0, s, a.packed, a.scales, zps, a.x, a.y, a.n, a.k, a.padded_k,
                        a.group_size, a.bias, a.perm);
 }
@@ -292,7 +308,12 @@ static void launch_variant(const W4Args& a, hipStream_t s) {
 template <int M>
 static int launch_m(const W4Args& a, hipStream_t s) {
     const bool fast_x = !a.perm && (a.k % 8 == 0) && ((reinterpret_cast<uintptr_t>(a.x) & 15) == 0);
-    if (a.tiled) {
+    if (a.glu) {
+        if (!(fast_x && a.tiled && !a.zp4))
+            return set_error(RUMUS_HIP_EINVAL, "w4 gemv: the SwiGLU input needs the decode layout, f32 zero-points, "
+                                               "k %% 8 == 0 and 16-byte aligned rows");
+        launch_variant<M, true, false, true, true>(a, s);
+    } else if (a.tiled) {
         if (fast_x) launch_variant<M, true, false, true>(a, s);
         else launch_variant<M, false, false, true>(a, s);
     } else if (a.zp4) {

@@ -267,10 +267,15 @@ class DecoderBlockW4:
             att = ops.attention(q, k_cache[:, :pos + 1], v_cache[:, :pos + 1], causal=False)
             k_out, v_out = k_cache, v_cache
         o = self.proj["o"](att.view(b * n, d))
-        x1 = ops.add(x2, o, out=o)
-        h2 = ops.rmsnorm(x1, self.norm2, self.eps, out=hn)
-        act = ops.swiglu_rows(self.gate_up(h2))
-        down = self.proj["down"](act)
+        x1, h2 = ops.add_rmsnorm(x2, o, self.norm2, self.eps, sum_out=o, out=hn)
+        gu = self.gate_up(h2)
+        dw = self.proj["down"]
+        if b * n <= DECODE_ROWS and dw.weight.decode is not None and dw.weight.perm is None:
+            # decode rows: the SwiGLU happens while the down projection reads its input
+            down = ops.qmatmul_int4_decode_swiglu(gu, *dw.weight.decode, dw.weight.k, dw.weight.group_size,
+                                                  bias=dw.bias)
+        else:
+            down = dw(ops.swiglu_rows(gu))
         y = ops.add(x1, down, out=down)
         return y.view(b, n, d), k_out, v_out
 

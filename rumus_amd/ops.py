@@ -187,6 +187,21 @@ def qmatmul_int4_decode(x, packed_t, scales_t, zp_t, k, group_size, bias=None, p
     return _w4_call("rumus_hip_qmatmul_int4_decode", x, packed_t, scales_t, zp_t, bias, perm, k, group_size, out)
 
 
+def qmatmul_int4_decode_swiglu(gate_up, packed_t, scales_t, zp_t, k, group_size, bias=None, out=None):
+    """``(silu(gate) * up) @ dequant(W)`` for ``gate_up`` ``[m, 2k]`` (gate | up), one launch."""
+    m = gate_up.shape[0]
+    n = packed_t.shape[1]
+    if gate_up.dim() != 2 or gate_up.shape[1] != 2 * k:
+        raise ValueError("qmatmul_int4_decode_swiglu: gate_up must be [m, 2k]")
+    padded_k, groups = w4_geometry(k, group_size) if group_size > 0 else (k, 0)
+    y = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=gate_up.device)
+    call("rumus_hip_qmatmul_int4_decode_swiglu", _dev(gate_up, torch.float32, "gate_up"),
+         _dev(packed_t, torch.int32, "packed_t"), _dev(scales_t, torch.float32, "scales_t"),
+         _dev(zp_t, torch.float32, "zero_points_t"), _opt(bias, torch.float32, "bias"),
+         _dev(y, torch.float32, "y"), m, k, n, padded_k, group_size, groups, _stream())
+    return y
+
+
 def qmatmul_int4_zp4(x, packed, scales, qzeros, k, group_size, bias=None, perm=None, out=None):
     m = x.shape[0]
     n = packed.shape[1]
@@ -255,6 +270,17 @@ def rmsnorm(x, weight, eps: float = 1e-6, out=None):
     call("rumus_hip_rmsnorm", _dev(x, torch.float32, "x"), _dev(weight, torch.float32, "weight"),
          _dev(y, torch.float32, "y"), rows, dim, float(eps), _stream())
     return y
+
+
+def add_rmsnorm(x, delta, weight, eps: float = 1e-6, sum_out=None, out=None):
+    """``s = x + delta; y = rmsnorm(s)`` in one launch; returns ``(s, y)``.  ``sum_out`` may be x or delta."""
+    rows, dim = x.shape
+    s = sum_out if sum_out is not None else torch.empty_like(x)
+    y = out if out is not None else torch.empty_like(x)
+    call("rumus_hip_add_rmsnorm", _dev(x, torch.float32, "x"), _dev(delta, torch.float32, "delta"),
+         _dev(weight, torch.float32, "weight"), _dev(s, torch.float32, "sum"), _dev(y, torch.float32, "y"),
+         rows, dim, float(eps), _stream())
+    return s, y
 
 
 def swiglu(gate, up, out=None):

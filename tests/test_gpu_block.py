@@ -40,6 +40,49 @@ def test_swiglu_and_add(ops):
     np.testing.assert_array_equal(host(ops.add(dev(g), dev(u))), g + u)
 
 
+@pytest.mark.parametrize("rows,dim", [(1, 4096), (7, 100), (3, 8200), (130, 11008)])
+def test_add_rmsnorm_is_add_then_rmsnorm(ops, rows, dim):
+    say(f"add_rmsnorm {rows}x{dim}")
+    rng = np.random.default_rng(rows * 3 + dim)
+    x = rng.normal(0, 2, (rows, dim)).astype(np.float32)
+    d = rng.normal(0, 1, (rows, dim)).astype(np.float32)
+    w = rng.normal(1, 0.1, dim).astype(np.float32)
+    s, y = ops.add_rmsnorm(dev(x), dev(d), dev(w), 1e-6)
+    np.testing.assert_array_equal(host(s), x + d)
+    close(host(y), oracle.rmsnorm(x + d, w, 1e-6), atol=1e-5)
+    # the same bits as the two separate launches
+    s2 = ops.add(dev(x), dev(d))
+    np.testing.assert_array_equal(host(y), host(ops.rmsnorm(s2, dev(w), 1e-6)))
+    # the sum written over the delta (the residual stream updated in place)
+    dd = dev(d)
+    s3, y3 = ops.add_rmsnorm(dev(x), dd, dev(w), 1e-6, sum_out=dd)
+    assert s3.data_ptr() == dd.data_ptr()
+    np.testing.assert_array_equal(host(s3), x + d)
+    np.testing.assert_array_equal(host(y3), host(y))
+    with pytest.raises(Exception, match="must not alias"):
+        ops.add_rmsnorm(dd, dd, dev(w), 1e-6, out=dd)
+
+
+@pytest.mark.parametrize("m,k,n,g", [(1, 11008, 4096, 128), (3, 512, 48, 64), (5, 264, 16, 256), (8, 1024, 272, 32)])
+def test_decode_gemv_with_swiglu_input(ops, m, k, n, g):
+    say(f"qmatmul_int4_decode_swiglu m={m} k={k} n={n} g={g}")
+    rng = np.random.default_rng(m + k + n)
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    gu = rng.normal(0, 2, (m, 2 * k)).astype(np.float32)
+    gu[0, :3] = [-100.0, 100.0, 0.0]
+    b = rng.normal(0, 0.01, n).astype(np.float32)
+    packed, scales, zp = oracle.w4_from_f32(w, g)
+    pt, st, zt = ops.w4_decode_layout(dev(packed), dev(scales), dev(zp), g)
+    got = host(ops.qmatmul_int4_decode_swiglu(dev(gu), pt, st, zt, k, g, bias=dev(b)))
+    x = oracle.swiglu(gu[:, :k], gu[:, k:]).astype(np.float32)
+    close(got, oracle.qmatmul_int4(x, packed, scales, zp, k, g, bias=b, threads=8))
+    # the same bits as the SwiGLU kernel followed by the decode kernel
+    act = ops.swiglu_rows(dev(gu))
+    np.testing.assert_array_equal(got, host(ops.qmatmul_int4_decode(act, pt, st, zt, k, g, bias=dev(b))))
+    with pytest.raises(Exception, match="gate_up must be"):
+        ops.qmatmul_int4_decode_swiglu(dev(gu[:, :k]), pt, st, zt, k, g)
+
+
 @pytest.mark.parametrize("b,h,nq,nkv,causal", [
     (1, 2, 64, 64, True), (2, 3, 100, 100, True), (1, 2, 70, 70, False), (1, 4, 33, 97, True),
     (2, 32, 1, 2048, False), (3, 2, 1, 1, False), (1, 2, 1, 300, True), (1, 1, 512, 512, True)])
