@@ -198,6 +198,171 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(AttnArgs a) {
             make_float4(acc[4 * i] * inv, acc[4 * i + 1] * inv, acc[4 * i + 2] * inv, acc[4 * i + 3] * inv);
 }
 
+// Prefill on the matrix cores (v_mfma_f32_32x32x2_f32, f32 in and out).  Workgroup = 128 query
+// rows of one (batch, head), 32 per wave; K/V tiles of 32 keys go through LDS.  Everything is
+// computed transposed so that no fragment ever has to be re-laid out:
+//   S^T = K Q^T   rows = keys (A operand, from LDS), columns = queries (B operand: the wave's Q
+//                 rows, kept in 64 registers per lane for the whole kernel).  In the result a
+//                 lane holds one query column and 16 of the tile's 32 keys, lane ^ 32 the other
+//                 16: the softmax statistics of a query need one exchange between the halves.
+//   O^T += V^T P^T  rows = dims (A operand, from LDS), columns = queries.  Result register r of
+//                 S^T is exactly the B operand of step r (k index = the keys that lane holds).
+// The 128 dims of the S^T product are walked as d = 64 * (lane / 32) + step, so that a lane's Q
+// and K fragments are contiguous floats.  LDS tiles are [32 rows][33 chunks of 16 bytes]: the
+// odd row stride spreads a column of chunks (the K fragment read, one row per lane) over all
+// banks, a row (the V fragment read) stays contiguous, and every address is one per-lane base
+// plus a compile-time offset.
+typedef float attn_v16f __attribute__((ext_vector_type(16)));
+
+constexpr uint32_t kAttnRowChunks = 33;
+__device__ __forceinline__ uint32_t attn_tile_pos(uint32_t row, uint32_t chunk) {
+    return row * kAttnRowChunks + chunk;
+}
+
+__global__ __launch_bounds__(256, 2) void attention_mfma_kernel(AttnArgs a) {
+    constexpr uint32_t BC = 32, BQ = 128;
+    __shared__ float4 ks[BC * kAttnRowChunks];
+    __shared__ float4 vs[BC * kAttnRowChunks];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t l32 = lane & 31, kb = lane >> 5;
+    // grid: x = (batch, head), y = block of 128 query rows, last block first: under a causal mask
+    // the late rows see the most keys, and the long workgroups should not be the last to start
+    const uint32_t bh = blockIdx.x, b = bh / a.heads, h = bh % a.heads;
+    const uint32_t qblock = gridDim.y - 1 - blockIdx.y;
+    const uint32_t shift = a.kv_len - a.q_len;                 // causal offset of the query rows
+    const uint32_t q0 = qblock * BQ + wave * 32;               // first query row of this wave
+    const uint32_t qrow = q0 + l32;                            // this lane's query
+    const bool wave_live = q0 < a.q_len;
+
+    // Q fragment, scaled by scale * log2(e) (the softmax runs on exp2): qf[s] = Q[qrow][64*kb + s]
+    float qf[64];
+    {
+        const float* qp = a.q + b * a.q_sb + h * a.q_sh + (uint64_t)min(qrow, a.q_len - 1) * a.q_sr + 64 * kb;
+        const float qs = a.scale * 1.44269504088896f;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const float4 t = *reinterpret_cast<const float4*>(qp + 4 * i);
+            qf[4 * i] = t.x * qs; qf[4 * i + 1] = t.y * qs; qf[4 * i + 2] = t.z * qs; qf[4 * i + 3] = t.w * qs;
+        }
+    }
+    attn_v16f oacc[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) oacc[dt][r] = 0.0f;
+    constexpr float kMasked = -1e30f;                          // finite: exp2 of differences stays defined
+    float mrun = kMasked, lrun = 0.0f;
+
+    // keys the workgroup, this wave and this lane's query need (exclusive ends)
+    const uint32_t wg_last = min(qblock * BQ + BQ - 1, a.q_len - 1);
+    const uint32_t kv_end = a.causal ? min(a.kv_len, wg_last + shift + 1) : a.kv_len;
+    const uint32_t wave_end = a.causal ? min(a.kv_len, min(q0 + 31, a.q_len - 1) + shift + 1) : a.kv_len;
+    const uint32_t my_end = a.causal ? min(a.kv_len, qrow + shift + 1) : a.kv_len;
+
+    // staging: a tile is 1024 chunks of K and of V, 4 of each per thread, fetched one tile ahead
+    const float* kbase = a.k + b * a.k_sb + h * a.k_sh;
+    const float* vbase = a.v + b * a.v_sb + h * a.v_sh;
+    // (this thread's chunks: rows tid/32 + 8t, chunk tid%32; loads past the last tile re-read it)
+    const uint32_t s_row = tid >> 5, s_chunk = tid & 31;
+    const float* kstage = kbase + 4 * s_chunk;
+    const float* vstage = vbase + 4 * s_chunk;
+    float4 kreg0, kreg1, kreg2, kreg3, vreg0, vreg1, vreg2, vreg3;
+#define RUMUS_ATTN_TILE_LOAD(J0)                                                                     \
+    {                                                                                               \
+        const uint32_t r0_ = min((J0) + s_row, a.kv_len - 1), r1_ = min((J0) + s_row + 8, a.kv_len - 1); \
+        const uint32_t r2_ = min((J0) + s_row + 16, a.kv_len - 1), r3_ = min((J0) + s_row + 24, a.kv_len - 1); \
+        kreg0 = *reinterpret_cast<const float4*>(kstage + (uint64_t)r0_ * a.k_sr);                  \
+        kreg1 = *reinterpret_cast<const float4*>(kstage + (uint64_t)r1_ * a.k_sr);                  \
+        kreg2 = *reinterpret_cast<const float4*>(kstage + (uint64_t)r2_ * a.k_sr);                  \
+        kreg3 = *reinterpret_cast<const float4*>(kstage + (uint64_t)r3_ * a.k_sr);                  \
+        vreg0 = *reinterpret_cast<const float4*>(vstage + (uint64_t)r0_ * a.v_sr);                  \
+        vreg1 = *reinterpret_cast<const float4*>(vstage + (uint64_t)r1_ * a.v_sr);                  \
+        vreg2 = *reinterpret_cast<const float4*>(vstage + (uint64_t)r2_ * a.v_sr);                  \
+        vreg3 = *reinterpret_cast<const float4*>(vstage + (uint64_t)r3_ * a.v_sr);                  \
+    }
+    RUMUS_ATTN_TILE_LOAD(0u)
+    for (uint32_t j0 = 0; j0 < kv_end; j0 += BC) {
+        __syncthreads();                                       // the previous tile has been consumed
+        {
+            const uint32_t pos = attn_tile_pos(s_row, s_chunk);
+            ks[pos] = kreg0; ks[pos + 8 * kAttnRowChunks] = kreg1;
+            ks[pos + 16 * kAttnRowChunks] = kreg2; ks[pos + 24 * kAttnRowChunks] = kreg3;
+            vs[pos] = vreg0; vs[pos + 8 * kAttnRowChunks] = vreg1;
+            vs[pos + 16 * kAttnRowChunks] = vreg2; vs[pos + 24 * kAttnRowChunks] = vreg3;
+        }
+        __syncthreads();
+        RUMUS_ATTN_TILE_LOAD(j0 + BC)                          // consumed at the top of the next round
+        if (!wave_live || j0 >= wave_end) continue;            // wave-uniform: nothing visible in this tile
+
+        // ---- S^T = K Q^T -----------------------------------------------------------------
+        attn_v16f sacc;
+#pragma unroll
+        for (int r = 0; r < 16; r++) sacc[r] = 0.0f;
+        const float4* kfrag = ks + attn_tile_pos(l32, 16 * kb);
+#pragma unroll
+        for (int s4 = 0; s4 < 16; s4++) {
+            const float4 kf = kfrag[s4];                       // K[key l32][64*kb + 4*s4 ..]
+            sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.x, qf[4 * s4], sacc, 0, 0, 0);
+            sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.y, qf[4 * s4 + 1], sacc, 0, 0, 0);
+            sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.z, qf[4 * s4 + 2], sacc, 0, 0, 0);
+            sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.w, qf[4 * s4 + 3], sacc, 0, 0, 0);
+        }
+        // ---- online softmax of this lane's query over its 16 keys + the other half's 16 ----
+        // register r holds key j0 + (r/4)*8 + kb*4 + r%4
+        float p[16];
+        float mloc = kMasked;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const uint32_t key = j0 + (r >> 2) * 8 + kb * 4 + (r & 3);
+            p[r] = key < my_end ? sacc[r] : kMasked;
+            mloc = fmaxf(mloc, p[r]);
+        }
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
+        const float mnew = fmaxf(mrun, mloc);
+        const float corr = exp2f(mrun - mnew);
+        float lloc = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const uint32_t key = j0 + (r >> 2) * 8 + kb * 4 + (r & 3);
+            p[r] = key < my_end ? exp2f(p[r] - mnew) : 0.0f;
+            lloc += p[r];
+        }
+        lloc += __shfl_xor(lloc, 32);
+        lrun = lrun * corr + lloc;
+        mrun = mnew;
+        if (__any(corr != 1.0f)) {                             // the running maxima settle after a few tiles
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) oacc[dt][r] *= corr;
+        }
+        // ---- O^T += V^T P^T: step s multiplies keys (s/4)*8 + kb*4 + s%4, i.e. p[s] ----------
+        const float* vfrag = reinterpret_cast<const float*>(vs + attn_tile_pos(kb * 4, 0)) + l32;
+#pragma unroll
+        for (int s = 0; s < 16; s++) {
+            constexpr uint32_t kRowFloats = kAttnRowChunks * 4;
+            const uint32_t krow = (s >> 2) * 8 + (s & 3);      // + kb * 4, already in vfrag
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) {
+                const float vv = vfrag[krow * kRowFloats + dt * 32];   // V[krow + 4*kb][dt*32 + l32]
+                oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv, p[s], oacc[dt], 0, 0, 0);
+            }
+        }
+    }
+#undef RUMUS_ATTN_TILE_LOAD
+    if (qrow >= a.q_len) return;
+    // oacc[dt][r] = O[qrow][dt*32 + (r/4)*8 + kb*4 + r%4]: four consecutive dims per r/4
+    const float inv = lrun > 0.0f ? 1.0f / lrun : 0.0f;
+    float* op = a.o + b * a.o_sb + h * a.o_sh + (uint64_t)qrow * a.o_sr;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+        for (int g = 0; g < 4; g++)
+            *reinterpret_cast<float4*>(op + dt * 32 + g * 8 + kb * 4) =
+                make_float4(oacc[dt][4 * g] * inv, oacc[dt][4 * g + 1] * inv, oacc[dt][4 * g + 2] * inv,
+                            oacc[dt][4 * g + 3] * inv);
+}
+
 // Decode case (q_len == 1): the keys of one (batch, head) are split over gridDim.x workgroups
 // so that the chip is covered; each writes (max, sum, unnormalised output) of its slice and
 // attention_merge_kernel combines the slices.  Within a workgroup: 4 lanes per key for the
@@ -391,6 +556,11 @@ int rumus_hip_attention(const float* q, const float* k, const float* v, float* o
         hipLaunchKernelGGL(attention_merge_kernel, dim3(batch * heads), dim3(kHeadDim), 0, s, a,
                            static_cast<const float*>(ws), slices);
         return check_launch("attention_merge_kernel");
+    }
+    if (q_len >= 64) {                                       // enough rows to fill 32-row matrix-core tiles
+        RUMUS_REQUIRE(ceil_div(q_len, 128) <= 65535, "attention: q_len %u beyond the grid limit", q_len);
+        hipLaunchKernelGGL(attention_mfma_kernel, dim3(batch * heads, ceil_div(q_len, 128)), dim3(256), 0, s, a);
+        return check_launch("attention_mfma_kernel");
     }
     hipLaunchKernelGGL(attention_rows_kernel, dim3(ceil_div(q_len, 64), batch * heads), dim3(256), 0, s, a);
     return check_launch("attention_rows_kernel");

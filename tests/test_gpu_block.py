@@ -85,7 +85,8 @@ def test_decode_gemv_with_swiglu_input(ops, m, k, n, g):
 
 @pytest.mark.parametrize("b,h,nq,nkv,causal", [
     (1, 2, 64, 64, True), (2, 3, 100, 100, True), (1, 2, 70, 70, False), (1, 4, 33, 97, True),
-    (2, 32, 1, 2048, False), (3, 2, 1, 1, False), (1, 2, 1, 300, True), (1, 1, 512, 512, True)])
+    (2, 32, 1, 2048, False), (3, 2, 1, 1, False), (1, 2, 1, 300, True), (1, 1, 512, 512, True),
+    (1, 2, 200, 333, True), (2, 2, 130, 130, True), (1, 3, 64, 500, False), (1, 1, 129, 160, True)])
 def test_attention_vs_float64(ops, b, h, nq, nkv, causal):
     say(f"attention b={b} h={h} nq={nq} nkv={nkv} causal={causal}")
     rng = np.random.default_rng(b * 1000 + nq + nkv)
