@@ -25,7 +25,13 @@ struct W4Args {
     // columns: packed_t[(c*word_rows + r)*16 + j] = packed[r*n + 16*c + j], likewise the metadata
     bool tiled;
     // w4_gemv_dot8 only: x holds rows of 2k floats, gate | up; the activations are silu(gate) * up
-    bool glu;
+    bool glu;    // w4_gemm_tile only (set by its launcher): activations split into hi and lo f16 planes in
+    // A-fragment order, block (row tile of 32, step of 16 k) = 64 lanes x 16 bytes, and the f32
+    // sum of every row's 16 values per step; xsteps = steps allocated per row tile
+    const uint8_t* xh;
+    const uint8_t* xl;
+    const float* xs;
+    uint32_t xsteps;
 };
 
 // zero-points of 4 (col % 4 == 0) or 2 (col % 2 == 0) adjacent columns from the packed form

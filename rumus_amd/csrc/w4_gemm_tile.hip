@@ -118,7 +118,12 @@ __device__ __forceinline__ float4 zp4_load(const uint32_t* zp4, uint32_t g, uint
 // The stage body is straight-line code: loads past the end of the work are clamped to valid
 // addresses and their results never used, instead of being skipped, and nothing is consumed
 // right after it was loaded, so that the memory counter never has to drain.
-template <int RT, int WM, int TN, int WAVES, int DEPTH, int FOLD, bool ZP4>
+//
+// PRE: the activations arrive already split into hi and lo f16 planes in A-fragment order, with
+// the sums of every 16 of them beside (w4_convert_x_kernel), and a stage is copied into LDS as
+// it is.  Without it every workgroup of a row tile converts the same activations again, once
+// per 512 columns of the output.
+template <int RT, int WM, int TN, int WAVES, int DEPTH, int FOLD, bool ZP4, bool PRE>
 __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, float* __restrict__ out,
                                                                       uint32_t stages_per_split) {
     // a.x: rows of a.k floats, a.k % 4 == 0, 16-byte aligned, columns already in weight order
@@ -153,8 +158,44 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
     // ---- staging role: thread t converts 16 consecutive k (MFMA step t%8) of row t/8 -----
     const uint32_t s_row = tid >> 3, s_step = tid & 7;
     const bool s_active = s_row < BM;            // 32 rows, 8 waves: half of the threads stage
+    // PRE: a stage is (BM/32) row tiles x 8 steps x 2 planes of 1 KB fragment blocks, NCH 16-byte
+    // chunks per thread, and BM x 8 sums, NS per thread
+    constexpr int T = 64 * WAVES;
+    constexpr int NCH = PRE ? (BM / 32) * 8 * 2 * 64 / T : 1;
+    constexpr int NS = PRE ? (BM * 8 + T - 1) / T : 1;
+    static_assert(!PRE || (BM * 8) % T == 0, "the sums of a stage divide evenly over the threads");
     float4 xraw[DEPTH][NI][4];                   // DEPTH stages of activations in flight, too
+    // PRE: this thread's chunks and sums of the stage in flight, as named registers (an array
+    // indexed through the staging lambdas is left in scratch memory by the compiler)
+    static_assert(!PRE || (DEPTH == 1 && (NCH == 4 || NCH == 8) && NS <= 2), "PRE staging shape");
+    float4 xp0, xp1, xp2, xp3, xp4, xp5, xp6, xp7;
+    float xsr0 = 0.0f, xsr1 = 0.0f;
+    auto pre_src = [&](uint64_t tile0, int i) __attribute__((always_inline)) {
+        const uint32_t c = tid + T * i, blk = c >> 6, ln = c & 63;
+        const uint32_t plane = blk / ((BM / 32) * 8), rt = (blk / 8) % (BM / 32), step = blk % 8;
+        const uint8_t* src = (plane ? a.xl : a.xh) + ((tile0 + (uint64_t)rt * a.xsteps + step) * 64 + ln) * 16;
+        return *reinterpret_cast<const float4*>(src);
+    };
+    auto pre_dst = [&](uint32_t buf, int i) __attribute__((always_inline)) {
+        const uint32_t c = tid + T * i, blk = c >> 6, ln = c & 63;
+        const uint32_t plane = blk / ((BM / 32) * 8), rt = (blk / 8) % (BM / 32), step = blk % 8;
+        return reinterpret_cast<float4*>(lds_a[buf][plane] + step * STEP + rt * 1024 + ln * 16);
+    };
+    auto pre_sum_src = [&](uint64_t tile0, int i) __attribute__((always_inline)) {
+        const uint32_t e = tid + T * i, step = e / BM, row = e % BM;
+        return a.xs[(tile0 + (uint64_t)(row / 32) * a.xsteps + step) * 32 + (row & 31)];
+    };
     auto stage_load = [&](uint32_t st, int slot) __attribute__((always_inline)) {
+        if constexpr (PRE) {
+            const uint32_t gstage = min(st, nstages - 1);      // past the end: any valid stage, never used
+            const uint64_t tile0 = (uint64_t)(m0 / 32) * a.xsteps + gstage * 8;
+            xp0 = pre_src(tile0, 0); xp1 = pre_src(tile0, 1); xp2 = pre_src(tile0, 2); xp3 = pre_src(tile0, 3);
+            if constexpr (NCH == 8) {
+                xp4 = pre_src(tile0, 4); xp5 = pre_src(tile0, 5); xp6 = pre_src(tile0, 6); xp7 = pre_src(tile0, 7);
+            }
+            xsr0 = pre_sum_src(tile0, 0);
+            if constexpr (NS == 2) xsr1 = pre_sum_src(tile0, 1);
+        } else {
         if (!s_active) return;
         const uint32_t k0 = st * kStageK + s_step * 16;
 #pragma unroll
@@ -164,12 +205,35 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
             for (int i = 0; i < 4; i++)
                 xraw[slot][it][i] = *reinterpret_cast<const float4*>(xrow + min(k0 + 4 * i, a.k - 4));
         }
+        }
     };
     // Conversion of the values loaded for stage `st`, in 2*NI pieces of 8 values so that it can
     // be spread over the MFMA steps of the stage being multiplied.
-    constexpr int PIECES = 2 * NI;
+    constexpr int PIECES = PRE ? 4 : 2 * NI;             // spread over the last steps of a stage: the
+    static_assert(!PRE || NCH % 4 == 0, "chunks per piece"); // loads were issued at its first step
     float xsum[NI];
     auto stage_store_piece = [&](uint32_t st, uint32_t buf, int piece, int slot) __attribute__((always_inline)) {
+        if constexpr (PRE) {                               // NCH/4 chunks per piece, the sums with the last
+            if constexpr (NCH == 4) {
+                switch (piece) {
+                    case 0: *pre_dst(buf, 0) = xp0; break;
+                    case 1: *pre_dst(buf, 1) = xp1; break;
+                    case 2: *pre_dst(buf, 2) = xp2; break;
+                    default: *pre_dst(buf, 3) = xp3; break;
+                }
+            } else {
+                switch (piece) {
+                    case 0: *pre_dst(buf, 0) = xp0; *pre_dst(buf, 1) = xp1; break;
+                    case 1: *pre_dst(buf, 2) = xp2; *pre_dst(buf, 3) = xp3; break;
+                    case 2: *pre_dst(buf, 4) = xp4; *pre_dst(buf, 5) = xp5; break;
+                    default: *pre_dst(buf, 6) = xp6; *pre_dst(buf, 7) = xp7; break;
+                }
+            }
+            if (piece == PIECES - 1) {
+                lds_xs[buf][tid / BM][tid % BM] = xsr0;
+                if constexpr (NS == 2) lds_xs[buf][(tid + T) / BM][(tid + T) % BM] = xsr1;
+            }
+        } else {
         if (!s_active) return;
         const int it = piece >> 1, b = piece & 1;         // b: which 8-k block of this thread's step
         const uint32_t row = s_row + RPP * it;
@@ -196,6 +260,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
         *reinterpret_cast<v8h*>(lds_a[buf][1] + off) = lo;
         xsum[it] = sum;
         if (b) lds_xs[buf][s_step][row] = sum;
+        }
     };
 
     // ---- weights: one load of TN words per MFMA step; a register is refilled for DEPTH stages
@@ -427,6 +492,55 @@ __global__ __launch_bounds__(256) void w4_prepare_x_kernel(const float* __restri
     xp[(uint64_t)row * k4 + j] = v;
 }
 
+// Activations -> the form the PRE tile kernel copies into LDS.  Workgroup = one row tile of 32
+// and four steps of 16 k; thread t holds 8 consecutive k (t % 8) of row t / 8, as the staging
+// role of the tile kernel does.  Per (row tile, step) it writes two 1 KB fragment blocks (hi, lo:
+// lane = 32 * (k block of 8) + row, 8 halves in the k order 0,4,1,5,2,6,3,7 of the weight
+// fragment) and 32 sums.  Rows beyond m and columns beyond k are written as zeros, so that the
+// tile kernel needs no mask.  perm: act-order gather (x[row][perm[j]]).
+template <bool VEC>
+__global__ __launch_bounds__(256) void w4_convert_x_kernel(const float* __restrict__ x,
+                                                           const int32_t* __restrict__ perm,
+                                                           uint8_t* __restrict__ xh, uint8_t* __restrict__ xl,
+                                                           float* __restrict__ xs, uint32_t m, uint32_t k,
+                                                           uint32_t xsteps) {
+    const uint32_t tid = threadIdx.x, row = tid >> 3, kblk = tid & 7;
+    const uint32_t tile = blockIdx.y, step = blockIdx.x * 4 + (kblk >> 1), kb = kblk & 1;
+    const uint32_t grow = tile * 32 + row, k0 = step * 16 + kb * 8;
+    float xv[8];
+    if (VEC) {                                               // no perm, k % 8 == 0, 16-byte aligned x
+        const bool in = grow < m && k0 < k;
+        const float* src = x + (uint64_t)(in ? grow : 0) * k + (in ? k0 : 0);
+        const float4 lo4 = *reinterpret_cast<const float4*>(src), hi4 = *reinterpret_cast<const float4*>(src + 4);
+        xv[0] = in ? lo4.x : 0.0f; xv[1] = in ? lo4.y : 0.0f; xv[2] = in ? lo4.z : 0.0f; xv[3] = in ? lo4.w : 0.0f;
+        xv[4] = in ? hi4.x : 0.0f; xv[5] = in ? hi4.y : 0.0f; xv[6] = in ? hi4.z : 0.0f; xv[7] = in ? hi4.w : 0.0f;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const bool in = grow < m && k0 + j < k;
+            const uint32_t kk = in ? k0 + j : 0;
+            const float v = x[(uint64_t)(in ? grow : 0) * k + (perm ? (uint32_t)perm[kk] : kk)];
+            xv[j] = in ? v : 0.0f;
+        }
+    }
+    v8h hi, lo;
+    float sum = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        const int j = (e >> 1) + 4 * (e & 1);                // fragment element e holds k offset j
+        const float v = xv[j];
+        const _Float16 h = (_Float16)v;
+        hi[e] = h;
+        lo[e] = (_Float16)(v - (float)h);                    // hi + lo equals v to 2^-22 |v|
+        sum += v;
+    }
+    sum += __shfl_xor(sum, 1);                               // the other 8 of this row's step
+    const uint64_t blk = (uint64_t)tile * xsteps + step;
+    *reinterpret_cast<v8h*>(xh + (blk * 64 + kb * 32 + row) * 16) = hi;
+    *reinterpret_cast<v8h*>(xl + (blk * 64 + kb * 32 + row) * 16) = lo;
+    if (kb == 0) xs[blk * 32 + row] = sum;
+}
+
 template <int RT, int WM, int TN, int WAVES, int DEPTH, int FOLD>
 static int launch_tile(const W4Args& a_in, hipStream_t s) {
     W4Args a = a_in;
@@ -434,17 +548,39 @@ static int launch_tile(const W4Args& a_in, hipStream_t s) {
     const uint32_t nstages = ceil_div(a.padded_k, kStageK);
     uint32_t sps = nstages;
     const uint32_t splits = pick_splits(tn * tm, nstages, &sps);
+    // 64-row tiles of eight waves: activations converted once, up front (10 % at m = 512).  The
+    // four-wave shape has no registers to spare for the staged chunks and converts in place.
+    constexpr bool PRE = RT * WM >= 2 && WAVES == 8;
+    constexpr uint32_t BM = 32 * RT * WM;
     // workspace: [activations in the form the kernel reads][partial tiles]
-    const bool prepare = a.perm || a.k % 4 != 0 || (reinterpret_cast<uintptr_t>(a.x) & 15) != 0;
+    const bool prepare = !PRE && (a.perm || a.k % 4 != 0 || (reinterpret_cast<uintptr_t>(a.x) & 15) != 0);
     const uint32_t k4 = (a.k + 3) & ~3u;
-    RUMUS_REQUIRE(!prepare || a.m <= 65535, "qmatmul_int4: m %u is beyond the grid limit of the activation copy", a.m);
-    const size_t x_bytes = prepare ? (((size_t)a.m * k4 * sizeof(float) + 255) & ~size_t(255)) : 0;
+    const uint32_t xtiles = tm * (BM / 32), xsteps = nstages * 8;   // whole workgroup tiles, whole stages
+    RUMUS_REQUIRE(!(prepare || PRE) || max(a.m, xtiles) <= 65535,
+                  "qmatmul_int4: m %u is beyond the grid limit of the activation copy", a.m);
+    const size_t plane_bytes = (size_t)xtiles * xsteps * 1024, sums_bytes = (size_t)xtiles * xsteps * 128;
+    const size_t x_bytes = PRE ? 2 * plane_bytes + sums_bytes
+                               : prepare ? (((size_t)a.m * k4 * sizeof(float) + 255) & ~size_t(255)) : 0;
     const size_t part_bytes = splits > 1 ? (size_t)splits * a.m * a.n * sizeof(float) : 0;
     float* out = a.y;
     if (x_bytes + part_bytes) {
         void* ws = nullptr;
         if (int rc = workspace_get(s, x_bytes + part_bytes, &ws)) return rc;
-        if (prepare) {
+        if (PRE) {
+            uint8_t* base = static_cast<uint8_t*>(ws);
+            const bool vec = !a.perm && a.k % 8 == 0 && (reinterpret_cast<uintptr_t>(a.x) & 15) == 0;
+            const dim3 grid(xsteps / 4, xtiles);
+            float* sums = reinterpret_cast<float*>(base + 2 * plane_bytes);
+            if (vec) hipLaunchKernelGGL(w4_convert_x_kernel<true>, grid, dim3(256), 0, s, a.x, a.perm, base,
+                                        base + plane_bytes, sums, a.m, a.k, xsteps);
+            else hipLaunchKernelGGL(w4_convert_x_kernel<false>, grid, dim3(256), 0, s, a.x, a.perm, base,
+                                    base + plane_bytes, sums, a.m, a.k, xsteps);
+            if (int rc = check_launch("w4_convert_x_kernel")) return rc;
+            a.xh = base;
+            a.xl = base + plane_bytes;
+            a.xs = sums;
+            a.xsteps = xsteps;
+        } else if (prepare) {
             float* xp = static_cast<float*>(ws);
             hipLaunchKernelGGL(w4_prepare_x_kernel, dim3(ceil_div(k4, 256), a.m), dim3(256), 0, s, a.x, a.perm, xp,
                                a.k, k4);
@@ -456,11 +592,11 @@ static int launch_tile(const W4Args& a_in, hipStream_t s) {
         if (splits > 1) out = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + x_bytes);
     }
     if (a.zp4)
-        hipLaunchKernelGGL((w4_gemm_tile_kernel<RT, WM, TN, WAVES, DEPTH, FOLD, true>), dim3(tn, tm, splits), dim3(64 * WAVES), 0,
-                           s, a, out, sps);
+        hipLaunchKernelGGL((w4_gemm_tile_kernel<RT, WM, TN, WAVES, DEPTH, FOLD, true, PRE>), dim3(tn, tm, splits),
+                           dim3(64 * WAVES), 0, s, a, out, sps);
     else
-        hipLaunchKernelGGL((w4_gemm_tile_kernel<RT, WM, TN, WAVES, DEPTH, FOLD, false>), dim3(tn, tm, splits), dim3(64 * WAVES), 0,
-                           s, a, out, sps);
+        hipLaunchKernelGGL((w4_gemm_tile_kernel<RT, WM, TN, WAVES, DEPTH, FOLD, false, PRE>), dim3(tn, tm, splits),
+                           dim3(64 * WAVES), 0, s, a, out, sps);
     if (int rc = check_launch("w4_gemm_tile_kernel")) return rc;
     if (splits > 1) {
         const uint32_t count4 = (uint32_t)((uint64_t)a.m * a.n / 4);
@@ -484,18 +620,18 @@ static int launch_fold(const W4Args& a, hipStream_t s) {
 int w4_launch_gemm(const W4Args& a, hipStream_t s) {
     RUMUS_REQUIRE((uint64_t)a.m * a.n < (1ull << 32), "qmatmul_int4: m * n must fit 32 bits");
     RUMUS_REQUIRE(a.m <= 65535 * 32, "qmatmul_int4: m %u is beyond the grid limit", a.m);
-    // Three shapes of workgroup, chosen by how many tiles the problem makes (measured on
-    // n = 4096 and n = 11008, m = 16 .. 4096):
-    //   up to 72 tiles of 32 rows: eight waves side by side, 32 rows x 64 columns each; the small
-    //       tile keeps more workgroups in flight when there are fewer tiles than CUs;
-    //   up to 255 tiles of 128 rows: the same eight waves with 64 rows each, so a converted weight
-    //       fragment serves two row tiles;
-    //   beyond: four waves side by side, 64 rows x 128 columns each, two such workgroups per CU
-    //       (fewer LDS fragment reads per MFMA, finer-grained rounds).
+    // Two shapes of workgroup, eight waves side by side over 512 columns, chosen by how many
+    // tiles the problem makes (measured on n = 4096 and n = 11008, m = 16 .. 8192):
+    //   up to 72 tiles of 32 rows: 32 rows x 64 columns per wave; the small tile keeps more
+    //       workgroups in flight when there are fewer tiles than CUs, and converts its few
+    //       activations itself;
+    //   beyond: 64 rows x 64 columns per wave, so that a converted weight fragment serves two row
+    //       tiles, on activations converted once by w4_convert_x_kernel.
+    // (Four waves of 64 x 128 each, two workgroups per CU, halve the LDS fragment reads but have
+    // no registers left for pre-converted activations: 3-20 % slower from m = 1024 to 4096.)
     const uint64_t col_tiles = ceil_div(a.n, kTileCols);
     if (ceil_div(a.m, 32) * col_tiles <= 72) return launch_fold<1, 1, 2, 8, 1>(a, s);
-    if (ceil_div(a.m, 128) * col_tiles < 256) return launch_fold<2, 1, 2, 8, 1>(a, s);
-    return launch_fold<2, 1, 4, 4, 1>(a, s);
+    return launch_fold<2, 1, 2, 8, 1>(a, s);
 }
 
 }  // namespace rumus
