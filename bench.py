@@ -93,7 +93,7 @@ def bench_gemv(torch, ops, steps, warmup):
             w = torch.randn((K, N), generator=gen, device=dev, dtype=torch.float32) * 0.02
         sets.append(ops.w4_quantize_pack(w, G))
         sets_dl.append(ops.w4_decode_layout(*sets[-1], G))
-        sets_awq.append(ops.w4_quantize_pack_awq(w, G))
+        sets_awq.append(ops.w4_decode_layout_zp4(*ops.w4_quantize_pack_awq(w, G), G))
         del w
     ys = [torch.empty((M, N), dtype=torch.float32, device=dev) for _ in range(WEIGHT_SETS)]
     torch.cuda.synchronize()
@@ -115,7 +115,7 @@ def bench_gemv(torch, ops, steps, warmup):
 
     def burst_rotating_awq():
         for (p, s, qz), y in zip(sets_awq, ys):
-            ops.qmatmul_int4_zp4(x, p, s, qz, K, G, out=y)
+            ops.qmatmul_int4_decode_zp4(x, p, s, qz, K, G, out=y)
 
     # the timed region of record: EXACTLY `steps` launches, bracketed by device syncs
     sec, launches, used_graph = time_graph(torch, burst_rotating, WEIGHT_SETS, steps, warmup)
@@ -465,7 +465,8 @@ def main():
         "awq_storage_u4_zero_points": {
             "ms_per_step": r["sec_awq"] / r["launches_awq"] * 1e3, "bytes_per_step": BYTES_U4_ZP,
             "gbs": BYTES_U4_ZP / (r["sec_awq"] / r["launches_awq"]) / 1e9,
-            "note": "same shape with integer zero-points packed eight per word (rumus_hip_qmatmul_int4_zp4)"},
+            "note": "same shape with integer zero-points packed eight per word, tile-major copy "
+                    "(rumus_hip_qmatmul_int4_decode_zp4)"},
         "cache_resident": {"gbs": BYTES_F32_ZP / per_launch_res / 1e9,
                            "ms_per_step": per_launch_res * 1e3,
                            "note": "single weight set, served by Infinity Cache / L2; not HBM"},

@@ -239,6 +239,23 @@ int rumus_hip_qmatmul_int4_decode(const float* x, const uint32_t* packed_t,
                                   uint32_t group_size, uint32_t num_groups,
                                   rumus_hip_stream_t stream);
 
+/* EXTENSION: the decode layout and its matmul for AWQ storage (u4 zero-points,
+ * rumus_hip_w4_quantize_pack_awq): packed_t and scales_t as in
+ * rumus_hip_w4_decode_layout; qzeros_t[(c*num_groups + g)*2 + h] =
+ * qzeros[g*(n/8) + 2*c + h], the two zero-point words of tile c's 16 columns.
+ * Same bits as rumus_hip_qmatmul_int4_zp4 on the row-major arrays for m <= 5.
+ * EINVAL as for the f32 zero-point forms.  No counterpart in the reference. */
+int rumus_hip_w4_decode_layout_zp4(const uint32_t* packed, const float* scales,
+                                   const uint32_t* qzeros, uint32_t padded_k, uint32_t n,
+                                   uint32_t group_size, uint32_t* packed_t, float* scales_t,
+                                   uint32_t* qzeros_t, rumus_hip_stream_t stream);
+int rumus_hip_qmatmul_int4_decode_zp4(const float* x, const uint32_t* packed_t,
+                                      const float* scales_t, const uint32_t* qzeros_t,
+                                      const float* bias, const int32_t* perm, float* y,
+                                      uint32_t m, uint32_t k, uint32_t n, uint32_t padded_k,
+                                      uint32_t group_size, uint32_t num_groups,
+                                      rumus_hip_stream_t stream);
+
 /* EXTENSION: rumus_hip_qmatmul_int4_decode whose input is the output of a
  * fused gate|up projection: gate_up [m, 2k] (gate in columns 0..k-1, up in
  * k..2k-1), x[m, j] = silu(gate[m, j]) * up[m, j] computed on the way in, so the

@@ -35,9 +35,11 @@ struct W4Args {
 };
 
 // zero-points of 4 (col % 4 == 0) or 2 (col % 2 == 0) adjacent columns from the packed form
-__device__ __forceinline__ float4 w4_zp4_load4(const uint32_t* zp4, uint32_t g, uint32_t n, uint32_t col) {
-    const uint32_t v = zp4[(uint64_t)g * (n / 8) + col / 8] >> ((col & 4u) * 4u);
+__device__ __forceinline__ float4 w4_zp4_unpack4(uint32_t v) {   // the four low nibbles
     return make_float4((float)(v & 15u), (float)((v >> 4) & 15u), (float)((v >> 8) & 15u), (float)((v >> 12) & 15u));
+}
+__device__ __forceinline__ float4 w4_zp4_load4(const uint32_t* zp4, uint32_t g, uint32_t n, uint32_t col) {
+    return w4_zp4_unpack4(zp4[(uint64_t)g * (n / 8) + col / 8] >> ((col & 4u) * 4u));
 }
 __device__ __forceinline__ float2 w4_zp4_load2(const uint32_t* zp4, uint32_t g, uint32_t n, uint32_t col) {
     const uint32_t v = zp4[(uint64_t)g * (n / 8) + col / 8] >> ((col & 6u) * 4u);

@@ -353,6 +353,23 @@ int rumus_hip_qmatmul_int4_decode(const float* x, const uint32_t* packed_t, cons
     return w4_launch_gemv_dot8(a, as_stream(stream));
 }
 
+int rumus_hip_qmatmul_int4_decode_zp4(const float* x, const uint32_t* packed_t, const float* scales_t,
+                                      const uint32_t* qzeros_t, const float* bias, const int32_t* perm, float* y,
+                                      uint32_t m, uint32_t k, uint32_t n, uint32_t padded_k, uint32_t group_size,
+                                      uint32_t num_groups, rumus_hip_stream_t stream) {
+    W4Args a{x, packed_t, scales_t, nullptr, bias, nullptr, perm, y, m, k, n, padded_k, group_size, num_groups,
+             qzeros_t, true};
+    if (int rc = validate(a, "qmatmul_int4_decode_zp4")) return rc;
+    RUMUS_REQUIRE(!perm || k == padded_k, "qmatmul_int4_decode_zp4: perm needs k == padded_k (%u vs %u)", k, padded_k);
+    RUMUS_REQUIRE(n % 16 == 0, "qmatmul_int4_decode_zp4: n must be a multiple of 16 (got %u)", n);
+    RUMUS_REQUIRE(m <= 8, "qmatmul_int4_decode_zp4: at most 8 rows (got %u); larger batches take qmatmul_int4_zp4", m);
+    if (m == 0 || n == 0) return RUMUS_HIP_OK;
+    RUMUS_REQUIRE(k > 0, "qmatmul_int4_decode_zp4: k must be > 0");
+    RUMUS_REQUIRE(w4_gemv_dot8_supported(a),
+                  "qmatmul_int4_decode_zp4: needs group_size %% 32 == 0 and 16-byte aligned buffers");
+    return w4_launch_gemv_dot8(a, as_stream(stream));
+}
+
 int rumus_hip_qmatmul_int4_decode_swiglu(const float* gate_up, const uint32_t* packed_t, const float* scales_t,
                                          const float* zero_points_t, const float* bias, float* y, uint32_t m,
                                          uint32_t k, uint32_t n, uint32_t padded_k, uint32_t group_size,

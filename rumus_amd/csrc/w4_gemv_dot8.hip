@@ -164,8 +164,11 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
         const uint64_t mo = TILED ? ((uint64_t)cchunk * (padded_k / group_size) + g) * kD8Cols + 4 * cq
                                   : (uint64_t)g * n + col_c;
         float4 sc = *reinterpret_cast<const float4*>(scales + mo);
-        const float4 zp = ZP4 ? w4_zp4_load4(reinterpret_cast<const uint32_t*>(zps), g, n, col_c)
-                              : *reinterpret_cast<const float4*>(zps + mo);
+        // ZP4 + TILED: the two zero-point words of a tile's 16 columns sit side by side per group
+        const float4 zp = !ZP4 ? *reinterpret_cast<const float4*>(zps + mo)
+                          : TILED ? w4_zp4_unpack4(reinterpret_cast<const uint32_t*>(zps)[
+                                        ((uint64_t)cchunk * (padded_k / group_size) + g) * 2 + (cq >> 1)] >> ((cq & 1) * 16))
+                                  : w4_zp4_load4(reinterpret_cast<const uint32_t*>(zps), g, n, col_c);
         if (!(live && col_ok)) sc = make_float4(0, 0, 0, 0);
 
         uint32_t wv[OCT][4];
@@ -313,6 +316,9 @@ static int launch_m(const W4Args& a, hipStream_t s) {
             return set_error(RUMUS_HIP_EINVAL, "w4 gemv: the SwiGLU input needs the decode layout, f32 zero-points, "
                                                "k %% 8 == 0 and 16-byte aligned rows");
         launch_variant<M, true, false, true, true>(a, s);
+    } else if (a.tiled && a.zp4) {
+        if (fast_x) launch_variant<M, true, true, true>(a, s);
+        else launch_variant<M, false, true, true>(a, s);
     } else if (a.tiled) {
         if (fast_x) launch_variant<M, true, false, true>(a, s);
         else launch_variant<M, false, false, true>(a, s);

@@ -116,6 +116,16 @@ __global__ __launch_bounds__(256) void w4_tile16_kernel(const uint4* __restrict_
     out[((uint64_t)(q >> 2) * rows + r) * 4 + (q & 3)] = in[(uint64_t)r * (n / 4) + q];
 }
 
+// Decode layout of u4 zero-points [groups, n/8]: the two words of a tile's 16 columns side by
+// side per group, out[(c*groups + g)*2 + h] = in[g*(n/8) + 2*c + h].
+__global__ __launch_bounds__(256) void w4_tile16_zp4_kernel(const uint32_t* __restrict__ in,
+                                                            uint32_t* __restrict__ out, uint32_t groups,
+                                                            uint32_t words_per_row) {
+    const uint32_t wd = blockIdx.x * 256 + threadIdx.x, g = blockIdx.y;
+    if (wd >= words_per_row) return;
+    out[((uint64_t)(wd >> 1) * groups + g) * 2 + (wd & 1)] = in[(uint64_t)g * words_per_row + wd];
+}
+
 // packed_sorted word (jr, col) gathers the nibbles of original rows
 // perm[8*jr .. 8*jr+7].
 __global__ __launch_bounds__(256) void w4_gather_rows_kernel(const uint32_t* __restrict__ packed,
@@ -182,10 +192,11 @@ int rumus_hip_w4_quantize_pack(const float* w, uint32_t k, uint32_t n, uint32_t 
     return quantize_pack<false>(w, k, n, group_size, packed, scales, zero_points, as_stream(stream));
 }
 
-int rumus_hip_w4_decode_layout(const uint32_t* packed, const float* scales, const float* zero_points,
-                               uint32_t padded_k, uint32_t n, uint32_t group_size, uint32_t* packed_t,
-                               float* scales_t, float* zero_points_t, rumus_hip_stream_t stream) {
-    RUMUS_REQUIRE(packed && scales && zero_points && packed_t && scales_t && zero_points_t,
+static int decode_layout(const uint32_t* packed, const float* scales, const float* zero_points,
+                         const uint32_t* qzeros, uint32_t padded_k, uint32_t n, uint32_t group_size,
+                         uint32_t* packed_t, float* scales_t, float* zero_points_t, uint32_t* qzeros_t,
+                         hipStream_t s) {
+    RUMUS_REQUIRE(packed && scales && packed_t && scales_t && ((zero_points && zero_points_t) || (qzeros && qzeros_t)),
                   "w4_decode_layout: null buffer");
     RUMUS_REQUIRE(n % 16 == 0, "w4_decode_layout: n must be a multiple of 16 (got %u)", n);
     RUMUS_REQUIRE(group_size > 0 && padded_k % group_size == 0 && group_size % 8 == 0,
@@ -197,15 +208,35 @@ int rumus_hip_w4_decode_layout(const uint32_t* packed, const float* scales, cons
     if (padded_k == 0 || n == 0) return RUMUS_HIP_OK;
     const uint32_t word_rows = padded_k / 8, groups = padded_k / group_size;
     RUMUS_REQUIRE(word_rows <= 65535, "w4_decode_layout: padded_k %u beyond the grid limit", padded_k);
-    hipStream_t s = as_stream(stream);
     const dim3 gx(ceil_div(n / 4, 256));
     hipLaunchKernelGGL(w4_tile16_kernel, dim3(gx.x, word_rows), dim3(256), 0, s,
                        reinterpret_cast<const uint4*>(packed), reinterpret_cast<uint4*>(packed_t), word_rows, n);
     hipLaunchKernelGGL(w4_tile16_kernel, dim3(gx.x, groups), dim3(256), 0, s,
                        reinterpret_cast<const uint4*>(scales), reinterpret_cast<uint4*>(scales_t), groups, n);
-    hipLaunchKernelGGL(w4_tile16_kernel, dim3(gx.x, groups), dim3(256), 0, s,
-                       reinterpret_cast<const uint4*>(zero_points), reinterpret_cast<uint4*>(zero_points_t), groups, n);
+    if (qzeros)
+        hipLaunchKernelGGL(w4_tile16_zp4_kernel, dim3(ceil_div(n / 8, 256), groups), dim3(256), 0, s, qzeros, qzeros_t,
+                           groups, n / 8);
+    else
+        hipLaunchKernelGGL(w4_tile16_kernel, dim3(gx.x, groups), dim3(256), 0, s,
+                           reinterpret_cast<const uint4*>(zero_points), reinterpret_cast<uint4*>(zero_points_t), groups,
+                           n);
     return check_launch("w4_tile16_kernel");
+}
+
+int rumus_hip_w4_decode_layout(const uint32_t* packed, const float* scales, const float* zero_points,
+                               uint32_t padded_k, uint32_t n, uint32_t group_size, uint32_t* packed_t,
+                               float* scales_t, float* zero_points_t, rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE(zero_points && zero_points_t, "w4_decode_layout: null buffer");
+    return decode_layout(packed, scales, zero_points, nullptr, padded_k, n, group_size, packed_t, scales_t,
+                         zero_points_t, nullptr, as_stream(stream));
+}
+
+int rumus_hip_w4_decode_layout_zp4(const uint32_t* packed, const float* scales, const uint32_t* qzeros,
+                                   uint32_t padded_k, uint32_t n, uint32_t group_size, uint32_t* packed_t,
+                                   float* scales_t, uint32_t* qzeros_t, rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE(qzeros && qzeros_t, "w4_decode_layout_zp4: null buffer");
+    return decode_layout(packed, scales, nullptr, qzeros, padded_k, n, group_size, packed_t, scales_t, nullptr,
+                         qzeros_t, as_stream(stream));
 }
 
 int rumus_hip_f16_to_f32(const uint16_t* in, float* out, uint64_t numel, rumus_hip_stream_t stream) {

@@ -187,6 +187,31 @@ def qmatmul_int4_decode(x, packed_t, scales_t, zp_t, k, group_size, bias=None, p
     return _w4_call("rumus_hip_qmatmul_int4_decode", x, packed_t, scales_t, zp_t, bias, perm, k, group_size, out)
 
 
+def w4_decode_layout_zp4(packed, scales, qzeros, group_size):
+    """Tile-major copies for AWQ storage: packed, scales as in w4_decode_layout, u4 zero-points with
+    the two words of a tile side by side."""
+    rows, n = packed.shape
+    out = (torch.empty_like(packed), torch.empty_like(scales), torch.empty_like(qzeros))
+    call("rumus_hip_w4_decode_layout_zp4", _dev(packed, torch.int32, "packed"), _dev(scales, torch.float32, "scales"),
+         _dev(qzeros, torch.int32, "qzeros"), rows * 8, n, group_size, out[0].data_ptr(), out[1].data_ptr(),
+         out[2].data_ptr(), _stream())
+    return out
+
+
+def qmatmul_int4_decode_zp4(x, packed_t, scales_t, qzeros_t, k, group_size, bias=None, perm=None, out=None):
+    m = x.shape[0]
+    n = packed_t.shape[1]
+    if x.dim() != 2 or x.shape[1] != k:
+        raise ValueError("qmatmul_int4_decode_zp4: x must be [m, k]")
+    padded_k, groups = w4_geometry(k, group_size) if group_size > 0 else (k, 0)
+    y = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=x.device)
+    call("rumus_hip_qmatmul_int4_decode_zp4", _dev(x, torch.float32, "x"), _dev(packed_t, torch.int32, "packed_t"),
+         _dev(scales_t, torch.float32, "scales_t"), _dev(qzeros_t, torch.int32, "qzeros_t"),
+         _opt(bias, torch.float32, "bias"), _opt(perm, torch.int32, "perm"),
+         _dev(y, torch.float32, "y"), m, k, n, padded_k, group_size, groups, _stream())
+    return y
+
+
 def qmatmul_int4_decode_swiglu(gate_up, packed_t, scales_t, zp_t, k, group_size, bias=None, out=None):
     """``(silu(gate) * up) @ dequant(W)`` for ``gate_up`` ``[m, 2k]`` (gate | up), one launch."""
     m = gate_up.shape[0]

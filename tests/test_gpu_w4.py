@@ -397,6 +397,31 @@ def test_decode_layout_is_bit_identical(ops, m, k, n, g):
         np.testing.assert_array_equal(got, host(ops.qmatmul_int4(dev(x), *d, k, g, bias=dev(b))))
 
 
+@pytest.mark.parametrize("m,k,n,g", [(1, 4096, 4096, 128), (3, 1000, 48, 64), (8, 512, 11008, 32), (5, 256, 16, 256)])
+def test_decode_layout_u4_zero_points(ops, m, k, n, g):
+    say(f"qmatmul_int4_decode_zp4 m={m} k={k} n={n} g={g}")
+    rng = np.random.default_rng(m + k + n + 1)
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    x = rng.normal(0, 1, (m, k)).astype(np.float32)
+    b = rng.normal(0, 0.01, n).astype(np.float32)
+    packed, scales, qzeros = oracle.w4_awq_from_f32(w, g)
+    d = [dev(a) for a in (packed, scales, qzeros)]
+    pt, st, qt = ops.w4_decode_layout_zp4(*d, g)
+    # the zero-point layout itself: the two words of a tile's 16 columns side by side per group
+    want_qt = qzeros.reshape(qzeros.shape[0], n // 16, 2).transpose(1, 0, 2).reshape(-1)
+    np.testing.assert_array_equal(host_u32(qt).reshape(-1), want_qt)
+    got = host(ops.qmatmul_int4_decode_zp4(dev(x), pt, st, qt, k, g, bias=dev(b)))
+    zp = oracle.w4_qzeros_unpack(qzeros, n)
+    assert_close(got, oracle.qmatmul_int4(x, packed, scales, zp, k, g, bias=b, threads=8))
+    if m <= 5:   # the row-major entry point runs the same kernel arithmetic on these shapes
+        np.testing.assert_array_equal(got, host(ops.qmatmul_int4_zp4(dev(x), *d, k, g, bias=dev(b))))
+    # act-order on top
+    if k % g == 0:
+        perm = rng.permutation(k).astype(np.int32)
+        got_p = host(ops.qmatmul_int4_decode_zp4(dev(x), pt, st, qt, k, g, perm=dev(perm)))
+        assert_close(got_p, oracle.qmatmul_int4(np.ascontiguousarray(x[:, perm]), packed, scales, zp, k, g, threads=8))
+
+
 def test_decode_layout_rejects_bad_arguments(ops):
     from rumus_amd._lib import RumusError
     import torch
