@@ -180,15 +180,17 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
 #pragma unroll
         for (int m = 0; m < M; m++) {
             // ---- 2. activations of the chunk -> nibble planes (registers) -----
-            float amax = 0.0f;
+            // largest magnitude of the chunk, compared as integers: the bits of non-negative floats
+            // order like the floats and a NaN sorts above infinity (a float max would skip it)
+            uint32_t amax = 0;
 #pragma unroll
             for (int t = 0; t < OPL; t++)
 #pragma unroll
-                for (int j = 0; j < 8; j++) amax = fmaxf(amax, fabsf(xv[m][t][j]));
-            amax = fmaxf(amax, RUMUS_DPP_F(amax, kDppXor1));
-            amax = fmaxf(amax, RUMUS_DPP_F(amax, kDppXor2));
+                for (int j = 0; j < 8; j++) amax = max(amax, __float_as_uint(xv[m][t][j]) & 0x7FFFFFFFu);
+            amax = max(amax, (uint32_t)RUMUS_DPP_I(amax, kDppXor1));
+            amax = max(amax, (uint32_t)RUMUS_DPP_I(amax, kDppXor2));
             // amax = a * 2^E (1 <= a < 2): scale by just under 2^(18-E) so that |x * f| < 2^19 - 1/2
-            const uint32_t ebits = __float_as_uint(amax) >> 23;   // biased exponent (amax >= 0)
+            const uint32_t ebits = amax >> 23;             // biased exponent
             // the factor 1 - 2^-20 keeps rint(amax * f) at 2^19 - 1 or below
             float f = __uint_as_float((272u - ebits) << 23) * 0.99999905f;
             float finv = __uint_as_float((ebits - 18u) << 23) * 1.00000095f;

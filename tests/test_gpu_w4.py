@@ -52,6 +52,30 @@ def test_quantize_pack_rejects_bad_group(ops):
         ops.w4_quantize_pack(dev(np.zeros((24, 4), np.float32)), 12)
 
 
+def test_quantize_pack_non_finite_weights(ops):
+    # quant.rs:69-73 compares with `<` and `>`, so a NaN never becomes min or max; `as i32`
+    # (quant.rs:96) saturates and turns NaN into 0.  Cases: a NaN among finite values, +inf, -inf,
+    # a group of NaNs only, and an inf whose quotient overflows the nibble range.
+    say("w4_quantize_pack non-finite weights")
+    nan, inf = np.float32(np.nan), np.float32(np.inf)
+    cols = [
+        [nan, 1, 2, 3, 0, 0, 0, 0],          # scale 0.2, zp 0 -> 0,5,10,15,0,...
+        [inf, 1, 0, 0, 0, 0, 0, 0],          # scale inf, zp -0: every quotient is 0 or NaN -> 0
+        [-inf, 1, 0, 0, 0, 0, 0, 0],         # scale inf, zp NaN -> 0
+        [nan] * 8,                           # min stays f32::MAX, max f32::MIN: range < 0 -> scale 1, zp 0
+        [nan, -3, 3, 1e30, 0, 0, 0, 0],
+    ]
+    w = np.array(cols, np.float32).T.copy()                 # [k = 8, n = 5]
+    want = oracle.w4_from_f32(w, 8)
+    assert [f"{v:08x}" for v in want[0].reshape(-1)[:4]] == ["0000fa50", "00000000", "00000000", "00000000"]
+    assert want[1][0, 3] == 1.0 and want[2][0, 3] == 0.0 and np.isinf(want[1][0, 1]) and np.isnan(want[2][0, 2])
+    got = ops.w4_quantize_pack(dev(w), 8)
+    np.testing.assert_array_equal(host_u32(got[0]), want[0])
+    for g, wv in ((host(got[1]), want[1]), (host(got[2]), want[2])):
+        np.testing.assert_array_equal(np.isnan(g), np.isnan(wv))
+        np.testing.assert_array_equal(g[~np.isnan(wv)].view(np.uint32), wv[~np.isnan(wv)].view(np.uint32))
+
+
 SHAPES = [
     # m, k, n, g, bias
     (1, 256, 64, 128, False),     # gemv, one pass
@@ -110,6 +134,31 @@ def test_zero_scale_group_contributes_nothing(ops):
     got = host(ops.qmatmul_int4(dev(x), dev(packed), dev(scales), dev(zp), k, g))
     assert np.isfinite(got).all()
     assert_close(got, want)
+
+
+@pytest.mark.parametrize("m", [2, 16])
+def test_non_finite_activations_poison_their_row_only(ops, m):
+    # the reference accumulates a * w in f32, so a NaN activation makes its whole output row NaN
+    # (NaN * 0 is NaN too) and leaves the other rows alone.  The decode kernel (m = 2) scales each
+    # chunk by its largest magnitude and the MFMA kernel (m = 16) splits activations into two
+    # halves: both must still deliver NaN, and both turn an infinite activation into NaN as well
+    # (the reference would give an infinity where all weights of the column agree in sign).
+    say(f"qmatmul_int4 non-finite activations m={m}")
+    rng = np.random.default_rng(50 + m)
+    k, n, g = 512, 64, 128
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    x = rng.normal(0, 1, (m, k)).astype(np.float32)
+    packed, scales, zp = oracle.w4_from_f32(w, g)
+    d = [dev(a) for a in (packed, scales, zp)]
+    clean = host(ops.qmatmul_int4(dev(x), *d, k, g))
+    for bad in (np.float32(np.nan), np.float32(np.inf)):
+        xb = x.copy()
+        xb[1, 300] = bad
+        got = host(ops.qmatmul_int4(dev(xb), *d, k, g))
+        assert np.isnan(got[1]).all()
+        np.testing.assert_array_equal(np.delete(got, 1, axis=0), np.delete(clean, 1, axis=0))
+    want = oracle.qmatmul_int4(np.where(np.isfinite(xb), xb, np.float32(np.nan)), packed, scales, zp, k, g)
+    assert np.isnan(want[1]).all() and np.isfinite(np.delete(want, 1, axis=0)).all()
 
 
 def test_reference_order_kernel_is_bit_exact(ops):
