@@ -161,6 +161,33 @@ def test_non_finite_activations_poison_their_row_only(ops, m):
     assert np.isnan(want[1]).all() and np.isfinite(np.delete(want, 1, axis=0)).all()
 
 
+@pytest.mark.parametrize("m", [1, 5, 16, 100])
+def test_weights_far_from_zero(ops, m):
+    # all weights near +10: the reference's zero-point is about -10 / scale, in the thousands and
+    # negative, and the zero-point term dwarfs the nibble term.  Every kernel forms
+    # scale * (sum x q - zp * sum x) per group instead of the reference's per-element products.
+    say(f"qmatmul_int4 offset weights m={m}")
+    rng = np.random.default_rng(70 + m)
+    k, n, g = 1024, 128, 128
+    w = (10.0 + rng.normal(0, 0.02, (k, n))).astype(np.float32)
+    w[:, 1] = -7.0 + rng.normal(0, 0.5, k)
+    x = rng.normal(0, 1, (m, k)).astype(np.float32)
+    packed, scales, zp = oracle.w4_from_f32(w, g)
+    assert zp.min() < -1000 and zp.max() > 30
+    want = oracle.qmatmul_int4(x, packed, scales, zp, k, g, threads=8)
+    got = host(ops.qmatmul_int4(dev(x), dev(packed), dev(scales), dev(zp), k, g))
+    # outputs reach +-500 here and some cancel to nearly zero, where abs 1e-4 is below what any f32
+    # summation order can promise: measure both results against float64 in units of the terms
+    # that were added up, and ask the kernels to be as accurate as the reference's own f32 loop
+    wd = oracle.w4_dequant(packed, scales, zp, k, g)
+    exact = x.astype(np.float64) @ wd
+    terms = np.abs(x).astype(np.float64) @ np.abs(wd)
+    err_ref = (np.abs(want - exact) / terms).max()
+    err_got = (np.abs(got - exact) / terms).max()
+    assert err_ref < 2e-6 and err_got < max(2e-7, 1.5 * err_ref), (err_got, err_ref)
+    np.testing.assert_allclose(got, want, rtol=1e-3, atol=1e-3)
+
+
 def test_reference_order_kernel_is_bit_exact(ops):
     # n % 4 != 0 routes to the one-thread-per-column kernel, which performs the oracle's
     # operations in the oracle's order: equality, not tolerance.
