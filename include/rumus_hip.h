@@ -239,11 +239,18 @@ int rumus_hip_qmatmul_int4_decode(const float* x, const uint32_t* packed_t,
                                   uint32_t group_size, uint32_t num_groups,
                                   rumus_hip_stream_t stream);
 
+/* Rows of x up to which the decode entry points are the faster way to run a
+ * [padded_k, n] weight (between 1 and 8, from measurements; beyond it
+ * rumus_hip_qmatmul_int4 takes the matrix cores).  The dispatch inside
+ * rumus_hip_qmatmul_int4 uses the same number.  No counterpart in the reference. */
+uint32_t rumus_hip_qmatmul_int4_decode_max_rows(uint32_t padded_k, uint32_t n);
+
 /* EXTENSION: the decode layout and its matmul for AWQ storage (u4 zero-points,
  * rumus_hip_w4_quantize_pack_awq): packed_t and scales_t as in
  * rumus_hip_w4_decode_layout; qzeros_t[(c*num_groups + g)*2 + h] =
  * qzeros[g*(n/8) + 2*c + h], the two zero-point words of tile c's 16 columns.
- * Same bits as rumus_hip_qmatmul_int4_zp4 on the row-major arrays for m <= 5.
+ * Same bits as rumus_hip_qmatmul_int4_zp4 on the row-major arrays while m is
+ * within rumus_hip_qmatmul_int4_decode_max_rows.
  * EINVAL as for the f32 zero-point forms.  No counterpart in the reference. */
 int rumus_hip_w4_decode_layout_zp4(const uint32_t* packed, const float* scales,
                                    const uint32_t* qzeros, uint32_t padded_k, uint32_t n,

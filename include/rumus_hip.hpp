@@ -184,10 +184,10 @@ struct QLinear {
     }
 
     // y[m, out] = x[m, in] . dequant(W) + bias; x and y are device pointers.
-    // Up to 5 rows take the decode kernel on the tile-major copy (same result bit for bit).
+    // Few rows take the decode kernel on the tile-major copy (same result bit for bit).
     void forward(const float* x, uint32_t m, float* y, hipStream_t stream = nullptr) const {
         const int32_t* perm = weight.perm.size() ? weight.perm.data() : nullptr;
-        if (m <= 5 && weight.has_decode_layout()) {
+        if (weight.has_decode_layout() && m <= rumus_hip_qmatmul_int4_decode_max_rows(weight.padded_k, weight.n)) {
             check(rumus_hip_qmatmul_int4_decode(x, weight.packed_t.data(), weight.scales_t.data(), weight.zp_t.data(),
                                                 bias.size() ? bias.data() : nullptr, perm, y, m, weight.k,
                                                 weight.n, weight.padded_k, weight.group_size, weight.num_groups,

@@ -59,6 +59,7 @@ PROTOTYPES = {
     "rumus_hip_w4_qzeros_unpack": (_i32, [_vp, _u32, _u32, _vp, _vp]),
     "rumus_hip_w4_decode_layout": (_i32, [_vp, _vp, _vp, _u32, _u32, _u32, _vp, _vp, _vp, _vp]),
     "rumus_hip_qmatmul_int4_decode": (_i32, [_vp] * 7 + [_u32] * 6 + [_vp]),
+    "rumus_hip_qmatmul_int4_decode_max_rows": (_u32, [_u32, _u32]),
     "rumus_hip_w4_decode_layout_zp4": (_i32, [_vp, _vp, _vp, _u32, _u32, _u32, _vp, _vp, _vp, _vp]),
     "rumus_hip_qmatmul_int4_decode_zp4": (_i32, [_vp] * 7 + [_u32] * 6 + [_vp]),
     "rumus_hip_qmatmul_int4_decode_swiglu": (_i32, [_vp] * 6 + [_u32] * 6 + [_vp]),

@@ -65,6 +65,7 @@ int w4_launch_gemv_dot8(const W4Args& a, hipStream_t s);
 // f16 MFMA kernel for larger m (needs group_size 32, 64 or a multiple of 128,
 // n % 4 == 0, 16-byte aligned buffers, no g_idx).
 bool w4_gemm_supported(const W4Args& a);
+uint32_t w4_decode_max_rows(uint32_t padded_k, uint32_t n);   // w4_gemv.hip
 int w4_launch_gemm(const W4Args& a, hipStream_t s);
 
 }  // namespace rumus

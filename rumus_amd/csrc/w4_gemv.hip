@@ -298,12 +298,22 @@ static int validate(const W4Args& a, const char* who) {
     return RUMUS_HIP_OK;
 }
 
+// Rows of x up to which the decode kernels beat the matrix-core kernel.  Measured on 4096 x 4096
+// and 4096 x 11008 (g128): a decode launch costs 2.5 + 0.82 W us for one row and 0.45 W us per
+// further row, W = millions of packed words; the matrix-core kernel 8.8 + 0.94 W us for any m up
+// to 32.  The crossing is at 7 rows for 4096 x 4096 and 3 rows for 4096 x 11008; the decode
+// kernels take at most 8.
+uint32_t w4_decode_max_rows(uint32_t padded_k, uint32_t n) {
+    const double mw = (double)(padded_k / 8) * n * 1e-6;
+    if (mw <= 0.0) return 8;
+    const double rows = 1.27 + 14.0 / mw;
+    return rows >= 8.0 ? 8u : rows < 1.0 ? 1u : (uint32_t)rows;
+}
+
 static int dispatch(const W4Args& a, hipStream_t s) {
     if (a.m == 0 || a.n == 0) return RUMUS_HIP_OK;
     RUMUS_REQUIRE(a.k > 0, "qmatmul_int4: k must be > 0");
-    // The decode kernels cost a fixed amount per row of x; from 6 rows on the matrix-core
-    // kernel (whose cost barely depends on m up to 32) is the faster one.
-    const bool few_rows = a.m <= 5 || !w4_gemm_supported(a);
+    const bool few_rows = a.m <= w4_decode_max_rows(a.padded_k, a.n) || !w4_gemm_supported(a);
     if (few_rows && w4_gemv_dot8_supported(a)) return w4_launch_gemv_dot8(a, s);
     if (few_rows && w4_gemv_supported(a)) return w4_launch_gemv(a, s);
     if (w4_gemm_supported(a)) return w4_launch_gemm(a, s);
@@ -351,6 +361,10 @@ int rumus_hip_qmatmul_int4_decode(const float* x, const uint32_t* packed_t, cons
     RUMUS_REQUIRE(w4_gemv_dot8_supported(a),
                   "qmatmul_int4_decode: needs group_size %% 32 == 0 and 16-byte aligned buffers");
     return w4_launch_gemv_dot8(a, as_stream(stream));
+}
+
+uint32_t rumus_hip_qmatmul_int4_decode_max_rows(uint32_t padded_k, uint32_t n) {
+    return w4_decode_max_rows(padded_k, n);
 }
 
 int rumus_hip_qmatmul_int4_decode_zp4(const float* x, const uint32_t* packed_t, const float* scales_t,

@@ -57,6 +57,9 @@ class QuantizedTensor:
         self.decode = None
         if n % 16 == 0 and group_size % 32 == 0 and packed.is_cuda:
             self.decode = ops.w4_decode_layout(packed, scales, zp, group_size)
+        # batches up to this many rows take the decode kernel (its cost grows with the rows, the
+        # matrix-core kernel's hardly does; the library knows where they cross for this shape)
+        self.decode_rows = ops.qmatmul_int4_decode_max_rows(padded_k, n) if self.decode is not None else 0
 
     @classmethod
     def from_f32(cls, data: torch.Tensor, k: int, n: int, group_size: int,
@@ -87,9 +90,6 @@ class QuantizedTensor:
         return cls(k, packed.shape[1], padded_k, group_size, groups, packed, scales, zp, perm)
 
 
-# batches up to this many rows take the decode kernel (its cost grows with the rows; from 6 on
-# the matrix-core kernel is faster)
-DECODE_ROWS = 5
 
 
 class QLinear:
@@ -109,7 +109,7 @@ class QLinear:
     def forward(self, x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``y = x @ dequant(W) + bias`` in one launch (the reference runs a second add_bias pass)."""
         w = self.weight
-        if w.decode is not None and x.shape[0] <= DECODE_ROWS:
+        if x.shape[0] <= w.decode_rows:
             return ops.qmatmul_int4_decode(x, *w.decode, w.k, w.group_size, bias=self.bias, perm=w.perm, out=out)
         return ops.qmatmul_int4_perm(x, w.packed_tensor, w.scales_tensor, w.zp_tensor, w.k,
                                      w.group_size, bias=self.bias, perm=w.perm, out=out)
@@ -270,7 +270,7 @@ class DecoderBlockW4:
         x1, h2 = ops.add_rmsnorm(x2, o, self.norm2, self.eps, sum_out=o, out=hn)
         gu = self.gate_up(h2)
         dw = self.proj["down"]
-        if b * n <= DECODE_ROWS and dw.weight.decode is not None and dw.weight.perm is None:
+        if b * n <= dw.weight.decode_rows and dw.weight.perm is None:
             # decode rows: the SwiGLU happens while the down projection reads its input
             down = ops.qmatmul_int4_decode_swiglu(gu, *dw.weight.decode, dw.weight.k, dw.weight.group_size,
                                                   bias=dw.bias)

@@ -187,6 +187,11 @@ def qmatmul_int4_decode(x, packed_t, scales_t, zp_t, k, group_size, bias=None, p
     return _w4_call("rumus_hip_qmatmul_int4_decode", x, packed_t, scales_t, zp_t, bias, perm, k, group_size, out)
 
 
+def qmatmul_int4_decode_max_rows(padded_k: int, n: int) -> int:
+    """Rows up to which the decode entry points beat the matrix-core kernel for this weight."""
+    return int(_lib.lib().rumus_hip_qmatmul_int4_decode_max_rows(padded_k, n))
+
+
 def w4_decode_layout_zp4(packed, scales, qzeros, group_size):
     """Tile-major copies for AWQ storage: packed, scales as in w4_decode_layout, u4 zero-points with
     the two words of a tile side by side."""

@@ -52,6 +52,7 @@ extern "C" {
                                          zero_points_t: *const f32, bias: *const f32, perm: *const i32,
                                          y: *mut f32, m: u32, k: u32, n: u32, padded_k: u32, group_size: u32,
                                          num_groups: u32, s: Stream) -> c_int;
+    pub fn rumus_hip_qmatmul_int4_decode_max_rows(padded_k: u32, n: u32) -> u32;
     pub fn rumus_hip_w4_decode_layout_zp4(packed: *const u32, scales: *const f32, qzeros: *const u32, padded_k: u32,
                                           n: u32, group_size: u32, packed_t: *mut u32, scales_t: *mut f32,
                                           qzeros_t: *mut u32, s: Stream) -> c_int;

@@ -469,7 +469,7 @@ def test_decode_layout_is_bit_identical(ops, m, k, n, g):
     np.testing.assert_array_equal(host(st).reshape(-1), want_st)
     got = host(ops.qmatmul_int4_decode(dev(x), pt, st, zt, k, g, bias=dev(b)))
     assert_close(got, oracle.qmatmul_int4(x, packed, scales, zp, k, g, bias=b, threads=8))
-    if m <= 5:   # the reference-layout entry point runs the same kernel on these shapes
+    if m <= ops.qmatmul_int4_decode_max_rows(packed.shape[0] * 8, n):   # the row-major entry point runs the same kernel then
         np.testing.assert_array_equal(got, host(ops.qmatmul_int4(dev(x), *d, k, g, bias=dev(b))))
 
 
@@ -489,7 +489,7 @@ def test_decode_layout_u4_zero_points(ops, m, k, n, g):
     got = host(ops.qmatmul_int4_decode_zp4(dev(x), pt, st, qt, k, g, bias=dev(b)))
     zp = oracle.w4_qzeros_unpack(qzeros, n)
     assert_close(got, oracle.qmatmul_int4(x, packed, scales, zp, k, g, bias=b, threads=8))
-    if m <= 5:   # the row-major entry point runs the same kernel arithmetic on these shapes
+    if m <= ops.qmatmul_int4_decode_max_rows(packed.shape[0] * 8, n):   # the row-major entry point runs the same kernel arithmetic then
         np.testing.assert_array_equal(got, host(ops.qmatmul_int4_zp4(dev(x), *d, k, g, bias=dev(b))))
     # act-order on top
     if k % g == 0:
