@@ -10,31 +10,59 @@
 
 namespace rumus {
 
-// Thread = one column of one group; workgroup = 256 adjacent columns, so every
-// row read and every word store is one contiguous 1 KiB segment per wave
-// quad.  The group is read twice (min/max, then quantize); the second read is
-// served by L2.
-template <bool SYM>
+// Thread = one column of one group; workgroup = 256 adjacent columns, so every row read and
+// every word store is one contiguous segment per wave.  GS = 32, 64 or 128: the group size is a
+// compile-time constant and the group is read once, all loads issued before the first use, and
+// kept in registers for the two passes (min/max, then quantize).  GS = 0: any group size, the
+// group is read twice (the second read is served by L2).  The arithmetic is the same, in the
+// same order, either way.
+template <int GS>
+struct GroupReader {
+    const float* w;
+    uint32_t k, n, col, r0;
+    float cache[GS > 0 ? GS : 1];
+    __device__ __forceinline__ GroupReader(const float* w_, uint32_t k_, uint32_t n_, uint32_t col_, uint32_t r0_)
+        : w(w_), k(k_), n(n_), col(col_), r0(r0_) {
+        if constexpr (GS > 0) {
+#pragma unroll
+            for (int i = 0; i < GS; i++) {
+                const uint32_t r = r0 + i;
+                const float v = w[(uint64_t)min(r, k - 1) * n + col];
+                cache[i] = r < k ? v : 0.0f;                 // rows >= k: the zero padding of quant.rs:50-56
+            }
+        }
+    }
+    __device__ __forceinline__ float operator[](uint32_t i) const {
+        if constexpr (GS > 0) return cache[i];
+        const uint32_t r = r0 + i;
+        return r < k ? w[(uint64_t)r * n + col] : 0.0f;
+    }
+};
+
+template <bool SYM, int GS>
 __global__ __launch_bounds__(256) void w4_quantize_pack_kernel(
-    const float* __restrict__ w, uint32_t k, uint32_t n, uint32_t gs,
+    const float* __restrict__ w, uint32_t k, uint32_t n, uint32_t gs_arg,
     uint32_t* __restrict__ packed, float* __restrict__ scales, float* __restrict__ zps) {
     const uint32_t col = blockIdx.x * 256 + threadIdx.x;
     const uint32_t g = blockIdx.y;
     if (col >= n) return;
+    const uint32_t gs = GS > 0 ? GS : gs_arg;
     const uint32_t r0 = g * gs;
+    const GroupReader<GS> group(w, k, n, col, r0);
 
     float scale, zp;
     if (SYM) {
         float amax = 0.0f;
-        for (uint32_t r = r0; r < r0 + gs && r < k; r++)
-            amax = fmaxf(amax, fabsf(w[(uint64_t)r * n + col]));
+#pragma unroll
+        for (uint32_t i = 0; i < gs; i++) amax = fmaxf(amax, fabsf(group[i]));
         scale = amax > 0.0f ? __fdiv_rn(amax, 7.0f) : 1.0f;
         zp = 8.0f;
     } else {
-        // quant.rs:66-74; rows >= k are the zero padding of quant.rs:50-56
+        // quant.rs:66-74
         float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
-        for (uint32_t r = r0; r < r0 + gs; r++) {
-            float v = r < k ? w[(uint64_t)r * n + col] : 0.0f;
+#pragma unroll
+        for (uint32_t i = 0; i < gs; i++) {
+            const float v = group[i];
             if (v < mn) mn = v;
             if (v > mx) mx = v;
         }
@@ -46,12 +74,12 @@ __global__ __launch_bounds__(256) void w4_quantize_pack_kernel(
     scales[(uint64_t)g * n + col] = scale;
     if (zps) zps[(uint64_t)g * n + col] = zp;
 
+#pragma unroll
     for (uint32_t wr = 0; wr < gs / 8; wr++) {
         uint32_t word = 0;
 #pragma unroll
         for (uint32_t j = 0; j < 8; j++) {
-            const uint32_t r = r0 + wr * 8 + j;
-            const float v = r < k ? w[(uint64_t)r * n + col] : 0.0f;
+            const float v = group[wr * 8 + j];
             float t;
             if (SYM) {
                 t = __fadd_rn(roundf(__fdiv_rn(v, scale)), 8.0f);
@@ -70,16 +98,20 @@ __global__ __launch_bounds__(256) void w4_quantize_pack_kernel(
 //   q = clamp(rint(w / scale) + z, 0, 15)        (rint: half to even)
 // Same thread layout as above; the eight lanes that share a zero-point word combine their
 // nibbles with lane exchanges (n % 8 == 0, so the eight are all inside or all outside).
+template <int GS>
 __global__ __launch_bounds__(256) void w4_quantize_pack_awq_kernel(
-    const float* __restrict__ w, uint32_t k, uint32_t n, uint32_t gs,
+    const float* __restrict__ w, uint32_t k, uint32_t n, uint32_t gs_arg,
     uint32_t* __restrict__ packed, float* __restrict__ scales, uint32_t* __restrict__ qzeros) {
     const uint32_t col = blockIdx.x * 256 + threadIdx.x;
     const uint32_t g = blockIdx.y;
     if (col >= n) return;
+    const uint32_t gs = GS > 0 ? GS : gs_arg;
     const uint32_t r0 = g * gs;
+    const GroupReader<GS> group(w, k, n, col, r0);
     float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
-    for (uint32_t r = r0; r < r0 + gs; r++) {
-        const float v = r < k ? w[(uint64_t)r * n + col] : 0.0f;
+#pragma unroll
+    for (uint32_t i = 0; i < gs; i++) {
+        const float v = group[i];
         if (v < mn) mn = v;
         if (v > mx) mx = v;
     }
@@ -93,12 +125,12 @@ __global__ __launch_bounds__(256) void w4_quantize_pack_awq_kernel(
     zw |= __shfl_xor(zw, 2);
     zw |= __shfl_xor(zw, 4);
     if ((col & 7) == 0) qzeros[(uint64_t)g * (n / 8) + col / 8] = zw;
+#pragma unroll
     for (uint32_t wr = 0; wr < gs / 8; wr++) {
         uint32_t word = 0;
 #pragma unroll
         for (uint32_t j = 0; j < 8; j++) {
-            const uint32_t r = r0 + wr * 8 + j;
-            const float v = r < k ? w[(uint64_t)r * n + col] : 0.0f;
+            const float v = group[wr * 8 + j];
             float t = __fadd_rn(rintf(__fdiv_rn(v, scale)), zf);
             t = fminf(fmaxf(t, 0.0f), 15.0f);
             word |= (uint32_t)t << (4 * j);
@@ -175,8 +207,13 @@ static int quantize_pack(const float* w, uint32_t k, uint32_t n, uint32_t gs, ui
     RUMUS_REQUIRE(w && packed && scales && (SYM || zps), "w4_quantize_pack: null buffer");
     if (n == 0 || k == 0) return RUMUS_HIP_OK;
     const uint32_t groups = ceil_div(k, gs);
-    hipLaunchKernelGGL((w4_quantize_pack_kernel<SYM>), dim3(ceil_div(n, 256), groups), dim3(256), 0,
-                       s, w, k, n, gs, packed, scales, zps);
+    const dim3 grid(ceil_div(n, 256), groups);
+    switch (gs) {                                        // common sizes: one pass over the weights
+        case 32: hipLaunchKernelGGL((w4_quantize_pack_kernel<SYM, 32>), grid, dim3(256), 0, s, w, k, n, gs, packed, scales, zps); break;
+        case 64: hipLaunchKernelGGL((w4_quantize_pack_kernel<SYM, 64>), grid, dim3(256), 0, s, w, k, n, gs, packed, scales, zps); break;
+        case 128: hipLaunchKernelGGL((w4_quantize_pack_kernel<SYM, 128>), grid, dim3(256), 0, s, w, k, n, gs, packed, scales, zps); break;
+        default: hipLaunchKernelGGL((w4_quantize_pack_kernel<SYM, 0>), grid, dim3(256), 0, s, w, k, n, gs, packed, scales, zps);
+    }
     return check_launch("w4_quantize_pack_kernel");
 }
 
@@ -271,8 +308,14 @@ int rumus_hip_w4_quantize_pack_awq(const float* w, uint32_t k, uint32_t n, uint3
     RUMUS_REQUIRE(w && packed && scales && qzeros, "w4_quantize_pack_awq: null buffer");
     if (k == 0 || n == 0) return RUMUS_HIP_OK;
     const uint32_t groups = ceil_div(k, group_size);
-    hipLaunchKernelGGL(w4_quantize_pack_awq_kernel, dim3(ceil_div(n, 256), groups), dim3(256), 0,
-                       as_stream(stream), w, k, n, group_size, packed, scales, qzeros);
+    const dim3 grid(ceil_div(n, 256), groups);
+    hipStream_t s = as_stream(stream);
+    switch (group_size) {
+        case 32: hipLaunchKernelGGL(w4_quantize_pack_awq_kernel<32>, grid, dim3(256), 0, s, w, k, n, group_size, packed, scales, qzeros); break;
+        case 64: hipLaunchKernelGGL(w4_quantize_pack_awq_kernel<64>, grid, dim3(256), 0, s, w, k, n, group_size, packed, scales, qzeros); break;
+        case 128: hipLaunchKernelGGL(w4_quantize_pack_awq_kernel<128>, grid, dim3(256), 0, s, w, k, n, group_size, packed, scales, qzeros); break;
+        default: hipLaunchKernelGGL(w4_quantize_pack_awq_kernel<0>, grid, dim3(256), 0, s, w, k, n, group_size, packed, scales, qzeros);
+    }
     return check_launch("w4_quantize_pack_awq_kernel");
 }
 
