@@ -183,6 +183,108 @@ __global__ __launch_bounds__(256) void matmul_q8_tiled_kernel(
     }
 }
 
+// block_size % 16 == 0, up to 8 rows per launch: bound by reading the weights once per launch
+// (more rows run as several launches, still well ahead of the LDS-tiled kernel below).  The rows of x are
+// staged in LDS (zero-padded to a multiple of 16 k).  A workgroup owns 32 columns, each of its
+// eight waves four of them; lane i takes the 16 bytes k = 16 i .. 16 i + 15 of each of the four
+// (one 128-bit load per column, all four in flight together; a run of 16 never straddles a block)
+// and multiplies them with one read of x.  The 64 partial sums of a column meet in a butterfly.
+// A column's bytes are contiguous in the Q8 layout, so a wave reads 1 KB runs.
+// Arithmetic: sum_k (a * f32(q)) per run of 16, times the block scale once per run
+// (matmul_q8.wgsl:77-80 multiplies by the scale per element).
+// run_magic = ceil(2^32 / runs_per_block): run / runs_per_block as a multiply (exact below 2^16);
+// 0 stands for one run per block.
+struct __attribute__((packed, aligned(4))) Q8Words4 { uint32_t x, y, z, w; };
+
+template <int M>
+__global__ __launch_bounds__(512) void matmul_q8_rows_kernel(
+    const float* __restrict__ a, const uint32_t* __restrict__ b, float* __restrict__ c, uint32_t k,
+    uint32_t n, uint32_t stride, uint32_t blocks_per_col, uint32_t kpad, uint32_t runs_per_block,
+    uint32_t run_magic) {
+    constexpr int CW = 4;                                     // columns per wave
+    // x in LDS as [row][quarter of a run][run][4]: the lanes of a wave, one run each, then read
+    // consecutive 16-byte pieces (run-major order would put them 64 bytes apart, 16 to a bank)
+    extern __shared__ float xs[];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t nruns = kpad / 16;
+    for (uint32_t r = 0; r < M; r++)
+        for (uint32_t kk = tid; kk < kpad; kk += 512)
+            xs[((r * 4 + (kk % 16) / 4) * nruns + kk / 16) * 4 + kk % 4] = kk < k ? a[(uint64_t)r * k + kk] : 0.0f;
+    __syncthreads();
+    const uint32_t col0 = blockIdx.x * 32 + wave * CW;
+    const uint32_t* colbase[CW];
+#pragma unroll
+    for (int cc = 0; cc < CW; cc++)
+        colbase[cc] = b + (uint64_t)min(col0 + cc, n - 1) * blocks_per_col * stride;   // past n: re-reads the last column
+    float acc[CW][M];
+#pragma unroll
+    for (int cc = 0; cc < CW; cc++)
+#pragma unroll
+        for (int r = 0; r < M; r++) acc[cc][r] = 0.0f;
+    for (uint32_t run = lane; run < nruns; run += 64) {
+        const uint32_t blk = run_magic ? __umulhi(run, run_magic) : run;   // magic 0: one run per block
+        const uint32_t in_blk = run - blk * runs_per_block;
+        const uint32_t off = blk * stride;                   // header word of the block; data follows
+        Q8Words4 w4[CW];
+        uint32_t hdr[CW];
+#pragma unroll
+        for (int cc = 0; cc < CW; cc++) {
+            hdr[cc] = colbase[cc][off];
+            w4[cc] = *reinterpret_cast<const Q8Words4*>(colbase[cc] + off + 1 + in_blk * 4);
+        }
+        float part[CW][M];
+#pragma unroll
+        for (int cc = 0; cc < CW; cc++)
+#pragma unroll
+            for (int r = 0; r < M; r++) part[cc][r] = 0.0f;
+#pragma unroll
+        for (int wi = 0; wi < 4; wi++) {
+            float4 xv[M];
+#pragma unroll
+            for (int r = 0; r < M; r++) xv[r] = *reinterpret_cast<const float4*>(xs + ((r * 4 + wi) * nruns + run) * 4);
+#pragma unroll
+            for (int cc = 0; cc < CW; cc++) {
+                const uint32_t word = wi == 0 ? w4[cc].x : wi == 1 ? w4[cc].y : wi == 2 ? w4[cc].z : w4[cc].w;
+                float q[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) q[j] = (float)(int)(int8_t)((word >> (8 * j)) & 0xFFu);
+#pragma unroll
+                for (int r = 0; r < M; r++) {
+                    part[cc][r] = fmaf(xv[r].x, q[0], part[cc][r]);
+                    part[cc][r] = fmaf(xv[r].y, q[1], part[cc][r]);
+                    part[cc][r] = fmaf(xv[r].z, q[2], part[cc][r]);
+                    part[cc][r] = fmaf(xv[r].w, q[3], part[cc][r]);
+                }
+            }
+        }
+#pragma unroll
+        for (int cc = 0; cc < CW; cc++) {
+            const float sc = header_scale(hdr[cc]);
+#pragma unroll
+            for (int r = 0; r < M; r++) acc[cc][r] = fmaf(part[cc][r], sc, acc[cc][r]);
+        }
+    }
+#pragma unroll
+    for (int cc = 0; cc < CW; cc++)
+#pragma unroll
+        for (int r = 0; r < M; r++) {
+            float v = acc[cc][r];
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+            if (lane == 0 && col0 + cc < n) c[(uint64_t)r * n + col0 + cc] = v;
+        }
+}
+
+template <int M>
+static int launch_q8_rows(const float* a, const uint32_t* b, float* c, uint32_t k, uint32_t n, uint32_t bs,
+                          uint32_t stride, uint32_t blocks_per_col, uint32_t kpad, hipStream_t s) {
+    const uint32_t runs_per_block = bs / 16;
+    const uint32_t run_magic = runs_per_block == 1 ? 0u : (uint32_t)((0x100000000ull + runs_per_block - 1) / runs_per_block);
+    hipLaunchKernelGGL(matmul_q8_rows_kernel<M>, dim3(ceil_div(n, 32)), dim3(512), (size_t)M * kpad * sizeof(float), s,
+                       a, b, c, k, n, stride, blocks_per_col, kpad, runs_per_block, run_magic);
+    return check_launch("matmul_q8_rows_kernel");
+}
+
 // Any block_size % 4 == 0: one thread per output, the reference's own loop.
 __global__ __launch_bounds__(256) void matmul_q8_naive_kernel(
     const float* __restrict__ a, const uint32_t* __restrict__ b, float* __restrict__ c,
@@ -282,6 +384,30 @@ int rumus_hip_matmul_q8(const float* a, const uint32_t* b, float* c, uint32_t m,
     RUMUS_REQUIRE(k > 0, "matmul_q8: k must be > 0");
     uint32_t blocks_per_col = ceil_div(k, block_size);
     uint32_t stride = (4 + block_size + 3) / 4;
+    const uint32_t kpad = (k + 15) & ~15u;
+    if (block_size % 16 == 0 && kpad <= 16384) {
+        // rows in groups whose x fits 64 KB of LDS: 4 rows at k = 4096, 1 at k = 11008, all 8 up to k = 2048
+        const uint32_t group = min(8u, 16384u / kpad);
+        hipStream_t s = as_stream(stream);
+        for (uint32_t r0 = 0; r0 < m; r0 += group) {
+            const uint32_t rows = min(group, m - r0);
+            const float* ar = a + (uint64_t)r0 * k;
+            float* cr = c + (uint64_t)r0 * n;
+            int rc;
+            switch (rows) {
+                case 1: rc = launch_q8_rows<1>(ar, b, cr, k, n, block_size, stride, blocks_per_col, kpad, s); break;
+                case 2: rc = launch_q8_rows<2>(ar, b, cr, k, n, block_size, stride, blocks_per_col, kpad, s); break;
+                case 3: rc = launch_q8_rows<3>(ar, b, cr, k, n, block_size, stride, blocks_per_col, kpad, s); break;
+                case 4: rc = launch_q8_rows<4>(ar, b, cr, k, n, block_size, stride, blocks_per_col, kpad, s); break;
+                case 5: rc = launch_q8_rows<5>(ar, b, cr, k, n, block_size, stride, blocks_per_col, kpad, s); break;
+                case 6: rc = launch_q8_rows<6>(ar, b, cr, k, n, block_size, stride, blocks_per_col, kpad, s); break;
+                case 7: rc = launch_q8_rows<7>(ar, b, cr, k, n, block_size, stride, blocks_per_col, kpad, s); break;
+                default: rc = launch_q8_rows<8>(ar, b, cr, k, n, block_size, stride, blocks_per_col, kpad, s); break;
+            }
+            if (rc) return rc;
+        }
+        return RUMUS_HIP_OK;
+    }
     if (block_size % 16 == 0) {
         dim3 grid(ceil_div(n, kQ8Tile), ceil_div(m, kQ8Tile));
         hipLaunchKernelGGL(matmul_q8_tiled_kernel, grid, dim3(256), 0, as_stream(stream), a, b, c,

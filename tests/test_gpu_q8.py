@@ -57,7 +57,12 @@ def test_q8_rejects_bad_block_size(ops):
 
 
 @pytest.mark.parametrize("m,k,n,bs", [(32, 512, 512, 512), (4, 64, 10, 64), (3, 96, 7, 32),
-                                      (2, 40, 5, 8), (70, 256, 130, 128), (5, 100, 9, 20)])
+                                      (2, 40, 5, 8), (70, 256, 130, 128), (5, 100, 9, 20),
+                                      (1, 4096, 1100, 4096),   # few-rows kernel, per-channel blocks
+                                      (8, 4096, 70, 128),      # two groups of four rows
+                                      (3, 1008, 64, 16),       # smallest block the few-rows kernel takes
+                                      (2, 11008, 40, 64),      # one row per launch
+                                      (7, 2048, 33, 2048)])
 def test_matmul_q8_vs_oracle(ops, m, k, n, bs):
     say(f"matmul_q8 m={m} k={k} n={n} bs={bs}")
     from rumus_amd import nn
