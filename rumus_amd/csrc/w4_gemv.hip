@@ -234,53 +234,61 @@ int w4_launch_gemv(const W4Args& a, hipStream_t s) {
 
 // ---------------------------------------------------------------------------
 // Transpose kernel (grad_x): out[m,k] = sum_n a[m,n] * dequant(W)[k,n]
-// (qmatmul_int4_transpose.wgsl:37-74).  A workgroup owns one word row (8
+// (qmatmul_int4_transpose.wgsl:37-74).  A workgroup owns KR word rows (8 KR
 // output columns k) and MR rows of a; threads stride over n, so packed words,
-// scales and zero-points are read once per workgroup row block, coalesced.
+// scales and zero-points are read coalesced, once per block of MR rows, and
+// every value of a once per 8 KR outputs.
 // ---------------------------------------------------------------------------
-template <int MR>
+template <int MR, int KR>
 __global__ __launch_bounds__(256) void w4_transpose_kernel(
     const float* __restrict__ a, const uint32_t* __restrict__ packed,
     const float* __restrict__ scales, const float* __restrict__ zp, float* __restrict__ out,
-    uint32_t m, uint32_t k, uint32_t n, uint32_t gs) {
-    __shared__ float red[4][MR][8];
-    const uint32_t kr = blockIdx.x, row0 = blockIdx.y * MR, tid = threadIdx.x;
-    const uint32_t g = (kr * 8) / gs;
-    float acc[MR][8];
+    uint32_t m, uint32_t k, uint32_t n, uint32_t gs, uint32_t word_rows) {
+    __shared__ float red[4][KR][MR][8];
+    const uint32_t kr0 = blockIdx.x * KR, row0 = blockIdx.y * MR, tid = threadIdx.x;
+    float acc[KR][MR][8];
 #pragma unroll
-    for (int r = 0; r < MR; r++)
+    for (int q = 0; q < KR; q++)
 #pragma unroll
-        for (int j = 0; j < 8; j++) acc[r][j] = 0.0f;
+        for (int r = 0; r < MR; r++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) acc[q][r][j] = 0.0f;
+#pragma unroll(MR * KR == 1 ? 4 : 1)
     for (uint32_t c = tid; c < n; c += 256) {
-        const uint32_t word = packed[(uint64_t)kr * n + c];
-        const float sc = scales[(uint64_t)g * n + c], z = zp[(uint64_t)g * n + c];
-        float wv[8];
+        float av[MR];
 #pragma unroll
-        for (int j = 0; j < 8; j++) wv[j] = ((float)((word >> (4 * j)) & 0xFu) - z) * sc;
+        for (int r = 0; r < MR; r++) av[r] = row0 + r < m ? a[(uint64_t)(row0 + r) * n + c] : 0.0f;
 #pragma unroll
-        for (int r = 0; r < MR; r++) {
-            if (row0 + r < m) {
-                const float av = a[(uint64_t)(row0 + r) * n + c];
+        for (int q = 0; q < KR; q++) {
+            const uint32_t kr = min(kr0 + q, word_rows - 1);        // past the end: recomputes the last row, not stored
+            const uint32_t g = (kr * 8) / gs;
+            const uint32_t word = packed[(uint64_t)kr * n + c];
+            const float sc = scales[(uint64_t)g * n + c], z = zp[(uint64_t)g * n + c];
 #pragma unroll
-                for (int j = 0; j < 8; j++) acc[r][j] = fmaf(av, wv[j], acc[r][j]);
+            for (int j = 0; j < 8; j++) {
+                const float wv = ((float)((word >> (4 * j)) & 0xFu) - z) * sc;
+#pragma unroll
+                for (int r = 0; r < MR; r++) acc[q][r][j] = fmaf(av[r], wv, acc[q][r][j]);
             }
         }
     }
 #pragma unroll
-    for (int r = 0; r < MR; r++)
+    for (int q = 0; q < KR; q++)
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            float v = acc[r][j];
+        for (int r = 0; r < MR; r++)
 #pragma unroll
-            for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
-            if ((tid & 63) == 0) red[tid >> 6][r][j] = v;
-        }
+            for (int j = 0; j < 8; j++) {
+                float v = acc[q][r][j];
+#pragma unroll
+                for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+                if ((tid & 63) == 0) red[tid >> 6][q][r][j] = v;
+            }
     __syncthreads();
-    if (tid < MR * 8) {
-        const uint32_t r = tid / 8, j = tid % 8;
-        const uint32_t kk = kr * 8 + j;
+    for (uint32_t e = tid; e < KR * MR * 8; e += 256) {
+        const uint32_t q = e / (MR * 8), r = (e / 8) % MR, j = e % 8;
+        const uint32_t kk = (kr0 + q) * 8 + j;
         if (row0 + r < m && kk < k)
-            out[(uint64_t)(row0 + r) * k + kk] = (red[0][r][j] + red[1][r][j]) + (red[2][r][j] + red[3][r][j]);
+            out[(uint64_t)(row0 + r) * k + kk] = (red[0][q][r][j] + red[1][q][r][j]) + (red[2][q][r][j] + red[3][q][r][j]);
     }
 }
 
@@ -417,9 +425,17 @@ int rumus_hip_qmatmul_int4_t(const float* a, const uint32_t* packed, const float
     W4Args v{a, packed, scales, zero_points, nullptr, nullptr, nullptr, out, m, k, n, padded_k, group_size, num_groups};
     if (int rc = validate(v, "qmatmul_int4_t")) return rc;
     if (m == 0 || k == 0) return RUMUS_HIP_OK;
-    constexpr int MR = 4;
-    hipLaunchKernelGGL((w4_transpose_kernel<MR>), dim3(ceil_div(k, 8), ceil_div(m, MR)), dim3(256), 0,
-                       as_stream(stream), a, packed, scales, zero_points, out, m, k, n, group_size);
+    // tile of a workgroup: 4 rows x 32 outputs from 3 rows on (each value of a is then read once per
+    // 32 outputs, each word once per 4 rows); single rows keep one word row per workgroup for
+    // the sake of parallelism
+    hipStream_t s = as_stream(stream);
+    const uint32_t word_rows = padded_k / 8;
+    if (m >= 3)
+        hipLaunchKernelGGL((w4_transpose_kernel<4, 4>), dim3(ceil_div(word_rows, 4), ceil_div(m, 4)), dim3(256), 0, s, a,
+                           packed, scales, zero_points, out, m, k, n, group_size, word_rows);
+    else
+        hipLaunchKernelGGL((w4_transpose_kernel<1, 1>), dim3(word_rows, m), dim3(256), 0, s, a, packed, scales,
+                           zero_points, out, m, k, n, group_size, word_rows);
     return check_launch("w4_transpose_kernel");
 }
 
