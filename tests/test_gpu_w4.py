@@ -90,12 +90,12 @@ SHAPES = [
     (64, 1024, 1024, 128, True),
     (100, 2048, 520, 256, False), # group spans two stages
     (20, 1000, 64, 64, True),     # K tail
-    (12, 256, 36, 8, False),      # group 8: not an MFMA case -> reference-order kernel
+    (12, 256, 36, 8, False),      # group 8: not an MFMA case -> the f32 decode kernel, a few rows per launch
     (7, 512, 128, 128, True),     # 6..8 rows already take the MFMA kernel
     (16, 4096, 4096, 128, True),  # few tiles: K split 16 ways over workgroups, ordered reduction
     (40, 1001, 64, 64, False),    # k % 4 != 0: activations are copied into padded rows first
     (100, 160, 520, 32, True),    # group 32: four settlements per stage, two row tiles
-    (24, 192, 48, 96, False),     # group 96 does not divide a stage -> reference-order kernel
+    (24, 192, 48, 96, False),     # group 96 does not divide a stage -> the f32 decode kernel in row chunks
     (1536, 256, 8192, 128, True), # more than 72 tiles: eight waves of 64 rows each
     (1500, 128, 8200, 64, False), # the same, group 64, ragged rows and columns
     (300, 160, 4100, 32, True),   # the same, group 32, K tail inside a stage
