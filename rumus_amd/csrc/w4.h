@@ -20,18 +20,19 @@ struct W4Args {
     uint32_t m, k, n, padded_k, group_size, num_groups;
     // AWQ storage (or null): integer zero-points, eight per word along n, column col in bits
     // 4*(col%8) of word g*(n/8) + col/8; `zp` is null then and n % 8 == 0
-    const uint32_t* zp4;
+    const uint32_t* zp4 = nullptr;
     // decode layout (w4_gemv_dot8 only): packed, scales and zp are tile-major copies, tile = 16
     // columns: packed_t[(c*word_rows + r)*16 + j] = packed[r*n + 16*c + j], likewise the metadata
-    bool tiled;
+    bool tiled = false;
     // w4_gemv_dot8 only: x holds rows of 2k floats, gate | up; the activations are silu(gate) * up
-    bool glu;    // w4_gemm_tile only (set by its launcher): activations split into hi and lo f16 planes in
+    bool glu = false;
+    // w4_gemm_tile only (set by its launcher): activations split into hi and lo f16 planes in
     // A-fragment order, block (row tile of 32, step of 16 k) = 64 lanes x 16 bytes, and the f32
     // sum of every row's 16 values per step; xsteps = steps allocated per row tile
-    const uint8_t* xh;
-    const uint8_t* xl;
-    const float* xs;
-    uint32_t xsteps;
+    const uint8_t* xh = nullptr;
+    const uint8_t* xl = nullptr;
+    const float* xs = nullptr;
+    uint32_t xsteps = 0;
 };
 
 // zero-points of 4 (col % 4 == 0) or 2 (col % 2 == 0) adjacent columns from the packed form
