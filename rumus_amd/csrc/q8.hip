@@ -285,6 +285,109 @@ static int launch_q8_rows(const float* a, const uint32_t* b, float* c, uint32_t 
     return check_launch("matmul_q8_rows_kernel");
 }
 
+// ---- batches on the matrix cores (one block per column, i.e. per-output-channel scales) ------
+// f32 activations cannot go into the int8 MFMA directly, but signed 7-bit digits can:
+//   x = (p0 + 128 p1 + 128^2 p2 + 128^3 p3) / f,  f a power of two with |x f| < 2^27 for the row,
+// so x . q = sum_p (p_p . q) 128^p / f, each p_p . q an exact i8 x i8 -> i32 product.  The four
+// digit planes are stacked as 4 m rows with row scales 128^p / f, the weights are copied out of
+// the block format once per call (dense int8 [n, k] + the header scales), the W8A8 kernel does
+// the rest and the four row blocks are added.  The activations keep 28 bits below the largest
+// magnitude of their row: with three planes (21 bits) a row with one entry 3e4 times the others
+// missed the tolerance tenfold, with four the error stays below that of an f32 accumulation.
+constexpr int kQ8Planes = 4;
+
+__global__ __launch_bounds__(256) void q8_split_rows_kernel(const float* __restrict__ a, int8_t* __restrict__ planes,
+                                                            float* __restrict__ sxp, uint32_t m, uint32_t k) {
+    __shared__ uint32_t red[4];
+    const uint32_t row = blockIdx.x, tid = threadIdx.x;
+    const float* ar = a + (uint64_t)row * k;
+    // largest magnitude as bits: orders like the floats, and a NaN sorts above infinity
+    uint32_t amax = 0;
+    for (uint32_t j = tid; j < k; j += 256) amax = max(amax, __float_as_uint(ar[j]) & 0x7FFFFFFFu);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) amax = max(amax, (uint32_t)__shfl_xor((int)amax, off));
+    if ((tid & 63) == 0) red[tid >> 6] = amax;
+    __syncthreads();
+    amax = max(max(red[0], red[1]), max(red[2], red[3]));
+    const uint32_t ebits = amax >> 23;                         // amax = a 2^(ebits-127), 1 <= a < 2
+    float f = __uint_as_float((280u - ebits) << 23);           // 2^(153 - ebits): |x f| < 2^27
+    uint32_t inv_bits = ebits - 26u;                           // 1 / f = 2^(ebits - 153), biased
+    if (ebits < 27) { f = 0.0f; inv_bits = 0; }                // zero or below 2^-100: contributes nothing
+    if (tid < kQ8Planes) {
+        float s = inv_bits ? __uint_as_float((inv_bits + 7u * tid) << 23) : 0.0f;
+        if (ebits == 255) s = __uint_as_float(0x7FC00000u);    // inf / nan in the row: poison it
+        sxp[tid * m + row] = s;
+    }
+    if (ebits == 255) f = 0.0f;
+    for (uint32_t j = 4 * tid; j < k; j += 1024) {             // k % 4 == 0
+        const float4 v = *reinterpret_cast<const float4*>(ar + j);
+        const float xv[4] = {v.x, v.y, v.z, v.w};
+        uint32_t word[kQ8Planes] = {};
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            int rest = (int)rintf(xv[e] * f);                  // exact: f is a power of two, |x f| < 2^27
+#pragma unroll
+            for (int p = 0; p < kQ8Planes; p++) {
+                const int digit = p + 1 < kQ8Planes ? ((rest + 64) & 127) - 64 : rest;   // the last one: -64 .. 64
+                rest = (rest - digit) >> 7;
+                word[p] |= (uint32_t)(digit & 0xFF) << (8 * e);
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < kQ8Planes; p++)
+            *reinterpret_cast<uint32_t*>(planes + ((uint64_t)p * m + row) * k + j) = word[p];
+    }
+}
+
+// Q8 buffer with one block per column -> dense int8 [n, k] and the n header scales
+__global__ __launch_bounds__(256) void q8_unpack_channels_kernel(const uint32_t* __restrict__ b,
+                                                                 uint32_t* __restrict__ wq, float* __restrict__ sw,
+                                                                 uint32_t kwords, uint32_t stride) {
+    const uint32_t w = blockIdx.x * 256 + threadIdx.x, col = blockIdx.y;
+    if (w >= kwords) return;
+    const uint32_t* bb = b + (uint64_t)col * stride;
+    wq[(uint64_t)col * kwords + w] = bb[1 + w];
+    if (w == 0) sw[col] = header_scale(bb[0]);
+}
+
+// c[r, :] = sum over the planes of yp[p m + r, :], smallest plane first
+__global__ __launch_bounds__(256) void q8_add_planes_kernel(const float* __restrict__ yp, float* __restrict__ c,
+                                                            uint64_t count) {
+    const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= count) return;
+    float v = yp[i];
+#pragma unroll
+    for (int p = 1; p < kQ8Planes; p++) v += yp[p * count + i];
+    c[i] = v;
+}
+
+static size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
+
+static int matmul_q8_mfma(const float* a, const uint32_t* b, float* c, uint32_t m, uint32_t k, uint32_t n,
+                          uint32_t stride, hipStream_t s) {
+    RUMUS_REQUIRE((uint64_t)kQ8Planes * m < (1ull << 31), "matmul_q8: m %u is beyond the grid limit", m);
+    const size_t planes_bytes = align256((size_t)kQ8Planes * m * k), sx_bytes = align256((size_t)kQ8Planes * m * sizeof(float));
+    const size_t wq_bytes = align256((size_t)n * k), sw_bytes = align256((size_t)n * sizeof(float));
+    const size_t y_bytes = (size_t)kQ8Planes * m * n * sizeof(float);
+    void* ws = nullptr;
+    if (int rc = workspace_get(s, planes_bytes + sx_bytes + wq_bytes + sw_bytes + y_bytes, &ws)) return rc;
+    uint8_t* base = static_cast<uint8_t*>(ws);
+    int8_t* planes = reinterpret_cast<int8_t*>(base);
+    float* sxp = reinterpret_cast<float*>(base + planes_bytes);
+    int8_t* wq = reinterpret_cast<int8_t*>(base + planes_bytes + sx_bytes);
+    float* sw = reinterpret_cast<float*>(base + planes_bytes + sx_bytes + wq_bytes);
+    float* yp = reinterpret_cast<float*>(base + planes_bytes + sx_bytes + wq_bytes + sw_bytes);
+    hipLaunchKernelGGL(q8_split_rows_kernel, dim3(m), dim3(256), 0, s, a, planes, sxp, m, k);
+    if (int rc = check_launch("q8_split_rows_kernel")) return rc;
+    hipLaunchKernelGGL(q8_unpack_channels_kernel, dim3(ceil_div(k / 4, 256), n), dim3(256), 0, s, b,
+                       reinterpret_cast<uint32_t*>(wq), sw, k / 4, stride);
+    if (int rc = check_launch("q8_unpack_channels_kernel")) return rc;
+    if (int rc = rumus_hip_i8_gemm(planes, wq, sxp, sw, nullptr, nullptr, yp, kQ8Planes * m, k, n, s)) return rc;
+    const uint64_t count = (uint64_t)m * n;
+    hipLaunchKernelGGL(q8_add_planes_kernel, dim3((uint32_t)((count + 255) / 256)), dim3(256), 0, s, yp, c, count);
+    return check_launch("q8_add_planes_kernel");
+}
+
 // Any block_size % 4 == 0: one thread per output, the reference's own loop.
 __global__ __launch_bounds__(256) void matmul_q8_naive_kernel(
     const float* __restrict__ a, const uint32_t* __restrict__ b, float* __restrict__ c,
@@ -384,6 +487,12 @@ int rumus_hip_matmul_q8(const float* a, const uint32_t* b, float* c, uint32_t m,
     RUMUS_REQUIRE(k > 0, "matmul_q8: k must be > 0");
     uint32_t blocks_per_col = ceil_div(k, block_size);
     uint32_t stride = (4 + block_size + 3) / 4;
+    // batches with per-output-channel blocks: the int8 matrix cores (from 8 rows on they are ahead of
+    // the kernel below, copy of the weights out of the block format included: 62 us either way at
+    // 8 x 4096 x 11008, 526 us = 351 TFLOP/s at 2048 rows)
+    if (blocks_per_col == 1 && k % 16 == 0 && m >= 8 && n <= 65535 &&
+        ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(c)) & 15) == 0)
+        return matmul_q8_mfma(a, b, c, m, k, n, stride, as_stream(stream));
     const uint32_t kpad = (k + 15) & ~15u;
     if (block_size % 16 == 0 && kpad <= 16384) {
         // rows in groups whose x fits 64 KB of LDS: 4 rows at k = 4096, 1 at k = 11008, all 8 up to k = 2048

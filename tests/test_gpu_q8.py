@@ -62,7 +62,10 @@ def test_q8_rejects_bad_block_size(ops):
                                       (8, 4096, 70, 128),      # two groups of four rows
                                       (3, 1008, 64, 16),       # smallest block the few-rows kernel takes
                                       (2, 11008, 40, 64),      # one row per launch
-                                      (7, 2048, 33, 2048)])
+                                      (7, 2048, 33, 2048),
+                                      (100, 1024, 300, 1024),  # digit planes on the int8 matrix cores
+                                      (8, 48, 20, 48),         # the smallest batch that goes there
+                                      (1000, 4096, 264, 4096)])
 def test_matmul_q8_vs_oracle(ops, m, k, n, bs):
     say(f"matmul_q8 m={m} k={k} n={n} bs={bs}")
     from rumus_amd import nn
@@ -79,6 +82,41 @@ def test_matmul_q8_vs_oracle(ops, m, k, n, bs):
     # Tensor::dequantize returns the buffer order ([N,K]) under the [K,N] shape
     deq = host(nn.dequantize(wq))
     np.testing.assert_array_equal(deq.reshape(-1), oracle.q8_dequantize(words, k * n, bs))
+
+
+def test_matmul_q8_batch_accuracy_and_non_finite_rows(ops):
+    # per-channel blocks and 8 rows or more: activations go through four 7-bit digit planes and
+    # the int8 matrix cores.  Judged against float64 in units of the summed terms (the planes keep
+    # 28 bits below the row maximum, so a row with one huge entry is the hard case), and a NaN or
+    # infinite activation must poison its own row only.
+    say("matmul_q8 digit-plane path")
+    rng = np.random.default_rng(77)
+    m, k, n = 64, 512, 96
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    a = rng.normal(0, 1, (m, k)).astype(np.float32)
+    a[3, 17] = 3.0e4                                        # dwarfs the rest of its row
+    a[5] *= 1e-30
+    a[6] = 0.0
+    words = oracle.tensor_quantize(w, k)
+    got = host(ops.matmul_q8(dev(a), dev(words), k, n, k))
+    want = oracle.matmul_q8(a, words, k, n, k, threads=8)
+    deq = oracle.q8_dequantize(words, k * n, k).reshape(n, k).T.astype(np.float64)
+    exact = a.astype(np.float64) @ deq
+    terms = np.abs(a).astype(np.float64) @ np.abs(deq) + 1e-300
+    err_ref = (np.abs(want - exact) / terms).max()
+    err_got = (np.abs(got - exact) / terms).max()
+    # ordinary rows come out more accurate than the f32 loop; the row with the outlier keeps 28 bits
+    # below 3e4 for its other entries and lands within a few times the f32 loop's own error
+    assert err_ref < 2e-6 and err_got < 1e-5, (err_got, err_ref)
+    assert (np.abs(np.delete(got, 3, axis=0) - np.delete(exact, 3, axis=0)) / np.delete(terms, 3, axis=0)).max() < 1e-7
+    assert_close(got, want)
+    np.testing.assert_array_equal(got[6], np.zeros(n, np.float32))
+    for bad in (np.float32(np.nan), np.float32(np.inf)):
+        ab = a.copy()
+        ab[9, 100] = bad
+        gb = host(ops.matmul_q8(dev(ab), dev(words), k, n, k))
+        assert np.isnan(gb[9]).all()
+        np.testing.assert_array_equal(np.delete(gb, 9, axis=0), np.delete(got, 9, axis=0))
 
 
 def test_matmul_q8_naive_kernel_is_bit_exact(ops):
