@@ -65,7 +65,15 @@ def test_q8_rejects_bad_block_size(ops):
                                       (7, 2048, 33, 2048),
                                       (100, 1024, 300, 1024),  # digit planes on the int8 matrix cores
                                       (8, 48, 20, 48),         # the smallest batch that goes there
-                                      (1000, 4096, 264, 4096)])
+                                      (1000, 4096, 264, 4096),
+                                      # blocks smaller than a column: block scales inside the MFMA loop
+                                      (11, 96, 20, 32),        # a fold per K half, K ends mid-step
+                                      (100, 1024, 300, 32),
+                                      (12, 192, 40, 96),       # blocks that straddle the K steps
+                                      (40, 4096, 64, 2048),    # two folds per block
+                                      (33, 512, 100, 64),
+                                      (1024, 512, 2048, 128),  # the largest tile
+                                      (1030, 256, 2050, 32)])
 def test_matmul_q8_vs_oracle(ops, m, k, n, bs):
     say(f"matmul_q8 m={m} k={k} n={n} bs={bs}")
     from rumus_amd import nn
@@ -84,12 +92,14 @@ def test_matmul_q8_vs_oracle(ops, m, k, n, bs):
     np.testing.assert_array_equal(deq.reshape(-1), oracle.q8_dequantize(words, k * n, bs))
 
 
-def test_matmul_q8_batch_accuracy_and_non_finite_rows(ops):
-    # per-channel blocks and 8 rows or more: activations go through four 7-bit digit planes and
-    # the int8 matrix cores.  Judged against float64 in units of the summed terms (the planes keep
+@pytest.mark.parametrize("bs", [512, 32, 128])
+def test_matmul_q8_batch_accuracy_and_non_finite_rows(ops, bs):
+    # 8 rows or more: activations go through four 7-bit digit planes and the int8 matrix cores
+    # (per-channel blocks: the W8A8 kernel; smaller blocks: block scales inside the loop).
+    # Judged against float64 in units of the summed terms (the planes keep
     # 28 bits below the row maximum, so a row with one huge entry is the hard case), and a NaN or
     # infinite activation must poison its own row only.
-    say("matmul_q8 digit-plane path")
+    say(f"matmul_q8 digit-plane path bs={bs}")
     rng = np.random.default_rng(77)
     m, k, n = 64, 512, 96
     w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
@@ -97,10 +107,10 @@ def test_matmul_q8_batch_accuracy_and_non_finite_rows(ops):
     a[3, 17] = 3.0e4                                        # dwarfs the rest of its row
     a[5] *= 1e-30
     a[6] = 0.0
-    words = oracle.tensor_quantize(w, k)
-    got = host(ops.matmul_q8(dev(a), dev(words), k, n, k))
-    want = oracle.matmul_q8(a, words, k, n, k, threads=8)
-    deq = oracle.q8_dequantize(words, k * n, k).reshape(n, k).T.astype(np.float64)
+    words = oracle.tensor_quantize(w, bs)
+    got = host(ops.matmul_q8(dev(a), dev(words), k, n, bs))
+    want = oracle.matmul_q8(a, words, k, n, bs, threads=8)
+    deq = oracle.q8_dequantize(words, k * n, bs).reshape(n, k).T.astype(np.float64)
     exact = a.astype(np.float64) @ deq
     terms = np.abs(a).astype(np.float64) @ np.abs(deq) + 1e-300
     err_ref = (np.abs(want - exact) / terms).max()
@@ -114,7 +124,7 @@ def test_matmul_q8_batch_accuracy_and_non_finite_rows(ops):
     for bad in (np.float32(np.nan), np.float32(np.inf)):
         ab = a.copy()
         ab[9, 100] = bad
-        gb = host(ops.matmul_q8(dev(ab), dev(words), k, n, k))
+        gb = host(ops.matmul_q8(dev(ab), dev(words), k, n, bs))
         assert np.isnan(gb[9]).all()
         np.testing.assert_array_equal(np.delete(gb, 9, axis=0), np.delete(got, 9, axis=0))
 
