@@ -390,18 +390,22 @@ static int matmul_q8_mfma(const float* a, const uint32_t* b, float* c, uint32_t 
 
 // q8_gemm.hip: the same digit planes against blocks smaller than a column
 int q8_gemm_blocks(const int8_t* planes, const float* sx, const uint32_t* b, float* c, uint32_t m, uint32_t k,
-                   uint32_t n, uint32_t bs, uint32_t stride, uint32_t bpc, hipStream_t s);
+                   uint32_t n, uint32_t bs, uint32_t stride, uint32_t bpc, float* part, uint32_t max_shares,
+                   hipStream_t s);
 
 static int matmul_q8_mfma_blocks(const float* a, const uint32_t* b, float* c, uint32_t m, uint32_t k, uint32_t n,
                                  uint32_t bs, uint32_t stride, uint32_t bpc, hipStream_t s) {
-    const size_t planes_bytes = align256((size_t)kQ8Planes * m * k);
+    const size_t planes_bytes = align256((size_t)kQ8Planes * m * k), sx_bytes = align256((size_t)kQ8Planes * m * sizeof(float));
+    // few rows: room for the partial results of up to 8 shares of K
+    const uint32_t max_shares = (uint64_t)m * n <= (1u << 22) ? 8 : 0;
     void* ws = nullptr;
-    if (int rc = workspace_get(s, planes_bytes + (size_t)kQ8Planes * m * sizeof(float), &ws)) return rc;
+    if (int rc = workspace_get(s, planes_bytes + sx_bytes + (size_t)max_shares * m * n * sizeof(float), &ws)) return rc;
     int8_t* planes = static_cast<int8_t*>(ws);
     float* sxp = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + planes_bytes);
+    float* part = max_shares ? reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + planes_bytes + sx_bytes) : nullptr;
     hipLaunchKernelGGL(q8_split_rows_kernel, dim3(m), dim3(256), 0, s, a, planes, sxp, m, k);
     if (int rc = check_launch("q8_split_rows_kernel")) return rc;
-    return q8_gemm_blocks(planes, sxp, b, c, m, k, n, bs, stride, bpc, s);   // sxp[0 .. m): the rows' 1 / f
+    return q8_gemm_blocks(planes, sxp, b, c, m, k, n, bs, stride, bpc, part, max_shares, s);   // sxp[0 .. m): the rows' 1 / f
 }
 
 // Any block_size % 4 == 0: one thread per output, the reference's own loop.
@@ -503,18 +507,18 @@ int rumus_hip_matmul_q8(const float* a, const uint32_t* b, float* c, uint32_t m,
     RUMUS_REQUIRE(k > 0, "matmul_q8: k must be > 0");
     uint32_t blocks_per_col = ceil_div(k, block_size);
     uint32_t stride = (4 + block_size + 3) / 4;
-    // batches with per-output-channel blocks: the int8 matrix cores (from 8 rows on they are ahead of
-    // the kernel below, copy of the weights out of the block format included: 62 us either way at
-    // 8 x 4096 x 11008, 526 us = 351 TFLOP/s at 2048 rows)
-    if (blocks_per_col == 1 && k % 16 == 0 && m >= 8 && n <= 65535 &&
-        ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(c)) & 15) == 0)
+    // Batches go to the int8 matrix cores as four digit planes of the activations.  Measured at
+    // 4096 x 11008 (us, whole call):          rows    5..32    128    512    2048
+    //   block-scale kernel, 32-element blocks         34..38    84    242     900     (few-rows kernel: 7.7 per row,
+    //   block-scale kernel, 128-element blocks        33..36    65    170     600      LDS-tiled kernel: 15 ms at 2048)
+    //   block-scale kernel, one block per column      29..33    65    170
+    //   W8A8 kernel on a dense copy of the weights        62    83    148     526     (one block per column only)
+    const bool aligned = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(c)) & 15) == 0;
+    const bool block_kernel = block_size % 32 == 0 && k % block_size == 0 && m >= 5 && aligned &&
+                              (uint64_t)k * block_size < (1ull << 32) && (uint64_t)kQ8Planes * m * k < (1ull << 40);
+    if (blocks_per_col == 1 && k % 16 == 0 && m >= (block_kernel ? 384u : 8u) && n <= 65535 && aligned)
         return matmul_q8_mfma(a, b, c, m, k, n, stride, as_stream(stream));
-    // batches against smaller blocks: the same on the int8 matrix cores, block scales applied in the loop
-    // (4096 x 11008, 32-element blocks: 83 us up to 32 rows against 7.7 us per row below;
-    // 2048 rows: 15.1 ms -> 1.24 ms, 128-element blocks 0.84 ms)
-    if (blocks_per_col > 1 && block_size % 32 == 0 && k % block_size == 0 && m >= 11 &&
-        (uint64_t)k * block_size < (1ull << 32) && (uint64_t)kQ8Planes * m * k < (1ull << 40) &&
-        (reinterpret_cast<uintptr_t>(a) & 15) == 0)
+    if (block_kernel)
         return matmul_q8_mfma_blocks(a, b, c, m, k, n, block_size, stride, blocks_per_col, as_stream(stream));
     const uint32_t kpad = (k + 15) & ~15u;
     if (block_size % 16 == 0 && kpad <= 16384) {

@@ -1,4 +1,4 @@
-// f32 x Q8 batches on the gfx950 i8 matrix cores when a column holds several blocks
+// f32 x Q8 batches on the gfx950 i8 matrix cores, block scales applied inside the K loop
 // (matmul_q8.wgsl:37-96 computes the same sums one output per thread).
 //
 //   c[m, n] = sum over the blocks kb of column n:  s[n, kb] * sum_{k in kb} x[m, k] * q[n, k]
@@ -13,108 +13,98 @@
 // which is 6 vector instructions per 4 accumulators.  With 32-element blocks that work, not the
 // matrix cores, sets the pace (96 instructions per 4 MFMAs and column tile).
 //
-// The weights are read where they lie: a 16-byte chunk of a block sits 4 bytes past a 4-byte
-// boundary because of the block header, which global loads take; the block scale of a lane's
-// column comes out of the same cache lines one K step ahead of its use.
+// The weights are read where they lie: a 16-byte chunk of a block sits 4 bytes past a 16-byte
+// boundary at best because of the block headers, which the loads take; the headers with the
+// block scales of the tile's columns ride along as 4-byte loads.
 //
-// Workgroup = WM x WN waves, block tile (32 WM) rows x (32 TN WN) columns, K step 64 bytes, two
-// LDS stages (global -> registers -> LDS of step t+1 under the MFMAs of step t), rows of 64 bytes
-// with the chunk swizzle of the W8A8 kernels.
+// Workgroup = WM x WN waves, block tile (32 WM) rows x (32 TN WN) columns, K step 64 bytes, NS
+// LDS stages filled by direct-to-LDS loads (NS - 1 steps in flight: with a single step in flight
+// a step took as long as a trip to memory, 1.3 to 1.7 us), rows of 64 bytes with the chunk
+// swizzle of the W8A8 kernels, one barrier per step.  Problems with few tiles share K out over
+// blockIdx.y as well and add the partial results in a second kernel, in a fixed order.
 #include <hip/hip_fp16.h>
 
 #include "i8_gemm.h"
 
 namespace rumus {
 
-typedef int v4i_a4 __attribute__((ext_vector_type(4), aligned(4)));
-
 constexpr int kQ8GemmPlanes = 4;
 
-template <int WM, int WN, int TN, bool EVERY>
+template <int WM, int WN, int TN, int NS, bool EVERY>
 __global__ __launch_bounds__(64 * WM * WN, 2) void q8_gemm_blocks_kernel(
     const int8_t* __restrict__ planes, const float* __restrict__ sx, const uint8_t* __restrict__ b,
     float* __restrict__ c, uint32_t M, uint32_t K, uint32_t N, uint32_t bs, uint32_t bs_magic,
-    uint32_t stride_bytes, uint32_t bpc, uint32_t period, uint32_t tiles_m, uint32_t tiles_n) {
+    uint32_t stride_bytes, uint32_t bpc, uint32_t period, uint32_t tiles_m, uint32_t tiles_n, uint32_t steps_per) {
     constexpr int P = kQ8GemmPlanes;
-    constexpr int T = 64 * WM * WN;
+    constexpr int WAVES = WM * WN;
     constexpr int BM = 32 * WM, BN = 32 * TN * WN;
     constexpr int A_ROWS = P * BM;
-    constexpr int A_BYTES = A_ROWS * kBK, B_BYTES = BN * kBK;
-    constexpr int ROWS_PER_PASS = T / 4;                       // 4 chunks of 16 bytes per row
-    constexpr int A_LOADS = A_ROWS / ROWS_PER_PASS, B_LOADS = BN / ROWS_PER_PASS;
-    static_assert(A_ROWS % ROWS_PER_PASS == 0 && BN % ROWS_PER_PASS == 0, "tile does not divide over the threads");
-    __shared__ __attribute__((aligned(16))) int8_t lds[2][A_BYTES + B_BYTES];
+    constexpr int A_BYTES = A_ROWS * kBK, B_BYTES = BN * kBK, S_BYTES = 2 * BN * 4;
+    constexpr int STAGE = A_BYTES + B_BYTES + S_BYTES;
+    // a wave-wide 16-byte LDS-DMA load fills 16 rows of 64 bytes, a 4-byte one 64 header words
+    constexpr int A_BLOCKS = A_ROWS / 16, B_BLOCKS = BN / 16, S_BLOCKS = 2 * BN / 64;
+    constexpr int A_LOADS = (A_BLOCKS + WAVES - 1) / WAVES, B_LOADS = (B_BLOCKS + WAVES - 1) / WAVES;
+    constexpr int S_LOADS = (S_BLOCKS + WAVES - 1) / WAVES;
+    constexpr int LOADS = A_LOADS + B_LOADS + S_LOADS;
+    static_assert(BN % 64 == 0, "a header load must stay inside one K half");
+    static_assert((NS - 2) * LOADS <= 63, "more loads in flight than the counter holds");
+    extern __shared__ __attribute__((aligned(16))) int8_t lds[];   // [NS][STAGE]
 
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: LDS-DMA destinations are
     const uint32_t wm = wave / WN, wn = wave % WN;
     const uint32_t tile = xcd_contiguous(blockIdx.x, tiles_m * tiles_n);
     const uint32_t m0 = (tile % tiles_m) * BM, n0 = (tile / tiles_m) * BN;
 
-    // ---- global -> LDS staging ----------------------------------------------------------------
-    const uint32_t ld_row = tid >> 2, ld_c = tid & 3;
-    const uint32_t ld_lds = ld_row * kBK + ((ld_c ^ row_swizzle(ld_row)) & 3) * 16;   // ROWS_PER_PASS % 16 == 0
+    // ---- global side of the LDS-DMA loads -----------------------------------------------------------
+    // lane l of a 16-row block fetches row l/4, logical chunk (l%4) ^ swizzle(row) and lands in
+    // physical chunk l%4; the swizzle only looks at row bits 1..3, the same for every block
+    const uint32_t lr = lane >> 2, lc = ((lane & 3) ^ row_swizzle(lr)) & 3;
     const int8_t* pa[A_LOADS];
     const uint8_t* pb[B_LOADS];
+    const uint8_t* ps[S_LOADS];
+    uint32_t blk_a[A_LOADS], blk_b[B_LOADS], blk_s[S_LOADS];
 #pragma unroll
     for (int i = 0; i < A_LOADS; i++) {
-        const uint32_t lr = ld_row + ROWS_PER_PASS * i;        // plane-major rows of the A tile
-        const uint32_t plane = lr / BM, r = lr % BM;
-        pa[i] = planes + ((uint64_t)plane * M + min(m0 + r, M - 1)) * K + ld_c * 16;
+        blk_a[i] = min(i * WAVES + wave, (uint32_t)A_BLOCKS - 1);
+        const uint32_t row = blk_a[i] * 16 + lr;               // plane-major rows of the A tile
+        const uint32_t plane = row / BM, r = row % BM;
+        pa[i] = planes + ((uint64_t)plane * M + min(m0 + r, M - 1)) * K;
     }
 #pragma unroll
     for (int i = 0; i < B_LOADS; i++) {
-        const uint32_t col = min(n0 + ld_row + ROWS_PER_PASS * i, N - 1);
+        blk_b[i] = min(i * WAVES + wave, (uint32_t)B_BLOCKS - 1);
+        const uint32_t col = min(n0 + blk_b[i] * 16 + lr, N - 1);
         pb[i] = b + (uint64_t)col * bpc * stride_bytes + 4;
     }
-    v4i ga[A_LOADS], gb[B_LOADS];
-    auto load_global = [&](uint32_t k0) {
-        const uint32_t kpos = k0 + ld_c * 16;
-        const bool ok = kpos < K;                              // K % 32 == 0: a chunk is all-in or all-out
+#pragma unroll
+    for (int i = 0; i < S_LOADS; i++) {
+        blk_s[i] = min(i * WAVES + wave, (uint32_t)S_BLOCKS - 1);
+        const uint32_t col = min(n0 + (blk_s[i] * 64 + lane) % BN, N - 1);
+        ps[i] = b + (uint64_t)col * bpc * stride_bytes;
+    }
+    // A K half past the end of K (K % 64 == 32) is fetched from the half before it: what it adds to
+    // the integer sums is never folded in, or folded in with scale 0.
+    auto issue = [&](uint32_t kt, uint32_t stage) {
+        int8_t* base = lds + stage * STAGE;
+        const uint32_t k0 = kt * kBK;
+        uint32_t kpos = k0 + lc * 16;
+        if (kpos >= K) kpos -= 32;
         const uint32_t blk = __umulhi(kpos, bs_magic);
         const uint32_t boff = blk * stride_bytes + (kpos - blk * bs);
 #pragma unroll
         for (int i = 0; i < A_LOADS; i++)
-            ga[i] = ok ? *reinterpret_cast<const v4i*>(pa[i] + k0) : v4i{0, 0, 0, 0};
-#pragma unroll
-        for (int i = 0; i < B_LOADS; i++) {
-            if (ok) {
-                const v4i_a4 v = *reinterpret_cast<const v4i_a4*>(pb[i] + boff);
-                gb[i] = v4i{v.x, v.y, v.z, v.w};
-            } else {
-                gb[i] = v4i{0, 0, 0, 0};
-            }
-        }
-    };
-    auto store_lds = [&](int stage) {
-        int8_t* base = lds[stage];
-#pragma unroll
-        for (int i = 0; i < A_LOADS; i++)
-            *reinterpret_cast<v4i*>(base + ld_lds + i * ROWS_PER_PASS * kBK) = ga[i];
+            __builtin_amdgcn_global_load_lds((gptr_t)(pa[i] + kpos), (lptr_t)(base + blk_a[i] * 1024), 16, 0, 0);
 #pragma unroll
         for (int i = 0; i < B_LOADS; i++)
-            *reinterpret_cast<v4i*>(base + A_BYTES + ld_lds + i * ROWS_PER_PASS * kBK) = gb[i];
-    };
-
-    // ---- block scales of this lane's columns -----------------------------------------------------
-    const uint32_t col_l = lane & 31;
-    const uint8_t* ph[TN];
+            __builtin_amdgcn_global_load_lds((gptr_t)(pb[i] + boff), (lptr_t)(base + A_BYTES + blk_b[i] * 1024), 16, 0, 0);
 #pragma unroll
-    for (int j = 0; j < TN; j++) {
-        const uint32_t col = min(n0 + (wn * TN + j) * 32 + col_l, N - 1);
-        ph[j] = b + (uint64_t)col * bpc * stride_bytes;
-    }
-    float sc_cur[2][TN], sc_nxt[2][TN];
-    auto load_scales = [&](uint32_t k0, float (&sc)[2][TN]) {
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-            const uint32_t kpos = k0 + 32 * h;
-            const uint32_t blk = min(__umulhi(kpos, bs_magic), bpc - 1);
-#pragma unroll
-            for (int j = 0; j < TN; j++) {
-                const uint32_t header = *reinterpret_cast<const uint32_t*>(ph[j] + (uint64_t)blk * stride_bytes);
-                const float s = __half2float(__ushort_as_half((unsigned short)(header & 0xFFFFu)));
-                sc[h][j] = kpos < K ? s : 0.0f;
-            }
+        for (int i = 0; i < S_LOADS; i++) {
+            uint32_t kh = k0 + 32 * (blk_s[i] * 64 / BN);
+            if (kh >= K) kh -= 32;
+            const uint32_t hb = __umulhi(kh, bs_magic);
+            __builtin_amdgcn_global_load_lds((gptr_t)(ps[i] + (uint64_t)hb * stride_bytes),
+                                             (lptr_t)(base + A_BYTES + B_BYTES + blk_s[i] * 256), 4, 0, 0);
         }
     };
 
@@ -127,6 +117,7 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void q8_gemm_blocks_kernel(
         a_off[s] = (wm * 32 + fr) * kBK + chunk * 16;
         b_off[s] = A_BYTES + (wn * 32 * TN + fr) * kBK + chunk * 16;
     }
+    const uint32_t s_off = A_BYTES + B_BYTES + (wn * TN * 32 + fr) * 4;
 
     v16i acc[P][TN];
     float out[TN][16];
@@ -141,21 +132,22 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void q8_gemm_blocks_kernel(
     }
     const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 
-    const uint32_t ksteps = (K + kBK - 1) / kBK;
+    // ---- pipeline: NS - 1 K steps in flight, one barrier per step -------------------------------------
+    // Every step issues exactly LOADS loads per wave, also past the end of K (the last step is then
+    // fetched again into a stage nobody reads any more), so the counter arithmetic has no tail cases.
+    // blockIdx.y picks the share of the K steps (a multiple of the fold period) this workgroup sums
+    const uint32_t kt0 = blockIdx.y * steps_per, ksteps = min((K + kBK - 1) / kBK, kt0 + steps_per);
     uint32_t left = period;                                    // K halves until the next fold
-    load_global(0);
-    load_scales(0, sc_cur);
-    store_lds(0);
-    __syncthreads();
-
-    for (uint32_t kt = 0; kt < ksteps; kt++) {
-        const int cur = kt & 1;
-        const bool more = kt + 1 < ksteps;
-        if (more) {
-            load_global((kt + 1) * kBK);
-            load_scales((kt + 1) * kBK, sc_nxt);
-        }
-        const int8_t* base = lds[cur];
+#pragma unroll
+    for (int s = 0; s < NS - 1; s++) issue(min(kt0 + s, ksteps - 1), s);
+    uint32_t cur = 0;
+    for (uint32_t kt = kt0; kt < ksteps; kt++) {
+        // step kt has landed once only the NS-2 younger steps are outstanding; past the barrier every
+        // wave has also finished reading the stage of step kt-1, which is refilled at once
+        RUMUS_WAIT_VMCNT((NS - 2) * LOADS);
+        __builtin_amdgcn_s_barrier();
+        issue(min(kt + (NS - 1), ksteps - 1), cur == 0 ? NS - 1 : cur - 1);
+        const int8_t* base = lds + cur * STAGE;
 #pragma unroll
         for (int s = 0; s < 2; s++) {
             v4i af[P], bf[TN];
@@ -177,9 +169,12 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void q8_gemm_blocks_kernel(
             }
             if (fold) {
                 left = period;
+                const bool live = kt * kBK + 32 * s < K;
 #pragma unroll
                 for (int j = 0; j < TN; j++) {
-                    const float s_lo = sc_cur[s][j], s_hi = s_lo * 16384.0f;
+                    const uint32_t header = *reinterpret_cast<const uint32_t*>(base + s_off + (s * BN + j * 32) * 4);
+                    const float s_lo = live ? __half2float(__ushort_as_half((unsigned short)(header & 0xFFFFu))) : 0.0f;
+                    const float s_hi = s_lo * 16384.0f;
 #pragma unroll
                     for (int r = 0; r < 16; r++) {
                         const int lo = acc[1][j][r] * 128 + acc[0][j][r];
@@ -194,16 +189,13 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void q8_gemm_blocks_kernel(
                 }
             }
         }
-        if (more) store_lds(cur ^ 1);
-        __syncthreads();
-#pragma unroll
-        for (int h = 0; h < 2; h++)
-#pragma unroll
-            for (int j = 0; j < TN; j++) sc_cur[h][j] = sc_nxt[h][j];
+        cur = cur + 1 == NS ? 0 : cur + 1;
     }
+    RUMUS_WAIT_VMCNT(0);         // no LDS-DMA write may outlive the workgroup
 
     // ---- rows back to their scale: register r of lane l is row 8 (r/4) + 4 (l/32) + r%4, column l%32 ----
-    const uint32_t row_l = (lane >> 5) * 4;
+    const uint32_t col_l = lane & 31, row_l = (lane >> 5) * 4;
+    c += (uint64_t)blockIdx.y * M * N;                         // partial sums of K share y when K is split
 #pragma unroll
     for (int j = 0; j < TN; j++) {
         const uint32_t col = n0 + (wn * TN + j) * 32 + col_l;
@@ -216,35 +208,69 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void q8_gemm_blocks_kernel(
     }
 }
 
-template <int WM, int WN, int TN, bool EVERY>
-static int launch_q8_gemm_blocks(const int8_t* planes, const float* sx, const uint32_t* b, float* c, uint32_t m,
-                                 uint32_t k, uint32_t n, uint32_t bs, uint32_t stride, uint32_t bpc, uint32_t period,
-                                 hipStream_t s) {
-    const uint32_t tm = ceil_div(m, 32 * WM), tn = ceil_div(n, 32 * TN * WN);
-    const uint32_t magic = (uint32_t)((0x100000000ull + bs - 1) / bs);
-    hipLaunchKernelGGL((q8_gemm_blocks_kernel<WM, WN, TN, EVERY>), dim3(tm * tn), dim3(64 * WM * WN), 0, s, planes, sx,
-                       reinterpret_cast<const uint8_t*>(b), c, m, k, n, bs, magic, stride * 4, bpc, period, tm, tn);
-    return check_launch("q8_gemm_blocks_kernel");
+// c = sum over the K shares of their partial results, in share order
+__global__ __launch_bounds__(256) void q8_gemm_add_shares_kernel(const float* __restrict__ part, float* __restrict__ c,
+                                                                 uint32_t count, uint32_t shares) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= count) return;
+    float v = part[i];
+    for (uint32_t z = 1; z < shares; z++) v += part[(uint64_t)z * count + i];
+    c[i] = v;
 }
 
+template <int WM, int WN, int TN, int NS, bool EVERY>
+static int launch_q8_gemm_blocks(const int8_t* planes, const float* sx, const uint32_t* b, float* c, uint32_t m,
+                                 uint32_t k, uint32_t n, uint32_t bs, uint32_t stride, uint32_t bpc, uint32_t period,
+                                 float* part, uint32_t max_shares, hipStream_t s) {
+    constexpr size_t lds_bytes = (size_t)NS * ((kQ8GemmPlanes * 32 * WM + 32 * TN * WN) * kBK + 2 * 32 * TN * WN * 4);
+    static_assert(lds_bytes <= 160 * 1024, "more LDS than a compute unit has");
+    static bool attr_set = false;   // benign race: setting the attribute is idempotent
+    if (!attr_set && lds_bytes > 64 * 1024) {
+        if (int rc = check_hip(hipFuncSetAttribute(
+                reinterpret_cast<const void*>(&q8_gemm_blocks_kernel<WM, WN, TN, NS, EVERY>),
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes), "hipFuncSetAttribute"))
+            return rc;
+        attr_set = true;
+    }
+    const uint32_t tm = ceil_div(m, 32 * WM), tn = ceil_div(n, 32 * TN * WN);
+    const uint32_t magic = (uint32_t)((0x100000000ull + bs - 1) / bs);
+    // too few tiles for the chip: K is shared out as well, in whole fold periods of at least 8 steps
+    const uint32_t ksteps = ceil_div(k, kBK);
+    uint32_t shares = 1, steps_per = ksteps;
+    if (part && tm * tn < 256) {
+        const uint32_t unit = period * ceil_div(8, period);
+        shares = min(min(max_shares, 512 / (tm * tn)), max(1u, ksteps / unit));
+        steps_per = ceil_div(ceil_div(ksteps, shares), unit) * unit;
+        shares = ceil_div(ksteps, steps_per);
+    }
+    hipLaunchKernelGGL((q8_gemm_blocks_kernel<WM, WN, TN, NS, EVERY>), dim3(tm * tn, shares), dim3(64 * WM * WN),
+                       lds_bytes, s, planes, sx, reinterpret_cast<const uint8_t*>(b), shares > 1 ? part : c, m, k, n, bs,
+                       magic, stride * 4, bpc, period, tm, tn, steps_per);
+    if (int rc = check_launch("q8_gemm_blocks_kernel")) return rc;
+    if (shares == 1) return RUMUS_HIP_OK;
+    hipLaunchKernelGGL(q8_gemm_add_shares_kernel, dim3(ceil_div(m * n, 256)), dim3(256), 0, s, part, c, m * n, shares);
+    return check_launch("q8_gemm_add_shares_kernel");
+}
+
+#define RUMUS_Q8_LAUNCH(WM, WN, TN, NS, EV) \
+    launch_q8_gemm_blocks<WM, WN, TN, NS, EV>(planes, sx, b, c, m, k, n, bs, stride, bpc, period, part, max_shares, s)
+
 // planes: [4][m][k] digit planes, sx: [m] the rows' 1 / f.  Needs bs % 32 == 0, k % bs == 0 and
-// k * bs < 2^32 (the division by bs is a multiply).
+// k * bs < 2^32 (the division by bs is a multiply).  part: room for max_shares x m x n partial
+// results (or null): small problems share K out over workgroups as well.
 int q8_gemm_blocks(const int8_t* planes, const float* sx, const uint32_t* b, float* c, uint32_t m, uint32_t k,
-                   uint32_t n, uint32_t bs, uint32_t stride, uint32_t bpc, hipStream_t s) {
+                   uint32_t n, uint32_t bs, uint32_t stride, uint32_t bpc, float* part, uint32_t max_shares,
+                   hipStream_t s) {
     // fold period in K halves: the largest divisor of the block's halves that keeps 1024 k between folds
     uint32_t period = 1;
     for (uint32_t d = 32; d > 1; d--)
         if ((bs / 32) % d == 0) { period = d; break; }
-    const bool small = m <= 32;
-    if (period == 1) {
-        // a fold per MFMA group: two column tiles per wave would not fit the registers next to the staging
-        if (small) return launch_q8_gemm_blocks<1, 2, 1, true>(planes, sx, b, c, m, k, n, bs, stride, bpc, period, s);
-        return launch_q8_gemm_blocks<2, 2, 1, true>(planes, sx, b, c, m, k, n, bs, stride, bpc, period, s);
-    }
-    if (small) return launch_q8_gemm_blocks<1, 2, 1, false>(planes, sx, b, c, m, k, n, bs, stride, bpc, period, s);
-    if ((uint64_t)ceil_div(m, 64) * ceil_div(n, 128) >= 256)
-        return launch_q8_gemm_blocks<2, 2, 2, false>(planes, sx, b, c, m, k, n, bs, stride, bpc, period, s);
-    return launch_q8_gemm_blocks<2, 2, 1, false>(planes, sx, b, c, m, k, n, bs, stride, bpc, period, s);
+    // measured at 4096 x 11008: with a fold per K half the 32-row tile is ahead at every batch size
+    // (the folds, not the operand traffic, set the pace); otherwise 64 x 128 tiles, two workgroups
+    // per compute unit, from 33 rows on
+    if (period == 1) return RUMUS_Q8_LAUNCH(1, 4, 1, 4, true);
+    if (m <= 32) return RUMUS_Q8_LAUNCH(1, 4, 1, 4, false);
+    return RUMUS_Q8_LAUNCH(2, 2, 2, 3, false);
 }
 
 }  // namespace rumus

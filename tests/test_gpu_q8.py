@@ -59,14 +59,16 @@ def test_q8_rejects_bad_block_size(ops):
 @pytest.mark.parametrize("m,k,n,bs", [(32, 512, 512, 512), (4, 64, 10, 64), (3, 96, 7, 32),
                                       (2, 40, 5, 8), (70, 256, 130, 128), (5, 100, 9, 20),
                                       (1, 4096, 1100, 4096),   # few-rows kernel, per-channel blocks
-                                      (8, 4096, 70, 128),      # two groups of four rows
+                                      (4, 8192, 70, 128),      # two groups of two rows
                                       (3, 1008, 64, 16),       # smallest block the few-rows kernel takes
                                       (2, 11008, 40, 64),      # one row per launch
                                       (7, 2048, 33, 2048),
-                                      (100, 1024, 300, 1024),  # digit planes on the int8 matrix cores
-                                      (8, 48, 20, 48),         # the smallest batch that goes there
+                                      (100, 1024, 300, 1024),  # digit planes on the int8 matrix cores, one block per column
+                                      (8, 48, 20, 48),         # W8A8 kernel on a dense copy: the smallest batch that goes there
+                                      (400, 512, 96, 512),     # and from 384 rows on
                                       (1000, 4096, 264, 4096),
-                                      # blocks smaller than a column: block scales inside the MFMA loop
+                                      # block scales inside the MFMA loop
+                                      (5, 64, 64, 32),         # the smallest batch that goes there
                                       (11, 96, 20, 32),        # a fold per K half, K ends mid-step
                                       (100, 1024, 300, 32),
                                       (12, 192, 40, 96),       # blocks that straddle the K steps
@@ -92,16 +94,16 @@ def test_matmul_q8_vs_oracle(ops, m, k, n, bs):
     np.testing.assert_array_equal(deq.reshape(-1), oracle.q8_dequantize(words, k * n, bs))
 
 
-@pytest.mark.parametrize("bs", [512, 32, 128])
-def test_matmul_q8_batch_accuracy_and_non_finite_rows(ops, bs):
-    # 8 rows or more: activations go through four 7-bit digit planes and the int8 matrix cores
-    # (per-channel blocks: the W8A8 kernel; smaller blocks: block scales inside the loop).
+@pytest.mark.parametrize("bs,m", [(512, 64), (32, 64), (128, 64), (512, 400)])
+def test_matmul_q8_batch_accuracy_and_non_finite_rows(ops, bs, m):
+    # batches: activations go through four 7-bit digit planes and the int8 matrix cores (block
+    # scales inside the loop; 400 rows and one block per column: the W8A8 kernel on a dense copy).
     # Judged against float64 in units of the summed terms (the planes keep
     # 28 bits below the row maximum, so a row with one huge entry is the hard case), and a NaN or
     # infinite activation must poison its own row only.
     say(f"matmul_q8 digit-plane path bs={bs}")
     rng = np.random.default_rng(77)
-    m, k, n = 64, 512, 96
+    k, n = 512, 96
     w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
     a = rng.normal(0, 1, (m, k)).astype(np.float32)
     a[3, 17] = 3.0e4                                        # dwarfs the rest of its row
