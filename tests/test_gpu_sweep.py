@@ -132,14 +132,14 @@ def test_i8_engine(ops, case):
     assert_close(host(y), oracle.i8_rescale_bias(acc_want, sx_want, sw_h, bias), "i8_gemm y")
 
 
-@pytest.mark.parametrize("case", range(16))
+@pytest.mark.parametrize("case", range(32))
 def test_q8_block_format(ops, case):
     rng = np.random.default_rng(4000 + case)
-    bs = int(rng.choice([4, 8, 32, 64, 256, 512]))
+    bs = int(rng.choice([4, 8, 32, 64, 256, 512] if case < 16 else [32, 64, 96, 128, 1024]))
     blocks_per_col = int(rng.integers(1, 5))
     k = bs * blocks_per_col
     n = draw(rng, [1, 7, 64, 130], 2)
-    m = draw(rng, [1, 5, 33], 1)
+    m = draw(rng, [1, 5, 33] if case < 16 else [5, 33, 70, 390], 1)   # few-rows kernel / the matrix-core paths
     say(f"sweep q8 case={case} m={m} k={k} n={n} bs={bs}")
     w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
     if case % 4 == 0:
