@@ -300,6 +300,33 @@ def bench_w4_gemm(torch, ops, m, steps=50, warmup=5):
             "tflops": flops / sec / 1e12, "f16_mfma_frac": flops / sec / 1e12 / F16_PEAK_TFLOPS}
 
 
+def bench_q8_matmul(torch, ops, steps=20, warmup=4):
+    """The reference's f32 x Q8 matmul (Tensor::matmul with a Q8 right-hand side), K=4096, N=11008,
+    at the block sizes that take different kernels: whole call, graph-timed."""
+    k, n = 4096, 11008
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev).manual_seed(3)
+    wt = ops.transpose_f32(torch.randn((k, n), generator=gen, device=dev) * 0.02).reshape(-1)
+    rows = []
+    for bs in (32, 128, 4096):
+        words = ops.q8_quantize(wt, bs)
+        for m in (1, 32, 2048):
+            a = torch.randn((m, k), generator=gen, device=dev)
+            c = torch.empty((m, n), dtype=torch.float32, device=dev)
+
+            def burst():
+                for _ in range(4):
+                    ops.matmul_q8(a, words, k, n, bs, out=c)
+
+            total, launches, _ = time_graph(torch, burst, 4, steps, warmup)
+            sec = total / launches
+            rows.append({"workload": f"matmul_q8_{m}x4096x11008_bs{bs}", "ms_per_call": sec * 1e3,
+                         "tflops": 2.0 * m * k * n / sec / 1e12,
+                         "weight_gbs": (k * n + 4 * n * (k // bs)) / sec / 1e9})
+        del words
+    return rows
+
+
 def bench_decoder_block(torch, ops):
     """Llama-7B-shaped block, all seven projections INT4 g128 with the reference's f32 zero-points:
     one decode step (batch 1, position 2047 of a 2048-entry cache) and one prefill of 8 x 512
@@ -489,6 +516,7 @@ def main():
         out["secondary"] = bench_i8_gemm(torch, ops)
         out["w4_gemv_wider"] = bench_gemv_shapes(torch, ops)
         out["w4_gemm"] = [bench_w4_gemm(torch, ops, 16), bench_w4_gemm(torch, ops, 128)]
+        out["q8_matmul"] = bench_q8_matmul(torch, ops)
         out["decoder_block"] = bench_decoder_block(torch, ops)
 
     if not args.no_cpu:

@@ -65,11 +65,13 @@ def q8_dequantize(words: torch.Tensor, numel: int, block_size: int) -> torch.Ten
     return out
 
 
-def matmul_q8(a: torch.Tensor, words: torch.Tensor, k: int, n: int, block_size: int) -> torch.Tensor:
+def matmul_q8(a: torch.Tensor, words: torch.Tensor, k: int, n: int, block_size: int, out=None) -> torch.Tensor:
     m = a.shape[0]
     if a.dim() != 2 or a.shape[1] != k:
         raise ValueError("matmul: inner dimension mismatch")
-    c = torch.empty((m, n), dtype=torch.float32, device=a.device)
+    c = torch.empty((m, n), dtype=torch.float32, device=a.device) if out is None else out
+    if c.shape != (m, n) or c.dtype != torch.float32 or not c.is_contiguous():
+        raise ValueError("matmul: out must be a contiguous f32 [m, n] tensor")
     call("rumus_hip_matmul_q8", _dev(a, torch.float32, "a"), _dev(words, torch.int32, "b"),
          c.data_ptr(), m, k, n, block_size, _stream())
     return c
