@@ -38,7 +38,7 @@ BYTES_U4_ZP = K * N // 2 + GROUPS * N * 4 + GROUPS * N // 2 + K * 4 + N * 4  # 9
 WEIGHT_SETS = 64
 # HBM bytes per GEMV launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by a 256 MiB copy
 # (profiles/w4_gemv_dot8_1x4096x4096_hbm_traffic.txt); a counter result, not measured by this script
-GEMV_TRAFFIC_BYTES = 9636889
+GEMV_TRAFFIC_BYTES = 9650224
 
 
 def log(msg):
