@@ -388,10 +388,52 @@ static int matmul_q8_mfma(const float* a, const uint32_t* b, float* c, uint32_t 
     return check_launch("q8_add_planes_kernel");
 }
 
+// Activations for the f16 variant of the block-scale kernel: x f = hi + lo, two f16 planes [2][m][k]
+// (22 bits of every element), f a power of two per row with |x f| < 2^15; sx[row] = 1 / f.
+__global__ __launch_bounds__(256) void q8_split_rows_f16_kernel(const float* __restrict__ a, _Float16* __restrict__ planes,
+                                                                float* __restrict__ sx, uint32_t m, uint32_t k) {
+    __shared__ uint32_t red[4];
+    const uint32_t row = blockIdx.x, tid = threadIdx.x;
+    const float* ar = a + (uint64_t)row * k;
+    uint32_t amax = 0;
+    for (uint32_t j = tid; j < k; j += 256) amax = max(amax, __float_as_uint(ar[j]) & 0x7FFFFFFFu);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) amax = max(amax, (uint32_t)__shfl_xor((int)amax, off));
+    if ((tid & 63) == 0) red[tid >> 6] = amax;
+    __syncthreads();
+    amax = max(max(red[0], red[1]), max(red[2], red[3]));
+    const uint32_t ebits = amax >> 23;                         // amax = a 2^(ebits-127), 1 <= a < 2
+    const bool poisoned = ebits == 255;                        // inf / nan in the row
+    const bool nothing = ebits < 15;                           // zero or below 2^-112: contributes nothing
+    const float f = (poisoned || nothing) ? 0.0f : __uint_as_float((268u - ebits) << 23);   // 2^(141 - ebits)
+    if (tid == 0)
+        sx[row] = poisoned ? __uint_as_float(0x7FC00000u) : nothing ? 0.0f : __uint_as_float((ebits - 14u) << 23);
+    _Float16* hi = planes + (uint64_t)row * k;
+    _Float16* lo = planes + ((uint64_t)m + row) * k;
+    for (uint32_t j = 4 * tid; j < k; j += 1024) {             // k % 4 == 0
+        const float4 v = *reinterpret_cast<const float4*>(ar + j);
+        const float xv[4] = {v.x, v.y, v.z, v.w};
+        _Float16 h[4], l[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const float t = poisoned ? 0.0f : xv[e] * f;       // exact: f is a power of two
+            h[e] = (_Float16)t;
+            l[e] = (_Float16)(t - (float)h[e]);
+        }
+        typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+        *reinterpret_cast<v4h*>(hi + j) = v4h{h[0], h[1], h[2], h[3]};
+        *reinterpret_cast<v4h*>(lo + j) = v4h{l[0], l[1], l[2], l[3]};
+    }
+}
+
 // q8_gemm.hip: the same digit planes against blocks smaller than a column
 int q8_gemm_blocks(const int8_t* planes, const float* sx, const uint32_t* b, float* c, uint32_t m, uint32_t k,
                    uint32_t n, uint32_t bs, uint32_t stride, uint32_t bpc, float* part, uint32_t max_shares,
                    hipStream_t s);
+
+int q8_gemm_blocks_f16(const _Float16* planes, const float* sx, const uint32_t* b, float* c, uint32_t m, uint32_t k,
+                       uint32_t n, uint32_t bs, uint32_t stride, uint32_t bpc, float* part, uint32_t max_shares,
+                       hipStream_t s);
 
 static int matmul_q8_mfma_blocks(const float* a, const uint32_t* b, float* c, uint32_t m, uint32_t k, uint32_t n,
                                  uint32_t bs, uint32_t stride, uint32_t bpc, hipStream_t s) {
@@ -403,6 +445,14 @@ static int matmul_q8_mfma_blocks(const float* a, const uint32_t* b, float* c, ui
     int8_t* planes = static_cast<int8_t*>(ws);
     float* sxp = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + planes_bytes);
     float* part = max_shares ? reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + planes_bytes + sx_bytes) : nullptr;
+    // small blocks (a fold at every or every other 32 k) and larger batches: two f16 planes; otherwise four
+    // exact digit planes on the int8 matrix cores
+    if (bs <= 64 || m > 64) {
+        _Float16* halves = reinterpret_cast<_Float16*>(ws);    // the same 4 m k bytes
+        hipLaunchKernelGGL(q8_split_rows_f16_kernel, dim3(m), dim3(256), 0, s, a, halves, sxp, m, k);
+        if (int rc = check_launch("q8_split_rows_f16_kernel")) return rc;
+        return q8_gemm_blocks_f16(halves, sxp, b, c, m, k, n, bs, stride, bpc, part, max_shares, s);
+    }
     hipLaunchKernelGGL(q8_split_rows_kernel, dim3(m), dim3(256), 0, s, a, planes, sxp, m, k);
     if (int rc = check_launch("q8_split_rows_kernel")) return rc;
     return q8_gemm_blocks(planes, sxp, b, c, m, k, n, bs, stride, bpc, part, max_shares, s);   // sxp[0 .. m): the rows' 1 / f
@@ -507,12 +557,12 @@ int rumus_hip_matmul_q8(const float* a, const uint32_t* b, float* c, uint32_t m,
     RUMUS_REQUIRE(k > 0, "matmul_q8: k must be > 0");
     uint32_t blocks_per_col = ceil_div(k, block_size);
     uint32_t stride = (4 + block_size + 3) / 4;
-    // Batches go to the int8 matrix cores as four digit planes of the activations.  Measured at
-    // 4096 x 11008 (us, whole call):          rows    5..32    128    512    2048
-    //   block-scale kernel, 32-element blocks         34..38    84    242     900     (few-rows kernel: 7.7 per row,
-    //   block-scale kernel, 128-element blocks        33..36    65    170     600      LDS-tiled kernel: 15 ms at 2048)
-    //   block-scale kernel, one block per column      29..33    65    170
-    //   W8A8 kernel on a dense copy of the weights        62    83    148     526     (one block per column only)
+    // Batches go to the matrix cores.  Measured at 4096 x 11008 (us, whole call):
+    //                                                 rows    5..32    128    512    2048
+    //   block-scale kernels, 32-element blocks (f16)          34..35     66    174     604   (few-rows kernel: 7.7 per row,
+    //   block-scale kernels, 128-element blocks               33..36     60    151     545    LDS-tiled kernel: 15 ms at 2048)
+    //   block-scale kernels, one block per column             29..33     60    151
+    //   W8A8 kernel on a dense copy of the weights                62     83    148     526   (one block per column only)
     const bool aligned = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(c)) & 15) == 0;
     const bool block_kernel = block_size % 32 == 0 && k % block_size == 0 && m >= 5 && aligned &&
                               (uint64_t)k * block_size < (1ull << 32) && (uint64_t)kQ8Planes * m * k < (1ull << 40);

@@ -67,15 +67,19 @@ def test_q8_rejects_bad_block_size(ops):
                                       (8, 48, 20, 48),         # W8A8 kernel on a dense copy: the smallest batch that goes there
                                       (400, 512, 96, 512),     # and from 384 rows on
                                       (1000, 4096, 264, 4096),
-                                      # block scales inside the MFMA loop
+                                      # block scales inside the MFMA loop: f16 planes for blocks up to 64 ...
                                       (5, 64, 64, 32),         # the smallest batch that goes there
-                                      (11, 96, 20, 32),        # a fold per K half, K ends mid-step
+                                      (11, 96, 20, 32),        # a fold per 32 k, K ends mid-step
                                       (100, 1024, 300, 32),
-                                      (12, 192, 40, 96),       # blocks that straddle the K steps
-                                      (40, 4096, 64, 2048),    # two folds per block
                                       (33, 512, 100, 64),
+                                      (1030, 256, 2050, 32),
+                                      # ... and for more than 64 rows
+                                      (70, 480, 40, 96),       # blocks that straddle the K steps, K ends mid-step
                                       (1024, 512, 2048, 128),  # the largest tile
-                                      (1030, 256, 2050, 32)])
+                                      # four int8 digit planes for larger blocks and up to 64 rows
+                                      (12, 192, 40, 96),
+                                      (40, 4096, 64, 2048),    # two folds per block, K shared over workgroups
+                                      (6, 1184, 16, 1184)])    # 37 K halves per block: a fold at every half
 def test_matmul_q8_vs_oracle(ops, m, k, n, bs):
     say(f"matmul_q8 m={m} k={k} n={n} bs={bs}")
     from rumus_amd import nn
@@ -94,13 +98,14 @@ def test_matmul_q8_vs_oracle(ops, m, k, n, bs):
     np.testing.assert_array_equal(deq.reshape(-1), oracle.q8_dequantize(words, k * n, bs))
 
 
-@pytest.mark.parametrize("bs,m", [(512, 64), (32, 64), (128, 64), (512, 400)])
+@pytest.mark.parametrize("bs,m", [(512, 64), (32, 64), (128, 64), (128, 100), (512, 400)])
 def test_matmul_q8_batch_accuracy_and_non_finite_rows(ops, bs, m):
-    # batches: activations go through four 7-bit digit planes and the int8 matrix cores (block
-    # scales inside the loop; 400 rows and one block per column: the W8A8 kernel on a dense copy).
-    # Judged against float64 in units of the summed terms (the planes keep
-    # 28 bits below the row maximum, so a row with one huge entry is the hard case), and a NaN or
-    # infinite activation must poison its own row only.
+    # batches: activations go through four 7-bit digit planes and the int8 matrix cores (block scales
+    # inside the loop; 400 rows and one block per column: the W8A8 kernel on a dense copy) or, for
+    # 32-element blocks and for 100 rows, through two f16 planes and the f16 matrix cores.
+    # Judged against float64 in units of the summed terms (the digit planes keep 28 bits below the
+    # row maximum, so a row with one huge entry is the hard case; the f16 planes keep 22 bits of
+    # every entry), and a NaN or infinite activation must poison its own row only.
     say(f"matmul_q8 digit-plane path bs={bs}")
     rng = np.random.default_rng(77)
     k, n = 512, 96
@@ -117,8 +122,8 @@ def test_matmul_q8_batch_accuracy_and_non_finite_rows(ops, bs, m):
     terms = np.abs(a).astype(np.float64) @ np.abs(deq) + 1e-300
     err_ref = (np.abs(want - exact) / terms).max()
     err_got = (np.abs(got - exact) / terms).max()
-    # ordinary rows come out more accurate than the f32 loop; the row with the outlier keeps 28 bits
-    # below 3e4 for its other entries and lands within a few times the f32 loop's own error
+    # ordinary rows come out at least as accurate as the f32 loop; the row with the outlier lands
+    # within a few times the f32 loop's own error
     assert err_ref < 2e-6 and err_got < 1e-5, (err_got, err_ref)
     assert (np.abs(np.delete(got, 3, axis=0) - np.delete(exact, 3, axis=0)) / np.delete(terms, 3, axis=0)).max() < 1e-7
     assert_close(got, want)
