@@ -89,7 +89,12 @@ int rumus_hip_q8_dequantize(const uint32_t* in, float* out, uint32_t numel,
 /* matmul_q8_dispatch (compute.rs:2021-2060) + matmul_q8_kernel
  * (shaders/matmul_q8.wgsl:37-98): c[m,n] = a[m,k] f32 x Q8 b, where column j
  * of b is the run of ceil(k/block_size) blocks starting at word
- * j*blocks_per_col*stride. */
+ * j*blocks_per_col*stride.  Results are within f32 summation error of the
+ * reference's loop (block_size % 16 != 0: the same operations in the same
+ * order).  Batches of 5 rows or more with block_size % 32 == 0 run on the
+ * matrix cores and use the stream's internal workspace (4 bytes per element
+ * of a, plus partial results for small m; one block per column from 384 rows
+ * on: also a dense copy of b). */
 int rumus_hip_matmul_q8(const float* a, const uint32_t* b, float* c, uint32_t m,
                         uint32_t k, uint32_t n, uint32_t block_size,
                         rumus_hip_stream_t stream);
