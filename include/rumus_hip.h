@@ -86,6 +86,14 @@ int rumus_hip_q8_quantize(const float* in, uint32_t* out, uint32_t numel,
 int rumus_hip_q8_dequantize(const uint32_t* in, float* out, uint32_t numel,
                             uint32_t block_size, rumus_hip_stream_t stream);
 
+/* The same values in the order of the tensor's shape: Tensor::quantize stores
+ * the transposed [N,K] tensor (ops.rs:2307), so rumus_hip_q8_dequantize - like
+ * Tensor::dequantize (ops.rs:2332-2352) - returns [N,K] order under the [K,N]
+ * shape.  This returns out[kk*n + col] = value at flat index col*k + kk, i.e.
+ * the dequantized [K,N] weight; bit-identical values, k*n = numel. */
+int rumus_hip_q8_dequantize_kn(const uint32_t* in, float* out, uint32_t k, uint32_t n,
+                               uint32_t block_size, rumus_hip_stream_t stream);
+
 /* matmul_q8_dispatch (compute.rs:2021-2060) + matmul_q8_kernel
  * (shaders/matmul_q8.wgsl:37-98): c[m,n] = a[m,k] f32 x Q8 b, where column j
  * of b is the run of ceil(k/block_size) blocks starting at word

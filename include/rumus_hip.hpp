@@ -247,6 +247,14 @@ inline DeviceBuffer<float> dequantize(const Q8Tensor& q, hipStream_t stream = nu
     return out;
 }
 
+// The dequantized [K, N] tensor with every value where the shape says it is (the buffer holds the
+// transposed tensor; Tensor::dequantize does not undo that).
+inline DeviceBuffer<float> dequantize_kn(const Q8Tensor& q, hipStream_t stream = nullptr) {
+    DeviceBuffer<float> out(q.numel());
+    check(rumus_hip_q8_dequantize_kn(q.buffer.data(), out.data(), q.k, q.n, q.block_size, stream));
+    return out;
+}
+
 // Tensor::matmul with a Q8 right-hand side (ops.rs:516-545): c[m,n] = a[m,k] x Q8.
 inline DeviceBuffer<float> matmul(const DeviceBuffer<float>& a, uint32_t m, const Q8Tensor& b,
                                   hipStream_t stream = nullptr) {

@@ -46,6 +46,7 @@ PROTOTYPES = {
     "rumus_hip_q8_buf_size": (_u64, [_u64, _u32]),
     "rumus_hip_q8_quantize": (_i32, [_vp, _vp, _u32, _u32, _vp]),
     "rumus_hip_q8_dequantize": (_i32, [_vp, _vp, _u32, _u32, _vp]),
+    "rumus_hip_q8_dequantize_kn": (_i32, [_vp, _vp, _u32, _u32, _u32, _vp]),
     "rumus_hip_matmul_q8": (_i32, [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
     "rumus_hip_add_bias": (_i32, [_vp, _vp, _vp, _u32, _u32, _vp]),
     "rumus_hip_transpose_f32": (_i32, [_vp, _vp, _u32, _u32, _vp]),

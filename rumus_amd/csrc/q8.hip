@@ -285,6 +285,38 @@ static int launch_q8_rows(const float* a, const uint32_t* b, float* c, uint32_t 
     return check_launch("matmul_q8_rows_kernel");
 }
 
+// Dequantize into the tensor's own [K, N] order: the buffer holds the transposed tensor ([N, K]
+// flattened, blocks of bs consecutive elements), so out[kk, col] = value at flat index col * k + kk.
+// 128 k x 32 columns per workgroup through LDS: words are read along k, rows written along n.
+__global__ __launch_bounds__(256) void q8_dequantize_kn_kernel(const uint32_t* __restrict__ in, float* __restrict__ out,
+                                                               uint32_t k, uint32_t n, uint32_t bs, uint32_t stride) {
+    __shared__ float t[32][129];
+    const uint32_t tx = threadIdx.x % 32, ty = threadIdx.x / 32;
+    const uint32_t k0 = blockIdx.x * 128, c0 = blockIdx.y * 32;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t cc = ty + 8 * i, col = c0 + cc;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {                         // element by element: col * k + kk need not be a multiple of 4
+            const uint32_t kk = k0 + 4 * tx + e;
+            float v = 0.0f;
+            if (col < n && kk < k) {
+                const uint64_t idx = (uint64_t)col * k + kk;
+                const uint32_t block = (uint32_t)(idx / bs), pos = (uint32_t)(idx % bs);
+                const uint32_t* ib = in + (uint64_t)block * stride;
+                const int q = (int)(int8_t)((ib[1 + pos / 4] >> (8 * (pos % 4))) & 0xFFu);
+                v = __fmul_rn((float)q, header_scale(ib[0]));
+            }
+            t[cc][4 * tx + e] = v;
+        }
+    }
+    __syncthreads();
+    for (uint32_t r = ty; r < 128; r += 8) {
+        const uint32_t kk = k0 + r, col = c0 + tx;
+        if (kk < k && col < n) out[(uint64_t)kk * n + col] = t[tx][r];
+    }
+}
+
 // ---- batches on the matrix cores (one block per column, i.e. per-output-channel scales) ------
 // f32 activations cannot go into the int8 MFMA directly, but signed 7-bit digits can:
 //   x = (p0 + 128 p1 + 128^2 p2 + 128^3 p3) / f,  f a power of two with |x f| < 2^27 for the row,
@@ -546,6 +578,19 @@ int rumus_hip_q8_dequantize(const uint32_t* in, float* out, uint32_t numel, uint
     hipLaunchKernelGGL(q8_dequantize_kernel, dim3(ceil_div(words, 256)), dim3(256), 0,
                        as_stream(stream), in, out, numel, block_size, stride);
     return check_launch("q8_dequantize_kernel");
+}
+
+int rumus_hip_q8_dequantize_kn(const uint32_t* in, float* out, uint32_t k, uint32_t n, uint32_t block_size,
+                               rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE(block_size > 0 && block_size % 4 == 0,
+                  "dequantize: block_size must be > 0 and divisible by 4 (got %u)", block_size);
+    RUMUS_REQUIRE(in && out, "dequantize: null buffer");
+    if (k == 0 || n == 0) return RUMUS_HIP_OK;
+    RUMUS_REQUIRE(n <= 65535u * 32u, "dequantize: n %u is beyond the grid limit", n);
+    const uint32_t stride = (4 + block_size + 3) / 4;
+    hipLaunchKernelGGL(q8_dequantize_kn_kernel, dim3(ceil_div(k, 128), ceil_div(n, 32)), dim3(256), 0, as_stream(stream),
+                       in, out, k, n, block_size, stride);
+    return check_launch("q8_dequantize_kn_kernel");
 }
 
 int rumus_hip_matmul_q8(const float* a, const uint32_t* b, float* c, uint32_t m, uint32_t k,

@@ -158,6 +158,16 @@ def dequantize(q: Q8Tensor) -> torch.Tensor:
     return ops.q8_dequantize(q.buffer, q.numel(), q.block_size).reshape(q.shape)
 
 
+def dequantize_kn(q: Q8Tensor) -> torch.Tensor:
+    """The dequantized tensor with every value where its shape says it is (``[K, N]`` order):
+    what ``Tensor::dequantize`` would return if it undid the transpose ``quantize`` applies."""
+    if not isinstance(q, Q8Tensor):
+        raise ValueError("dequantize: tensor is not Q8")
+    if len(q.shape) != 2:
+        raise ValueError("dequantize_kn: tensor is not 2-D")
+    return ops.q8_dequantize_kn(q.buffer, q.shape[0], q.shape[1], q.block_size)
+
+
 def matmul(lhs: torch.Tensor, rhs) -> torch.Tensor:
     """``Tensor::matmul`` with a Q8 right-hand side (ops.rs:516-545)."""
     if isinstance(lhs, Q8Tensor):

@@ -13,7 +13,7 @@ from . import _lib
 from ._lib import RumusError, call
 
 __all__ = [
-    "q8_buf_size", "q8_quantize", "q8_dequantize", "matmul_q8", "add_bias", "transpose_f32",
+    "q8_buf_size", "q8_quantize", "q8_dequantize", "q8_dequantize_kn", "matmul_q8", "add_bias", "transpose_f32",
     "i8_quantize_rows", "i8_quantize_cols_t", "i8_gemm", "w4_quantize_pack", "qmatmul_int4",
     "qmatmul_int4_t", "w4_actorder_prepare", "qmatmul_int4_perm", "w4_geometry", "RumusError",
 ]
@@ -62,6 +62,13 @@ def q8_dequantize(words: torch.Tensor, numel: int, block_size: int) -> torch.Ten
     out = torch.empty(numel, dtype=torch.float32, device=words.device)
     call("rumus_hip_q8_dequantize", _dev(words, torch.int32, "in"), out.data_ptr(), numel,
          block_size, _stream())
+    return out
+
+
+def q8_dequantize_kn(words: torch.Tensor, k: int, n: int, block_size: int) -> torch.Tensor:
+    """The dequantized weight in its own ``[k, n]`` order (the buffer holds the transposed tensor)."""
+    out = torch.empty((k, n), dtype=torch.float32, device=words.device)
+    call("rumus_hip_q8_dequantize_kn", _dev(words, torch.int32, "in"), out.data_ptr(), k, n, block_size, _stream())
     return out
 
 

@@ -25,6 +25,7 @@ extern "C" {
     pub fn rumus_hip_q8_buf_size(numel: u64, block_size: u32) -> u64;
     pub fn rumus_hip_q8_quantize(input: *const f32, out: *mut u32, numel: u32, block_size: u32, s: Stream) -> c_int;
     pub fn rumus_hip_q8_dequantize(input: *const u32, out: *mut f32, numel: u32, block_size: u32, s: Stream) -> c_int;
+    pub fn rumus_hip_q8_dequantize_kn(input: *const u32, out: *mut f32, k: u32, n: u32, block_size: u32, s: Stream) -> c_int;
     pub fn rumus_hip_matmul_q8(a: *const f32, b: *const u32, c: *mut f32, m: u32, k: u32, n: u32,
                                block_size: u32, s: Stream) -> c_int;
     pub fn rumus_hip_add_bias(mat: *const f32, bias: *const f32, out: *mut f32, m: u32, n: u32, s: Stream) -> c_int;
@@ -111,6 +112,11 @@ pub fn quantize_dispatch(stream: Stream, input: DevPtr, output: DevPtr, numel: u
 /// `dequantize_dispatch(ctx, input, output, numel, block_size)` (compute.rs:1985-1991).
 pub fn dequantize_dispatch(stream: Stream, input: DevPtr, output: DevPtr, numel: u32, block_size: u32) {
     check(unsafe { rumus_hip_q8_dequantize(input.0 as *const u32, output.0 as *mut f32, numel, block_size, stream) });
+}
+
+/// The dequantized `[k, n]` tensor in the order of its shape (the Q8 buffer holds the transposed tensor).
+pub fn dequantize_kn_dispatch(stream: Stream, input: DevPtr, output: DevPtr, k: u32, n: u32, block_size: u32) {
+    check(unsafe { rumus_hip_q8_dequantize_kn(input.0 as *const u32, output.0 as *mut f32, k, n, block_size, stream) });
 }
 
 /// `matmul_q8_dispatch(ctx, a, b, c, m, k, n, block_size)` (compute.rs:2021-2028).

@@ -85,6 +85,14 @@ static void test_q8(uint32_t m, uint32_t k, uint32_t n, uint32_t bs) {
     CHECK(close(matmul(da, m, q).download(), want, "matmul (Q8 rhs)"), "matmul_q8");
     orc_q8_dequantize(words.data(), deq.data(), k * n, bs);
     CHECK(dequantize(q).download() == deq, "dequantize is not bit-exact");
+    {
+        std::vector<float> kn = dequantize_kn(q).download();
+        bool same = kn.size() == deq.size();
+        for (uint32_t r = 0; same && r < k; r++)
+            for (uint32_t c = 0; c < n; c++)
+                if (kn[(size_t)r * n + c] != deq[(size_t)c * k + r]) { same = false; break; }
+        CHECK(same, "dequantize_kn is not the transposed dequantize");
+    }
 }
 
 static void test_int8_linear(uint32_t m, uint32_t k, uint32_t n) {

@@ -48,6 +48,27 @@ def test_q8_quantize_dequantize_bit_exact(ops, numel, bs):
                                   oracle.q8_dequantize(want, numel, bs))
 
 
+@pytest.mark.parametrize("k,n,bs", [(512, 512, 512), (96, 7, 32), (100, 9, 20), (130, 33, 64), (4096, 264, 4096),
+                                    (257, 70, 8)])
+def test_q8_dequantize_kn_is_the_transposed_dequantize(ops, k, n, bs):
+    # values in the order of the tensor's shape: bit-identical to the reference-order output, moved
+    say(f"q8 dequantize_kn k={k} n={n} bs={bs}")
+    from rumus_amd import nn
+    rng = np.random.default_rng(k + n + bs)
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    words = oracle.tensor_quantize(w, bs)
+    want = oracle.q8_dequantize(words, k * n, bs).reshape(n, k).T
+    got = host(ops.q8_dequantize_kn(dev(words), k, n, bs))
+    np.testing.assert_array_equal(got, want)
+    wq = nn.quantize(dev(w), bs)
+    np.testing.assert_array_equal(host(nn.dequantize_kn(wq)), want)
+    # and it is the weight again, to quantization error: half a step, plus the f16 rounding of the
+    # block scale (2^-11 of the value); blocks line up with columns when bs divides k
+    if k % bs == 0:
+        scale = np.abs(w).reshape(k // bs, bs, n).max(axis=1).repeat(bs, axis=0) / 127.0
+        assert (np.abs(got - w) <= scale * 0.501 + np.abs(w) * 6e-4 + 1e-12).all()
+
+
 def test_q8_rejects_bad_block_size(ops):
     say("q8 bad block size")
     with pytest.raises(ops.RumusError):
