@@ -247,6 +247,13 @@ inline DeviceBuffer<float> dequantize(const Q8Tensor& q, hipStream_t stream = nu
     return out;
 }
 
+// Tensor::data() on a Q8 tensor (core.rs:612-691): dequantize on the GPU, then download.
+inline std::vector<float> data(const Q8Tensor& q, hipStream_t stream = nullptr) {
+    DeviceBuffer<float> f = dequantize(q, stream);
+    check(rumus_hip_sync(stream));
+    return f.download();
+}
+
 // The dequantized [K, N] tensor with every value where the shape says it is (the buffer holds the
 // transposed tensor; Tensor::dequantize does not undo that).
 inline DeviceBuffer<float> dequantize_kn(const Q8Tensor& q, hipStream_t stream = nullptr) {

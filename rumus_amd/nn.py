@@ -137,6 +137,15 @@ class Q8Tensor:
     def numel(self) -> int:
         return self.shape[0] * self.shape[1]
 
+    def data(self):
+        """``Tensor::data()`` on a Q8 tensor (core.rs:612-691): dequantize on the GPU, download the
+        f32 values (buffer order, as the reference does) and keep the host copy for later calls."""
+        host = getattr(self, "_host", None)
+        if host is None:
+            host = ops.q8_dequantize(self.buffer, self.numel(), self.block_size).cpu().numpy()
+            object.__setattr__(self, "_host", host)
+        return host
+
 
 def quantize(t, block_size: int) -> Q8Tensor:
     """``Tensor::quantize`` (ops.rs:2290-2327): transpose the last two dims, then block-quantize."""

@@ -85,6 +85,7 @@ static void test_q8(uint32_t m, uint32_t k, uint32_t n, uint32_t bs) {
     CHECK(close(matmul(da, m, q).download(), want, "matmul (Q8 rhs)"), "matmul_q8");
     orc_q8_dequantize(words.data(), deq.data(), k * n, bs);
     CHECK(dequantize(q).download() == deq, "dequantize is not bit-exact");
+    CHECK(data(q) == deq, "data() of a Q8 tensor is not the dequantized buffer");
     {
         std::vector<float> kn = dequantize_kn(q).download();
         bool same = kn.size() == deq.size();

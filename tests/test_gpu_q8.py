@@ -62,6 +62,9 @@ def test_q8_dequantize_kn_is_the_transposed_dequantize(ops, k, n, bs):
     np.testing.assert_array_equal(got, want)
     wq = nn.quantize(dev(w), bs)
     np.testing.assert_array_equal(host(nn.dequantize_kn(wq)), want)
+    # Tensor::data() on a Q8 tensor: the dequantized buffer (reference order), downloaded once
+    np.testing.assert_array_equal(wq.data(), oracle.q8_dequantize(words, k * n, bs))
+    assert wq.data() is wq.data()
     # and it is the weight again, to quantization error: half a step, plus the f16 rounding of the
     # block scale (2^-11 of the value); blocks line up with columns when bs divides k
     if k % bs == 0:
