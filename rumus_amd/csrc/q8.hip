@@ -328,19 +328,46 @@ __global__ __launch_bounds__(256) void q8_dequantize_kn_kernel(const uint32_t* _
 // missed the tolerance tenfold, with four the error stays below that of an f32 accumulation.
 constexpr int kQ8Planes = 4;
 
-__global__ __launch_bounds__(256) void q8_split_rows_kernel(const float* __restrict__ a, int8_t* __restrict__ planes,
-                                                            float* __restrict__ sxp, uint32_t m, uint32_t k) {
-    __shared__ uint32_t red[4];
-    const uint32_t row = blockIdx.x, tid = threadIdx.x;
-    const float* ar = a + (uint64_t)row * k;
-    // largest magnitude as bits: orders like the floats, and a NaN sorts above infinity
+// largest magnitude of a row as bits (orders like the floats, and a NaN sorts above infinity).  Rows of
+// up to 8192 elements stay in registers between the two passes: all loads of a thread are in flight at
+// once instead of one trip to memory per 256 elements, and the row is read once.
+constexpr int kSplitCache = 8;                                 // float4 per thread: 256 x 8 x 4 = 8192 elements
+
+__device__ __forceinline__ uint32_t q8_row_amax(const float* __restrict__ ar, uint32_t k, uint32_t tid, bool cached,
+                                                float4 (&v)[kSplitCache], uint32_t* red) {
     uint32_t amax = 0;
-    for (uint32_t j = tid; j < k; j += 256) amax = max(amax, __float_as_uint(ar[j]) & 0x7FFFFFFFu);
+    if (cached) {
+#pragma unroll
+        for (int i = 0; i < kSplitCache; i++) {
+            const uint32_t j = 4 * tid + 1024 * i;
+            v[i] = j < k ? *reinterpret_cast<const float4*>(ar + j) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
+#pragma unroll
+        for (int i = 0; i < kSplitCache; i++)
+            amax = max(max(amax, max(__float_as_uint(v[i].x) & 0x7FFFFFFFu, __float_as_uint(v[i].y) & 0x7FFFFFFFu)),
+                       max(__float_as_uint(v[i].z) & 0x7FFFFFFFu, __float_as_uint(v[i].w) & 0x7FFFFFFFu));
+    } else {
+        for (uint32_t j = 4 * tid; j < k; j += 1024) {
+            const float4 t = *reinterpret_cast<const float4*>(ar + j);
+            amax = max(max(amax, max(__float_as_uint(t.x) & 0x7FFFFFFFu, __float_as_uint(t.y) & 0x7FFFFFFFu)),
+                       max(__float_as_uint(t.z) & 0x7FFFFFFFu, __float_as_uint(t.w) & 0x7FFFFFFFu));
+        }
+    }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) amax = max(amax, (uint32_t)__shfl_xor((int)amax, off));
     if ((tid & 63) == 0) red[tid >> 6] = amax;
     __syncthreads();
-    amax = max(max(red[0], red[1]), max(red[2], red[3]));
+    return max(max(red[0], red[1]), max(red[2], red[3]));
+}
+
+__global__ __launch_bounds__(256) void q8_split_rows_kernel(const float* __restrict__ a, int8_t* __restrict__ planes,
+                                                            float* __restrict__ sxp, uint32_t m, uint32_t k) {
+    __shared__ uint32_t red[4];
+    const uint32_t row = blockIdx.x, tid = threadIdx.x;
+    const float* ar = a + (uint64_t)row * k;                   // k % 4 == 0
+    const bool cached = k <= 1024u * kSplitCache;
+    float4 cache[kSplitCache];
+    const uint32_t amax = q8_row_amax(ar, k, tid, cached, cache, red);
     const uint32_t ebits = amax >> 23;                         // amax = a 2^(ebits-127), 1 <= a < 2
     float f = __uint_as_float((280u - ebits) << 23);           // 2^(153 - ebits): |x f| < 2^27
     uint32_t inv_bits = ebits - 26u;                           // 1 / f = 2^(ebits - 153), biased
@@ -350,14 +377,13 @@ __global__ __launch_bounds__(256) void q8_split_rows_kernel(const float* __restr
         if (ebits == 255) s = __uint_as_float(0x7FC00000u);    // inf / nan in the row: poison it
         sxp[tid * m + row] = s;
     }
-    if (ebits == 255) f = 0.0f;
-    for (uint32_t j = 4 * tid; j < k; j += 1024) {             // k % 4 == 0
-        const float4 v = *reinterpret_cast<const float4*>(ar + j);
+    const bool poisoned = ebits == 255;
+    auto emit = [&](uint32_t j, const float4& v) {
         const float xv[4] = {v.x, v.y, v.z, v.w};
         uint32_t word[kQ8Planes] = {};
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            int rest = (int)rintf(xv[e] * f);                  // exact: f is a power of two, |x f| < 2^27
+            int rest = poisoned ? 0 : (int)rintf(xv[e] * f);   // exact: f is a power of two, |x f| < 2^27
 #pragma unroll
             for (int p = 0; p < kQ8Planes; p++) {
                 const int digit = p + 1 < kQ8Planes ? ((rest + 64) & 127) - 64 : rest;   // the last one: -64 .. 64
@@ -368,6 +394,15 @@ __global__ __launch_bounds__(256) void q8_split_rows_kernel(const float* __restr
 #pragma unroll
         for (int p = 0; p < kQ8Planes; p++)
             *reinterpret_cast<uint32_t*>(planes + ((uint64_t)p * m + row) * k + j) = word[p];
+    };
+    if (cached) {
+#pragma unroll
+        for (int i = 0; i < kSplitCache; i++) {
+            const uint32_t j = 4 * tid + 1024 * i;
+            if (j < k) emit(j, cache[i]);
+        }
+    } else {
+        for (uint32_t j = 4 * tid; j < k; j += 1024) emit(j, *reinterpret_cast<const float4*>(ar + j));
     }
 }
 
@@ -426,14 +461,10 @@ __global__ __launch_bounds__(256) void q8_split_rows_f16_kernel(const float* __r
                                                                 float* __restrict__ sx, uint32_t m, uint32_t k) {
     __shared__ uint32_t red[4];
     const uint32_t row = blockIdx.x, tid = threadIdx.x;
-    const float* ar = a + (uint64_t)row * k;
-    uint32_t amax = 0;
-    for (uint32_t j = tid; j < k; j += 256) amax = max(amax, __float_as_uint(ar[j]) & 0x7FFFFFFFu);
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) amax = max(amax, (uint32_t)__shfl_xor((int)amax, off));
-    if ((tid & 63) == 0) red[tid >> 6] = amax;
-    __syncthreads();
-    amax = max(max(red[0], red[1]), max(red[2], red[3]));
+    const float* ar = a + (uint64_t)row * k;                   // k % 4 == 0
+    const bool cached = k <= 1024u * kSplitCache;
+    float4 cache[kSplitCache];
+    const uint32_t amax = q8_row_amax(ar, k, tid, cached, cache, red);
     const uint32_t ebits = amax >> 23;                         // amax = a 2^(ebits-127), 1 <= a < 2
     const bool poisoned = ebits == 255;                        // inf / nan in the row
     const bool nothing = ebits < 15;                           // zero or below 2^-112: contributes nothing
@@ -442,8 +473,8 @@ __global__ __launch_bounds__(256) void q8_split_rows_f16_kernel(const float* __r
         sx[row] = poisoned ? __uint_as_float(0x7FC00000u) : nothing ? 0.0f : __uint_as_float((ebits - 14u) << 23);
     _Float16* hi = planes + (uint64_t)row * k;
     _Float16* lo = planes + ((uint64_t)m + row) * k;
-    for (uint32_t j = 4 * tid; j < k; j += 1024) {             // k % 4 == 0
-        const float4 v = *reinterpret_cast<const float4*>(ar + j);
+    typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+    auto emit = [&](uint32_t j, const float4& v) {
         const float xv[4] = {v.x, v.y, v.z, v.w};
         _Float16 h[4], l[4];
 #pragma unroll
@@ -452,9 +483,17 @@ __global__ __launch_bounds__(256) void q8_split_rows_f16_kernel(const float* __r
             h[e] = (_Float16)t;
             l[e] = (_Float16)(t - (float)h[e]);
         }
-        typedef _Float16 v4h __attribute__((ext_vector_type(4)));
         *reinterpret_cast<v4h*>(hi + j) = v4h{h[0], h[1], h[2], h[3]};
         *reinterpret_cast<v4h*>(lo + j) = v4h{l[0], l[1], l[2], l[3]};
+    };
+    if (cached) {
+#pragma unroll
+        for (int i = 0; i < kSplitCache; i++) {
+            const uint32_t j = 4 * tid + 1024 * i;
+            if (j < k) emit(j, cache[i]);
+        }
+    } else {
+        for (uint32_t j = 4 * tid; j < k; j += 1024) emit(j, *reinterpret_cast<const float4*>(ar + j));
     }
 }
 
