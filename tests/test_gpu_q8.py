@@ -189,7 +189,9 @@ def test_api_errors_mirror_reference_asserts(ops):
 
 # ---- W8A8 extension -------------------------------------------------------------
 
-@pytest.mark.parametrize("rows,cols", [(32, 512), (7, 100), (3, 4096), (1, 5), (130, 1024)])
+@pytest.mark.parametrize("rows,cols", [(32, 512), (7, 100), (3, 4096), (1, 5), (130, 1024),
+                                       (3, 6000), (5, 11008), (2, 12288),   # rows held in registers: 8 and 12 K
+                                       (2, 12292), (2, 20001)])             # longer rows are read twice
 def test_i8_quantize_rows_bit_exact(ops, rows, cols):
     say(f"i8_quantize_rows {rows}x{cols}")
     rng = np.random.default_rng(rows * cols)
