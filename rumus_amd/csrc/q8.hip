@@ -22,8 +22,16 @@ __device__ __forceinline__ int quant_i8(float v, float inv) {
     return (int)t;
 }
 
-// One wave per block: abs-max by wave reduction, then quantize and pack.
-// quantize.wgsl:29-100.
+__device__ __forceinline__ uint32_t quant_word(const float4& v, float inv) {
+    return ((uint32_t)quant_i8(v.x, inv) & 0xFFu) | (((uint32_t)quant_i8(v.y, inv) & 0xFFu) << 8) |
+           (((uint32_t)quant_i8(v.z, inv) & 0xFFu) << 16) | (((uint32_t)quant_i8(v.w, inv) & 0xFFu) << 24);
+}
+
+// One wave per block: abs-max by wave reduction, then quantize and pack.  quantize.wgsl:29-100.
+// A block of up to 4096 elements stays in registers between the two passes (16 float4 per lane, all
+// loads in flight at once); longer blocks are read twice.
+constexpr int kBlockCache = 16;
+
 __global__ __launch_bounds__(256) void q8_quantize_kernel(const float* __restrict__ in,
                                                           uint32_t* __restrict__ out,
                                                           uint32_t numel, uint32_t bs,
@@ -34,10 +42,21 @@ __global__ __launch_bounds__(256) void q8_quantize_kernel(const float* __restric
     const uint64_t start = (uint64_t)block * bs;
     const uint32_t words = bs / 4;
     const bool full = start + bs <= numel && ((reinterpret_cast<uintptr_t>(in) & 15) == 0);
+    const bool cached = full && words <= 64u * kBlockCache;
+    const float4* p = reinterpret_cast<const float4*>(in + start);
+    float4 cache[kBlockCache];
 
     float amax = 0.0f;
-    if (full) {
-        const float4* p = reinterpret_cast<const float4*>(in + start);
+    if (cached) {
+#pragma unroll
+        for (int i = 0; i < kBlockCache; i++) {
+            const uint32_t w = lane + 64 * i;
+            cache[i] = w < words ? p[w] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
+#pragma unroll
+        for (int i = 0; i < kBlockCache; i++)
+            amax = fmaxf(amax, fmaxf(fmaxf(fabsf(cache[i].x), fabsf(cache[i].y)), fmaxf(fabsf(cache[i].z), fabsf(cache[i].w))));
+    } else if (full) {
         for (uint32_t w = lane; w < words; w += 64) {
             float4 v = p[w];
             amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
@@ -53,16 +72,14 @@ __global__ __launch_bounds__(256) void q8_quantize_kernel(const float* __restric
     uint32_t* ob = out + (uint64_t)block * stride;
     if (lane == 0) ob[0] = (uint32_t)__half_as_ushort(__float2half_rn(scale));  // :71-74
 
-    if (full) {
-        const float4* p = reinterpret_cast<const float4*>(in + start);
-        for (uint32_t w = lane; w < words; w += 64) {
-            float4 v = p[w];
-            uint32_t word = ((uint32_t)quant_i8(v.x, inv) & 0xFFu) |
-                            (((uint32_t)quant_i8(v.y, inv) & 0xFFu) << 8) |
-                            (((uint32_t)quant_i8(v.z, inv) & 0xFFu) << 16) |
-                            (((uint32_t)quant_i8(v.w, inv) & 0xFFu) << 24);
-            ob[1 + w] = word;
+    if (cached) {
+#pragma unroll
+        for (int i = 0; i < kBlockCache; i++) {
+            const uint32_t w = lane + 64 * i;
+            if (w < words) ob[1 + w] = quant_word(cache[i], inv);
         }
+    } else if (full) {
+        for (uint32_t w = lane; w < words; w += 64) ob[1 + w] = quant_word(p[w], inv);
     } else {
         for (uint32_t w = lane; w < words; w += 64) {
             uint32_t word = 0;
@@ -74,6 +91,40 @@ __global__ __launch_bounds__(256) void q8_quantize_kernel(const float* __restric
             ob[1 + w] = word;
         }
     }
+}
+
+// Blocks of up to 256 elements: LPB lanes per block (one float4 each), 256 / LPB blocks per
+// workgroup, so that a 32-element block does not leave 56 lanes of a wave idle.
+template <int LPB>
+__global__ __launch_bounds__(256) void q8_quantize_small_kernel(const float* __restrict__ in, uint32_t* __restrict__ out,
+                                                                uint32_t numel, uint32_t bs, uint32_t num_blocks,
+                                                                uint32_t stride) {
+    const uint32_t sub = threadIdx.x % LPB;
+    const uint32_t block = blockIdx.x * (256 / LPB) + threadIdx.x / LPB;
+    if (block >= num_blocks) return;                           // whole groups of LPB lanes leave together
+    const uint64_t start = (uint64_t)block * bs;
+    const uint32_t words = bs / 4;                             // <= LPB
+    const bool full = start + bs <= numel && ((reinterpret_cast<uintptr_t>(in) & 15) == 0);
+    float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (sub < words) {
+        if (full) {
+            v = reinterpret_cast<const float4*>(in + start)[sub];
+        } else {
+            const uint64_t g = start + 4 * sub;
+            v.x = g < numel ? in[g] : 0.0f;
+            v.y = g + 1 < numel ? in[g + 1] : 0.0f;
+            v.z = g + 2 < numel ? in[g + 2] : 0.0f;
+            v.w = g + 3 < numel ? in[g + 3] : 0.0f;
+        }
+    }
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+#pragma unroll
+    for (int off = LPB / 2; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
+    const float scale = amax == 0.0f ? 1.0f : __fdiv_rn(amax, 127.0f);  // :66
+    const float inv = amax == 0.0f ? 0.0f : __fdiv_rn(127.0f, amax);    // :67
+    uint32_t* ob = out + (uint64_t)block * stride;
+    if (sub == 0) ob[0] = (uint32_t)__half_as_ushort(__float2half_rn(scale));  // :71-74
+    if (sub < words) ob[1 + sub] = quant_word(v, inv);         // elements past numel quantize to 0
 }
 
 __device__ __forceinline__ float header_scale(uint32_t header) {
@@ -601,8 +652,22 @@ int rumus_hip_q8_quantize(const float* in, uint32_t* out, uint32_t numel, uint32
     if (numel == 0) return RUMUS_HIP_OK;
     uint32_t num_blocks = ceil_div(numel, block_size);
     uint32_t stride = (4 + block_size + 3) / 4;
-    hipLaunchKernelGGL(q8_quantize_kernel, dim3(ceil_div(num_blocks, 4)), dim3(256), 0,
-                       as_stream(stream), in, out, numel, block_size, num_blocks, stride);
+    hipStream_t s = as_stream(stream);
+    if (block_size <= 32)
+        hipLaunchKernelGGL(q8_quantize_small_kernel<8>, dim3(ceil_div(num_blocks, 32)), dim3(256), 0, s, in, out, numel,
+                           block_size, num_blocks, stride);
+    else if (block_size <= 64)
+        hipLaunchKernelGGL(q8_quantize_small_kernel<16>, dim3(ceil_div(num_blocks, 16)), dim3(256), 0, s, in, out, numel,
+                           block_size, num_blocks, stride);
+    else if (block_size <= 128)
+        hipLaunchKernelGGL(q8_quantize_small_kernel<32>, dim3(ceil_div(num_blocks, 8)), dim3(256), 0, s, in, out, numel,
+                           block_size, num_blocks, stride);
+    else if (block_size <= 256)
+        hipLaunchKernelGGL(q8_quantize_small_kernel<64>, dim3(ceil_div(num_blocks, 4)), dim3(256), 0, s, in, out, numel,
+                           block_size, num_blocks, stride);
+    else
+        hipLaunchKernelGGL(q8_quantize_kernel, dim3(ceil_div(num_blocks, 4)), dim3(256), 0, s, in, out, numel,
+                           block_size, num_blocks, stride);
     return check_launch("q8_quantize_kernel");
 }
 
