@@ -136,20 +136,23 @@ __global__ __launch_bounds__(256) void q8_dequantize_kernel(const uint32_t* __re
                                                             float* __restrict__ out,
                                                             uint32_t numel, uint32_t bs,
                                                             uint32_t stride) {
-    const uint64_t w = (uint64_t)blockIdx.x * 256 + threadIdx.x;  // data-word index
-    const uint64_t e0 = w * 4;
-    if (e0 >= numel) return;
-    const uint32_t block = (uint32_t)(e0 / bs);
-    const uint32_t pos = (uint32_t)(e0 % bs);
+    const uint32_t w = blockIdx.x * 256 + threadIdx.x;         // data-word index; numel fits 32 bits
+    if (w >= numel / 4 + (numel % 4 != 0)) return;
+    const uint32_t e0 = w * 4;                                 // < numel <= 2^32 - 1: the last word starts below 2^32 - 3
+    const uint32_t block = e0 / bs;
+    const uint32_t pos = e0 - block * bs;
     const uint32_t* ib = in + (uint64_t)block * stride;
     const float scale = header_scale(ib[0]);
     const uint32_t word = ib[1 + pos / 4];
+    float v[4];
 #pragma unroll
-    for (int b = 0; b < 4; b++) {
-        if (e0 + b < numel) {
-            int q = (int)(int8_t)((word >> (8 * b)) & 0xFFu);
-            out[e0 + b] = __fmul_rn((float)q, scale);
-        }
+    for (int b = 0; b < 4; b++) v[b] = __fmul_rn((float)(int)(int8_t)((word >> (8 * b)) & 0xFFu), scale);
+    if (numel - e0 >= 4 && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+        *reinterpret_cast<float4*>(out + e0) = make_float4(v[0], v[1], v[2], v[3]);
+    } else {
+#pragma unroll
+        for (int b = 0; b < 4; b++)
+            if (b < (int)(numel - e0)) out[e0 + b] = v[b];
     }
 }
 
@@ -632,6 +635,33 @@ __global__ __launch_bounds__(256) void transpose_kernel(const float* __restrict_
     }
 }
 
+// 64x64 tile, 128-bit accesses on both sides (rows % 4 == 0, cols % 4 == 0, 16-byte aligned buffers).
+// Thread (q = tid % 16, p = tid / 16): reads float4 at row p + 16 i, columns 4 q .. 4 q + 3; writes the
+// float4 of output row (= input column) p + 16 i, output columns (= input rows) 4 q .. 4 q + 3, which it
+// gathers from LDS rows of 65 floats: bank 4 q + e + p + 16 i (mod 64), distinct across a wave.
+__global__ __launch_bounds__(256) void transpose64_kernel(const float* __restrict__ in, float* __restrict__ out,
+                                                          uint32_t rows, uint32_t cols) {
+    __shared__ float t[64][65];
+    const uint32_t q = threadIdx.x % 16, p = threadIdx.x / 16;
+    const uint32_t r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t r = r0 + p + 16 * i, cc = c0 + 4 * q;
+        float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (r < rows && cc < cols) v = *reinterpret_cast<const float4*>(in + (uint64_t)r * cols + cc);
+        float* d = &t[p + 16 * i][4 * q];
+        d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t cc = c0 + p + 16 * i, r = r0 + 4 * q;
+        if (cc < cols && r < rows)
+            *reinterpret_cast<float4*>(out + (uint64_t)cc * rows + r) =
+                make_float4(t[4 * q][p + 16 * i], t[4 * q + 1][p + 16 * i], t[4 * q + 2][p + 16 * i], t[4 * q + 3][p + 16 * i]);
+    }
+}
+
 }  // namespace rumus
 
 using namespace rumus;
@@ -678,7 +708,7 @@ int rumus_hip_q8_dequantize(const uint32_t* in, float* out, uint32_t numel, uint
     RUMUS_REQUIRE(in && out, "dequantize: null buffer");
     if (numel == 0) return RUMUS_HIP_OK;
     uint32_t stride = (4 + block_size + 3) / 4;
-    uint32_t words = ceil_div(numel, 4);
+    uint32_t words = numel / 4 + (numel % 4 != 0);
     hipLaunchKernelGGL(q8_dequantize_kernel, dim3(ceil_div(words, 256)), dim3(256), 0,
                        as_stream(stream), in, out, numel, block_size, stride);
     return check_launch("q8_dequantize_kernel");
@@ -769,6 +799,13 @@ int rumus_hip_transpose_f32(const float* in, float* out, uint32_t rows, uint32_t
                             rumus_hip_stream_t stream) {
     RUMUS_REQUIRE(in && out, "transpose: null buffer");
     if (rows == 0 || cols == 0) return RUMUS_HIP_OK;
+    if (rows % 4 == 0 && cols % 4 == 0 &&
+        ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
+        RUMUS_REQUIRE(ceil_div(rows, 64) <= 65535, "transpose: rows %u beyond the grid limit", rows);
+        hipLaunchKernelGGL(transpose64_kernel, dim3(ceil_div(cols, 64), ceil_div(rows, 64)), dim3(256), 0,
+                           as_stream(stream), in, out, rows, cols);
+        return check_launch("transpose64_kernel");
+    }
     dim3 grid(ceil_div(cols, 32), ceil_div(rows, 32));
     hipLaunchKernelGGL(transpose_kernel, grid, dim3(256), 0, as_stream(stream), in, out, rows, cols);
     return check_launch("transpose_kernel");

@@ -72,6 +72,17 @@ def test_q8_dequantize_kn_is_the_transposed_dequantize(ops, k, n, bs):
         assert (np.abs(got - w) <= scale * 0.501 + np.abs(w) * 6e-4 + 1e-12).all()
 
 
+@pytest.mark.parametrize("rows,cols", [(64, 64), (4096, 264), (1000, 4100), (1001, 4101), (4, 8), (3, 1), (1, 7),
+                                       (68, 132), (130, 64)])
+def test_transpose_is_exact(ops, rows, cols):
+    # the transpose in front of the block quantizer (ops.rs:2307); 64 x 64 tiles with 128-bit accesses
+    # when both sides are multiples of 4, 32 x 32 tiles otherwise
+    say(f"transpose rows={rows} cols={cols}")
+    rng = np.random.default_rng(rows * 7 + cols)
+    w = rng.normal(0, 1, (rows, cols)).astype(np.float32)
+    np.testing.assert_array_equal(host(ops.transpose_f32(dev(w))), np.ascontiguousarray(w.T))
+
+
 def test_q8_rejects_bad_block_size(ops):
     say("q8 bad block size")
     with pytest.raises(ops.RumusError):
