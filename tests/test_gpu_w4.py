@@ -271,7 +271,14 @@ def test_act_order_rejects_unbalanced_groups(ops):
         ops.w4_actorder_prepare(dev(np.zeros((k // 8, n), np.uint32)), dev(bad), g)
 
 
-@pytest.mark.parametrize("m,k,n,g", [(3, 72, 20, 8), (16, 512, 300, 128), (1, 1000, 64, 64)])
+@pytest.mark.parametrize("m,k,n,g", [(3, 72, 20, 8), (16, 512, 300, 128), (1, 1000, 64, 64),
+                                     # from 16 rows on and group % 128 == 0: the f16 matrix cores
+                                     (64, 4096, 1100, 128),     # n shared over workgroups
+                                     (130, 1000, 264, 128),     # k ends inside the last group, three row tiles
+                                     (100, 256, 4100, 256),     # n ends 4 past a step of 32
+                                     (2050, 256, 516, 128),     # many row tiles
+                                     (16, 128, 4, 128),         # the smallest n
+                                     (40, 512, 300, 64)])       # other group sizes keep the vector kernel
 def test_qmatmul_int4_transpose(ops, m, k, n, g):
     say(f"qmatmul_int4_t m={m} k={k} n={n} g={g}")
     rng = np.random.default_rng(k + n)
@@ -282,6 +289,39 @@ def test_qmatmul_int4_transpose(ops, m, k, n, g):
     got = host(ops.qmatmul_int4_t(dev(gy), dev(packed), dev(scales), dev(zp), k, g))
     assert got.shape == (m, k)
     assert_close(got, want)
+
+
+def test_qmatmul_int4_transpose_scaling_and_non_finite_rows(ops):
+    # the matrix-core grad_x rescales every row of grad_y and the scales by powers of two: rows of very
+    # different magnitude, tiny and huge scales, a zero row; inf / nan poison their own row only
+    say("qmatmul_int4_t row scaling")
+    rng = np.random.default_rng(11)
+    m, k, n, g = 48, 256, 520, 128
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    w[:, :100] *= 1e-4                                       # scales over four decades
+    w[:, 100:200] *= 50.0
+    gy = rng.normal(0, 1, (m, n)).astype(np.float32)
+    gy[1] *= 1e-12
+    gy[2] *= 1e9
+    gy[3, 7] = 2.0e4                                         # dwarfs the rest of its row
+    gy[4] = 0.0
+    packed, scales, zp = oracle.w4_from_f32(w, g)
+    d = [dev(a) for a in (packed, scales, zp)]
+    want = oracle.qmatmul_int4_t(gy, packed, scales, zp, k, g, threads=8)
+    got = host(ops.qmatmul_int4_t(dev(gy), *d, k, g))
+    # judged in units of the summed terms, like the forward kernels with wide-ranging operands
+    deq = oracle.w4_dequant(packed, scales, zp, k, g).astype(np.float64)          # [k, n]
+    exact = gy.astype(np.float64) @ deq.T
+    terms = np.abs(gy).astype(np.float64) @ np.abs(deq).T + 1e-300
+    assert (np.abs(want - exact) / terms).max() < 2e-6                            # the f32 loop itself
+    assert (np.abs(got - exact) / terms).max() < 2e-6
+    np.testing.assert_array_equal(got[4], np.zeros(k, np.float32))
+    for bad in (np.float32(np.nan), np.float32(np.inf)):
+        gb = gy.copy()
+        gb[9, 33] = bad
+        out = host(ops.qmatmul_int4_t(dev(gb), *d, k, g))
+        assert np.isnan(out[9]).all()
+        np.testing.assert_array_equal(np.delete(out, 9, axis=0), np.delete(got, 9, axis=0))
 
 
 def test_gptq_actorder_config_full_size(ops):
