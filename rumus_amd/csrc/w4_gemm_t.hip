@@ -12,10 +12,10 @@
 // accuracy: the 2^-23 the f16 planes lose of A is then multiplied by q instead of by q - zp, which
 // near-zero weights make many times larger than the term itself.)  A workgroup owns 64 rows x 128 consecutive k of one
 // group (group_size % 128 == 0) and walks n in steps of 32:
-//   * staging (all 256 threads, 8 values each): a = (gy f_row) (s / S) with f_row and S powers of two
+//   * conversion (all 256 threads, 8 values each): a = (gy f_row) (s / S) with f_row and S powers of two
 //     that put |a| below 2^14 (w4t_prepare_kernel: row maxima of gy, maximum of the scales), split into
 //     hi + lo f16 (22 bits), written to LDS in A-fragment rows of 64 bytes; c accumulates in f32;
-//   * every wave owns 32 of the 128 k: lane (k = lane % 32, half = lane / 32) loads the 8 consecutive
+//   * every wave owns 32 of the 128 k: lane (k = lane % 32, half = lane / 32) reads the 8 consecutive
 //     words of word row k / 8 that hold its 8 values of n, takes nibble k % 8 of each, and splices them
 //     under the mantissa of 1024 (minus 1024, two at a time): 20 instructions per B fragment, which
 //     serves 4 MFMAs (two row tiles x hi, lo);
@@ -30,140 +30,184 @@ typedef _Float16 t8h __attribute__((ext_vector_type(8)));
 typedef _Float16 t2h __attribute__((ext_vector_type(2)));
 typedef float t16f __attribute__((ext_vector_type(16)));
 
-constexpr int kTScaleParts = 64;                               // partial maxima of the scales
 constexpr int kTMaxSplits = 8;
 
-// blocks [0, m): f_row = 2^(140 - e) for a row maximum a 2^(e - 127), 1 <= a < 2, so |gy f| < 2^14
-// (0 for an all-zero or tiny row, NaN marker for a row with inf / nan); blocks [m, m + 64): partial
-// maxima of the scales as bits.
+// Per call, before the GEMM:
+//   blocks [0, m): f_row = 2^(140 - e) for a row maximum a 2^(e - 127), 1 <= a < 2, so |gy f| < 2^14
+//       (0 for an all-zero or tiny row, NaN marker for a row with inf / nan);
+//   blocks [m, m + groups): for group g, S_g = the power of two at or above its largest scale, and per
+//       column the three things the GEMM needs of scale and zero-point: s / S_g (f32, at most 1),
+//       zp - rint(zp) (f32) and 1024 + rint(zp) (f16), so that no workgroup works them out again.
+//       sgrp[g] = S_g; 0 when every scale of the group is zero or denormal, NaN when one is not finite
+//       or S_g or 1 / S_g would leave the normal range: the GEMM then writes zeros / NaNs for the group.
 __global__ __launch_bounds__(256) void w4t_prepare_kernel(const float* __restrict__ gy, const float* __restrict__ scales,
-                                                          float* __restrict__ rowf, uint32_t* __restrict__ smax_part,
-                                                          uint32_t m, uint32_t n, uint64_t nscales) {
+                                                          const float* __restrict__ zp, float* __restrict__ rowf,
+                                                          float* __restrict__ sgrp, float* __restrict__ sp,
+                                                          float* __restrict__ zf, _Float16* __restrict__ zo,
+                                                          uint32_t m, uint32_t n) {
     __shared__ uint32_t red[4];
     const uint32_t tid = threadIdx.x;
+    const bool is_row = blockIdx.x < m;
+    const float* r = is_row ? gy + (uint64_t)blockIdx.x * n : scales + (uint64_t)(blockIdx.x - m) * n;   // n % 4 == 0, aligned
     uint32_t amax = 0;
-    if (blockIdx.x < m) {
-        const float* r = gy + (uint64_t)blockIdx.x * n;        // n % 4 == 0, 16-byte aligned
-        for (uint32_t j = 4 * tid; j < n; j += 1024) {
-            const float4 t = *reinterpret_cast<const float4*>(r + j);
-            amax = max(max(amax, max(__float_as_uint(t.x) & 0x7FFFFFFFu, __float_as_uint(t.y) & 0x7FFFFFFFu)),
-                       max(__float_as_uint(t.z) & 0x7FFFFFFFu, __float_as_uint(t.w) & 0x7FFFFFFFu));
-        }
-    } else {
-        const uint32_t part = blockIdx.x - m;
-        const uint64_t per = (nscales + kTScaleParts - 1) / kTScaleParts;
-        const uint64_t lo = part * per, hi = min(nscales, lo + per);
-        for (uint64_t j = lo + tid; j < hi; j += 256) amax = max(amax, __float_as_uint(scales[j]) & 0x7FFFFFFFu);
+#pragma unroll 4
+    for (uint32_t j = 4 * tid; j < n; j += 1024) {
+        const float4 t = *reinterpret_cast<const float4*>(r + j);
+        amax = max(max(amax, max(__float_as_uint(t.x) & 0x7FFFFFFFu, __float_as_uint(t.y) & 0x7FFFFFFFu)),
+                   max(__float_as_uint(t.z) & 0x7FFFFFFFu, __float_as_uint(t.w) & 0x7FFFFFFFu));
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) amax = max(amax, (uint32_t)__shfl_xor((int)amax, off));
     if ((tid & 63) == 0) red[tid >> 6] = amax;
     __syncthreads();
-    if (tid != 0) return;
     amax = max(max(red[0], red[1]), max(red[2], red[3]));
-    if (blockIdx.x >= m) {
-        smax_part[blockIdx.x - m] = amax;
+    if (is_row) {
+        const uint32_t e = amax >> 23;
+        if (tid == 0)
+            rowf[blockIdx.x] = e >= 255 ? __uint_as_float(0x7FC00000u) : e < 14 ? 0.0f : __uint_as_float((267u - e) << 23);
         return;
     }
-    const uint32_t e = amax >> 23;
-    float f = e >= 255 ? __uint_as_float(0x7FC00000u) : e < 14 ? 0.0f : __uint_as_float((267u - e) << 23);
-    rowf[blockIdx.x] = f;
+    const uint32_t g = blockIdx.x - m;
+    const uint32_t se = (amax >> 23) + ((amax & 0x7FFFFFu) ? 1u : 0u);      // S_g = 2^(se - 127)
+    const bool ok = se >= 1 && se <= 253;                      // S_g and 1 / S_g are normal floats
+    const float s_inv = ok ? __uint_as_float((254u - se) << 23) : 0.0f;
+    if (tid == 0) sgrp[g] = ok ? __uint_as_float(se << 23) : (amax >= 0x7F000000u ? __uint_as_float(0x7FC00000u) : 0.0f);
+    const float* zr = zp + (uint64_t)g * n;
+    typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+#pragma unroll 4
+    for (uint32_t j = 4 * tid; j < n; j += 1024) {             // independent iterations: their loads overlap
+        const float4 sv = *reinterpret_cast<const float4*>(r + j), z = *reinterpret_cast<const float4*>(zr + j);
+        const float4 z0 = make_float4(rintf(z.x), rintf(z.y), rintf(z.z), rintf(z.w));
+        // s / S_g is exact (a power of two); 1024 + z0 is exact for |z0| <= 1024, zero-points are 0 .. 15
+        *reinterpret_cast<float4*>(sp + (uint64_t)g * n + j) = make_float4(sv.x * s_inv, sv.y * s_inv, sv.z * s_inv, sv.w * s_inv);
+        *reinterpret_cast<float4*>(zf + (uint64_t)g * n + j) = make_float4(z.x - z0.x, z.y - z0.y, z.z - z0.z, z.w - z0.w);
+        *reinterpret_cast<v4h*>(zo + (uint64_t)g * n + j) =
+            v4h{(_Float16)(1024.0f + z0.x), (_Float16)(1024.0f + z0.y), (_Float16)(1024.0f + z0.z), (_Float16)(1024.0f + z0.w)};
+    }
 }
 
 // One workgroup: rows [64 y, 64 y + 64), k [128 x, 128 x + 128), n steps [z steps_per, ..).
+//
+// Operands travel global -> LDS by direct-to-LDS loads, kTStages steps deep: per step the raw tile of
+// grad_y (64 rows x 32 floats), the 16 word rows x 32 words of the weights and the group's 32 scaled
+// scales, 32 zero-point fractions and 32 f16 zero-point integers, 10.5 KB.  The raw tile of step t+1
+// is converted into the A-fragment buffer (double-buffered) while the MFMAs of step t run; one barrier
+// per step.
+constexpr int kTRawGy = 64 * 128, kTRawW = 16 * 128, kTRawSz = 256, kTRawZo = 256;   // 64 bytes of zero-point integers used
+constexpr int kTRaw = kTRawGy + kTRawW + kTRawSz + kTRawZo;   // bytes of one raw stage
+constexpr int kTAbuf = 2 * 64 * 64;                           // hi, lo planes
+constexpr int kTLoads = 3;                                    // wave-wide loads per wave and step: 12 in all
+constexpr size_t w4t_lds_bytes(int stages) { return (size_t)stages * kTRaw + 2 * kTAbuf + 64 * sizeof(float); }
+
+template <int kTStages>
 __global__ __launch_bounds__(256, 2) void w4t_gemm_kernel(
-    const float* __restrict__ gy, const uint32_t* __restrict__ packed, const float* __restrict__ scales,
-    const float* __restrict__ zp, const float* __restrict__ rowf, const uint32_t* __restrict__ smax_part,
-    float* __restrict__ out, uint32_t m, uint32_t k, uint32_t n, uint32_t gs, uint32_t steps_per) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds_a[2][2][64 * 64];   // [buffer][hi, lo][row][32 n] f16
-    __shared__ __attribute__((aligned(16))) _Float16 lds_z[2][32];          // [buffer][n]: 1024 + z0
-    __shared__ float lds_c[64];
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const float* __restrict__ gy, const uint32_t* __restrict__ packed, const float* __restrict__ sp,
+    const float* __restrict__ zf, const _Float16* __restrict__ zo, const float* __restrict__ rowf,
+    const float* __restrict__ sgrp, float* __restrict__ out, uint32_t m, uint32_t k, uint32_t n, uint32_t gs,
+    uint32_t steps_per) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    uint8_t* const raw = lds;                                  // [kTStages][kTRaw]
+    uint8_t* const abuf = lds + kTStages * kTRaw;              // [2][kTAbuf]
+    float* const lds_c = reinterpret_cast<float*>(abuf + 2 * kTAbuf);
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t k0 = blockIdx.x * 128, m0 = blockIdx.y * 64;
     const uint32_t g = k0 / gs;
     const uint32_t nsteps = (n + 31) / 32;
-    const uint32_t st0 = blockIdx.z * steps_per, st1 = min(nsteps, st0 + steps_per);
+    const uint32_t st0 = blockIdx.z * steps_per, st1 = min(nsteps, st0 + steps_per);   // st0 < st1 by the launch
 
-    // ---- S: the power of two at or above the largest scale -------------------------------------------
-    uint32_t smax = smax_part[lane];                           // kTScaleParts == 64
+    // ---- global side of the direct-to-LDS loads: load q = 4 i + wave of a step --------------------------
+    //   q 0..7: rows 8 q .. 8 q + 7 of grad_y (lane: row lane / 8, floats 4 (lane % 8) .. + 3)
+    //   q 8, 9: word rows 8 (q - 8) .. + 7 of the weights (lane: row lane / 8, words 4 (lane % 8) .. + 3)
+    //   q 10: lanes 0..31 scaled scale, 32..63 zero-point fraction of column lane % 32
+    //   q 11: lanes 0..15 two f16 zero-point integers each (columns 2 lane, 2 lane + 1); the other lanes
+    //         fetch the same words again, into the unused tail of the stage
+    const uint32_t l8 = lane >> 3, p8 = lane & 7;
+    const uint8_t* src[kTLoads];
+    uint32_t dst[kTLoads], colw[kTLoads], esz[kTLoads];        // colw: the lane's first column inside a step
+    bool wide[kTLoads];
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) smax = max(smax, (uint32_t)__shfl_xor((int)smax, off));
-    const uint32_t se = (smax >> 23) + ((smax & 0x7FFFFFu) ? 1u : 0u);      // S = 2^(se - 127)
-    // se in 1 .. 253: both S and 1 / S are normal floats; otherwise (all scales zero or denormal,
-    // or huge / inf / nan) the workgroup writes what the plain product would: zeros or NaNs
-    const bool s_ok = se >= 1 && se <= 253;
-    const float s_inv = s_ok ? __uint_as_float((254u - se) << 23) : 0.0f;
-    const float s_big = s_ok ? __uint_as_float(se << 23) : (smax >= 0x7F000000u ? __uint_as_float(0x7FC00000u) : 0.0f);
+    for (int i = 0; i < kTLoads; i++) {
+        const uint32_t q = 4 * i + wave;
+        if (q < 8) {
+            const uint32_t row = min(m0 + 8 * q + l8, m - 1);
+            src[i] = reinterpret_cast<const uint8_t*>(gy + (uint64_t)row * n);
+            dst[i] = q * 1024; colw[i] = 4 * p8; wide[i] = true; esz[i] = 4;
+        } else if (q < 10) {
+            const uint32_t wr = k0 / 8 + 8 * (q - 8) + l8;     // < padded_k / 8: whole groups exist in the arrays
+            src[i] = reinterpret_cast<const uint8_t*>(packed + (uint64_t)wr * n);
+            dst[i] = kTRawGy + (q - 8) * 1024; colw[i] = 4 * p8; wide[i] = true; esz[i] = 4;
+        } else if (q == 10) {
+            src[i] = reinterpret_cast<const uint8_t*>((lane < 32 ? sp : zf) + (uint64_t)g * n);
+            dst[i] = kTRawGy + kTRawW; colw[i] = lane & 31; wide[i] = false; esz[i] = 4;
+        } else {
+            src[i] = reinterpret_cast<const uint8_t*>(zo + (uint64_t)g * n);
+            dst[i] = kTRawGy + kTRawW + kTRawSz; colw[i] = 2 * (lane & 15); wide[i] = false; esz[i] = 2;
+        }
+    }
+    // columns past n are fetched from column 0: the conversion turns them into zeros
+    auto issue = [&](uint32_t st, uint32_t stage) {
+        uint8_t* base = raw + stage * kTRaw;
+        const uint32_t c0 = min(st, st1 - 1) * 32;
+#pragma unroll
+        for (int i = 0; i < kTLoads; i++) {
+            const uint32_t col = c0 + colw[i] < n ? c0 + colw[i] : 0;
+            if (wide[i])
+                __builtin_amdgcn_global_load_lds((gptr_t)(src[i] + (uint64_t)col * esz[i]), (lptr_t)(base + dst[i]), 16, 0, 0);
+            else
+                __builtin_amdgcn_global_load_lds((gptr_t)(src[i] + (uint64_t)col * esz[i]), (lptr_t)(base + dst[i]), 4, 0, 0);
+        }
+    };
 
-    // ---- staging role: 8 consecutive n (chunk tid % 4) of row tid / 4 --------------------------------
+    // ---- conversion role: 8 consecutive n (chunk tid % 4) of row tid / 4 ------------------------------
     const uint32_t s_row = tid >> 2, s_ch = tid & 3;
-    const uint32_t grow = min(m0 + s_row, m - 1);
-    const float frow_raw = rowf[grow];
-    const bool row_bad = frow_raw != frow_raw;                 // inf / nan in the row of gy
-    const float frow = row_bad ? 0.0f : frow_raw;
-    const float* gy_r = gy + (uint64_t)grow * n;
-    const float* sc_g = scales + (uint64_t)g * n;
-    const float* zp_g = zp + (uint64_t)g * n;
+    const float frow_raw = rowf[min(m0 + s_row, m - 1)];
+    const float frow = frow_raw != frow_raw ? 0.0f : frow_raw; // inf / nan in the row: NaN times 0 poisons it below
     const uint32_t s_lds = s_row * 64 + ((s_ch ^ row_swizzle(s_row)) & 3) * 16;
-    float4 gv0, gv1, sv0, sv1, zv0, zv1;
-    auto load_stage = [&](uint32_t st) {
-        const uint32_t c0 = st * 32 + s_ch * 8;
-        const bool in0 = c0 < n, in1 = c0 + 4 < n;             // n % 4 == 0: a float4 is all-in or all-out
-        const uint32_t a0 = in0 ? c0 : 0, a1 = in1 ? c0 + 4 : 0;
-        gv0 = *reinterpret_cast<const float4*>(gy_r + a0);
-        gv1 = *reinterpret_cast<const float4*>(gy_r + a1);
-        sv0 = *reinterpret_cast<const float4*>(sc_g + a0);
-        sv1 = *reinterpret_cast<const float4*>(sc_g + a1);
-        zv0 = *reinterpret_cast<const float4*>(zp_g + a0);
-        zv1 = *reinterpret_cast<const float4*>(zp_g + a1);
-        if (!in0) gv0 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        if (!in1) gv1 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-    };
     float csum = 0.0f;
-    auto store_stage = [&](int buf) {
-        const float gvv[8] = {gv0.x, gv0.y, gv0.z, gv0.w, gv1.x, gv1.y, gv1.z, gv1.w};
-        const float svv[8] = {sv0.x, sv0.y, sv0.z, sv0.w, sv1.x, sv1.y, sv1.z, sv1.w};
-        const float zvv[8] = {zv0.x, zv0.y, zv0.z, zv0.w, zv1.x, zv1.y, zv1.z, zv1.w};
-        t8h hi, lo, zoff;
+    auto convert = [&](uint32_t st, uint32_t stage, int buf) {
+        const uint8_t* base = raw + stage * kTRaw;
+        const float4 g0 = *reinterpret_cast<const float4*>(base + s_row * 128 + s_ch * 32);
+        const float4 g1 = *reinterpret_cast<const float4*>(base + s_row * 128 + s_ch * 32 + 16);
+        const float4 s0 = *reinterpret_cast<const float4*>(base + kTRawGy + kTRawW + s_ch * 32);
+        const float4 s1 = *reinterpret_cast<const float4*>(base + kTRawGy + kTRawW + s_ch * 32 + 16);
+        const float4 z0 = *reinterpret_cast<const float4*>(base + kTRawGy + kTRawW + 128 + s_ch * 32);
+        const float4 z1 = *reinterpret_cast<const float4*>(base + kTRawGy + kTRawW + 128 + s_ch * 32 + 16);
+        const uint32_t c0 = st * 32 + s_ch * 8;
+        // n % 4 == 0: four columns are all-in or all-out; the columns past n hold values of column 0
+        const float f0 = c0 < n ? frow : 0.0f, f1 = c0 + 4 < n ? frow : 0.0f;
+        // powers of two first: gy f is exact, the product with s / S is rounded once
+        const float a[8] = {(g0.x * f0) * s0.x, (g0.y * f0) * s0.y, (g0.z * f0) * s0.z, (g0.w * f0) * s0.w,
+                            (g1.x * f1) * s1.x, (g1.y * f1) * s1.y, (g1.z * f1) * s1.z, (g1.w * f1) * s1.w};
+        const float zv[8] = {z0.x, z0.y, z0.z, z0.w, z1.x, z1.y, z1.z, z1.w};
+        uint32_t hi[4], lo[4];
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
-            // powers of two first: (gy f) and (s / S) are exact, their product is rounded once
-            const float a = (gvv[e] * frow) * (svv[e] * s_inv);
-            const float z0 = rintf(zvv[e]);
-            csum = fmaf(a, zvv[e] - z0, csum);
-            zoff[e] = (_Float16)(1024.0f + z0);                // exact for |z0| <= 1024; zero-points are 0 .. 15
-            // hi = a rounded to 11 bits by integer arithmetic, so that it converts to f16 exactly: left to
-            // the compiler, (_Float16)a of a product becomes v_fma_mixlo_f16 (one rounding of the exact
-            // product) in one place and a conversion of the rounded f32 in another, and on a tie the two
-            // differ by a whole f16 step, which hi + lo then misses
-            const float a_hi = __uint_as_float((__float_as_uint(a) + 0x1000u) & 0xFFFFE000u);
-            const _Float16 h = (_Float16)a_hi;                 // exact above 2^-14; below, any rounding does
-            hi[e] = h;
-            lo[e] = (_Float16)(a - (float)h);
+        for (int e = 0; e < 8; e += 2) {
+            csum = fmaf(a[e], zv[e], csum);
+            csum = fmaf(a[e + 1], zv[e + 1], csum);
+            // hi = a cut to 11 bits (one instruction for two values), lo = the rest cut to 11 bits: 2^-21 of a
+            // is lost at most.  The explicit conversion also keeps the compiler from rounding a product
+            // to f16 in two different ways (v_fma_mixlo_f16 of the exact product here, a conversion of the
+            // rounded f32 there), which on a tie differ by a whole f16 step that hi + lo then misses.
+            const auto h2 = __builtin_amdgcn_cvt_pkrtz(a[e], a[e + 1]);
+            const auto l2 = __builtin_amdgcn_cvt_pkrtz(a[e] - (float)h2[0], a[e + 1] - (float)h2[1]);
+            hi[e / 2] = __builtin_bit_cast(uint32_t, h2);
+            lo[e / 2] = __builtin_bit_cast(uint32_t, l2);
         }
-        *reinterpret_cast<t8h*>(&lds_a[buf][0][s_lds]) = hi;
-        *reinterpret_cast<t8h*>(&lds_a[buf][1][s_lds]) = lo;
-        if (s_row == 0) *reinterpret_cast<t8h*>(&lds_z[buf][8 * s_ch]) = zoff;
+        uint8_t* ab = abuf + buf * kTAbuf;
+        *reinterpret_cast<uint4*>(ab + s_lds) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+        *reinterpret_cast<uint4*>(ab + 64 * 64 + s_lds) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
     };
 
-    // ---- B role: lane (k = 32 wave + lane % 32, half = lane / 32) -----------------------------------
+    // ---- B role: lane (k = 32 wave + lane % 32, half = lane / 32): 8 words of word row 4 wave + k / 8 ----
     const uint32_t bc = lane & 31, bh = lane >> 5;
-    const uint32_t kk = k0 + 32 * wave + bc;                   // < padded_k: whole groups exist in the arrays
-    const uint32_t shift = 4 * (kk & 7);
-    const uint32_t* wrow = packed + (uint64_t)(kk >> 3) * n;
-    uint4 bw[2][2];                                            // [MFMA step t][low, high four words]
-    auto load_b = [&](uint32_t st) {
-#pragma unroll
-        for (int t = 0; t < 2; t++) {
-            const uint32_t c0 = st * 32 + 16 * t + 8 * bh;
-            const uint32_t a0 = c0 < n ? c0 : 0, a1 = c0 + 4 < n ? c0 + 4 : 0;   // past n: any words, times a = 0
-            bw[t][0] = *reinterpret_cast<const uint4*>(wrow + a0);
-            bw[t][1] = *reinterpret_cast<const uint4*>(wrow + a1);
-        }
-    };
-    auto b_frag = [&](int t, int buf) {
-        const uint32_t w[8] = {bw[t][0].x, bw[t][0].y, bw[t][0].z, bw[t][0].w, bw[t][1].x, bw[t][1].y, bw[t][1].z, bw[t][1].w};
-        const t8h off = *reinterpret_cast<const t8h*>(&lds_z[buf][16 * t + 8 * bh]);   // 1024 + z0 of this lane's 8 n
+    const uint32_t shift = 4 * (bc & 7);
+    const uint32_t b_off = kTRawGy + (4 * wave + (bc >> 3)) * 128 + bh * 32;
+    auto b_frag = [&](int t, uint32_t stage) {
+        const uint8_t* sb = raw + stage * kTRaw;
+        const uint4 w0 = *reinterpret_cast<const uint4*>(sb + b_off + t * 64), w1 = *reinterpret_cast<const uint4*>(sb + b_off + t * 64 + 16);
+        const uint32_t w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+        const t8h off = *reinterpret_cast<const t8h*>(sb + kTRawGy + kTRawW + kTRawSz + 32 * t + 16 * bh);   // 1024 + z0
         t2h h[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -185,42 +229,49 @@ __global__ __launch_bounds__(256, 2) void w4t_gemm_kernel(
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[i][r] = 0.0f;
 
-    if (st0 < st1) {
-        load_stage(st0);
-        load_b(st0);
-        store_stage(0);
-    }
-    __syncthreads();
+    // ---- pipeline -----------------------------------------------------------------------------------------
+    // Every step issues exactly kTLoads loads per wave, also past the end (the last step again, into a
+    // stage nobody reads any more), so the counter arithmetic has no tail cases.
+#pragma unroll
+    for (int s = 0; s < kTStages - 1; s++) issue(st0 + s, s);
+    RUMUS_WAIT_VMCNT((kTStages - 2) * kTLoads);               // step st0 has landed
+    __builtin_amdgcn_s_barrier();
+    convert(st0, 0, 0);
+    uint32_t cur = 0;                                          // raw stage of step st
     for (uint32_t st = st0; st < st1; st++) {
-        const int cur = (st - st0) & 1;
-        const bool more = st + 1 < st1;
-        const t8h b0 = b_frag(0, cur), b1 = b_frag(1, cur);    // the words of this step, loaded a step ago
-        if (more) {
-            load_stage(st + 1);
-            load_b(st + 1);
-        }
+        const int ab = (st - st0) & 1;
+        const uint32_t nxt = cur + 1 == kTStages ? 0 : cur + 1, prv = cur == 0 ? kTStages - 1 : cur - 1;
+        // step st+1 has landed once only the kTStages-3 younger steps are outstanding; past the barrier
+        // the A fragments of step st are visible and the stage of step st-1 is free
+        RUMUS_WAIT_VMCNT((kTStages - 3) * kTLoads);
+        __builtin_amdgcn_s_barrier();
+        issue(st + (kTStages - 1), prv);
+        const t8h b0 = b_frag(0, cur), b1 = b_frag(1, cur);
+        const uint8_t* abp = abuf + ab * kTAbuf;
 #pragma unroll
         for (int i = 0; i < 2; i++) {
-            const uint8_t* hi = &lds_a[cur][0][i * 32 * 64];
-            const uint8_t* lo = &lds_a[cur][1][i * 32 * 64];
+            const uint8_t* hi = abp + i * 32 * 64;
+            const uint8_t* lo = abp + 64 * 64 + i * 32 * 64;
             acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const t8h*>(hi + a_off[0]), b0, acc[i], 0, 0, 0);
             acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const t8h*>(lo + a_off[0]), b0, acc[i], 0, 0, 0);
             acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const t8h*>(hi + a_off[1]), b1, acc[i], 0, 0, 0);
             acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const t8h*>(lo + a_off[1]), b1, acc[i], 0, 0, 0);
         }
-        if (more) store_stage(cur ^ 1);
-        __syncthreads();
+        if (st + 1 < st1) convert(st + 1, nxt, ab ^ 1);
+        cur = nxt;
     }
+    RUMUS_WAIT_VMCNT(0);         // no direct-to-LDS write may outlive the workgroup
 
-    // ---- c[row]: the four staging threads of a row are neighbours in a wave ----------------------------
+    // ---- c[row]: the four conversion threads of a row are neighbours in a wave ------------------------
     csum += __shfl_xor(csum, 1);
     csum += __shfl_xor(csum, 2);
     if (s_ch == 0) lds_c[s_row] = csum;
     __syncthreads();
 
     // ---- register r of lane l is row 8 (r/4) + 4 (l/32) + r%4, column l%32 of its 32 x 32 tile -------
-    float* dst = out + (uint64_t)blockIdx.z * m * k;
+    float* dst_out = out + (uint64_t)blockIdx.z * m * k;
     const uint32_t col = k0 + 32 * wave + bc;
+    const float s_big = sgrp[g];
     if (col < k) {
 #pragma unroll
         for (int i = 0; i < 2; i++)
@@ -231,7 +282,7 @@ __global__ __launch_bounds__(256, 2) void w4t_gemm_kernel(
                 const float f = rowf[row];
                 // 1 / f_row = 2^(e - 140): from the bits of f (f = 2^(140 - e), biased exponent 267 - e)
                 const float finv = f != f ? f : f == 0.0f ? 0.0f : __uint_as_float((254u - (__float_as_uint(f) >> 23)) << 23);
-                dst[(uint64_t)row * k + col] = ((acc[i][r] - lds_c[lr]) * finv) * s_big;
+                dst_out[(uint64_t)row * k + col] = ((acc[i][r] - lds_c[lr]) * finv) * s_big;
             }
     }
 }
@@ -258,35 +309,67 @@ bool w4_gemm_t_supported(uint32_t m, uint32_t k, uint32_t n, uint32_t group_size
            (uint64_t)m * k < (1ull << 32) && (uint64_t)m * n < (1ull << 40);
 }
 
+template <int NS>
+static int launch_w4t(uint32_t ktiles, uint32_t mtiles, uint32_t shares, hipStream_t s, const float* gy,
+                      const uint32_t* packed, const float* sp, const float* zf, const _Float16* zo, const float* rowf,
+                      const float* sgrp, float* out, uint32_t m, uint32_t k, uint32_t n, uint32_t gs, uint32_t steps_per) {
+    constexpr size_t lds_bytes = w4t_lds_bytes(NS);
+    static bool attr_set = false;   // benign race: setting the attribute is idempotent
+    if (!attr_set && lds_bytes > 64 * 1024) {
+        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&w4t_gemm_kernel<NS>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes),
+                               "hipFuncSetAttribute"))
+            return rc;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(w4t_gemm_kernel<NS>, dim3(ktiles, mtiles, shares), dim3(256), lds_bytes, s, gy, packed, sp, zf, zo,
+                       rowf, sgrp, out, m, k, n, gs, steps_per);
+    return check_launch("w4t_gemm_kernel");
+}
+
 int w4_launch_gemm_t(const float* gy, const uint32_t* packed, const float* scales, const float* zp, float* out,
                      uint32_t m, uint32_t k, uint32_t n, uint32_t padded_k, uint32_t group_size, uint32_t num_groups,
                      hipStream_t s) {
     const uint32_t ktiles = padded_k / 128, mtiles = ceil_div(m, 64), nsteps = ceil_div(n, 32);
     RUMUS_REQUIRE(mtiles <= 65535, "qmatmul_int4_t: m %u is beyond the grid limit", m);
-    // few tiles: n is shared out too, in shares of at least 16 steps
+    // fewer tiles than two per compute unit: n is shared out too, in shares of at least 16 steps
     uint32_t shares = 1, steps_per = nsteps;
     const uint64_t tiles = (uint64_t)ktiles * mtiles;
-    if (tiles < 256) {
-        shares = (uint32_t)(512 / tiles);
+    if (tiles < 512) {
+        shares = (uint32_t)(1024 / tiles);
         if (shares > (uint32_t)kTMaxSplits) shares = kTMaxSplits;
         if (shares > nsteps / 16) shares = nsteps / 16;
         if (shares < 1) shares = 1;
         steps_per = ceil_div(nsteps, shares);
         shares = ceil_div(nsteps, steps_per);
     }
-    const size_t rowf_bytes = ((size_t)m * sizeof(float) + 255) & ~size_t(255);
+    auto up = [](size_t v) { return (v + 255) & ~size_t(255); };
+    const size_t gn = (size_t)num_groups * n;
+    const size_t rowf_bytes = up((size_t)m * sizeof(float)), sgrp_bytes = up((size_t)num_groups * sizeof(float));
+    const size_t sp_bytes = up(gn * sizeof(float)), zo_bytes = up(gn * sizeof(_Float16) + 64);
     const size_t part_bytes = shares > 1 ? (size_t)shares * m * k * sizeof(float) : 0;
     void* ws = nullptr;
-    if (int rc = workspace_get(s, rowf_bytes + 256 + part_bytes, &ws)) return rc;
-    float* rowf = static_cast<float*>(ws);
-    uint32_t* smax_part = reinterpret_cast<uint32_t*>(static_cast<uint8_t*>(ws) + rowf_bytes);
-    float* part = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + rowf_bytes + 256);
-    hipLaunchKernelGGL(w4t_prepare_kernel, dim3(m + kTScaleParts), dim3(256), 0, s, gy, scales, rowf, smax_part, m, n,
-                       (uint64_t)num_groups * n);
+    if (int rc = workspace_get(s, rowf_bytes + sgrp_bytes + 2 * sp_bytes + zo_bytes + part_bytes, &ws)) return rc;
+    uint8_t* b = static_cast<uint8_t*>(ws);
+    float* rowf = reinterpret_cast<float*>(b);
+    float* sgrp = reinterpret_cast<float*>(b + rowf_bytes);
+    float* sp = reinterpret_cast<float*>(b + rowf_bytes + sgrp_bytes);
+    float* zf = reinterpret_cast<float*>(b + rowf_bytes + sgrp_bytes + sp_bytes);
+    _Float16* zo = reinterpret_cast<_Float16*>(b + rowf_bytes + sgrp_bytes + 2 * sp_bytes);
+    float* part = reinterpret_cast<float*>(b + rowf_bytes + sgrp_bytes + 2 * sp_bytes + zo_bytes);
+    hipLaunchKernelGGL(w4t_prepare_kernel, dim3(m + num_groups), dim3(256), 0, s, gy, scales, zp, rowf, sgrp, sp, zf, zo, m,
+                       n);
     if (int rc = check_launch("w4t_prepare_kernel")) return rc;
-    hipLaunchKernelGGL(w4t_gemm_kernel, dim3(ktiles, mtiles, shares), dim3(256), 0, s, gy, packed, scales, zp, rowf,
-                       smax_part, shares > 1 ? part : out, m, k, n, group_size, steps_per);
-    if (int rc = check_launch("w4t_gemm_kernel")) return rc;
+    // stages of loads in flight: the step rate does not depend on them (3 to 5 measured within 4 %: the
+    // vector ALU work of the conversion sets the pace), so the count follows occupancy: four stages and
+    // two workgroups per compute unit up to two rounds of them, three stages and three workgroups beyond
+    const int ns = tiles * shares <= 1024 ? 4 : 3;
+    int rc;
+    switch (ns) {
+        case 4: rc = launch_w4t<4>(ktiles, mtiles, shares, s, gy, packed, sp, zf, zo, rowf, sgrp, shares > 1 ? part : out, m, k, n, group_size, steps_per); break;
+        default: rc = launch_w4t<3>(ktiles, mtiles, shares, s, gy, packed, sp, zf, zo, rowf, sgrp, shares > 1 ? part : out, m, k, n, group_size, steps_per); break;
+    }
+    if (rc) return rc;
     if (shares == 1) return RUMUS_HIP_OK;
     const uint32_t count4 = (uint32_t)((uint64_t)m * k / 4);
     hipLaunchKernelGGL(w4t_add_shares_kernel, dim3(ceil_div(count4, 256)), dim3(256), 0, s,

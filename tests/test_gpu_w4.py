@@ -272,7 +272,8 @@ def test_act_order_rejects_unbalanced_groups(ops):
 
 
 @pytest.mark.parametrize("m,k,n,g", [(3, 72, 20, 8), (16, 512, 300, 128), (1, 1000, 64, 64),
-                                     # from 16 rows on and group % 128 == 0: the f16 matrix cores
+                                     # from 8 rows on and group % 128 == 0: the f16 matrix cores
+                                     (8, 256, 64, 128),
                                      (64, 4096, 1100, 128),     # n shared over workgroups
                                      (130, 1000, 264, 128),     # k ends inside the last group, three row tiles
                                      (100, 256, 4100, 256),     # n ends 4 past a step of 32
