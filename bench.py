@@ -300,6 +300,32 @@ def bench_w4_gemm(torch, ops, m, steps=50, warmup=5):
             "tflops": flops / sec / 1e12, "f16_mfma_frac": flops / sec / 1e12 / F16_PEAK_TFLOPS}
 
 
+def bench_grad_x(torch, ops, steps=20, warmup=4):
+    """grad_x of the INT4 Linear (QLinearBackward: grad_y . dequant(W)^T), K=4096, N=11008, g128:
+    whole call, graph-timed."""
+    k, n = 4096, 11008
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev).manual_seed(4)
+    w = torch.randn((k, n), generator=gen, device=dev) * 0.02
+    packed, scales, zp = ops.w4_quantize_pack(w, G)
+    del w
+    rows = []
+    for m in (1, 16, 128, 2048):
+        gy = torch.randn((m, n), generator=gen, device=dev)
+        out = torch.empty((m, k), dtype=torch.float32, device=dev)
+
+        def burst():
+            for _ in range(4):
+                ops.qmatmul_int4_t(gy, packed, scales, zp, k, G, out=out)
+
+        total, launches, _ = time_graph(torch, burst, 4, steps, warmup)
+        sec = total / launches
+        rows.append({"workload": f"w4_grad_x_{m}x4096x11008_g128", "ms_per_call": sec * 1e3,
+                     "tflops": 2.0 * m * k * n / sec / 1e12,
+                     "weight_gbs": (k * n // 2 + 2 * (k // G) * n * 4) / sec / 1e9})
+    return rows
+
+
 def bench_q8_matmul(torch, ops, steps=20, warmup=4):
     """The reference's f32 x Q8 matmul (Tensor::matmul with a Q8 right-hand side), K=4096, N=11008,
     at the block sizes that take different kernels: whole call, graph-timed."""
@@ -517,6 +543,7 @@ def main():
         out["w4_gemv_wider"] = bench_gemv_shapes(torch, ops)
         out["w4_gemm"] = [bench_w4_gemm(torch, ops, 16), bench_w4_gemm(torch, ops, 128)]
         out["q8_matmul"] = bench_q8_matmul(torch, ops)
+        out["w4_grad_x"] = bench_grad_x(torch, ops)
         out["decoder_block"] = bench_decoder_block(torch, ops)
 
     if not args.no_cpu:

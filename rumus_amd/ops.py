@@ -278,12 +278,15 @@ def qmatmul_int4_perm(x, packed_sorted, scales, zp, k, group_size, bias=None, pe
                     group_size, out)
 
 
-def qmatmul_int4_t(a, packed, scales, zp, k, group_size):
+def qmatmul_int4_t(a, packed, scales, zp, k, group_size, out=None):
     m, n = a.shape
     if packed.shape[1] != n:
         raise ValueError("qmatmul_int4_t: a must be [m, n]")
     padded_k, groups = w4_geometry(k, group_size)
-    out = torch.empty((m, k), dtype=torch.float32, device=a.device)
+    if out is None:
+        out = torch.empty((m, k), dtype=torch.float32, device=a.device)
+    elif out.shape != (m, k) or out.dtype != torch.float32 or not out.is_contiguous():
+        raise ValueError("qmatmul_int4_t: out must be a contiguous f32 [m, k] tensor")
     call("rumus_hip_qmatmul_int4_t", _dev(a, torch.float32, "a"), _dev(packed, torch.int32, "packed"),
          _dev(scales, torch.float32, "scales"), _dev(zp, torch.float32, "zero_points"),
          out.data_ptr(), m, k, n, padded_k, group_size, groups, _stream())
