@@ -37,7 +37,8 @@ constexpr int kTMaxSplits = 16;
 //       (0 for an all-zero or tiny row, NaN marker for a row with inf / nan);
 //   blocks [m, m + groups): for group g, S_g = the power of two at or above its largest scale, and per
 //       column the three things the GEMM needs of scale and zero-point: s / S_g (f32, at most 1),
-//       zp - rint(zp) (f32) and 1024 + rint(zp) (f16), so that no workgroup works them out again.
+//       zp - z0 (f32) and 1024 + z0 (f16), z0 = rint(zp) held within +-1000, so that no workgroup works
+//       them out again.
 //       sgrp[g] = S_g; 0 when every scale of the group is zero or denormal, NaN when one is not finite
 //       or S_g or 1 / S_g would leave the normal range: the GEMM then writes zeros / NaNs for the group.
 __global__ __launch_bounds__(256) void w4t_prepare_kernel(const float* __restrict__ gy, const float* __restrict__ scales,
@@ -77,8 +78,11 @@ __global__ __launch_bounds__(256) void w4t_prepare_kernel(const float* __restric
 #pragma unroll 4
     for (uint32_t j = 4 * tid; j < n; j += 1024) {             // independent iterations: their loads overlap
         const float4 sv = *reinterpret_cast<const float4*>(r + j), z = *reinterpret_cast<const float4*>(zr + j);
-        const float4 z0 = make_float4(rintf(z.x), rintf(z.y), rintf(z.z), rintf(z.w));
-        // s / S_g is exact (a power of two); 1024 + z0 is exact for |z0| <= 1024, zero-points are 0 .. 15
+        // zero-points are 0 .. 15 unless a group's weights sit far from zero (zp = -min / scale); beyond
+        // +-1000 the integer part stops growing and the rest goes into the f32 correction with the fraction
+        auto whole = [](float v) { return fminf(fmaxf(rintf(v), -1000.0f), 1000.0f); };
+        const float4 z0 = make_float4(whole(z.x), whole(z.y), whole(z.z), whole(z.w));
+        // s / S_g is exact (a power of two); 1024 + z0 is exact in f16 for |z0| <= 1024
         *reinterpret_cast<float4*>(sp + (uint64_t)g * n + j) = make_float4(sv.x * s_inv, sv.y * s_inv, sv.z * s_inv, sv.w * s_inv);
         *reinterpret_cast<float4*>(zf + (uint64_t)g * n + j) = make_float4(z.x - z0.x, z.y - z0.y, z.z - z0.z, z.w - z0.w);
         *reinterpret_cast<v4h*>(zo + (uint64_t)g * n + j) =

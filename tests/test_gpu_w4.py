@@ -301,6 +301,8 @@ def test_qmatmul_int4_transpose_scaling_and_non_finite_rows(ops):
     w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
     w[:, :100] *= 1e-4                                       # scales over four decades
     w[:, 100:200] *= 50.0
+    w[:128, 200:230] += 3.0                                  # weights far from zero: zero-points near -300
+    w[:128, 230:240] = 1.0 + 1e-5 * w[:128, 230:240]         # and beyond -1000
     gy = rng.normal(0, 1, (m, n)).astype(np.float32)
     gy[1] *= 1e-12
     gy[2] *= 1e9
