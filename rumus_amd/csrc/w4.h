@@ -69,7 +69,7 @@ bool w4_gemm_supported(const W4Args& a);
 uint32_t w4_decode_max_rows(uint32_t padded_k, uint32_t n);   // w4_gemv.hip
 int w4_launch_gemm(const W4Args& a, hipStream_t s);
 
-// grad_x on the f16 matrix cores (w4_gemm_t.hip): group_size % 128 == 0, n % 4 == 0, k % 4 == 0,
+// grad_x on the f16 matrix cores (w4_gemm_t.hip): group_size 32, 64 or a multiple of 128, n % 4 == 0, k % 4 == 0,
 // 16-byte aligned buffers.
 bool w4_gemm_t_supported(uint32_t m, uint32_t k, uint32_t n, uint32_t group_size, const void* gy, const void* packed,
                          const void* scales, const void* zp, const void* out);

@@ -11,7 +11,7 @@
 // per group of output columns.  (Taking the whole zero-point out, q against c = sum A zp, costs
 // accuracy: the 2^-23 the f16 planes lose of A is then multiplied by q instead of by q - zp, which
 // near-zero weights make many times larger than the term itself.)  A workgroup owns 64 rows x 128 consecutive k of one
-// group (group_size % 128 == 0) and walks n in steps of 32:
+// group (group_size % 128 == 0; 64 or 32 k for groups of 64 or 32) and walks n in steps of 32:
 //   * conversion (all 256 threads, 8 values each): a = (gy f_row) (s / S) with f_row and S powers of two
 //     that put |a| below 2^14 (w4t_prepare_kernel: row maxima of gy, maximum of the scales), split into
 //     hi + lo f16 (22 bits), written to LDS in A-fragment rows of 64 bytes; c accumulates in f32;
@@ -100,11 +100,14 @@ __global__ __launch_bounds__(256) void w4t_prepare_kernel(const float* __restric
 constexpr int kTRawGy = 64 * 128, kTRawW = 16 * 128, kTRawSz = 256, kTRawZo = 256;   // 64 bytes of zero-point integers used
 constexpr int kTRaw = kTRawGy + kTRawW + kTRawSz + kTRawZo;   // bytes of one raw stage
 constexpr int kTAbuf = 2 * 64 * 64;                           // hi, lo planes
-constexpr int kTLoads = 3;                                    // wave-wide loads per wave and step: 12 in all
+constexpr int kTSlots = 12;                                   // wave-wide loads per step: 8 grad_y, 1-2 weights, 2 tables
 constexpr size_t w4t_lds_bytes(int stages) { return (size_t)stages * kTRaw + 2 * kTAbuf + 64 * sizeof(float); }
 
-template <int kTStages>
-__global__ __launch_bounds__(256, 2) void w4t_gemm_kernel(
+// KW = waves per workgroup = 32-column slices of k per tile: 4 when groups are multiples of 128, 2 for
+// groups of 64, 1 for groups of 32 (a tile must lie inside one group, since the activations are re-scaled
+// per group; the smaller workgroups convert the same 64 x 32 activations for fewer output columns).
+template <int kTStages, int KW>
+__global__ __launch_bounds__(64 * KW, 2) void w4t_gemm_kernel(
     const float* __restrict__ gy, const uint32_t* __restrict__ packed, const float* __restrict__ sp,
     const float* __restrict__ zf, const _Float16* __restrict__ zo, const float* __restrict__ rowf,
     const float* __restrict__ sgrp, float* __restrict__ out, uint32_t m, uint32_t k, uint32_t n, uint32_t gs,
@@ -115,33 +118,38 @@ __global__ __launch_bounds__(256, 2) void w4t_gemm_kernel(
     float* const lds_c = reinterpret_cast<float*>(abuf + 2 * kTAbuf);
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t k0 = blockIdx.x * 128, m0 = blockIdx.y * 64;
+    constexpr int kTLoads = kTSlots / KW;                      // per wave and step
+    constexpr int WS = KW == 4 ? 2 : 1;                        // slots of weight words (8 word rows each)
+    const uint32_t k0 = blockIdx.x * (32 * KW), m0 = blockIdx.y * 64;
     const uint32_t g = k0 / gs;
     const uint32_t nsteps = (n + 31) / 32;
     const uint32_t st0 = blockIdx.z * steps_per, st1 = min(nsteps, st0 + steps_per);   // st0 < st1 by the launch
 
     // ---- global side of the direct-to-LDS loads: load q = 4 i + wave of a step --------------------------
     //   q 0..7: rows 8 q .. 8 q + 7 of grad_y (lane: row lane / 8, floats 4 (lane % 8) .. + 3)
-    //   q 8, 9: word rows 8 (q - 8) .. + 7 of the weights (lane: row lane / 8, words 4 (lane % 8) .. + 3)
-    //   q 10: lanes 0..31 scaled scale, 32..63 zero-point fraction of column lane % 32
-    //   q 11: lanes 0..15 two f16 zero-point integers each (columns 2 lane, 2 lane + 1); the other lanes
-    //         fetch the same words again, into the unused tail of the stage
+    //   q 8 (and 9 when KW = 4): word rows 8 (q - 8) .. + 7 of the weights (lane: row lane / 8, words
+    //         4 (lane % 8) .. + 3)
+    //   next: lanes 0..31 scaled scale, 32..63 zero-point fraction of column lane % 32
+    //   last (and any slot left over): lanes 0..15 two f16 zero-point integers each (columns 2 lane,
+    //         2 lane + 1); the other lanes fetch the same words again, into the unused tail of the stage
     const uint32_t l8 = lane >> 3, p8 = lane & 7;
     const uint8_t* src[kTLoads];
     uint32_t dst[kTLoads], colw[kTLoads], esz[kTLoads];        // colw: the lane's first column inside a step
     bool wide[kTLoads];
 #pragma unroll
     for (int i = 0; i < kTLoads; i++) {
-        const uint32_t q = 4 * i + wave;
+        const uint32_t q = KW * i + wave;
         if (q < 8) {
             const uint32_t row = min(m0 + 8 * q + l8, m - 1);
             src[i] = reinterpret_cast<const uint8_t*>(gy + (uint64_t)row * n);
             dst[i] = q * 1024; colw[i] = 4 * p8; wide[i] = true; esz[i] = 4;
-        } else if (q < 10) {
-            const uint32_t wr = k0 / 8 + 8 * (q - 8) + l8;     // < padded_k / 8: whole groups exist in the arrays
+        } else if (q < 8 + WS) {
+            // the tile's 4 KW word rows (< padded_k / 8: whole groups exist in the arrays); lanes past them
+            // fetch its last row again, into room the stage keeps for that
+            const uint32_t wr = k0 / 8 + min(8 * (q - 8) + l8, 4u * KW - 1);
             src[i] = reinterpret_cast<const uint8_t*>(packed + (uint64_t)wr * n);
             dst[i] = kTRawGy + (q - 8) * 1024; colw[i] = 4 * p8; wide[i] = true; esz[i] = 4;
-        } else if (q == 10) {
+        } else if (q == 8 + WS) {
             src[i] = reinterpret_cast<const uint8_t*>((lane < 32 ? sp : zf) + (uint64_t)g * n);
             dst[i] = kTRawGy + kTRawW; colw[i] = lane & 31; wide[i] = false; esz[i] = 4;
         } else {
@@ -163,13 +171,14 @@ __global__ __launch_bounds__(256, 2) void w4t_gemm_kernel(
         }
     };
 
-    // ---- conversion role: 8 consecutive n (chunk tid % 4) of row tid / 4 ------------------------------
-    const uint32_t s_row = tid >> 2, s_ch = tid & 3;
+    // ---- conversion role: row tid / KW, its chunks of 8 consecutive n: 4 / KW of them from (tid % KW) 4 / KW ----
+    constexpr int CPT = 4 / KW;
+    const uint32_t s_row = tid / KW, s_ch0 = (tid % KW) * CPT;
     const float frow_raw = rowf[min(m0 + s_row, m - 1)];
     const float frow = frow_raw != frow_raw ? 0.0f : frow_raw; // inf / nan in the row: NaN times 0 poisons it below
-    const uint32_t s_lds = s_row * 64 + ((s_ch ^ row_swizzle(s_row)) & 3) * 16;
     float csum = 0.0f;
-    auto convert = [&](uint32_t st, uint32_t stage, int buf) {
+    auto convert_chunk = [&](uint32_t st, uint32_t stage, int buf, uint32_t s_ch) {
+        const uint32_t s_lds = s_row * 64 + ((s_ch ^ row_swizzle(s_row)) & 3) * 16;
         const uint8_t* base = raw + stage * kTRaw;
         const float4 g0 = *reinterpret_cast<const float4*>(base + s_row * 128 + s_ch * 32);
         const float4 g1 = *reinterpret_cast<const float4*>(base + s_row * 128 + s_ch * 32 + 16);
@@ -201,6 +210,10 @@ __global__ __launch_bounds__(256, 2) void w4t_gemm_kernel(
         uint8_t* ab = abuf + buf * kTAbuf;
         *reinterpret_cast<uint4*>(ab + s_lds) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
         *reinterpret_cast<uint4*>(ab + 64 * 64 + s_lds) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+    };
+    auto convert = [&](uint32_t st, uint32_t stage, int buf) {
+#pragma unroll
+        for (int cc = 0; cc < CPT; cc++) convert_chunk(st, stage, buf, s_ch0 + cc);
     };
 
     // ---- B role: lane (k = 32 wave + lane % 32, half = lane / 32): 8 words of word row 4 wave + k / 8 ----
@@ -266,10 +279,10 @@ __global__ __launch_bounds__(256, 2) void w4t_gemm_kernel(
     }
     RUMUS_WAIT_VMCNT(0);         // no direct-to-LDS write may outlive the workgroup
 
-    // ---- c[row]: the four conversion threads of a row are neighbours in a wave ------------------------
-    csum += __shfl_xor(csum, 1);
-    csum += __shfl_xor(csum, 2);
-    if (s_ch == 0) lds_c[s_row] = csum;
+    // ---- c[row]: the KW conversion threads of a row are neighbours in a wave ---------------------------
+    if (KW >= 2) csum += __shfl_xor(csum, 1);
+    if (KW == 4) csum += __shfl_xor(csum, 2);
+    if (tid % KW == 0) lds_c[s_row] = csum;
     __syncthreads();
 
     // ---- register r of lane l is row 8 (r/4) + 4 (l/32) + r%4, column l%32 of its 32 x 32 tile -------
@@ -309,32 +322,37 @@ bool w4_gemm_t_supported(uint32_t m, uint32_t k, uint32_t n, uint32_t group_size
     const uintptr_t bits = reinterpret_cast<uintptr_t>(gy) | reinterpret_cast<uintptr_t>(packed) |
                            reinterpret_cast<uintptr_t>(scales) | reinterpret_cast<uintptr_t>(zp) |
                            reinterpret_cast<uintptr_t>(out);
-    return group_size % 128 == 0 && n % 4 == 0 && k % 4 == 0 && (bits & 15) == 0 &&
+    return (group_size % 128 == 0 || group_size == 64 || group_size == 32) && n % 4 == 0 && k % 4 == 0 && (bits & 15) == 0 &&
            (uint64_t)m * k < (1ull << 32) && (uint64_t)m * n < (1ull << 40);
 }
 
-template <int NS>
+template <int NS, int KW>
 static int launch_w4t(uint32_t ktiles, uint32_t mtiles, uint32_t shares, hipStream_t s, const float* gy,
                       const uint32_t* packed, const float* sp, const float* zf, const _Float16* zo, const float* rowf,
                       const float* sgrp, float* out, uint32_t m, uint32_t k, uint32_t n, uint32_t gs, uint32_t steps_per) {
     constexpr size_t lds_bytes = w4t_lds_bytes(NS);
     static bool attr_set = false;   // benign race: setting the attribute is idempotent
     if (!attr_set && lds_bytes > 64 * 1024) {
-        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&w4t_gemm_kernel<NS>),
+        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&w4t_gemm_kernel<NS, KW>),
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes),
                                "hipFuncSetAttribute"))
             return rc;
         attr_set = true;
     }
-    hipLaunchKernelGGL(w4t_gemm_kernel<NS>, dim3(ktiles, mtiles, shares), dim3(256), lds_bytes, s, gy, packed, sp, zf, zo,
+    hipLaunchKernelGGL((w4t_gemm_kernel<NS, KW>), dim3(ktiles, mtiles, shares), dim3(64 * KW), lds_bytes, s, gy, packed, sp, zf, zo,
                        rowf, sgrp, out, m, k, n, gs, steps_per);
     return check_launch("w4t_gemm_kernel");
 }
 
+#define RUMUS_W4T_LAUNCH(NS, KW)                                                                                  \
+    launch_w4t<NS, KW>(ktiles, mtiles, shares, s, gy, packed, sp, zf, zo, rowf, sgrp, shares > 1 ? part : out, m, k, n, \
+                       group_size, steps_per)
+
 int w4_launch_gemm_t(const float* gy, const uint32_t* packed, const float* scales, const float* zp, float* out,
                      uint32_t m, uint32_t k, uint32_t n, uint32_t padded_k, uint32_t group_size, uint32_t num_groups,
                      hipStream_t s) {
-    const uint32_t ktiles = padded_k / 128, mtiles = ceil_div(m, 64), nsteps = ceil_div(n, 32);
+    const int kw = group_size % 128 == 0 ? 4 : group_size / 32;   // waves per workgroup: 32-column slices of one group
+    const uint32_t ktiles = padded_k / (32 * kw), mtiles = ceil_div(m, 64), nsteps = ceil_div(n, 32);
     RUMUS_REQUIRE(mtiles <= 65535, "qmatmul_int4_t: m %u is beyond the grid limit", m);
     // fewer tiles than two per compute unit: n is shared out too, in shares of at least 16 steps
     uint32_t shares = 1, steps_per = nsteps;
@@ -373,8 +391,12 @@ int w4_launch_gemm_t(const float* gy, const uint32_t* packed, const float* scale
     const int ns = tiles * shares <= 1024 ? 4 : 3;
     int rc;
     switch (ns) {
-        case 4: rc = launch_w4t<4>(ktiles, mtiles, shares, s, gy, packed, sp, zf, zo, rowf, sgrp, shares > 1 ? part : out, m, k, n, group_size, steps_per); break;
-        default: rc = launch_w4t<3>(ktiles, mtiles, shares, s, gy, packed, sp, zf, zo, rowf, sgrp, shares > 1 ? part : out, m, k, n, group_size, steps_per); break;
+        case 4:
+            rc = kw == 4 ? RUMUS_W4T_LAUNCH(4, 4) : kw == 2 ? RUMUS_W4T_LAUNCH(4, 2) : RUMUS_W4T_LAUNCH(4, 1);
+            break;
+        default:
+            rc = kw == 4 ? RUMUS_W4T_LAUNCH(3, 4) : kw == 2 ? RUMUS_W4T_LAUNCH(3, 2) : RUMUS_W4T_LAUNCH(3, 1);
+            break;
     }
     if (rc) return rc;
     if (shares == 1) return RUMUS_HIP_OK;

@@ -446,8 +446,10 @@ int rumus_hip_qmatmul_int4_t(const float* a, const uint32_t* packed, const float
     // 32 outputs, each word once per 4 rows); single rows keep one word row per workgroup for
     // the sake of parallelism
     hipStream_t s = as_stream(stream);
-    // from 8 rows on the matrix-core kernel is ahead (4096 x 11008: 60 us for up to 64 rows against 8.6 us per row)
-    if (m >= 8 && w4_gemm_t_supported(m, k, n, group_size, a, packed, scales, zero_points, out))
+    // where the matrix-core kernel is ahead of the one below (4096 x 11008: 45 us for up to 64 rows with groups
+    // of 128, 85 us with 64, 176 us with 32, against 67 us per 8 rows)
+    const uint32_t mfma_from = group_size % 128 == 0 ? 8 : group_size == 64 ? 12 : 24;
+    if (m >= mfma_from && w4_gemm_t_supported(m, k, n, group_size, a, packed, scales, zero_points, out))
         return w4_launch_gemm_t(a, packed, scales, zero_points, out, m, k, n, padded_k, group_size, num_groups, s);
     const uint32_t word_rows = padded_k / 8;
     if (m >= 3)

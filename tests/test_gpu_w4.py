@@ -279,7 +279,10 @@ def test_act_order_rejects_unbalanced_groups(ops):
                                      (100, 256, 4100, 256),     # n ends 4 past a step of 32
                                      (2050, 256, 516, 128),     # many row tiles
                                      (16, 128, 4, 128),         # the smallest n
-                                     (40, 512, 300, 64)])       # other group sizes keep the vector kernel
+                                     (40, 512, 300, 64),        # groups of 64: two waves per workgroup
+                                     (70, 256, 132, 32),        # groups of 32: one
+                                     (300, 200, 64, 32),        # k ends inside a group of 32
+                                     (9, 96, 40, 16)])          # other group sizes keep the vector kernel
 def test_qmatmul_int4_transpose(ops, m, k, n, g):
     say(f"qmatmul_int4_t m={m} k={k} n={n} g={g}")
     rng = np.random.default_rng(k + n)
