@@ -150,7 +150,7 @@ template <int TM, int TN, int WM, int WN, int NS>
 __global__ __launch_bounds__(64 * WM * WN) void i8_gemm_dma_kernel(
     const int8_t* __restrict__ A, const int8_t* __restrict__ B, const float* __restrict__ sx,
     const float* __restrict__ sw, const float* __restrict__ bias, int32_t* __restrict__ acc_out,
-    float* __restrict__ y, uint32_t M, uint32_t K, uint32_t N, uint32_t tiles_m, uint32_t tiles_n) {
+    float* __restrict__ y, uint32_t M, uint32_t K, uint32_t N, uint32_t tiles_m, uint32_t tiles_n, uint32_t steps_per) {
     constexpr int WAVES = WM * WN;
     constexpr int BM = 32 * TM * WM, BN = 32 * TN * WN;
     constexpr int A_BYTES = BM * kBK, B_BYTES = BN * kBK, STAGE = A_BYTES + B_BYTES;
@@ -168,6 +168,11 @@ __global__ __launch_bounds__(64 * WM * WN) void i8_gemm_dma_kernel(
     const uint32_t wm = wave / WN, wn = wave % WN;
     const uint32_t tile = xcd_contiguous(blockIdx.x, tiles_m * tiles_n);
     const uint32_t m0 = (tile % tiles_m) * BM, n0 = (tile / tiles_m) * BN;
+
+    // blockIdx.y picks a share of the K steps (small problems: more workgroups than tiles); the shares'
+    // accumulators go to acc_out + share * M * N and are added by i8_splitk_finish_kernel
+    const uint32_t kt_base = blockIdx.y * steps_per;
+    const uint32_t ksteps = min(K / kBK - kt_base, steps_per);
 
     // ---- global side of the LDS-DMA loads ------------------------------------
     // block b = i*WAVES + wave holds rows 16b .. 16b+15 of the operand tile
@@ -192,7 +197,7 @@ __global__ __launch_bounds__(64 * WM * WN) void i8_gemm_dma_kernel(
     // loads [first, first + count) of a step: A blocks, then B blocks
     auto issue_part = [&](uint32_t kt, uint32_t stage, int first, int count) {
         int8_t* base = lds + stage * STAGE;
-        const uint32_t k0 = kt * kBK;
+        const uint32_t k0 = (kt_base + kt) * kBK;
 #pragma unroll
         for (int q = 0; q < LOADS; q++) {
             if (q < first || q >= first + count) continue;
@@ -233,7 +238,6 @@ __global__ __launch_bounds__(64 * WM * WN) void i8_gemm_dma_kernel(
     // Every step issues exactly LOADS loads, also past the end of K (the last
     // step is then fetched again into a stage nobody reads any more): the memory
     // counter arithmetic below needs no tail cases and the loop stays branch-free.
-    const uint32_t ksteps = K / kBK;
 #pragma unroll
     for (int s = 0; s < NS - 1; s++) issue(min((uint32_t)s, ksteps - 1), s);
 
@@ -298,7 +302,25 @@ __global__ __launch_bounds__(64 * WM * WN) void i8_gemm_dma_kernel(
     mfma_half(1);
     RUMUS_WAIT_VMCNT(0);         // no LDS-DMA write may outlive the workgroup
 
+    if (gridDim.y > 1) acc_out += (uint64_t)blockIdx.y * M * N;
     i8_epilogue<TM, TN, BM, BN>(acc, sx, sw, bias, acc_out, y, M, N, m0, n0, wm, wn, lane);
+}
+
+// Sum of the K shares' i32 accumulators (exact, any order), then the rescale and bias of the epilogue.
+__global__ __launch_bounds__(256) void i8_splitk_finish_kernel(const int32_t* __restrict__ part, uint32_t shares,
+                                                               const float* __restrict__ sx, const float* __restrict__ sw,
+                                                               const float* __restrict__ bias, int32_t* __restrict__ acc_out,
+                                                               float* __restrict__ y, uint32_t M, uint32_t N) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;         // M * N fits 32 bits for the shapes that split K
+    if (i >= M * N) return;
+    int32_t a = part[i];
+    for (uint32_t z = 1; z < shares; z++) a += part[(uint64_t)z * M * N + i];
+    if (acc_out) acc_out[i] = a;
+    if (y) {
+        float v = __fmul_rn(__fmul_rn((float)a, sx[i / N]), sw[i % N]);
+        if (bias) v = __fadd_rn(v, bias[i % N]);
+        y[i] = v;
+    }
 }
 
 template <int TM, int TN, int WM, int WN, int NS>
@@ -317,8 +339,40 @@ static int launch_dma(const int8_t* A, const int8_t* B, const float* sx, const f
     }
     uint32_t tm = ceil_div(M, BM), tn = ceil_div(N, BN);
     hipLaunchKernelGGL((i8_gemm_dma_kernel<TM, TN, WM, WN, NS>), dim3(tm * tn), dim3(64 * WM * WN),
-                       lds_bytes, s, A, B, sx, sw, bias, acc, y, M, K, N, tm, tn);
+                       lds_bytes, s, A, B, sx, sw, bias, acc, y, M, K, N, tm, tn, K / kBK);
     return check_launch("i8_gemm_dma_kernel");
+}
+
+// Few tiles (K % 64 == 0): one wave per 64 x 64 tile, eight stages of direct-to-LDS loads deep, and K
+// shared over up to 8 workgroups per tile so that the weights stream from all of the chip.  The
+// register-staged kernel with one K step in flight spent a trip to memory per step on these shapes
+// (32 x 4096 x 11008: 29 us for 45 MB of weights).
+static int launch_small(const int8_t* A, const int8_t* B, const float* sx, const float* sw, const float* bias,
+                        int32_t* acc, float* y, uint32_t M, uint32_t K, uint32_t N, hipStream_t s) {
+    constexpr int NS = 8;
+    constexpr size_t lds_bytes = (size_t)NS * 128 * kBK;       // 64 KB
+    const uint32_t tm = ceil_div(M, 64), tn = ceil_div(N, 64), ksteps = K / kBK;
+    uint32_t shares = 512 / (tm * tn);
+    if (shares > 8) shares = 8;
+    if (shares > ksteps / 8) shares = ksteps / 8;
+    if (shares < 1) shares = 1;
+    const uint32_t steps_per = ceil_div(ksteps, shares);
+    shares = ceil_div(ksteps, steps_per);
+    if (shares == 1) {
+        hipLaunchKernelGGL((i8_gemm_dma_kernel<2, 2, 1, 1, NS>), dim3(tm * tn, 1), dim3(64), lds_bytes, s, A, B, sx, sw,
+                           bias, acc, y, M, K, N, tm, tn, steps_per);
+        return check_launch("i8_gemm_dma_kernel");
+    }
+    void* ws = nullptr;
+    if (int rc = workspace_get(s, (size_t)shares * M * N * sizeof(int32_t), &ws)) return rc;
+    int32_t* part = static_cast<int32_t*>(ws);
+    hipLaunchKernelGGL((i8_gemm_dma_kernel<2, 2, 1, 1, NS>), dim3(tm * tn, shares), dim3(64), lds_bytes, s, A, B,
+                       (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, part, (float*)nullptr, M, K, N,
+                       tm, tn, steps_per);
+    if (int rc = check_launch("i8_gemm_dma_kernel")) return rc;
+    hipLaunchKernelGGL(i8_splitk_finish_kernel, dim3(ceil_div(M * N, 256)), dim3(256), 0, s, part, shares, sx, sw, bias, acc,
+                       y, M, N);
+    return check_launch("i8_splitk_finish_kernel");
 }
 
 template <int TM, int TN, int OCC>
@@ -356,6 +410,10 @@ extern "C" int rumus_hip_i8_gemm(const int8_t* xq, const int8_t* wq, const float
         return launch_dma<2, 2, 4, 2, 5>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
     }
     if (big >= 256) return launch<4, 2, 2>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
+    // up to 128 rows, or a long K: the deep-pipelined one-wave tiles with K shared over workgroups
+    // (4096 x 11008: 28 -> 17-21 us up to 128 rows, but 33 -> 39 us at 256; 11008 x 4096: 66 -> 18-25 us, 69 -> 39 us)
+    if (k % kBK == 0 && (m <= 128 || k >= 8192) && (uint64_t)m * n < (1ull << 28))
+        return launch_small(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
     if (mid >= 256) return launch<2, 2, 2>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
     return launch<1, 1, 2>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
 }

@@ -229,7 +229,12 @@ def test_i8_quantize_cols_t_bit_exact(ops, k, n):
 
 
 @pytest.mark.parametrize("m,k,n", [(32, 512, 512), (1, 16, 1), (77, 208, 133), (256, 1024, 384),
-                                   (300, 4096, 260), (2048, 256, 2304)])
+                                   (300, 4096, 260), (2048, 256, 2304),
+                                   # few tiles, K % 64 == 0: one-wave tiles, K shared over workgroups
+                                   (32, 4096, 1100),          # eight shares
+                                   (1, 4096, 64), (128, 1088, 70),   # 17 K steps in two shares of 9 and 8
+                                   (5, 576, 200),             # 9 steps: a single share
+                                   (300, 8192, 130)])         # long K beyond 128 rows
 def test_i8_gemm_accumulators_bit_exact(ops, m, k, n):
     check_i8_gemm(ops, m, k, n)
 
