@@ -232,7 +232,9 @@ def test_i8_quantize_cols_t_bit_exact(ops, k, n):
                                    (300, 4096, 260), (2048, 256, 2304),
                                    # few tiles, K % 64 == 0: one-wave tiles, K shared over workgroups
                                    (32, 4096, 1100),          # eight shares
-                                   (1, 4096, 64), (128, 1088, 70),   # 17 K steps in two shares of 9 and 8
+                                   (6, 4096, 64), (128, 1088, 70),   # 17 K steps in two shares of 9 and 8
+                                   # up to 4 rows: the dot4 decode kernel
+                                   (1, 4096, 1100), (2, 11008, 130), (3, 5008, 67), (4, 4096, 260), (4, 48, 5),
                                    (5, 576, 200),             # 9 steps: a single share
                                    (300, 8192, 130)])         # long K beyond 128 rows
 def test_i8_gemm_accumulators_bit_exact(ops, m, k, n):
