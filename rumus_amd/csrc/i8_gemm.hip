@@ -400,9 +400,8 @@ extern "C" int rumus_hip_i8_gemm(const int8_t* xq, const int8_t* wq, const float
                   "i8_gemm: operands must be 16-byte aligned");
     if (m == 0 || n == 0) return RUMUS_HIP_OK;
     hipStream_t s = as_stream(stream);
-    // decode: up to 4 rows on v_dot4_i32_i8 (4096 x 11008 from a HIP graph, one cache-resident copy of the weights:
-    // 7.8, 9.0, 11.6 us for 1, 2, 4 rows against 15.5 us for the one-wave MFMA tiles; at 8 rows the dot products
-    // cost 19.8 us; rotating copies from HBM: 11.2 us for one row)
+    // decode: up to 4 rows on v_dot4_i32_i8 (4096 x 11008 from a HIP graph over rotating weight copies: 9.3, 10.0,
+    // 12.7 us for 1, 2, 4 rows against 18.3 us for 8 rows on the one-wave MFMA tiles)
     if (m <= 4) return i8_launch_gemv(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
     // Largest tile that still gives every CU a workgroup.
     const uint64_t big = (uint64_t)ceil_div(m, 256) * ceil_div(n, 128);
