@@ -28,6 +28,10 @@ int i8_gemm_launch_wide(int tn, const int8_t* A, const int8_t* B, const float* s
 int i8_launch_gemv(const int8_t* xq, const int8_t* wq, const float* sx, const float* sw, const float* bias, int32_t* acc,
                    float* y, uint32_t m, uint32_t k, uint32_t n, hipStream_t s);
 
+// 5 to 32 rows, K % 256 == 0: MFMA tiles fed straight from global memory (i8_gemv.hip).
+int i8_launch_stream(const int8_t* xq, const int8_t* wq, const float* sx, const float* sw, const float* bias, int32_t* acc,
+                     float* y, uint32_t m, uint32_t k, uint32_t n, hipStream_t s);
+
 // chunk swizzle of an LDS row: bit0 = b1 ^ b3, bit1 = b2 of the row index
 __device__ __forceinline__ uint32_t row_swizzle(uint32_t row) {
     return (((row >> 1) ^ (row >> 3)) & 1u) | ((row >> 1) & 2u);

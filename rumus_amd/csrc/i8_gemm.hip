@@ -352,7 +352,7 @@ static int launch_small(const int8_t* A, const int8_t* B, const float* sx, const
     constexpr int NS = 8;
     constexpr size_t lds_bytes = (size_t)NS * 128 * kBK;       // 64 KB
     const uint32_t tm = ceil_div(M, 64), tn = ceil_div(N, 64), ksteps = K / kBK;
-    uint32_t shares = 512 / (tm * tn);
+    uint32_t shares = 512 / (tm * tn);   // more shares cost more in partial sums than they gain (1024: 25.7 us against 20.8)
     if (shares > 8) shares = 8;
     if (shares > ksteps / 8) shares = ksteps / 8;
     if (shares < 1) shares = 1;
@@ -403,6 +403,11 @@ extern "C" int rumus_hip_i8_gemm(const int8_t* xq, const int8_t* wq, const float
     // decode: up to 4 rows on v_dot4_i32_i8 (4096 x 11008 from a HIP graph over rotating weight copies: 9.3, 10.0,
     // 12.7 us for 1, 2, 4 rows against 18.3 us for 8 rows on the one-wave MFMA tiles)
     if (m <= 4) return i8_launch_gemv(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
+    // 5 to 16 rows (to 32 on smaller weights): MFMA tiles fed straight from global memory, a workgroup per 16 columns
+    // (from HBM, 8 rows: 4096 x 11008 14.5 us against 18.1 us for the LDS-staged tiles below, 4096 x 4096 7.4 against 12.8;
+    // 32 rows: 22.5 against 20.6 and 10.8 against 14.6)
+    if (k % 256 == 0 && (m <= 16 || (m <= 32 && (uint64_t)n * k <= (32ull << 20))))
+        return i8_launch_stream(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
     // Largest tile that still gives every CU a workgroup.
     const uint64_t big = (uint64_t)ceil_div(m, 256) * ceil_div(n, 128);
     const uint64_t mid = (uint64_t)ceil_div(m, 128) * ceil_div(n, 128);

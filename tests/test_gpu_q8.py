@@ -233,6 +233,8 @@ def test_i8_quantize_cols_t_bit_exact(ops, k, n):
                                    # few tiles, K % 64 == 0: one-wave tiles, K shared over workgroups
                                    (32, 4096, 1100),          # eight shares
                                    (6, 4096, 64), (128, 1088, 70),   # 17 K steps in two shares of 9 and 8
+                                   # 5 to 32 rows, K % 256 == 0: MFMA tiles fed straight from global memory
+                                   (5, 256, 16), (16, 1024, 100), (17, 1024, 40), (32, 2816, 70), (9, 11008, 30),
                                    # up to 4 rows: the dot4 decode kernel
                                    (1, 4096, 1100), (2, 11008, 130), (3, 5008, 67), (4, 4096, 260), (4, 48, 5),
                                    (5, 576, 200),             # 9 steps: a single share
