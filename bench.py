@@ -300,6 +300,29 @@ def bench_w4_gemm(torch, ops, m, steps=50, warmup=5):
             "tflops": flops / sec / 1e12, "f16_mfma_frac": flops / sec / 1e12 / F16_PEAK_TFLOPS}
 
 
+def bench_i8_small(torch, ops, steps=48, warmup=16):
+    """W8A8 at decode batch sizes, 4096 x 11008, rotating over 8 copies of the weights (361 MB: HBM,
+    not the Infinity Cache); graph-timed."""
+    k, n = 4096, 11008
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev).manual_seed(5)
+    wq, sw = ops.i8_quantize_cols_t(torch.randn((k, n), generator=gen, device=dev) * 0.02)
+    copies = [wq] + [wq.clone() for _ in range(7)]
+    rows = []
+    for m in (1, 4, 8, 32):
+        xq, sx = ops.i8_quantize_rows(torch.randn((m, k), generator=gen, device=dev))
+
+        def burst():
+            for c in copies:
+                ops.i8_gemm(xq, c, sx, sw, None)
+
+        total, launches, _ = time_graph(torch, burst, len(copies), steps, warmup)
+        sec = total / launches
+        rows.append({"workload": f"int8_gemm_{m}x4096x11008", "ms_per_launch": sec * 1e3, "weight_gbs": k * n / sec / 1e9,
+                     "hbm_frac": k * n / sec / 1e9 / HBM_PEAK_GBS})
+    return rows
+
+
 def bench_grad_x(torch, ops, steps=20, warmup=4):
     """grad_x of the INT4 Linear (QLinearBackward: grad_y . dequant(W)^T), K=4096, N=11008, g128:
     whole call, graph-timed."""
@@ -544,6 +567,7 @@ def main():
         out["w4_gemm"] = [bench_w4_gemm(torch, ops, 16), bench_w4_gemm(torch, ops, 128)]
         out["q8_matmul"] = bench_q8_matmul(torch, ops)
         out["w4_grad_x"] = bench_grad_x(torch, ops)
+        out["int8_decode"] = bench_i8_small(torch, ops)
         out["decoder_block"] = bench_decoder_block(torch, ops)
 
     if not args.no_cpu:
