@@ -375,6 +375,39 @@ static int launch_small(const int8_t* A, const int8_t* B, const float* sx, const
     return check_launch("i8_splitk_finish_kernel");
 }
 
+// Between the two (K % 64 == 0): 128 x 128 tiles of four waves, two workgroups per CU, K shared over workgroups
+// while the tiles alone would leave CUs idle.
+static int launch_mid(const int8_t* A, const int8_t* B, const float* sx, const float* sw, const float* bias,
+                      int32_t* acc, float* y, uint32_t M, uint32_t K, uint32_t N, hipStream_t s) {
+    constexpr int NS = 4;
+    constexpr size_t lds_bytes = (size_t)NS * 256 * kBK;       // 64 KB
+    const uint32_t tm = ceil_div(M, 128), tn = ceil_div(N, 128), ksteps = K / kBK;
+    // K shares: towards 256 workgroups, but the partial sums are paid per share: from 64 tiles on only a long K is
+    // shared (256 x 4096 x 4096, 64 tiles: 18.5 us whole, 20.1 in four shares; 256 x 11008 x 4096: 53.0 and 28.4)
+    const uint32_t tiles = tm * tn, min_steps = tiles < 64 ? 16 : 32;
+    uint32_t shares = 256 / tiles;
+    if (shares > 8) shares = 8;
+    if (shares > ksteps / min_steps) shares = ksteps / min_steps;
+    if (shares < 1 || (tiles >= 64 && ksteps < 128)) shares = 1;
+    const uint32_t steps_per = ceil_div(ksteps, shares);
+    shares = ceil_div(ksteps, steps_per);
+    if (shares == 1) {
+        hipLaunchKernelGGL((i8_gemm_dma_kernel<2, 2, 2, 2, NS>), dim3(tm * tn, 1), dim3(256), lds_bytes, s, A, B, sx, sw,
+                           bias, acc, y, M, K, N, tm, tn, steps_per);
+        return check_launch("i8_gemm_dma_kernel");
+    }
+    void* ws = nullptr;
+    if (int rc = workspace_get(s, (size_t)shares * M * N * sizeof(int32_t), &ws)) return rc;
+    int32_t* part = static_cast<int32_t*>(ws);
+    hipLaunchKernelGGL((i8_gemm_dma_kernel<2, 2, 2, 2, NS>), dim3(tm * tn, shares), dim3(256), lds_bytes, s, A, B,
+                       (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, part, (float*)nullptr, M, K, N,
+                       tm, tn, steps_per);
+    if (int rc = check_launch("i8_gemm_dma_kernel")) return rc;
+    hipLaunchKernelGGL(i8_splitk_finish_kernel, dim3(ceil_div(M * N, 256)), dim3(256), 0, s, part, shares, sx, sw, bias, acc,
+                       y, M, N);
+    return check_launch("i8_splitk_finish_kernel");
+}
+
 template <int TM, int TN, int OCC>
 static int launch(const int8_t* A, const int8_t* B, const float* sx, const float* sw,
                   const float* bias, int32_t* acc, float* y, uint32_t M, uint32_t K, uint32_t N,
@@ -418,9 +451,13 @@ extern "C" int rumus_hip_i8_gemm(const int8_t* xq, const int8_t* wq, const float
         return launch_dma<2, 2, 4, 2, 5>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
     }
     if (big >= 256) return launch<4, 2, 2>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
-    // up to 128 rows, or a long K: the deep-pipelined one-wave tiles with K shared over workgroups
-    // (4096 x 11008: 28 -> 17-21 us up to 128 rows, but 33 -> 39 us at 256; 11008 x 4096: 66 -> 18-25 us, 69 -> 39 us)
-    if (k % kBK == 0 && (m <= 128 || k >= 8192) && (uint64_t)m * n < (1ull << 28))
+    // more than 128 rows, fewer than 256 of the big tiles: 128 x 128 tiles, two workgroups per CU
+    // (1024 x 4096 x 4096: 39.6 -> 24.2 us, 1024 x 11008 x 4096: 97.5 -> 59.1 us, 256 x 4096 x 11008: 32.9 -> 22.9 us)
+    if (k % kBK == 0 && m > 128 && (uint64_t)m * n < (1ull << 28))
+        return launch_mid(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
+    // up to 128 rows: the deep-pipelined one-wave tiles with K shared over workgroups
+    // (4096 x 11008: 28 -> 17-21 us; 11008 x 4096: 66 -> 18-25 us)
+    if (k % kBK == 0 && (uint64_t)m * n < (1ull << 28))
         return launch_small(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
     if (mid >= 256) return launch<2, 2, 2>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
     return launch<1, 1, 2>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);

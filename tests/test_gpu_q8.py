@@ -238,7 +238,10 @@ def test_i8_quantize_cols_t_bit_exact(ops, k, n):
                                    # up to 4 rows: the dot4 decode kernel
                                    (1, 4096, 1100), (2, 11008, 130), (3, 5008, 67), (4, 4096, 260), (4, 48, 5),
                                    (5, 576, 200),             # 9 steps: a single share
-                                   (300, 8192, 130)])         # long K beyond 128 rows
+                                   (300, 8192, 130),          # 128 x 128 tiles, six of them, K in eight shares
+                                   (129, 1024, 129),          # the same tiles, four, ragged both ways, one share
+                                   (200, 4160, 384),          # 65 K steps in four shares of 17, 17, 17 and 14
+                                   (1000, 8192, 1100)])       # 72 tiles, three shares of 43, 43 and 42 steps
 def test_i8_gemm_accumulators_bit_exact(ops, m, k, n):
     check_i8_gemm(ops, m, k, n)
 
