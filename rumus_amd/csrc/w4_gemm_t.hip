@@ -386,9 +386,17 @@ int w4_launch_gemm_t(const float* gy, const uint32_t* packed, const float* scale
                        n);
     if (int rc = check_launch("w4t_prepare_kernel")) return rc;
     // stages of loads in flight: the step rate does not depend on them (3 to 5 measured within 4 %: the
-    // vector ALU work of the conversion sets the pace), so the count follows occupancy: four stages and
-    // two workgroups per compute unit up to two rounds of them, three stages and three workgroups beyond
-    const int ns = tiles * shares <= 1024 ? 4 : 3;
+    // vector ALU work of the conversion sets the pace), so the count follows occupancy: four stages leave
+    // LDS for two workgroups per compute unit, three stages for three.  Workgroups run in rounds of that many
+    // per CU and a round lasts the same whether it is full or not (544 workgroups: 678 us with four stages,
+    // 437 us with three), so the cheaper of the two by the measured round times (us at 4096 x 11008, g128; only
+    // their ratios matter) is taken.
+    auto rounds_cost = [](uint64_t wgs, uint32_t per_cu, const uint32_t* round_us) {
+        const uint64_t slots = 256ull * per_cu, rest = wgs % slots;
+        return (wgs / slots) * round_us[per_cu] + round_us[(rest + 255) / 256];
+    };
+    static const uint32_t us4[3] = {0, 225, 350}, us3[4] = {0, 260, 383, 465};   // by workgroups per CU in the round
+    const int ns = rounds_cost(tiles * shares, 3, us3) < rounds_cost(tiles * shares, 2, us4) ? 3 : 4;
     int rc;
     switch (ns) {
         case 4:
