@@ -86,47 +86,78 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(uint32_t* __restrict__ p
     if (i < n) p[i] = 0u;
 }
 
-// Pass 1: column abs-max.  Thread = one column, workgroup = 256 columns x one
-// K slice; slices combine with an integer atomic max on the float bits (exact
-// and order-independent for non-negative floats).
+// Pass 1: column abs-max.  Thread = four adjacent columns (one 128-bit load per row), workgroup = 1024 columns x
+// one K slice; slices combine with an integer atomic max on the float bits (exact and order-independent for
+// non-negative floats).
 __global__ __launch_bounds__(256) void col_absmax_kernel(const float* __restrict__ w,
                                                          uint32_t* __restrict__ amax_bits,
                                                          uint32_t k, uint32_t n, uint32_t kslice) {
-    const uint32_t col = blockIdx.x * 256 + threadIdx.x;
+    const uint32_t col = (blockIdx.x * 256 + threadIdx.x) * 4;
     if (col >= n) return;
     const uint32_t k0 = blockIdx.y * kslice, k1 = min(k, k0 + kslice);
-    float amax = 0.0f;
-    for (uint32_t r = k0; r < k1; r++) amax = fmaxf(amax, fabsf(w[(uint64_t)r * n + col]));
-    atomicMax(amax_bits + col, __float_as_uint(amax));
+    float amax[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (n % 4 == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0) {
+        for (uint32_t r = k0; r < k1; r++) {
+            const float4 v = *reinterpret_cast<const float4*>(w + (uint64_t)r * n + col);
+            amax[0] = fmaxf(amax[0], fabsf(v.x)); amax[1] = fmaxf(amax[1], fabsf(v.y));
+            amax[2] = fmaxf(amax[2], fabsf(v.z)); amax[3] = fmaxf(amax[3], fabsf(v.w));
+        }
+    } else {
+        for (uint32_t r = k0; r < k1; r++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (col + j < n) amax[j] = fmaxf(amax[j], fabsf(w[(uint64_t)r * n + col + j]));
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+        if (col + j < n) atomicMax(amax_bits + col + j, __float_as_uint(amax[j]));
 }
 
-// Pass 2: 64x64 tile, quantize with the column's inv and write transposed.
+// Pass 2: 64x64 tile, quantize with the column's inv and write transposed.  Reads are 128-bit over
+// four adjacent columns, writes 128-bit over sixteen consecutive k of one column; the tile turns in LDS.
 __global__ __launch_bounds__(256) void quantize_cols_t_kernel(const float* __restrict__ w,
                                                               const float* __restrict__ amax,
                                                               int8_t* __restrict__ wq, uint32_t k,
                                                               uint32_t n) {
-    __shared__ int8_t t[64][64 + 4];   // [col][k]
+    __shared__ __attribute__((aligned(16))) int8_t t[64][64 + 16];   // [col][k]; rows 16-byte aligned
     const uint32_t k0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
-    const uint32_t tx = threadIdx.x % 64, ty = threadIdx.x / 64;  // 64 cols x 4 rows
-    const uint32_t col = c0 + tx;
-    float inv = 0.0f;
-    if (col < n) {
-        float am = amax[col];
-        inv = am == 0.0f ? 0.0f : __fdiv_rn(127.0f, am);
+    const uint32_t tx = threadIdx.x % 16, ty = threadIdx.x / 16;  // 16 groups of 4 columns x 16 rows
+    const uint32_t col = c0 + 4 * tx;
+    const bool vec = n % 4 == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0;   // then col + 3 < n whenever col < n
+    float inv[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const float am = col + j < n ? amax[col + j] : 0.0f;
+        inv[j] = am == 0.0f ? 0.0f : __fdiv_rn(127.0f, am);
     }
-    for (uint32_t r = ty; r < 64; r += 4) {
-        uint32_t kk = k0 + r;
-        int q = 0;
-        if (kk < k && col < n) q = q_i8(w[(uint64_t)kk * n + col], inv);
-        t[tx][r] = (int8_t)q;
+#pragma unroll
+    for (uint32_t r = ty; r < 64; r += 16) {
+        const uint32_t kk = k0 + r;
+        float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (kk < k) {
+            if (vec && col < n) {
+                const float4 q = *reinterpret_cast<const float4*>(w + (uint64_t)kk * n + col);
+                v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if (col + j < n) v[j] = w[(uint64_t)kk * n + col + j];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) t[4 * tx + j][r] = (int8_t)q_i8(v[j], inv[j]);
     }
     __syncthreads();
     // write: thread handles one column row, 16 consecutive k bytes
     const uint32_t oc = threadIdx.x / 4, seg = (threadIdx.x % 4) * 16;
-    if (c0 + oc < n) {
+    if (c0 + oc < n && k0 + seg < k) {
         int8_t* dst = wq + (uint64_t)(c0 + oc) * k + k0 + seg;
-        for (uint32_t i = 0; i < 16; i++)
-            if (k0 + seg + i < k) dst[i] = t[oc][seg + i];
+        if (k % 16 == 0 && (reinterpret_cast<uintptr_t>(wq) & 15) == 0) {
+            *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(&t[oc][seg]);
+        } else {
+            for (uint32_t i = 0; i < 16; i++)
+                if (k0 + seg + i < k) dst[i] = t[oc][seg + i];
+        }
     }
 }
 
@@ -171,8 +202,8 @@ int rumus_hip_i8_quantize_cols_t(const float* w, int8_t* wq, float* sw, uint32_t
     // sw doubles as the abs-max accumulator until pass 3 turns it into scales.
     hipLaunchKernelGGL(fill_zero_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, s,
                        reinterpret_cast<uint32_t*>(sw), n);
-    const uint32_t kslice = 128;
-    hipLaunchKernelGGL(col_absmax_kernel, dim3(ceil_div(n, 256), ceil_div(k, kslice)), dim3(256), 0,
+    const uint32_t kslice = 64;
+    hipLaunchKernelGGL(col_absmax_kernel, dim3(ceil_div(n, 1024), ceil_div(k, kslice)), dim3(256), 0,
                        s, w, reinterpret_cast<uint32_t*>(sw), k, n, kslice);
     hipLaunchKernelGGL(quantize_cols_t_kernel, dim3(ceil_div(n, 64), ceil_div(k, 64)), dim3(256), 0,
                        s, w, sw, wq, k, n);

@@ -215,7 +215,7 @@ def test_i8_quantize_rows_bit_exact(ops, rows, cols):
     np.testing.assert_array_equal(host(s), ws)
 
 
-@pytest.mark.parametrize("k,n", [(512, 512), (100, 37), (4096, 200), (64, 1)])
+@pytest.mark.parametrize("k,n", [(512, 512), (100, 37), (4096, 200), (64, 1), (208, 130), (72, 64), (1024, 2052)])
 def test_i8_quantize_cols_t_bit_exact(ops, k, n):
     say(f"i8_quantize_cols_t k={k} n={n}")
     rng = np.random.default_rng(k + n)
