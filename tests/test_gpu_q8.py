@@ -241,7 +241,8 @@ def test_i8_quantize_cols_t_bit_exact(ops, k, n):
                                    (300, 8192, 130),          # 128 x 128 tiles, six of them, K in eight shares
                                    (129, 1024, 129),          # the same tiles, four, ragged both ways, one share
                                    (200, 4160, 384),          # 65 K steps in four shares of 17, 17, 17 and 14
-                                   (1000, 8192, 1100)])       # 72 tiles, three shares of 43, 43 and 42 steps
+                                   (1000, 8192, 1100),        # 72 tiles, three shares of 43, 43 and 42 steps
+                                   (300, 208, 260), (2048, 208, 2304)])   # K % 64 != 0: the register-staged tiles
 def test_i8_gemm_accumulators_bit_exact(ops, m, k, n):
     check_i8_gemm(ops, m, k, n)
 
