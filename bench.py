@@ -323,6 +323,40 @@ def bench_i8_small(torch, ops, steps=48, warmup=16):
     return rows
 
 
+def bench_i8_mid(torch, ops, steps=20, warmup=4):
+    """W8A8 GEMM between the decode and the prefill shapes (1024 rows on the square and the down-projection
+    weights): the 128 x 128 tile kernel; graph-timed, the vendor library's i32-output GEMM beside it."""
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev).manual_seed(6)
+    rows = []
+    for (m, k, n) in ((1024, 4096, 4096), (1024, 11008, 4096), (256, 4096, 11008)):
+        wq, sw = ops.i8_quantize_cols_t(torch.randn((k, n), generator=gen, device=dev) * 0.02)
+        xq, sx = ops.i8_quantize_rows(torch.randn((m, k), generator=gen, device=dev))
+        y = torch.empty((m, n), dtype=torch.float32, device=dev)
+
+        def burst():
+            for _ in range(4):
+                ops.i8_gemm(xq, wq, sx, sw, None, out=y)
+
+        total, launches, _ = time_graph(torch, burst, 4, steps, warmup)
+        sec = total / launches
+        row = {"workload": f"int8_gemm_{m}x{k}x{n}", "ms_per_launch": sec * 1e3, "tops": 2.0 * m * k * n / sec / 1e12}
+        try:
+            wt = wq.t()
+
+            def vendor():
+                for _ in range(4):
+                    torch._int_mm(xq, wt)
+
+            vt, vl, _ = time_graph(torch, vendor, 4, steps, warmup)
+            row["vendor_int_mm_tops"] = 2.0 * m * k * n / (vt / vl) / 1e12
+        except Exception as e:                      # not every torch build can capture it
+            row["vendor_int_mm_tops"] = None
+            log(f"vendor int_mm skipped: {e}")
+        rows.append(row)
+    return rows
+
+
 def bench_grad_x(torch, ops, steps=20, warmup=4):
     """grad_x of the INT4 Linear (QLinearBackward: grad_y . dequant(W)^T), K=4096, N=11008, g128:
     whole call, graph-timed."""
@@ -568,6 +602,7 @@ def main():
         out["q8_matmul"] = bench_q8_matmul(torch, ops)
         out["w4_grad_x"] = bench_grad_x(torch, ops)
         out["int8_decode"] = bench_i8_small(torch, ops)
+        out["int8_mid"] = bench_i8_mid(torch, ops)
         out["decoder_block"] = bench_decoder_block(torch, ops)
 
     if not args.no_cpu:
