@@ -57,7 +57,7 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-constexpr int kTileCols = 512;   // columns per workgroup (every wave-grid shape covers 512)
+constexpr int kTileCols = 512;   // columns per workgroup of eight waves
 constexpr int kStageK = 128;     // rows of K staged per barrier (8 MFMA steps of 16)
 constexpr int kMaxSplits = 16;
 
@@ -106,9 +106,9 @@ __device__ __forceinline__ float4 zp4_load(const uint32_t* zp4, uint32_t g, uint
     return w4_zp4_load4(zp4, g, n, col);
 }
 
-// The 8 waves of a workgroup form a WM x (8/WM) grid; a wave owns RT row tiles of 32 and TN
+// The WAVES (8 or 4) waves of a workgroup form a WM x (WAVES/WM) grid; a wave owns RT row tiles of 32 and TN
 // column tiles (its lanes hold TN adjacent columns each), so the workgroup covers
-// BM = 32*RT*WM rows and 512 columns.  Wide wave tiles matter: every wave reads the A fragments
+// BM = 32*RT*WM rows and 32*TN*WAVES/WM columns (512 with eight waves side by side).  Wide wave tiles matter: every wave reads the A fragments
 // of its rows from LDS at every step, and with 64-column waves (TN = 2) side by side those
 // reads, not the MFMAs, bound the 128-row tile.
 // DEPTH = stages of weights in flight; FOLD = MFMA steps between settlements of the zero-point
@@ -132,7 +132,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
     typedef typename WVec<TN>::floats floats_t;
     constexpr int WN = WAVES / WM;
     constexpr int RPP = 8 * WAVES;               // rows staged per pass: 8 threads per row
-    static_assert(WN * 32 * TN == kTileCols, "a workgroup covers 512 columns");
+    constexpr int COLS = WN * 32 * TN;           // columns per workgroup
     constexpr int BM = 32 * RT * WM;
     // bytes of one k16 step of one plane: [row tile][k block][row] x 16, plus 128 bytes of skew so
     // that the eight staging lanes of a row (one step each) do not write to the same banks
@@ -146,7 +146,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
     const uint32_t wm = wave / WN, wn = wave % WN;
     const uint32_t l32 = lane & 31, kb = lane >> 5;
     const uint32_t m0 = blockIdx.y * BM;
-    const uint32_t colbase = blockIdx.x * kTileCols + wn * (32 * TN) + TN * l32;   // this lane's TN columns
+    const uint32_t colbase = blockIdx.x * COLS + wn * (32 * TN) + TN * l32;   // this lane's TN columns
     const bool col_ok = colbase < a.n;                   // n % 4 == 0
     const uint32_t col_c = col_ok ? colbase : 0;
     const uint32_t nstages = (a.padded_k + kStageK - 1) / kStageK;
@@ -544,13 +544,13 @@ __global__ __launch_bounds__(256) void w4_convert_x_kernel(const float* __restri
 template <int RT, int WM, int TN, int WAVES, int DEPTH, int FOLD>
 static int launch_tile(const W4Args& a_in, hipStream_t s) {
     W4Args a = a_in;
-    const uint32_t tn = ceil_div(a.n, kTileCols), tm = ceil_div(a.m, 32 * RT * WM);
+    const uint32_t tn = ceil_div(a.n, (WAVES / WM) * 32 * TN), tm = ceil_div(a.m, 32 * RT * WM);
     const uint32_t nstages = ceil_div(a.padded_k, kStageK);
     uint32_t sps = nstages;
     const uint32_t splits = pick_splits(tn * tm, nstages, &sps);
     // 64-row tiles of eight waves: activations converted once, up front (10 % at m = 512).  The
     // four-wave shape has no registers to spare for the staged chunks and converts in place.
-    constexpr bool PRE = RT * WM >= 2 && WAVES == 8;
+    constexpr bool PRE = RT * WM >= 2 && (WAVES == 8 || (WAVES == 4 && TN == 2));
     constexpr uint32_t BM = 32 * RT * WM;
     // workspace: [activations in the form the kernel reads][partial tiles]
     const bool prepare = !PRE && (a.perm || a.k % 4 != 0 || (reinterpret_cast<uintptr_t>(a.x) & 15) != 0);
@@ -631,6 +631,16 @@ int w4_launch_gemm(const W4Args& a, hipStream_t s) {
     // no registers left for pre-converted activations: 3-20 % slower from m = 1024 to 4096.)
     const uint64_t col_tiles = ceil_div(a.n, kTileCols);
     if (ceil_div(a.m, 32) * col_tiles <= 72) return launch_fold<1, 1, 2, 8, 1>(a, s);
+    // The 64-row workgroups run one per CU, in rounds of 256 that last the same full or not (4096 x 11008, 1024 rows:
+    // 352 workgroups take as long as 512).  When the last round would be poorly filled, the same tile with four
+    // waves over 256 columns runs two per CU and a CU's last one alone at 3/4 of the time, while a pair costs 5 %
+    // more than one eight-wave workgroup (1024 rows: 255 -> 220 us, 768: 251 -> 210, but 2048: 405 -> 425).  Same
+    // order of the sums over K, same bits.
+    const uint64_t row_tiles = ceil_div(a.m, 64);
+    const uint64_t full_rounds = ceil_div(row_tiles * col_tiles, 256);
+    const uint64_t halves = ceil_div(row_tiles * ceil_div(a.n, kTileCols / 2), 256);       // on the busiest CU
+    if (row_tiles * col_tiles >= 192 && (halves / 2) * 105 + (halves % 2) * 75 < full_rounds * 97)
+        return launch_fold<2, 1, 2, 4, 1>(a, s);
     return launch_fold<2, 1, 2, 8, 1>(a, s);
 }
 

@@ -96,12 +96,12 @@ SHAPES = [
     (40, 1001, 64, 64, False),    # k % 4 != 0: activations are copied into padded rows first
     (100, 160, 520, 32, True),    # group 32: four settlements per stage, two row tiles
     (24, 192, 48, 96, False),     # group 96 does not divide a stage -> the f32 decode kernel in row chunks
-    (1536, 256, 8192, 128, True), # more than 72 tiles: eight waves of 64 rows each
+    (1536, 256, 8192, 128, True), # 384 tiles of 64 rows: four waves over 256 columns, two workgroups per CU
     (1500, 128, 8200, 64, False), # the same, group 64, ragged rows and columns
     (300, 160, 4100, 32, True),   # the same, group 32, K tail inside a stage
-    (2048, 256, 8192, 128, True), # 256 tiles of 128 rows: four-wave workgroups, 64 x 128 per wave
-    (1990, 192, 8200, 64, False), # four-wave workgroups, group 64, ragged rows and columns
-    (2100, 96, 8192, 32, True),   # four-wave workgroups, group 32, K shorter than a stage
+    (2048, 256, 8192, 128, True), # 512 tiles of 64 rows: two full rounds of eight-wave workgroups
+    (1990, 192, 8200, 64, False), # 544 tiles: four-wave workgroups, group 64, ragged rows and columns
+    (2100, 96, 8192, 32, True),   # 528 tiles: four-wave workgroups, group 32, K shorter than a stage
 ]
 
 
@@ -457,7 +457,8 @@ def test_awq_rejects_bad_shapes(ops):
     (3, 200, 24, 8, True),          # group 8 -> reference-order kernel
     (16, 4096, 4096, 128, True),    # MFMA kernel, K split
     (70, 512, 520, 32, False),      # MFMA kernel, group 32
-    (300, 256, 8192, 128, True),    # MFMA kernel, 128-row tiles
+    (300, 256, 8192, 128, True),    # MFMA kernel, eight-wave 64-row tiles
+    (1536, 128, 8192, 128, False),  # MFMA kernel, four-wave 64-row tiles (384 tiles: a poorly filled second round)
 ])
 def test_qmatmul_int4_zp4_vs_oracle(ops, m, k, n, g, with_bias):
     say(f"qmatmul_int4_zp4 m={m} k={k} n={n} g={g}")
