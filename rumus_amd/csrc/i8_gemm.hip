@@ -448,6 +448,21 @@ extern "C" int rumus_hip_i8_gemm(const int8_t* xq, const int8_t* wq, const float
         // one round of 256 x (256..352) tiles when the shape divides that way
         if (const int tn = i8_gemm_wide_width(m, n, 256))
             return i8_gemm_launch_wide(tn, xq, wq, sx, sw, bias, acc, y, m, k, n, s);
+        // The 256 x 128 tiles run one per CU in rounds of 256 that last the same full or not.  When the column
+        // tiles divide a round and the last round would be at most half full, the rows of the whole rounds and
+        // the rest are launched apart: the rest then takes the smaller tiles below at about 0.6 of a round
+        // (3072 x 11008 x 4096: 177 -> 1.6 rounds).  Rows are independent, so the results are the same.
+        const uint32_t col_tiles = ceil_div(n, 128), row_tiles = ceil_div(m, 256);
+        if (256 % col_tiles == 0) {
+            const uint32_t per_round = 256 / col_tiles, rest = row_tiles % per_round;
+            if (row_tiles > per_round && rest != 0 && 2 * rest <= per_round) {
+                const uint32_t m1 = (row_tiles - rest) * 256;
+                if (int rc = rumus_hip_i8_gemm(xq, wq, sx, sw, bias, acc, y, m1, k, n, stream)) return rc;
+                return rumus_hip_i8_gemm(xq + (uint64_t)m1 * k, wq, sx ? sx + m1 : nullptr, sw, bias,
+                                         acc ? acc + (uint64_t)m1 * n : nullptr, y ? y + (uint64_t)m1 * n : nullptr,
+                                         m - m1, k, n, stream);
+            }
+        }
         return launch_dma<2, 2, 4, 2, 5>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
     }
     if (big >= 256) return launch<4, 2, 2>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);

@@ -242,7 +242,8 @@ def test_i8_quantize_cols_t_bit_exact(ops, k, n):
                                    (129, 1024, 129),          # the same tiles, four, ragged both ways, one share
                                    (200, 4160, 384),          # 65 K steps in four shares of 17, 17, 17 and 14
                                    (1000, 8192, 1100),        # 72 tiles, three shares of 43, 43 and 42 steps
-                                   (300, 208, 260), (2048, 208, 2304)])   # K % 64 != 0: the register-staged tiles
+                                   (300, 208, 260), (2048, 208, 2304),   # K % 64 != 0: the register-staged tiles
+                                   (2250, 128, 4096)])        # one whole round of 256 x 128 tiles, the other 202 rows apart
 def test_i8_gemm_accumulators_bit_exact(ops, m, k, n):
     check_i8_gemm(ops, m, k, n)
 
