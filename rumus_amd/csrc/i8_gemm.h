@@ -17,9 +17,7 @@ typedef void __attribute__((address_space(3)))* lptr_t;
 // s_waitcnt with only vmcnt set (gfx9 encoding: vmcnt[3:0] | expcnt 7 | lgkmcnt 15 | vmcnt[5:4] << 14)
 #define RUMUS_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | 0x70 | 0xF00)
 
-// Wide-tile kernel (i8_gemm_wide.hip): tile width in 32-column units that deals the
-// problem to `cus` compute units in whole rounds with little padding, 0 if none does.
-int i8_gemm_wide_width(uint32_t M, uint32_t N, uint32_t cus);
+// Wide-block kernel (i8_gemm_wide.hip): 256 x 32*tn blocks, tn = 8..12.
 int i8_gemm_launch_wide(int tn, const int8_t* A, const int8_t* B, const float* sx, const float* sw,
                         const float* bias, int32_t* acc, float* y, uint32_t M, uint32_t K, uint32_t N,
                         hipStream_t s);

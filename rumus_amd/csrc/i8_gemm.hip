@@ -418,6 +418,27 @@ static int launch(const int8_t* A, const int8_t* B, const float* sx, const float
     return check_launch("i8_gemm_kernel");
 }
 
+// Launch cost by rounds, in units of one round of 256 x 256 blocks (the wide kernel at width 8; 70 us at K = 4096,
+// 161 us at K = 11008), from measurements on N = 4096 .. 22016: a round of 256 x 32w blocks costs w/8; a round of
+// 256 x 128 tiles 0.63 (half the area: the wide blocks are the better kernel where they fill their rounds); below
+// 256 of those tiles the 128 x 128 tiles run two per CU, a pair at 0.83 and a single one at 0.38.
+struct I8Plan { double cost; int wide; };    // wide: block width in 32-column units, 0 = the narrower tiles
+static double i8_round_cost(int w) { return w ? w / 8.0 : 0.63; }
+static I8Plan i8_plan_single(uint32_t m, uint32_t n) {
+    const uint64_t narrow = (uint64_t)ceil_div(m, 256) * ceil_div(n, 128);
+    if (narrow < 256) {
+        const uint64_t per_cu = ((uint64_t)ceil_div(m, 128) * ceil_div(n, 128) + 255) / 256;
+        return {(per_cu / 2) * 0.83 + (per_cu % 2) * 0.38, 0};
+    }
+    I8Plan best{(double)((narrow + 255) / 256) * i8_round_cost(0), 0};
+    for (int w = 8; w <= 12; w++) {
+        const uint64_t blocks = (uint64_t)ceil_div(m, 256) * ceil_div(n, 32 * w);
+        const double c = (double)((blocks + 255) / 256) * i8_round_cost(w);
+        if (c < best.cost) best = {c, w};
+    }
+    return best;
+}
+
 }  // namespace rumus
 
 using namespace rumus;
@@ -445,24 +466,32 @@ extern "C" int rumus_hip_i8_gemm(const int8_t* xq, const int8_t* wq, const float
     const uint64_t big = (uint64_t)ceil_div(m, 256) * ceil_div(n, 128);
     const uint64_t mid = (uint64_t)ceil_div(m, 128) * ceil_div(n, 128);
     if (big >= 256 && k % kBK == 0) {
-        // one round of 256 x (256..352) tiles when the shape divides that way
-        if (const int tn = i8_gemm_wide_width(m, n, 256))
-            return i8_gemm_launch_wide(tn, xq, wq, sx, sw, bias, acc, y, m, k, n, s);
-        // The 256 x 128 tiles run one per CU in rounds of 256 that last the same full or not.  When the column
-        // tiles divide a round and the last round would be at most half full, the rows of the whole rounds and
-        // the rest are launched apart: the rest then takes the smaller tiles below at about 0.6 of a round
-        // (3072 x 11008 x 4096: 177 -> 1.6 rounds).  Rows are independent, so the results are the same.
-        const uint32_t col_tiles = ceil_div(n, 128), row_tiles = ceil_div(m, 256);
-        if (256 % col_tiles == 0) {
-            const uint32_t per_round = 256 / col_tiles, rest = row_tiles % per_round;
-            if (row_tiles > per_round && rest != 0 && 2 * rest <= per_round) {
-                const uint32_t m1 = (row_tiles - rest) * 256;
-                if (int rc = rumus_hip_i8_gemm(xq, wq, sx, sw, bias, acc, y, m1, k, n, stream)) return rc;
-                return rumus_hip_i8_gemm(xq + (uint64_t)m1 * k, wq, sx ? sx + m1 : nullptr, sw, bias,
-                                         acc ? acc + (uint64_t)m1 * n : nullptr, y ? y + (uint64_t)m1 * n : nullptr,
-                                         m - m1, k, n, stream);
-            }
+        // Workgroups of the large tiles run one per CU, in rounds of 256 that last the same full or not, so the
+        // kernel is chosen by rounds: see i8_plan_single.  Rows are independent, so when whole rounds of one
+        // kernel plus a cheaper launch for the rest cost less than any single launch (6144 x 11008 x 4096: three
+        // rounds of 256 x 128 tiles 357 us; 4096 rows in one round of 256 x 256 blocks + 2048 rows 263 us), the
+        // two parts are launched apart; same results.
+        const I8Plan one = i8_plan_single(m, n);
+        uint32_t split_rows = 0;
+        double split_cost = one.cost * 0.97;                     // a second launch has to pay for itself
+        for (int w = 0; w <= 12; w = w ? w + 1 : 8) {            // 0: the 256 x 128 tiles
+            const uint32_t cols = ceil_div(n, w ? 32 * w : 128);
+            if (cols > 256) continue;
+            const uint32_t rows_per_round = (256 / cols) * 256;
+            if (m <= rows_per_round) continue;
+            const uint32_t m1 = (m / rows_per_round) * rows_per_round;
+            if (m1 == m) continue;
+            const double c = (m1 / rows_per_round) * i8_round_cost(w) + i8_plan_single(m - m1, n).cost;
+            if (c < split_cost) { split_cost = c; split_rows = m1; }
         }
+        if (split_rows) {
+            const uint32_t m1 = split_rows;
+            if (int rc = rumus_hip_i8_gemm(xq, wq, sx, sw, bias, acc, y, m1, k, n, stream)) return rc;
+            return rumus_hip_i8_gemm(xq + (uint64_t)m1 * k, wq, sx ? sx + m1 : nullptr, sw, bias,
+                                     acc ? acc + (uint64_t)m1 * n : nullptr, y ? y + (uint64_t)m1 * n : nullptr,
+                                     m - m1, k, n, stream);
+        }
+        if (one.wide) return i8_gemm_launch_wide(one.wide, xq, wq, sx, sw, bias, acc, y, m, k, n, s);
         return launch_dma<2, 2, 4, 2, 5>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
     }
     if (big >= 256) return launch<4, 2, 2>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);

@@ -219,20 +219,6 @@ static int launch_wide(const int8_t* A, const int8_t* B, const float* sx, const 
     return check_launch("i8_gemm_wide_kernel");
 }
 
-// Picks the block width (in 32-column units, 8..12) that leaves the fewest idle
-// CU slots when the blocks are dealt to `cus` compute units; 0 = not worth it.
-int i8_gemm_wide_width(uint32_t M, uint32_t N, uint32_t cus) {
-    int best = 0;
-    double best_eff = 0.80;     // below this the narrow kernel's finer tiles win
-    for (int w = 8; w <= 12; w++) {
-        const uint64_t tiles = (uint64_t)ceil_div(M, kWideBM) * ceil_div(N, 32 * w);
-        const uint64_t rounds = (tiles + cus - 1) / cus;
-        const double eff = ((double)M * N) / ((double)rounds * cus * kWideBM * 32 * w);
-        if (eff > best_eff) { best_eff = eff; best = w; }
-    }
-    return best;
-}
-
 int i8_gemm_launch_wide(int w, const int8_t* A, const int8_t* B, const float* sx, const float* sw,
                         const float* bias, int32_t* acc, float* y, uint32_t M, uint32_t K, uint32_t N,
                         hipStream_t s) {

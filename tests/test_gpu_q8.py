@@ -243,7 +243,7 @@ def test_i8_quantize_cols_t_bit_exact(ops, k, n):
                                    (200, 4160, 384),          # 65 K steps in four shares of 17, 17, 17 and 14
                                    (1000, 8192, 1100),        # 72 tiles, three shares of 43, 43 and 42 steps
                                    (300, 208, 260), (2048, 208, 2304),   # K % 64 != 0: the register-staged tiles
-                                   (2250, 128, 4096)])        # one whole round of 256 x 128 tiles, the other 202 rows apart
+                                   (2250, 128, 4096)])        # 144 blocks of 256 x 256: one partly filled round
 def test_i8_gemm_accumulators_bit_exact(ops, m, k, n):
     check_i8_gemm(ops, m, k, n)
 
@@ -253,7 +253,9 @@ def test_i8_gemm_accumulators_bit_exact(ops, m, k, n):
 # pipeline stages included), a ragged last row block and N that is not a multiple of 32.
 @pytest.mark.parametrize("m,k,n", [(4096, 192, 4096), (2048, 64, 9216), (2048, 128, 10240),
                                    (2048, 320, 11008), (2000, 64, 10990), (2048, 64, 12288),
-                                   (1990, 128, 12281)])
+                                   (1990, 128, 12281),
+                                   # whole rounds and the rest launched apart: 4096 + 2048 rows, 1024 + 512 rows
+                                   (6144, 64, 4096), (1536, 64, 16384), (1500, 128, 16300)])
 def test_i8_gemm_wide_blocks_bit_exact(ops, m, k, n):
     check_i8_gemm(ops, m, k, n)
 
