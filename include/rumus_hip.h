@@ -54,15 +54,22 @@ const char* rumus_hip_version(void);
 int rumus_hip_sync(rumus_hip_stream_t stream);
 
 /* Workspace.  The reference takes every temporary from its BufferPool
- * (rumus/src/backend/gpu/pool.rs:34-75) and returns it on drop; here the only
- * temporaries are those of qmatmul_int4 / _perm / _zp4 with m > 5 (the partial
- * sums when K is split over workgroups, and a copy of x when it has to be
- * gathered or padded) and of attention with q_len == 1 (partial results per
- * slice of 256 keys).  They live in one device buffer per (device, stream),
- * grown on demand inside the call that needs it.  A caller that must not
- * allocate later (graph capture, serving loop) reserves the size up front:
- * at most (m * k + 16 * m * n) * 4 + 256 bytes per matmul call and
- * batch * heads * ceil(kv_len / 256) * 520 bytes per attention call.
+ * (rumus/src/backend/gpu/pool.rs:34-75) and returns it on drop; here the
+ * temporaries live in one device buffer per (device, stream), grown on demand
+ * inside the call that needs it.  A caller that must not allocate later
+ * (graph capture, serving loop) reserves the largest size up front.  Upper
+ * bounds per call, in bytes:
+ *   qmatmul_int4 / _perm / _zp4, m > 5: 5 * (m + 64) * (k + 128) (activations
+ *       in matrix-core order) + 64 * m * n (partial sums, only while the
+ *       output has fewer than 192 tiles of 64 x 512) + 256;
+ *   qmatmul_int4_t, m >= 8: 64 * m * k (partial sums, only below 512 tiles of
+ *       64 x 128) + 10 * num_groups * n + 4 * (m + num_groups) + 2048;
+ *   i8_gemm: 32 * m * n, and only while the output has fewer than 512 tiles of
+ *       64 x 64 (K shared over workgroups): at most 16 MiB;
+ *   matmul_q8, m >= 5: 4 * m * k * 4 (digit planes of a) + 4 * m * n * 4 + 32 MiB
+ *       (partial sums of the int8 GEMM inside); with one block per column from
+ *       384 rows on also k * n + 4 * n;
+ *   attention with q_len == 1: batch * heads * ceil(kv_len / 256) * 520.
  * rumus_hip_shutdown frees every workspace (no launch may be in flight). */
 int rumus_hip_workspace_reserve(rumus_hip_stream_t stream, uint64_t bytes);
 int rumus_hip_shutdown(void);

@@ -16,6 +16,18 @@ int check_hip(hipError_t e, const char* what);
 
 // Device workspace of at least `bytes` for work queued on `stream` (runtime.hip).
 int workspace_get(hipStream_t stream, size_t bytes, void** out);
+// A call that holds workspace memory and then calls another entry point that takes workspace of its own on the
+// same stream (the Q8 matmul around the int8 GEMM) asks for both sizes at once and keeps one of these alive over
+// the inner call: workspace_get then hands out the part of the buffer behind `offset`, and fails instead of
+// growing (growing would free what the outer call still uses).
+struct WorkspaceNest {
+    explicit WorkspaceNest(size_t offset);
+    ~WorkspaceNest();
+    WorkspaceNest(const WorkspaceNest&) = delete;
+    WorkspaceNest& operator=(const WorkspaceNest&) = delete;
+  private:
+    size_t prev_;
+};
 
 // hipGetLastError() after a kernel launch.
 inline int check_launch(const char* kernel) { return check_hip(hipGetLastError(), kernel); }

@@ -418,6 +418,15 @@ static int launch(const int8_t* A, const int8_t* B, const float* sx, const float
     return check_launch("i8_gemm_kernel");
 }
 
+size_t i8_gemm_workspace_bound(uint32_t m, uint32_t n) {
+    // launch_small shares K below 512 tiles of 64 x 64, launch_mid below 128 tiles of 128 x 128 (the same area);
+    // the two parts of a row split are each smaller than the whole
+    // (shares <= 512 / tiles and <= 256 / tiles: at most 16 MiB of partial sums whatever the shape)
+    if ((uint64_t)ceil_div(m, 64) * ceil_div(n, 64) > 1024) return 0;
+    const size_t all = (size_t)8 * m * n * sizeof(int32_t), cap = size_t(32) << 20;
+    return all < cap ? all : cap;
+}
+
 // Launch cost by rounds, in units of one round of 256 x 256 blocks (the wide kernel at width 8; 70 us at K = 4096,
 // 161 us at K = 11008), from measurements on N = 4096 .. 22016: a round of 256 x 32w blocks costs w/8; a round of
 // 256 x 128 tiles 0.63 (half the area: the wide blocks are the better kernel where they fill their rounds); below

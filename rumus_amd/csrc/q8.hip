@@ -6,6 +6,7 @@
 #include <hip/hip_fp16.h>
 
 #include "common.h"
+#include "i8_gemm.h"
 
 namespace rumus {
 
@@ -490,8 +491,13 @@ static int matmul_q8_mfma(const float* a, const uint32_t* b, float* c, uint32_t 
     const size_t planes_bytes = align256((size_t)kQ8Planes * m * k), sx_bytes = align256((size_t)kQ8Planes * m * sizeof(float));
     const size_t wq_bytes = align256((size_t)n * k), sw_bytes = align256((size_t)n * sizeof(float));
     const size_t y_bytes = (size_t)kQ8Planes * m * n * sizeof(float);
+    // the int8 GEMM below shares K over workgroups on small outputs and keeps the partial sums in the workspace
+    // too: room for them behind this call's own buffers
+    const size_t own_bytes = align256(planes_bytes + sx_bytes + wq_bytes + sw_bytes + y_bytes);
+    const size_t gemm_bytes = i8_gemm_workspace_bound(kQ8Planes * m, n);
     void* ws = nullptr;
-    if (int rc = workspace_get(s, planes_bytes + sx_bytes + wq_bytes + sw_bytes + y_bytes, &ws)) return rc;
+    if (int rc = workspace_get(s, own_bytes + gemm_bytes, &ws)) return rc;
+    WorkspaceNest nest(own_bytes);
     uint8_t* base = static_cast<uint8_t*>(ws);
     int8_t* planes = reinterpret_cast<int8_t*>(base);
     float* sxp = reinterpret_cast<float*>(base + planes_bytes);

@@ -49,11 +49,22 @@ std::mutex g_arena_mutex;
 std::unordered_map<ArenaKey, Arena, ArenaKeyHash> g_arenas;
 }  // namespace
 
+static thread_local size_t g_nest_offset = 0;
+WorkspaceNest::WorkspaceNest(size_t offset) : prev_(g_nest_offset) { g_nest_offset = offset; }
+WorkspaceNest::~WorkspaceNest() { g_nest_offset = prev_; }
+
 int workspace_get(hipStream_t stream, size_t bytes, void** out) {
     int device = 0;
     if (int rc = check_hip(hipGetDevice(&device), "hipGetDevice")) return rc;
     std::lock_guard<std::mutex> lock(g_arena_mutex);
     Arena& a = g_arenas[ArenaKey{device, stream}];
+    if (const size_t offset = g_nest_offset) {
+        if (a.bytes < offset + bytes)
+            return set_error(RUMUS_HIP_EINVAL, "nested workspace of %zu bytes behind %zu does not fit the %zu reserved", bytes,
+                             offset, a.bytes);
+        *out = static_cast<uint8_t*>(a.ptr) + offset;
+        return RUMUS_HIP_OK;
+    }
     if (a.bytes < bytes) {
         hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
         if (stream && hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)

@@ -102,6 +102,8 @@ def test_q8_rejects_bad_block_size(ops):
                                       (8, 48, 20, 48),         # W8A8 kernel on a dense copy: the smallest batch that goes there
                                       (400, 512, 96, 512),     # and from 384 rows on
                                       (1000, 4096, 264, 4096),
+                                      (400, 8192, 256, 8192),  # the int8 GEMM inside shares K eight ways: its partial sums sit
+                                      (384, 2048, 128, 2048),  # behind this call's planes in the workspace (two ways here)
                                       # block scales inside the MFMA loop: f16 planes for blocks up to 64 ...
                                       (5, 64, 64, 32),         # the smallest batch that goes there
                                       (11, 96, 20, 32),        # a fold per 32 k, K ends mid-step
