@@ -59,7 +59,7 @@ int rumus_hip_sync(rumus_hip_stream_t stream);
  * inside the call that needs it.  A caller that must not allocate later
  * (graph capture, serving loop) reserves the largest size up front.  Upper
  * bounds per call, in bytes:
- *   qmatmul_int4 / _perm / _zp4, m > 5: 5 * (m + 64) * (k + 128) (activations
+ *   qmatmul_int4 / _perm / _zp4, m > 5: 5 * (m + 64) * (padded_k + 128) (activations
  *       in matrix-core order) + 64 * m * n (partial sums, only while the
  *       output has fewer than 192 tiles of 64 x 512) + 256;
  *   qmatmul_int4_t, m >= 8: 64 * m * k (partial sums, only below 512 tiles of
