@@ -598,7 +598,8 @@ def main():
     if not args.only_gemv:
         out["secondary"] = bench_i8_gemm(torch, ops)
         out["w4_gemv_wider"] = bench_gemv_shapes(torch, ops)
-        out["w4_gemm"] = [bench_w4_gemm(torch, ops, 16), bench_w4_gemm(torch, ops, 128)]
+        out["w4_gemm"] = [bench_w4_gemm(torch, ops, 16), bench_w4_gemm(torch, ops, 128),
+                          bench_w4_gemm(torch, ops, 1024, steps=10, warmup=2), bench_w4_gemm(torch, ops, 2048, steps=10, warmup=2)]
         out["q8_matmul"] = bench_q8_matmul(torch, ops)
         out["w4_grad_x"] = bench_grad_x(torch, ops)
         out["int8_decode"] = bench_i8_small(torch, ops)
