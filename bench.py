@@ -5,10 +5,13 @@
 
 Headline workload (the one the metric is quoted on): the INT4 AWQ-style W4 GEMV,
 M=1, K=4096, N=4096, group size 128, f32 activations, f32 scale + f32
-zero-point per group (the reference's storage).  A step is one GEMV launch over
-one weight set; the run rotates through 64 distinct weight sets (> 600 MB) so
-that the 256 MB Infinity Cache cannot serve the weights, with all inputs
-resident in HBM before the timed region.  The INT8 prefill GEMM
+zero-point per group (the reference's storage).  A step is one pass over the
+batch of synthetic input: 64 GEMV launches, one per distinct weight set
+(> 600 MB in all, so that the 256 MB Infinity Cache cannot serve the weights),
+replayed from one HIP graph, with all inputs resident in HBM before the timed
+region.  --steps K times exactly K such passes, each between its own pair of
+HIP events on the launch stream; the figure of record is the median pass.  The
+INT8 prefill GEMM
 (2048 x 4096 x 11008 on the i8 matrix cores) is timed in the same run and
 reported under "secondary".  One JSON line is printed on stdout.
 """
@@ -45,9 +48,11 @@ def log(msg):
     print(msg, file=sys.stderr, flush=True)
 
 
-def time_graph(torch, launch_all, launches_per_replay, steps, warmup):
-    """Capture `launch_all` (a burst of launches) in a HIP graph and time replays with HIP events
-    on the stream the kernels run on.  Returns (seconds_total, launches_timed, used_graph)."""
+def time_graph(torch, launch_all, launches_per_replay, replays, warmup_replays):
+    """Capture `launch_all` (a burst of `launches_per_replay` launches) in a HIP graph and time exactly
+    `replays` replays after `warmup_replays` untimed ones, every replay between its own pair of HIP
+    events on the stream the kernels run on.  Returns a dict: seconds per LAUNCH as median / mean / min /
+    max over the replays, the replay count and whether a graph was used."""
     stream = torch.cuda.current_stream()
     graph = None
     try:
@@ -65,17 +70,27 @@ def time_graph(torch, launch_all, launches_per_replay, steps, warmup):
         log(f"[bench] HIP graph capture unavailable ({e!r}); timing direct launches")
         torch.cuda.synchronize()
     run = graph.replay if graph is not None else launch_all
-    for _ in range(max(1, -(-warmup // launches_per_replay))):
+    replays = max(1, int(replays))
+    for _ in range(max(0, int(warmup_replays))):
         run()
     torch.cuda.synchronize()
-    replays = max(1, -(-steps // launches_per_replay))
-    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(replays):
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(replays + 1)]
+    marks[0].record()
+    for i in range(replays):
         run()
-    end.record()
+        marks[i + 1].record()
     torch.cuda.synchronize()
-    return start.elapsed_time(end) * 1e-3, replays * launches_per_replay, graph is not None
+    per = np.array([marks[i].elapsed_time(marks[i + 1]) for i in range(replays)]) * 1e-3 / launches_per_replay
+    return {"median": float(np.median(per)), "mean": float(marks[0].elapsed_time(marks[replays]) * 1e-3
+                                                              / (replays * launches_per_replay)),
+            "min": float(per.min()), "max": float(per.max()), "replays": replays,
+            "launches_per_replay": launches_per_replay, "graph": graph is not None}
+
+
+def spread(t):
+    """The per-replay statistics of time_graph, in microseconds per launch, for the JSON line."""
+    return {"replays": t["replays"], "launches_per_replay": t["launches_per_replay"],
+            "us_median": t["median"] * 1e6, "us_mean": t["mean"] * 1e6, "us_min": t["min"] * 1e6, "us_max": t["max"] * 1e6}
 
 
 def bench_gemv(torch, ops, steps, warmup):
@@ -117,22 +132,16 @@ def bench_gemv(torch, ops, steps, warmup):
         for (p, s, qz), y in zip(sets_awq, ys):
             ops.qmatmul_int4_decode_zp4(x, p, s, qz, K, G, out=y)
 
-    # the timed region of record: EXACTLY `steps` launches, bracketed by device syncs
-    sec, launches, used_graph = time_graph(torch, burst_rotating, WEIGHT_SETS, steps, warmup)
-    sec_res, launches_res, _ = time_graph(torch, burst_resident, WEIGHT_SETS, steps, warmup)
+    # the timed region of record: EXACTLY `steps` passes over the 64 weight sets
+    t = time_graph(torch, burst_rotating, WEIGHT_SETS, steps, warmup)
+    t_res = time_graph(torch, burst_resident, WEIGHT_SETS, steps, warmup)
     y0 = ys[0].cpu().numpy()
-    sec_awq, launches_awq, _ = time_graph(torch, burst_rotating_awq, WEIGHT_SETS, steps, warmup)
-    sec_ref, launches_ref, _ = time_graph(torch, burst_rotating_ref, WEIGHT_SETS, steps, warmup)
-    return {
-        "sec_ref": sec_ref, "launches_ref": launches_ref,
-        "sec_awq": sec_awq, "launches_awq": launches_awq,
-        "sec": sec, "launches": launches, "graph": used_graph,
-        "sec_resident": sec_res, "launches_resident": launches_res,
-        "x": x0, "w": w0, "y0": y0,
-    }
+    t_awq = time_graph(torch, burst_rotating_awq, WEIGHT_SETS, steps, warmup)
+    t_ref = time_graph(torch, burst_rotating_ref, WEIGHT_SETS, steps, warmup)
+    return {"t": t, "t_resident": t_res, "t_awq": t_awq, "t_ref": t_ref, "x": x0, "w": w0, "y0": y0}
 
 
-def bench_i8_gemm(torch, ops, steps=30, warmup=5):
+def bench_i8_gemm(torch, ops, replays=12, warmup=3):
     m, k, n = 2048, 4096, 11008
     dev = torch.device("cuda:0")
     gen = torch.Generator(device=dev).manual_seed(1)
@@ -142,24 +151,24 @@ def bench_i8_gemm(torch, ops, steps=30, warmup=5):
     wq, sw = ops.i8_quantize_cols_t(w)
     del w
     y = torch.empty((m, n), dtype=torch.float32, device=dev)
-    for _ in range(warmup):
-        ops.i8_gemm(xq, wq, sx, sw, None, out=y)
-    torch.cuda.synchronize()
-    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(steps):
-        ops.i8_gemm(xq, wq, sx, sw, None, out=y)
-    end.record()
-    torch.cuda.synchronize()
-    sec = start.elapsed_time(end) * 1e-3 / steps
+    per_graph = 10
+
+    def burst():
+        for _ in range(per_graph):
+            ops.i8_gemm(xq, wq, sx, sw, None, out=y)
+
+    t = time_graph(torch, burst, per_graph, replays, warmup)
+    sec = t["median"]
     ops_per = 2.0 * m * k * n
+
     # dynamic activation quantizer, timed separately (it precedes every GEMM in a forward)
-    start.record()
-    for _ in range(steps):
-        ops.i8_quantize_rows(x)
-    end.record()
-    torch.cuda.synchronize()
-    sec_q = start.elapsed_time(end) * 1e-3 / steps
+    xq2, sx2 = torch.empty_like(xq), torch.empty_like(sx)
+
+    def burst_q():
+        for _ in range(per_graph):
+            ops.i8_quantize_rows(x, out=(xq2, sx2))
+
+    sec_q = time_graph(torch, burst_q, per_graph, replays, warmup)["median"]
     tops = ops_per / sec / 1e12
     # Two yardsticks measured in the same run, on the same operands where it applies:
     # the matrix cores alone (MFMA from registers, random operand bits, no memory traffic:
@@ -169,18 +178,17 @@ def bench_i8_gemm(torch, ops, steps=30, warmup=5):
     vendor = None
     try:
         wt = wq.t()
-        for _ in range(warmup):
-            torch._int_mm(xq, wt)
-        start.record()
-        for _ in range(steps):
-            torch._int_mm(xq, wt)
-        end.record()
-        torch.cuda.synchronize()
-        vendor = ops_per / (start.elapsed_time(end) * 1e-3 / steps) / 1e12
+
+        def burst_vendor():
+            for _ in range(per_graph):
+                torch._int_mm(xq, wt)
+
+        vendor = ops_per / time_graph(torch, burst_vendor, per_graph, replays, warmup)["median"] / 1e12
     except Exception as exc:   # informational only
         log(f"[bench] vendor int8 GEMM not timed: {exc}")
     return {
-        "workload": "int8_gemm_2048x4096x11008", "ms_per_launch": sec * 1e3, "tops": tops,
+        "workload": "int8_gemm_2048x4096x11008", "ms_per_launch": sec * 1e3, "tops": tops, "hip_graph": t["graph"],
+        "timing": spread(t),
         "roofline": {"bound": "mfma", "achieved": tops, "peak": I8_PEAK_TOPS, "unit": "TOP/s",
                      "frac": tops / I8_PEAK_TOPS, "traffic": None},
         "mfma_only_random_operands": ceiling,
@@ -194,9 +202,9 @@ def bench_i8_gemm(torch, ops, steps=30, warmup=5):
 def probe_launch_floor():
     """What a single launch of the GEMV's size can reach on this GPU: an empty kernel, and a
     kernel that only reads 8 MiB (the packed weights) from 64 rotating buffers, both replayed
-    from a HIP graph (rumus_amd/csrc/probe_mfma.hip).  None when the probe library is absent."""
+    from a HIP graph (bench/probe_mfma.hip).  None when the probe library is absent."""
     import ctypes
-    path = os.path.join(ROOT, "rumus_amd", "librumus_probe.so")
+    path = os.path.join(ROOT, "bench", "librumus_probe.so")
     if not os.path.exists(path):
         return None
     lib = ctypes.CDLL(path)
@@ -214,9 +222,9 @@ def probe_launch_floor():
 
 def probe_mfma_ceiling():
     """int8 TOP/s of v_mfma_i32_32x32x32_i8 issued back to back from registers with random
-    operand bits (rumus_amd/csrc/probe_mfma.hip, its own small library), or None."""
+    operand bits (bench/probe_mfma.hip, its own small library), or None."""
     import ctypes
-    path = os.path.join(ROOT, "rumus_amd", "librumus_probe.so")
+    path = os.path.join(ROOT, "bench", "librumus_probe.so")
     if not os.path.exists(path):
         return None
     lib = ctypes.CDLL(path)
@@ -229,7 +237,7 @@ def probe_mfma_ceiling():
     return {"tops": tops.value, "shader_mhz": mhz.value}
 
 
-def bench_gemv_shapes(torch, ops, steps=400, warmup=40):
+def bench_gemv_shapes(torch, ops, replays=10, warmup=2):
     """The same decode kernel on the wider projections of a Llama-7B block (q|k|v, gate|up, down),
     each rotating over enough weight sets (> 600 MB) to defeat the Infinity Cache.  The longer a
     launch, the smaller the share of its fixed start-up and drain."""
@@ -237,7 +245,7 @@ def bench_gemv_shapes(torch, ops, steps=400, warmup=40):
     dev = torch.device("cuda:0")
     gen = torch.Generator(device=dev).manual_seed(5)
     probe = None
-    path = os.path.join(ROOT, "rumus_amd", "librumus_probe.so")
+    path = os.path.join(ROOT, "bench", "librumus_probe.so")
     if os.path.exists(path):
         probe = ctypes.CDLL(path)
         probe.rumus_probe_read_launch.restype = ctypes.c_int
@@ -259,9 +267,7 @@ def bench_gemv_shapes(torch, ops, steps=400, warmup=40):
             for p, s, z in sets:
                 ops.qmatmul_int4_decode(x, p, s, z, k, G, out=y)
 
-        launches = max(nsets, (steps // nsets) * nsets)
-        sec, timed, _ = time_graph(torch, burst, nsets, launches, warmup)
-        per = sec / timed
+        per = time_graph(torch, burst, nsets, replays, warmup)["median"]
         row = {"workload": f"w4_gemv_1x{k}x{n}_g128", "weight_sets_rotated": nsets, "bytes_per_step": nbytes,
                "ms_per_step": per * 1e3, "gbs": nbytes / per / 1e9, "hbm_frac": nbytes / per / 1e9 / HBM_PEAK_GBS}
         if probe is not None:
@@ -274,7 +280,7 @@ def bench_gemv_shapes(torch, ops, steps=400, warmup=40):
     return rows
 
 
-def bench_w4_gemm(torch, ops, m, steps=50, warmup=5):
+def bench_w4_gemm(torch, ops, m, replays=10, warmup=2):
     """W4 GEMM with act-order (GPTQ style), K=4096, N=11008, g128, symmetric zp=8."""
     k, n = 4096, 11008
     dev = torch.device("cuda:0")
@@ -291,8 +297,7 @@ def bench_w4_gemm(torch, ops, m, steps=50, warmup=5):
         for _ in range(10):
             ops.qmatmul_int4_perm(x, packed_sorted, scales, zp, k, G, perm=perm, out=y)
 
-    total, launches, _ = time_graph(torch, burst, 10, steps, warmup)
-    sec = total / launches
+    sec = time_graph(torch, burst, 10, replays, warmup)["median"]
     nbytes = k * n // 2 + (k // G) * n * 4 + k * 4 + m * k * 4 + m * n * 4
     flops = 2.0 * m * k * n
     return {"workload": f"w4_gemm_actorder_{m}x4096x11008_g128", "hip_graph": True, "ms_per_launch": sec * 1e3,
@@ -300,7 +305,7 @@ def bench_w4_gemm(torch, ops, m, steps=50, warmup=5):
             "tflops": flops / sec / 1e12, "f16_mfma_frac": flops / sec / 1e12 / F16_PEAK_TFLOPS}
 
 
-def bench_i8_small(torch, ops, steps=48, warmup=16):
+def bench_i8_small(torch, ops, replays=10, warmup=2):
     """W8A8 at decode batch sizes, 4096 x 11008, rotating over 8 copies of the weights (361 MB: HBM,
     not the Infinity Cache); graph-timed."""
     k, n = 4096, 11008
@@ -316,14 +321,13 @@ def bench_i8_small(torch, ops, steps=48, warmup=16):
             for c in copies:
                 ops.i8_gemm(xq, c, sx, sw, None)
 
-        total, launches, _ = time_graph(torch, burst, len(copies), steps, warmup)
-        sec = total / launches
+        sec = time_graph(torch, burst, len(copies), replays, warmup)["median"]
         rows.append({"workload": f"int8_gemm_{m}x4096x11008", "ms_per_launch": sec * 1e3, "weight_gbs": k * n / sec / 1e9,
                      "hbm_frac": k * n / sec / 1e9 / HBM_PEAK_GBS})
     return rows
 
 
-def bench_i8_mid(torch, ops, steps=20, warmup=4):
+def bench_i8_mid(torch, ops, replays=10, warmup=2):
     """W8A8 GEMM between the decode and the prefill shapes (1024 rows on the square and the down-projection
     weights): the 128 x 128 tile kernel; graph-timed, the vendor library's i32-output GEMM beside it."""
     dev = torch.device("cuda:0")
@@ -338,8 +342,7 @@ def bench_i8_mid(torch, ops, steps=20, warmup=4):
             for _ in range(4):
                 ops.i8_gemm(xq, wq, sx, sw, None, out=y)
 
-        total, launches, _ = time_graph(torch, burst, 4, steps, warmup)
-        sec = total / launches
+        sec = time_graph(torch, burst, 4, replays, warmup)["median"]
         row = {"workload": f"int8_gemm_{m}x{k}x{n}", "ms_per_launch": sec * 1e3, "tops": 2.0 * m * k * n / sec / 1e12}
         try:
             wt = wq.t()
@@ -348,8 +351,7 @@ def bench_i8_mid(torch, ops, steps=20, warmup=4):
                 for _ in range(4):
                     torch._int_mm(xq, wt)
 
-            vt, vl, _ = time_graph(torch, vendor, 4, steps, warmup)
-            row["vendor_int_mm_tops"] = 2.0 * m * k * n / (vt / vl) / 1e12
+            row["vendor_int_mm_tops"] = 2.0 * m * k * n / time_graph(torch, vendor, 4, replays, warmup)["median"] / 1e12
         except Exception as e:                      # not every torch build can capture it
             row["vendor_int_mm_tops"] = None
             log(f"vendor int_mm skipped: {e}")
@@ -357,7 +359,7 @@ def bench_i8_mid(torch, ops, steps=20, warmup=4):
     return rows
 
 
-def bench_grad_x(torch, ops, steps=20, warmup=4):
+def bench_grad_x(torch, ops, replays=10, warmup=2):
     """grad_x of the INT4 Linear (QLinearBackward: grad_y . dequant(W)^T), K=4096, N=11008, g128:
     whole call, graph-timed."""
     k, n = 4096, 11008
@@ -375,15 +377,14 @@ def bench_grad_x(torch, ops, steps=20, warmup=4):
             for _ in range(4):
                 ops.qmatmul_int4_t(gy, packed, scales, zp, k, G, out=out)
 
-        total, launches, _ = time_graph(torch, burst, 4, steps, warmup)
-        sec = total / launches
+        sec = time_graph(torch, burst, 4, replays, warmup)["median"]
         rows.append({"workload": f"w4_grad_x_{m}x4096x11008_g128", "ms_per_call": sec * 1e3,
                      "tflops": 2.0 * m * k * n / sec / 1e12,
                      "weight_gbs": (k * n // 2 + 2 * (k // G) * n * 4) / sec / 1e9})
     return rows
 
 
-def bench_q8_matmul(torch, ops, steps=20, warmup=4):
+def bench_q8_matmul(torch, ops, replays=10, warmup=2):
     """The reference's f32 x Q8 matmul (Tensor::matmul with a Q8 right-hand side), K=4096, N=11008,
     at the block sizes that take different kernels: whole call, graph-timed."""
     k, n = 4096, 11008
@@ -401,8 +402,7 @@ def bench_q8_matmul(torch, ops, steps=20, warmup=4):
                 for _ in range(4):
                     ops.matmul_q8(a, words, k, n, bs, out=c)
 
-            total, launches, _ = time_graph(torch, burst, 4, steps, warmup)
-            sec = total / launches
+            sec = time_graph(torch, burst, 4, replays, warmup)["median"]
             rows.append({"workload": f"matmul_q8_{m}x4096x11008_bs{bs}", "ms_per_call": sec * 1e3,
                          "tflops": 2.0 * m * k * n / sec / 1e12,
                          "weight_gbs": (k * n + 4 * n * (k // bs)) / sec / 1e9})
@@ -507,17 +507,28 @@ def cpu_baseline(x, w, budget_s=12.0):
         y = oracle.qmatmul_int4(x, packed, scales, zp, K, G, threads=1)
         times.append(time.perf_counter() - t0)
     med = float(np.median(times))
-    cores = os.cpu_count() or 1
-    cores = min(cores, 16)
-    t0 = time.perf_counter()
-    oracle.qmatmul_int4(x, packed, scales, zp, K, G, threads=cores)
-    t_mt = time.perf_counter() - t0
+    # every core the job may use: the GPU box gives a one-GPU job 16 threads whatever the host shows
+    visible = os.cpu_count() or 1
+    try:
+        allowed = len(os.sched_getaffinity(0))
+    except AttributeError:
+        allowed = visible
+    cores = max(1, min(allowed, int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or 16))
+    mt = []
+    for _ in range(7):
+        t0 = time.perf_counter()
+        oracle.qmatmul_int4(x, packed, scales, zp, K, G, threads=cores)
+        mt.append(time.perf_counter() - t0)
+    t_mt = float(np.median(mt))
     return {
         "value": BYTES_F32_ZP / med / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
         "sample": f"{len(times)} full 1x4096x4096 g128 GEMVs, median, scalar C restatement of "
                   "qmatmul_int4.wgsl (reference has no CPU kernel for this op)",
         "ms_per_gemv": med * 1e3,
-        "all_cores": {"value": BYTES_F32_ZP / t_mt / 1e9, "cores": cores, "ms_per_gemv": t_mt * 1e3},
+        "host_cpus_visible": visible, "host_cpus_allowed": allowed,
+        "all_cores": {"value": BYTES_F32_ZP / t_mt / 1e9, "cores": cores, "ms_per_gemv": t_mt * 1e3,
+                      "samples": len(mt), "ms_min": min(mt) * 1e3, "ms_max": max(mt) * 1e3,
+                      "note": "the same C restatement, OpenMP over output columns, median"},
         "quantize_pack_from_f32_s": t_pack,
     }, y
 
@@ -525,8 +536,9 @@ def cpu_baseline(x, w, budget_s=12.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=6400)
-    ap.add_argument("--warmup", type=int, default=640)
+    ap.add_argument("--steps", type=int, default=100,
+                    help="timed passes over the 64 weight sets (64 GEMV launches each)")
+    ap.add_argument("--warmup", type=int, default=10, help="untimed passes before them")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-gemv", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -544,8 +556,9 @@ def main():
     _lib.call("rumus_hip_init", 0)
     torch.cuda.set_device(0)
 
-    steps = max(WEIGHT_SETS, (args.steps // WEIGHT_SETS) * WEIGHT_SETS)
-    warmup = max(0, args.warmup)
+    if args.steps < 1 or args.warmup < 0:
+        sys.exit("bench.py: --steps must be at least 1 and --warmup at least 0")
+    steps, warmup = args.steps, args.warmup
 
     torch.cuda.synchronize()
     wall0 = time.perf_counter()
@@ -553,32 +566,41 @@ def main():
     wall = time.perf_counter() - wall0
     log(f"[bench] gemv leg wall {wall:.1f}s (includes building {WEIGHT_SETS} weight sets)")
 
-    per_launch = r["sec"] / r["launches"]
+    t = r["t"]
+    per_launch = t["median"]                        # seconds per GEMV launch, median over the timed passes
     gbs = BYTES_F32_ZP / per_launch / 1e9
-    per_launch_res = r["sec_resident"] / r["launches_resident"]
+    per_launch_res, per_launch_ref, per_launch_awq = r["t_resident"]["median"], r["t_ref"]["median"], r["t_awq"]["median"]
 
     out = {
         "metric": "W4 GEMV GB/s (%HBM peak) @1x4096x4096; INT8 GEMM TOPS (%MFMA peak)",
-        "value": gbs, "unit": "GB/s", "n_gpus": 1, "steps": r["launches"], "warmup": warmup,
-        "ms_per_step": per_launch * 1e3, "higher_is_better": True, "scaling": "weak",
+        "value": gbs, "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": per_launch * WEIGHT_SETS * 1e3, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "w4_gemv_1x4096x4096_g128_awq_f32zp", "weight_layout": "tile-major copy (16 columns)", "weight_sets_rotated": WEIGHT_SETS,
-                   "hip_graph": r["graph"], "bytes_per_step": BYTES_F32_ZP},
+        "config": {"workload": "w4_gemv_1x4096x4096_g128_awq_f32zp", "weight_layout": "tile-major copy (16 columns)",
+                   "step": "one pass over 64 distinct weight sets = 64 GEMV launches replayed from one HIP graph",
+                   "launches_per_step": WEIGHT_SETS, "weight_sets_rotated": WEIGHT_SETS,
+                   "hip_graph": t["graph"], "bytes_per_launch": BYTES_F32_ZP, "bytes_per_step": BYTES_F32_ZP * WEIGHT_SETS},
+        "us_per_launch": per_launch * 1e6,
+        "timing": {"statistic": "median over the timed steps, each between its own pair of HIP events on the launch stream",
+                   **spread(t)},
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": gbs / HBM_PEAK_GBS, "traffic": GEMV_TRAFFIC_BYTES},
+                     "frac": gbs / HBM_PEAK_GBS, "traffic": GEMV_TRAFFIC_BYTES,
+                     "achieved_from": "9,469,952 algorithmic bytes / median launch time of this run",
+                     "traffic_from": "profiles/w4_gemv_dot8_1x4096x4096_hbm_traffic.txt (rocprofv3 counters of an "
+                                     "earlier run of this kernel, not measured by this script)"},
         "gbs_at_u4_zero_point_bytes": BYTES_U4_ZP / per_launch / 1e9,
         "reference_layout_entry": {
-            "ms_per_step": r["sec_ref"] / r["launches_ref"] * 1e3,
-            "gbs": BYTES_F32_ZP / (r["sec_ref"] / r["launches_ref"]) / 1e9,
+            "us_per_launch": per_launch_ref * 1e6,
+            "gbs": BYTES_F32_ZP / per_launch_ref / 1e9,
             "note": "rumus_hip_qmatmul_int4 on the reference's row-major arrays; the headline uses the "
                     "tile-major copy QuantizedTensor builds once (same words, same bytes)"},
         "awq_storage_u4_zero_points": {
-            "ms_per_step": r["sec_awq"] / r["launches_awq"] * 1e3, "bytes_per_step": BYTES_U4_ZP,
-            "gbs": BYTES_U4_ZP / (r["sec_awq"] / r["launches_awq"]) / 1e9,
+            "us_per_launch": per_launch_awq * 1e6, "bytes_per_launch": BYTES_U4_ZP,
+            "gbs": BYTES_U4_ZP / per_launch_awq / 1e9,
             "note": "same shape with integer zero-points packed eight per word, tile-major copy "
                     "(rumus_hip_qmatmul_int4_decode_zp4)"},
         "cache_resident": {"gbs": BYTES_F32_ZP / per_launch_res / 1e9,
-                           "ms_per_step": per_launch_res * 1e3,
+                           "us_per_launch": per_launch_res * 1e6,
                            "note": "single weight set, served by Infinity Cache / L2; not HBM"},
     }
 
@@ -599,7 +621,7 @@ def main():
         out["secondary"] = bench_i8_gemm(torch, ops)
         out["w4_gemv_wider"] = bench_gemv_shapes(torch, ops)
         out["w4_gemm"] = [bench_w4_gemm(torch, ops, 16), bench_w4_gemm(torch, ops, 128),
-                          bench_w4_gemm(torch, ops, 1024, steps=10, warmup=2), bench_w4_gemm(torch, ops, 2048, steps=10, warmup=2)]
+                          bench_w4_gemm(torch, ops, 1024), bench_w4_gemm(torch, ops, 2048)]
         out["q8_matmul"] = bench_q8_matmul(torch, ops)
         out["w4_grad_x"] = bench_grad_x(torch, ops)
         out["int8_decode"] = bench_i8_small(torch, ops)

@@ -19,7 +19,13 @@
  *     rumus_hip_last_error() then returns a thread-local message.  The
  *     reference panics on the same preconditions (assert!/expect); a Rust
  *     shim turns a non-zero status into panic! to keep that behaviour;
- *   - functions are re-entrant and thread-safe.
+ *   - functions are re-entrant and thread-safe: any number of host threads may
+ *     call any entry point at once, on the same or on different streams (the
+ *     reference runs ops from several threads, rumus/src/nn/parallel.rs:84).  A
+ *     call that queues several kernels which share the stream's workspace holds
+ *     that stream's workspace lock until its last kernel is queued, so calls of
+ *     two threads on one stream are queued one whole call after the other; calls
+ *     on different streams never wait for each other.
  */
 #ifndef RUMUS_HIP_H
 #define RUMUS_HIP_H
@@ -64,8 +70,8 @@ int rumus_hip_sync(rumus_hip_stream_t stream);
  *       output has fewer than 192 tiles of 64 x 512) + 256;
  *   qmatmul_int4_t, m >= 8: 64 * m * k (partial sums, only below 512 tiles of
  *       64 x 128) + 10 * num_groups * n + 4 * (m + num_groups) + 2048;
- *   i8_gemm: 32 * m * n, and only while the output has fewer than 512 tiles of
- *       64 x 64 (K shared over workgroups): at most 16 MiB;
+ *   i8_gemm: rumus_hip_i8_gemm_workspace_size(m, k, n) exactly; at most
+ *       min(32 * m * n, 16 MiB);
  *   matmul_q8, m >= 5: 4 * m * k * 4 (digit planes of a) + 4 * m * n * 4 + 32 MiB
  *       (partial sums of the int8 GEMM inside); with one block per column from
  *       384 rows on also k * n + 4 * n;
@@ -147,6 +153,13 @@ int rumus_hip_i8_quantize_cols_t(const float* w, int8_t* wq, float* sw,
 int rumus_hip_i8_gemm(const int8_t* xq, const int8_t* wq, const float* sx,
                       const float* sw, const float* bias, int32_t* acc, float* y,
                       uint32_t m, uint32_t k, uint32_t n, rumus_hip_stream_t stream);
+
+/* Workspace bytes rumus_hip_i8_gemm takes on its stream for an m x k x n
+ * product: i32 partial sums where K is shared over workgroups (outputs of few
+ * tiles), 0 otherwise; never more than 16 MiB.  Host arithmetic only, for
+ * rumus_hip_workspace_reserve.  No counterpart in the reference (its BufferPool
+ * sizes temporaries inside the op, rumus/src/backend/gpu/pool.rs:34-75). */
+uint64_t rumus_hip_i8_gemm_workspace_size(uint32_t m, uint32_t k, uint32_t n);
 
 /* ---- INT4 engine --------------------------------------------------------- */
 
@@ -349,6 +362,23 @@ int rumus_hip_add(const float* a, const float* b, float* out, uint64_t numel,
 int rumus_hip_attention(const float* q, const float* k, const float* v, float* out,
                         uint32_t batch, uint32_t heads, uint32_t q_len, uint32_t kv_len,
                         uint32_t head_dim, const uint64_t* strides, int causal,
+                        rumus_hip_stream_t stream);
+
+/* KV-cache append of a decoder block: the keys and values of `rows` new tokens
+ * (prefill: all of them, decode: one) are written at positions pos .. pos+rows-1
+ * of the cache.  Shape contract of the cache: rumus-serve/src/model.rs:11-14,
+ * K and V [batch, heads, cached_len, head_dim]; there the new entries are
+ * concatenated by the tensor library, here they are written in place into a
+ * cache allocated for cache_len positions.
+ * strides: HOST array of 12 element strides (floats, multiples of 4), in the
+ * order of rumus_hip_attention: {knew_batch, knew_head, knew_row, vnew_batch,
+ * vnew_head, vnew_row, kcache_batch, kcache_head, kcache_row, vcache_batch,
+ * vcache_head, vcache_row}; head_dim is contiguous.  The reference's layout is
+ * {H*T*d, T*d, d}; a token-major cache [batch, T, heads, d] is {T*H*d, d, H*d}.
+ * EINVAL unless head_dim % 4 == 0, pos + rows <= cache_len, 16-byte aligned. */
+int rumus_hip_kv_append(const float* k_new, const float* v_new, float* k_cache, float* v_cache,
+                        uint32_t batch, uint32_t heads, uint32_t rows, uint32_t head_dim,
+                        uint32_t pos, uint32_t cache_len, const uint64_t* strides,
                         rumus_hip_stream_t stream);
 
 #ifdef __cplusplus

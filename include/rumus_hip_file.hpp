@@ -357,6 +357,17 @@ inline std::map<std::string, QLinear> load_w4(const std::string& path, hipStream
                                                         nullptr, stream);
             if (pm) {
                 require(k == padded_k, "perm needs k to be a multiple of group_size");
+                // the kernels gather activations through perm without a bounds check of their own: every
+                // input feature 0..k-1 must appear exactly once (checked on the host, before the upload)
+                std::vector<int32_t> host_perm(k);
+                require(fseek(f.get(), (long)(h.data_start + pm->begin), SEEK_SET) == 0, "seek failed");
+                require(fread(host_perm.data(), 4, k, f.get()) == k, "file ended early");
+                std::vector<char> seen(k, 0);
+                for (uint32_t j = 0; j < k; j++) {
+                    const int32_t v = host_perm[j];
+                    require(v >= 0 && (uint32_t)v < k && !seen[v], "perm is not a permutation of 0..k-1");
+                    seen[v] = 1;
+                }
                 layer.weight.perm = DeviceBuffer<int32_t>(k);
                 up.fetch(h.data_start + pm->begin, pm->end - pm->begin, layer.weight.perm.data());
             }

@@ -158,8 +158,10 @@ def save_w4(path: str, layers: Dict[str, QLinear], zero_points: str = "f32") -> 
         tensors[f"{name}.scales"] = _host(w.scales_tensor)
         zp = _host(w.zp_tensor)
         if zero_points == "u4":
-            zi = zp.astype(np.int64)
-            if w.n % 8 != 0 or not (np.array_equal(zi.astype(np.float32), zp) and zi.min() >= 0 and zi.max() <= 15):
+            finite = bool(np.isfinite(zp).all())              # a NaN cast to an integer is undefined
+            zi = np.where(np.isfinite(zp), zp, 0).astype(np.int64)
+            if w.n % 8 != 0 or not (finite and np.array_equal(zi.astype(np.float32), zp) and zi.min() >= 0
+                                    and zi.max() <= 15):
                 raise ValueError(f"{name}: zero-points are not integers in 0..15 over a multiple of 8 columns; "
                                  f"store them as f32")
             z8 = zi.reshape(w.num_groups, w.n // 8, 8).astype(np.uint32)
@@ -176,6 +178,17 @@ def save_w4(path: str, layers: Dict[str, QLinear], zero_points: str = "f32") -> 
         meta[f"{name}.k"] = w.k
         meta[f"{name}.group_size"] = w.group_size
     write_safetensors(path, tensors, meta)
+
+
+def check_perm(perm: np.ndarray, k: int, what: str) -> None:
+    """Raise ValueError unless ``perm`` holds every input feature 0..k-1 exactly once."""
+    perm = np.asarray(perm)
+    if perm.shape != (k,):
+        raise ValueError(f"{what} has shape {perm.shape}, expected ({k},)")
+    if perm.size and (perm.min() < 0 or perm.max() >= k):
+        raise ValueError(f"{what} has entries outside [0, {k})")
+    if not np.array_equal(np.sort(perm), np.arange(k, dtype=perm.dtype)):
+        raise ValueError(f"{what} is not a permutation of 0..{k - 1}")
 
 
 def load_w4(path: str, device="cuda:0") -> Dict[str, QLinear]:
@@ -236,6 +249,9 @@ def load_w4(path: str, device="cuda:0") -> Dict[str, QLinear]:
             if perm is not None:
                 if k != padded_k:
                     raise ValueError(f"{path}: {name}.perm needs k to be a multiple of group_size")
+                # the kernels gather activations through perm without a bounds check of their own:
+                # an entry outside [0, k) in a damaged file would read outside x
+                check_perm(perm.cpu().numpy(), k, f"{path}: {name}.perm")
                 weight = QuantizedTensor(k, n, padded_k, group_size, groups, packed, scales, zp, perm)
             else:
                 weight = QuantizedTensor.from_packed(packed, scales, zp, k, group_size, g_idx=g_idx)

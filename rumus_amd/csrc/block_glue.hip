@@ -466,6 +466,32 @@ __global__ __launch_bounds__(kHeadDim) void attention_merge_kernel(AttnArgs a, c
     a.o[b * a.o_sb + h * a.o_sh + dim] = o / l;
 }
 
+// ---- KV-cache append: the new tokens' keys and values go to positions pos .. pos + rows - 1 -------
+// Every operand carries (batch, head, row) strides like the attention operands, so the projection
+// output [batch * rows, heads * dim] is read in place and the cache may be the reference's
+// [batch, heads, positions, dim] (rumus-serve/src/model.rs:11-14) or token-major.  One launch
+// moves both tensors: blockIdx.z picks K or V; a thread moves 16 bytes.
+struct KvAppendArgs {
+    const float* src[2];
+    float* dst[2];
+    uint64_t sb[2], sh[2], sr[2];     // source strides: batch, head, row
+    uint64_t db[2], dh[2], dr[2];     // cache strides
+    uint32_t heads, rows, dim4, pos;  // dim4 = head_dim / 4
+};
+
+__global__ __launch_bounds__(256) void kv_append_kernel(KvAppendArgs a) {
+    const uint32_t which = blockIdx.z;
+    const uint32_t per_row = a.heads * a.dim4;
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;        // (row, head, chunk) of this batch entry
+    if (i >= a.rows * per_row) return;
+    const uint32_t row = i / per_row, rem = i % per_row, head = rem / a.dim4, c = rem % a.dim4;
+    const uint32_t b = blockIdx.y;
+    const float4 v = *reinterpret_cast<const float4*>(a.src[which] + b * a.sb[which] + head * a.sh[which] +
+                                                      row * a.sr[which] + 4 * c);
+    *reinterpret_cast<float4*>(a.dst[which] + b * a.db[which] + head * a.dh[which] +
+                               (uint64_t)(a.pos + row) * a.dr[which] + 4 * c) = v;
+}
+
 }  // namespace rumus
 
 using namespace rumus;
@@ -549,7 +575,8 @@ int rumus_hip_attention(const float* q, const float* k, const float* v, float* o
     if (q_len == 1) {
         const uint32_t slices = ceil_div(kv_len, kDecodeSlice);
         void* ws = nullptr;
-        if (int rc = workspace_get(s, (size_t)batch * heads * slices * (kHeadDim + 2) * sizeof(float), &ws)) return rc;
+        WorkspaceLease lease;                                // until both kernels are queued
+        if (int rc = workspace_get(s, (size_t)batch * heads * slices * (kHeadDim + 2) * sizeof(float), &ws, lease)) return rc;
         hipLaunchKernelGGL(attention_decode_kernel, dim3(slices, batch * heads), dim3(256), 0, s, a,
                            static_cast<float*>(ws));
         if (int rc = check_launch("attention_decode_kernel")) return rc;
@@ -564,6 +591,31 @@ int rumus_hip_attention(const float* q, const float* k, const float* v, float* o
     }
     hipLaunchKernelGGL(attention_rows_kernel, dim3(ceil_div(q_len, 64), batch * heads), dim3(256), 0, s, a);
     return check_launch("attention_rows_kernel");
+}
+
+int rumus_hip_kv_append(const float* k_new, const float* v_new, float* k_cache, float* v_cache, uint32_t batch,
+                        uint32_t heads, uint32_t rows, uint32_t head_dim, uint32_t pos, uint32_t cache_len,
+                        const uint64_t* strides, rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE(k_new && v_new && k_cache && v_cache && strides, "kv_append: null buffer");
+    RUMUS_REQUIRE(head_dim > 0 && head_dim % 4 == 0, "kv_append: head_dim %u must be a positive multiple of 4", head_dim);
+    RUMUS_REQUIRE((uint64_t)pos + rows <= cache_len, "kv_append: positions %u..%llu do not fit a cache of %u", pos,
+                  (unsigned long long)pos + rows, cache_len);
+    if (batch == 0 || heads == 0 || rows == 0) return RUMUS_HIP_OK;
+    for (int i = 0; i < 12; i++)
+        RUMUS_REQUIRE(strides[i] % 4 == 0, "kv_append: stride %d (%llu) must be a multiple of 4 floats", i,
+                      (unsigned long long)strides[i]);
+    RUMUS_REQUIRE(((reinterpret_cast<uintptr_t>(k_new) | reinterpret_cast<uintptr_t>(v_new) |
+                    reinterpret_cast<uintptr_t>(k_cache) | reinterpret_cast<uintptr_t>(v_cache)) & 15) == 0,
+                  "kv_append: operands must be 16-byte aligned");
+    const uint64_t per_batch = (uint64_t)rows * heads * (head_dim / 4);
+    RUMUS_REQUIRE(batch <= 65535 && per_batch < (1ull << 32), "kv_append: shape beyond the grid limit");
+    KvAppendArgs a{{k_new, v_new}, {k_cache, v_cache},
+                   {strides[0], strides[3]}, {strides[1], strides[4]}, {strides[2], strides[5]},
+                   {strides[6], strides[9]}, {strides[7], strides[10]}, {strides[8], strides[11]},
+                   heads, rows, head_dim / 4, pos};
+    hipLaunchKernelGGL(kv_append_kernel, dim3((uint32_t)((per_batch + 255) / 256), batch, 2), dim3(256), 0,
+                       as_stream(stream), a);
+    return check_launch("kv_append_kernel");
 }
 
 }  // extern "C"

@@ -14,8 +14,26 @@ int set_error(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3
 // Converts a HIP status into a return code (0 when hipSuccess).
 int check_hip(hipError_t e, const char* what);
 
-// Device workspace of at least `bytes` for work queued on `stream` (runtime.hip).
-int workspace_get(hipStream_t stream, size_t bytes, void** out);
+// Exclusive use of one stream's workspace, from workspace_get until the holder goes out of scope.  A call that
+// queues several kernels which talk to each other through the workspace keeps its lease until the last of them
+// is queued: another host thread on the same stream then cannot slip launches of its own between them (they
+// would overwrite the partial results), and cannot grow - that is, free - the buffer under them.  The lock
+// behind it is per (device, stream) and recursive, so calls on different streams never wait for each other and
+// an entry point may call another one while it holds the lease.
+class WorkspaceLease {
+  public:
+    WorkspaceLease() = default;
+    ~WorkspaceLease();
+    WorkspaceLease(const WorkspaceLease&) = delete;
+    WorkspaceLease& operator=(const WorkspaceLease&) = delete;
+  private:
+    friend int workspace_get(hipStream_t, size_t, void**, WorkspaceLease&);
+    void* arena_ = nullptr;
+};
+
+// Device workspace of at least `bytes` for work queued on `stream` (runtime.hip); `lease` then holds the
+// stream's workspace lock.
+int workspace_get(hipStream_t stream, size_t bytes, void** out, WorkspaceLease& lease);
 // A call that holds workspace memory and then calls another entry point that takes workspace of its own on the
 // same stream (the Q8 matmul around the int8 GEMM) asks for both sizes at once and keeps one of these alive over
 // the inner call: workspace_get then hands out the part of the buffer behind `offset`, and fails instead of

@@ -22,9 +22,9 @@ int i8_gemm_launch_wide(int tn, const int8_t* A, const int8_t* B, const float* s
                         const float* bias, int32_t* acc, float* y, uint32_t M, uint32_t K, uint32_t N,
                         hipStream_t s);
 
-// Upper bound of the workspace rumus_hip_i8_gemm takes for an m x n output: up to 8 shares of K with i32 partial
-// sums, only on outputs of fewer than 512 tiles of 64 x 64.
-size_t i8_gemm_workspace_bound(uint32_t m, uint32_t n);
+// Workspace bytes rumus_hip_i8_gemm takes for an m x k x n product (i32 partial sums where K is shared over
+// workgroups); replays the dispatch, no device call.
+size_t i8_gemm_workspace_need(uint32_t m, uint32_t k, uint32_t n);
 
 // Decode kernel for m <= 4 on v_dot4_i32_i8 (i8_gemv.hip).
 int i8_launch_gemv(const int8_t* xq, const int8_t* wq, const float* sx, const float* sw, const float* bias, int32_t* acc,

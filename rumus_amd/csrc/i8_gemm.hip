@@ -343,6 +343,32 @@ static int launch_dma(const int8_t* A, const int8_t* B, const float* sx, const f
     return check_launch("i8_gemm_dma_kernel");
 }
 
+// K shares of launch_small: towards 512 one-wave tiles in flight; more shares cost more in partial sums than
+// they gain (1024: 25.7 us against 20.8).
+static uint32_t small_shares(uint32_t M, uint32_t K, uint32_t N, uint32_t* steps_per) {
+    const uint32_t tm = ceil_div(M, 64), tn = ceil_div(N, 64), ksteps = K / kBK;
+    uint32_t shares = 512 / (tm * tn);
+    if (shares > 8) shares = 8;
+    if (shares > ksteps / 8) shares = ksteps / 8;
+    if (shares < 1) shares = 1;
+    *steps_per = ceil_div(ksteps, shares);
+    return ceil_div(ksteps, *steps_per);
+}
+
+// K shares of launch_mid: towards 256 workgroups, but the partial sums are paid per share: from 64 tiles on only
+// a long K is shared (256 x 4096 x 4096, 64 tiles: 18.5 us whole, 20.1 in four shares; 256 x 11008 x 4096: 53.0
+// and 28.4).
+static uint32_t mid_shares(uint32_t M, uint32_t K, uint32_t N, uint32_t* steps_per) {
+    const uint32_t tm = ceil_div(M, 128), tn = ceil_div(N, 128), ksteps = K / kBK;
+    const uint32_t tiles = tm * tn, min_steps = tiles < 64 ? 16 : 32;
+    uint32_t shares = 256 / tiles;
+    if (shares > 8) shares = 8;
+    if (shares > ksteps / min_steps) shares = ksteps / min_steps;
+    if (shares < 1 || (tiles >= 64 && ksteps < 128)) shares = 1;
+    *steps_per = ceil_div(ksteps, shares);
+    return ceil_div(ksteps, *steps_per);
+}
+
 // Few tiles (K % 64 == 0): one wave per 64 x 64 tile, eight stages of direct-to-LDS loads deep, and K
 // shared over up to 8 workgroups per tile so that the weights stream from all of the chip.  The
 // register-staged kernel with one K step in flight spent a trip to memory per step on these shapes
@@ -351,20 +377,17 @@ static int launch_small(const int8_t* A, const int8_t* B, const float* sx, const
                         int32_t* acc, float* y, uint32_t M, uint32_t K, uint32_t N, hipStream_t s) {
     constexpr int NS = 8;
     constexpr size_t lds_bytes = (size_t)NS * 128 * kBK;       // 64 KB
-    const uint32_t tm = ceil_div(M, 64), tn = ceil_div(N, 64), ksteps = K / kBK;
-    uint32_t shares = 512 / (tm * tn);   // more shares cost more in partial sums than they gain (1024: 25.7 us against 20.8)
-    if (shares > 8) shares = 8;
-    if (shares > ksteps / 8) shares = ksteps / 8;
-    if (shares < 1) shares = 1;
-    const uint32_t steps_per = ceil_div(ksteps, shares);
-    shares = ceil_div(ksteps, steps_per);
+    const uint32_t tm = ceil_div(M, 64), tn = ceil_div(N, 64);
+    uint32_t steps_per = 0;
+    const uint32_t shares = small_shares(M, K, N, &steps_per);
     if (shares == 1) {
         hipLaunchKernelGGL((i8_gemm_dma_kernel<2, 2, 1, 1, NS>), dim3(tm * tn, 1), dim3(64), lds_bytes, s, A, B, sx, sw,
                            bias, acc, y, M, K, N, tm, tn, steps_per);
         return check_launch("i8_gemm_dma_kernel");
     }
     void* ws = nullptr;
-    if (int rc = workspace_get(s, (size_t)shares * M * N * sizeof(int32_t), &ws)) return rc;
+    WorkspaceLease lease;                                    // until both kernels are queued
+    if (int rc = workspace_get(s, (size_t)shares * M * N * sizeof(int32_t), &ws, lease)) return rc;
     int32_t* part = static_cast<int32_t*>(ws);
     hipLaunchKernelGGL((i8_gemm_dma_kernel<2, 2, 1, 1, NS>), dim3(tm * tn, shares), dim3(64), lds_bytes, s, A, B,
                        (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, part, (float*)nullptr, M, K, N,
@@ -381,23 +404,17 @@ static int launch_mid(const int8_t* A, const int8_t* B, const float* sx, const f
                       int32_t* acc, float* y, uint32_t M, uint32_t K, uint32_t N, hipStream_t s) {
     constexpr int NS = 4;
     constexpr size_t lds_bytes = (size_t)NS * 256 * kBK;       // 64 KB
-    const uint32_t tm = ceil_div(M, 128), tn = ceil_div(N, 128), ksteps = K / kBK;
-    // K shares: towards 256 workgroups, but the partial sums are paid per share: from 64 tiles on only a long K is
-    // shared (256 x 4096 x 4096, 64 tiles: 18.5 us whole, 20.1 in four shares; 256 x 11008 x 4096: 53.0 and 28.4)
-    const uint32_t tiles = tm * tn, min_steps = tiles < 64 ? 16 : 32;
-    uint32_t shares = 256 / tiles;
-    if (shares > 8) shares = 8;
-    if (shares > ksteps / min_steps) shares = ksteps / min_steps;
-    if (shares < 1 || (tiles >= 64 && ksteps < 128)) shares = 1;
-    const uint32_t steps_per = ceil_div(ksteps, shares);
-    shares = ceil_div(ksteps, steps_per);
+    const uint32_t tm = ceil_div(M, 128), tn = ceil_div(N, 128);
+    uint32_t steps_per = 0;
+    const uint32_t shares = mid_shares(M, K, N, &steps_per);
     if (shares == 1) {
         hipLaunchKernelGGL((i8_gemm_dma_kernel<2, 2, 2, 2, NS>), dim3(tm * tn, 1), dim3(256), lds_bytes, s, A, B, sx, sw,
                            bias, acc, y, M, K, N, tm, tn, steps_per);
         return check_launch("i8_gemm_dma_kernel");
     }
     void* ws = nullptr;
-    if (int rc = workspace_get(s, (size_t)shares * M * N * sizeof(int32_t), &ws)) return rc;
+    WorkspaceLease lease;                                    // until both kernels are queued
+    if (int rc = workspace_get(s, (size_t)shares * M * N * sizeof(int32_t), &ws, lease)) return rc;
     int32_t* part = static_cast<int32_t*>(ws);
     hipLaunchKernelGGL((i8_gemm_dma_kernel<2, 2, 2, 2, NS>), dim3(tm * tn, shares), dim3(256), lds_bytes, s, A, B,
                        (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, part, (float*)nullptr, M, K, N,
@@ -416,15 +433,6 @@ static int launch(const int8_t* A, const int8_t* B, const float* sx, const float
     hipLaunchKernelGGL((i8_gemm_kernel<TM, TN, OCC>), dim3(tm * tn), dim3(256), 0, s, A, B, sx, sw,
                        bias, acc, y, M, K, N, tm, tn);
     return check_launch("i8_gemm_kernel");
-}
-
-size_t i8_gemm_workspace_bound(uint32_t m, uint32_t n) {
-    // launch_small shares K below 512 tiles of 64 x 64, launch_mid below 128 tiles of 128 x 128 (the same area);
-    // the two parts of a row split are each smaller than the whole
-    // (shares <= 512 / tiles and <= 256 / tiles: at most 16 MiB of partial sums whatever the shape)
-    if ((uint64_t)ceil_div(m, 64) * ceil_div(n, 64) > 1024) return 0;
-    const size_t all = (size_t)8 * m * n * sizeof(int32_t), cap = size_t(32) << 20;
-    return all < cap ? all : cap;
 }
 
 // Launch cost by rounds, in units of one round of 256 x 256 blocks (the wide kernel at width 8; 70 us at K = 4096,
@@ -448,29 +456,19 @@ static I8Plan i8_plan_single(uint32_t m, uint32_t n) {
     return best;
 }
 
-}  // namespace rumus
+// Which kernel takes an m x k x n product.  Pure host arithmetic: rumus_hip_i8_gemm launches what this returns,
+// and rumus_hip_i8_gemm_workspace_size replays it to size the workspace.
+enum class I8Route { Gemv, Stream, SplitRows, Wide, Dma256, Reg4x2, Mid, Small, Reg2x2, Reg1x1 };
+struct I8Choice { I8Route route; uint32_t split_rows; int wide; };
 
-using namespace rumus;
-
-extern "C" int rumus_hip_i8_gemm(const int8_t* xq, const int8_t* wq, const float* sx,
-                                 const float* sw, const float* bias, int32_t* acc, float* y,
-                                 uint32_t m, uint32_t k, uint32_t n, rumus_hip_stream_t stream) {
-    RUMUS_REQUIRE(xq && wq, "i8_gemm: null operand");
-    RUMUS_REQUIRE(acc || y, "i8_gemm: both outputs are null");
-    RUMUS_REQUIRE(!y || (sx && sw), "i8_gemm: y needs sx and sw");
-    RUMUS_REQUIRE(k > 0 && k % 16 == 0, "i8_gemm: k must be a positive multiple of 16 (got %u)", k);
-    RUMUS_REQUIRE(((reinterpret_cast<uintptr_t>(xq) | reinterpret_cast<uintptr_t>(wq)) & 15) == 0,
-                  "i8_gemm: operands must be 16-byte aligned");
-    if (m == 0 || n == 0) return RUMUS_HIP_OK;
-    hipStream_t s = as_stream(stream);
+static I8Choice i8_choose(uint32_t m, uint32_t k, uint32_t n) {
     // decode: up to 4 rows on v_dot4_i32_i8 (4096 x 11008 from a HIP graph over rotating weight copies: 9.3, 10.0,
     // 12.7 us for 1, 2, 4 rows against 18.3 us for 8 rows on the one-wave MFMA tiles)
-    if (m <= 4) return i8_launch_gemv(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
+    if (m <= 4) return {I8Route::Gemv, 0, 0};
     // 5 to 16 rows (to 32 on smaller weights): MFMA tiles fed straight from global memory, a workgroup per 16 columns
     // (from HBM, 8 rows: 4096 x 11008 14.5 us against 18.1 us for the LDS-staged tiles below, 4096 x 4096 7.4 against 12.8;
     // 32 rows: 22.5 against 20.6 and 10.8 against 14.6)
-    if (k % 256 == 0 && (m <= 16 || (m <= 32 && (uint64_t)n * k <= (32ull << 20))))
-        return i8_launch_stream(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
+    if (k % 256 == 0 && (m <= 16 || (m <= 32 && (uint64_t)n * k <= (32ull << 20)))) return {I8Route::Stream, 0, 0};
     // Largest tile that still gives every CU a workgroup.
     const uint64_t big = (uint64_t)ceil_div(m, 256) * ceil_div(n, 128);
     const uint64_t mid = (uint64_t)ceil_div(m, 128) * ceil_div(n, 128);
@@ -493,25 +491,76 @@ extern "C" int rumus_hip_i8_gemm(const int8_t* xq, const int8_t* wq, const float
             const double c = (m1 / rows_per_round) * i8_round_cost(w) + i8_plan_single(m - m1, n).cost;
             if (c < split_cost) { split_cost = c; split_rows = m1; }
         }
-        if (split_rows) {
-            const uint32_t m1 = split_rows;
+        if (split_rows) return {I8Route::SplitRows, split_rows, 0};
+        if (one.wide) return {I8Route::Wide, 0, one.wide};
+        return {I8Route::Dma256, 0, 0};
+    }
+    if (big >= 256) return {I8Route::Reg4x2, 0, 0};
+    // more than 128 rows, fewer than 256 of the big tiles: 128 x 128 tiles, two workgroups per CU
+    // (1024 x 4096 x 4096: 39.6 -> 24.2 us, 1024 x 11008 x 4096: 97.5 -> 59.1 us, 256 x 4096 x 11008: 32.9 -> 22.9 us)
+    if (k % kBK == 0 && m > 128 && (uint64_t)m * n < (1ull << 28)) return {I8Route::Mid, 0, 0};
+    // up to 128 rows: the deep-pipelined one-wave tiles with K shared over workgroups
+    // (4096 x 11008: 28 -> 17-21 us; 11008 x 4096: 66 -> 18-25 us)
+    if (k % kBK == 0 && (uint64_t)m * n < (1ull << 28)) return {I8Route::Small, 0, 0};
+    if (mid >= 256) return {I8Route::Reg2x2, 0, 0};
+    return {I8Route::Reg1x1, 0, 0};
+}
+
+// Workspace bytes rumus_hip_i8_gemm takes for this shape: the i32 partial sums of the K shares of the 64 x 64
+// and 128 x 128 tile kernels (at most 8 and 16 MiB), for the larger of the two parts when the rows are split.
+size_t i8_gemm_workspace_need(uint32_t m, uint32_t k, uint32_t n) {
+    if (m == 0 || n == 0 || k == 0 || k % 16 != 0) return 0;
+    const I8Choice c = i8_choose(m, k, n);
+    uint32_t steps_per = 0, shares = 1;
+    switch (c.route) {
+        case I8Route::SplitRows: {
+            const size_t a = i8_gemm_workspace_need(c.split_rows, k, n), b = i8_gemm_workspace_need(m - c.split_rows, k, n);
+            return a > b ? a : b;
+        }
+        case I8Route::Small: shares = small_shares(m, k, n, &steps_per); break;
+        case I8Route::Mid: shares = mid_shares(m, k, n, &steps_per); break;
+        default: break;
+    }
+    return shares > 1 ? (size_t)shares * m * n * sizeof(int32_t) : 0;
+}
+
+}  // namespace rumus
+
+using namespace rumus;
+
+extern "C" int rumus_hip_i8_gemm(const int8_t* xq, const int8_t* wq, const float* sx,
+                                 const float* sw, const float* bias, int32_t* acc, float* y,
+                                 uint32_t m, uint32_t k, uint32_t n, rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE(xq && wq, "i8_gemm: null operand");
+    RUMUS_REQUIRE(acc || y, "i8_gemm: both outputs are null");
+    RUMUS_REQUIRE(!y || (sx && sw), "i8_gemm: y needs sx and sw");
+    RUMUS_REQUIRE(k > 0 && k % 16 == 0, "i8_gemm: k must be a positive multiple of 16 (got %u)", k);
+    RUMUS_REQUIRE(((reinterpret_cast<uintptr_t>(xq) | reinterpret_cast<uintptr_t>(wq)) & 15) == 0,
+                  "i8_gemm: operands must be 16-byte aligned");
+    if (m == 0 || n == 0) return RUMUS_HIP_OK;
+    hipStream_t s = as_stream(stream);
+    const I8Choice c = i8_choose(m, k, n);
+    switch (c.route) {
+        case I8Route::Gemv: return i8_launch_gemv(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
+        case I8Route::Stream: return i8_launch_stream(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
+        case I8Route::SplitRows: {
+            const uint32_t m1 = c.split_rows;
             if (int rc = rumus_hip_i8_gemm(xq, wq, sx, sw, bias, acc, y, m1, k, n, stream)) return rc;
             return rumus_hip_i8_gemm(xq + (uint64_t)m1 * k, wq, sx ? sx + m1 : nullptr, sw, bias,
                                      acc ? acc + (uint64_t)m1 * n : nullptr, y ? y + (uint64_t)m1 * n : nullptr,
                                      m - m1, k, n, stream);
         }
-        if (one.wide) return i8_gemm_launch_wide(one.wide, xq, wq, sx, sw, bias, acc, y, m, k, n, s);
-        return launch_dma<2, 2, 4, 2, 5>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
+        case I8Route::Wide: return i8_gemm_launch_wide(c.wide, xq, wq, sx, sw, bias, acc, y, m, k, n, s);
+        case I8Route::Dma256: return launch_dma<2, 2, 4, 2, 5>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
+        case I8Route::Reg4x2: return launch<4, 2, 2>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
+        case I8Route::Mid: return launch_mid(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
+        case I8Route::Small: return launch_small(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
+        case I8Route::Reg2x2: return launch<2, 2, 2>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
+        case I8Route::Reg1x1: return launch<1, 1, 2>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
     }
-    if (big >= 256) return launch<4, 2, 2>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
-    // more than 128 rows, fewer than 256 of the big tiles: 128 x 128 tiles, two workgroups per CU
-    // (1024 x 4096 x 4096: 39.6 -> 24.2 us, 1024 x 11008 x 4096: 97.5 -> 59.1 us, 256 x 4096 x 11008: 32.9 -> 22.9 us)
-    if (k % kBK == 0 && m > 128 && (uint64_t)m * n < (1ull << 28))
-        return launch_mid(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
-    // up to 128 rows: the deep-pipelined one-wave tiles with K shared over workgroups
-    // (4096 x 11008: 28 -> 17-21 us; 11008 x 4096: 66 -> 18-25 us)
-    if (k % kBK == 0 && (uint64_t)m * n < (1ull << 28))
-        return launch_small(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
-    if (mid >= 256) return launch<2, 2, 2>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
-    return launch<1, 1, 2>(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
+    return set_error(RUMUS_HIP_EINVAL, "i8_gemm: no kernel for %u x %u x %u", m, k, n);
+}
+
+extern "C" uint64_t rumus_hip_i8_gemm_workspace_size(uint32_t m, uint32_t k, uint32_t n) {
+    return i8_gemm_workspace_need(m, k, n);
 }

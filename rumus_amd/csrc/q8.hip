@@ -494,9 +494,10 @@ static int matmul_q8_mfma(const float* a, const uint32_t* b, float* c, uint32_t 
     // the int8 GEMM below shares K over workgroups on small outputs and keeps the partial sums in the workspace
     // too: room for them behind this call's own buffers
     const size_t own_bytes = align256(planes_bytes + sx_bytes + wq_bytes + sw_bytes + y_bytes);
-    const size_t gemm_bytes = i8_gemm_workspace_bound(kQ8Planes * m, n);
+    const size_t gemm_bytes = i8_gemm_workspace_need(kQ8Planes * m, k, n);
     void* ws = nullptr;
-    if (int rc = workspace_get(s, own_bytes + gemm_bytes, &ws)) return rc;
+    WorkspaceLease lease;                                    // until the last kernel of this call is queued
+    if (int rc = workspace_get(s, own_bytes + gemm_bytes, &ws, lease)) return rc;
     WorkspaceNest nest(own_bytes);
     uint8_t* base = static_cast<uint8_t*>(ws);
     int8_t* planes = reinterpret_cast<int8_t*>(base);
@@ -572,7 +573,8 @@ static int matmul_q8_mfma_blocks(const float* a, const uint32_t* b, float* c, ui
     // few rows: room for the partial results of up to 8 shares of K
     const uint32_t max_shares = (uint64_t)m * n <= (1u << 22) ? 8 : 0;
     void* ws = nullptr;
-    if (int rc = workspace_get(s, planes_bytes + sx_bytes + (size_t)max_shares * m * n * sizeof(float), &ws)) return rc;
+    WorkspaceLease lease;                                    // until the last kernel of this call is queued
+    if (int rc = workspace_get(s, planes_bytes + sx_bytes + (size_t)max_shares * m * n * sizeof(float), &ws, lease)) return rc;
     int8_t* planes = static_cast<int8_t*>(ws);
     float* sxp = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + planes_bytes);
     float* part = max_shares ? reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + planes_bytes + sx_bytes) : nullptr;

@@ -34,6 +34,7 @@ namespace {
 struct Arena {
     void* ptr = nullptr;
     size_t bytes = 0;
+    std::recursive_mutex in_use;     // held by a WorkspaceLease
 };
 struct ArenaKey {
     int device;
@@ -53,11 +54,23 @@ static thread_local size_t g_nest_offset = 0;
 WorkspaceNest::WorkspaceNest(size_t offset) : prev_(g_nest_offset) { g_nest_offset = offset; }
 WorkspaceNest::~WorkspaceNest() { g_nest_offset = prev_; }
 
-int workspace_get(hipStream_t stream, size_t bytes, void** out) {
+WorkspaceLease::~WorkspaceLease() {
+    if (arena_) static_cast<Arena*>(arena_)->in_use.unlock();
+}
+
+int workspace_get(hipStream_t stream, size_t bytes, void** out, WorkspaceLease& lease) {
     int device = 0;
     if (int rc = check_hip(hipGetDevice(&device), "hipGetDevice")) return rc;
-    std::lock_guard<std::mutex> lock(g_arena_mutex);
-    Arena& a = g_arenas[ArenaKey{device, stream}];
+    if (lease.arena_) return set_error(RUMUS_HIP_EINVAL, "workspace lease used twice");
+    Arena* found = nullptr;
+    {
+        // the table lock covers the lookup only; entries of an unordered_map do not move
+        std::lock_guard<std::mutex> lock(g_arena_mutex);
+        found = &g_arenas[ArenaKey{device, stream}];
+    }
+    found->in_use.lock();            // from here on this thread alone queues work that uses the buffer
+    lease.arena_ = found;
+    Arena& a = *found;
     if (const size_t offset = g_nest_offset) {
         if (a.bytes < offset + bytes)
             return set_error(RUMUS_HIP_EINVAL, "nested workspace of %zu bytes behind %zu does not fit the %zu reserved", bytes,
@@ -107,7 +120,8 @@ extern "C" {
 int rumus_hip_workspace_reserve(rumus_hip_stream_t stream, uint64_t bytes) {
     void* p = nullptr;
     if (bytes == 0) return RUMUS_HIP_OK;
-    return rumus::workspace_get(rumus::as_stream(stream), (size_t)bytes, &p);
+    rumus::WorkspaceLease lease;
+    return rumus::workspace_get(rumus::as_stream(stream), (size_t)bytes, &p, lease);
 }
 
 int rumus_hip_shutdown(void) { return rumus::workspace_release_all(); }

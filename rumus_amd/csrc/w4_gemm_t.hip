@@ -374,7 +374,8 @@ int w4_launch_gemm_t(const float* gy, const uint32_t* packed, const float* scale
     const size_t sp_bytes = up(gn * sizeof(float)), zo_bytes = up(gn * sizeof(_Float16) + 64);
     const size_t part_bytes = shares > 1 ? (size_t)shares * m * k * sizeof(float) : 0;
     void* ws = nullptr;
-    if (int rc = workspace_get(s, rowf_bytes + sgrp_bytes + 2 * sp_bytes + zo_bytes + part_bytes, &ws)) return rc;
+    WorkspaceLease lease;                                    // until the last kernel of this call is queued
+    if (int rc = workspace_get(s, rowf_bytes + sgrp_bytes + 2 * sp_bytes + zo_bytes + part_bytes, &ws, lease)) return rc;
     uint8_t* b = static_cast<uint8_t*>(ws);
     float* rowf = reinterpret_cast<float*>(b);
     float* sgrp = reinterpret_cast<float*>(b + rowf_bytes);

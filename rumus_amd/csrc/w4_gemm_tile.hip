@@ -563,9 +563,10 @@ static int launch_tile(const W4Args& a_in, hipStream_t s) {
                                : prepare ? (((size_t)a.m * k4 * sizeof(float) + 255) & ~size_t(255)) : 0;
     const size_t part_bytes = splits > 1 ? (size_t)splits * a.m * a.n * sizeof(float) : 0;
     float* out = a.y;
+    WorkspaceLease lease;                                    // until the last kernel of this call is queued
     if (x_bytes + part_bytes) {
         void* ws = nullptr;
-        if (int rc = workspace_get(s, x_bytes + part_bytes, &ws)) return rc;
+        if (int rc = workspace_get(s, x_bytes + part_bytes, &ws, lease)) return rc;
         if (PRE) {
             uint8_t* base = static_cast<uint8_t*>(ws);
             const bool vec = !a.perm && a.k % 8 == 0 && (reinterpret_cast<uintptr_t>(a.x) & 15) == 0;

@@ -281,8 +281,7 @@ class DecoderBlockW4:
         else:
             if n != 1:
                 raise ValueError("DecoderBlockW4: decode takes one token per sequence")
-            k_cache[:, pos].copy_(k[:, 0])
-            v_cache[:, pos].copy_(v[:, 0])
+            ops.kv_append(k, v, k_cache, v_cache, pos)
             att = ops.attention(q, k_cache[:, :pos + 1], v_cache[:, :pos + 1], causal=False)
             k_out, v_out = k_cache, v_cache
         o = self.proj["o"](att.view(b * n, d))

@@ -103,10 +103,17 @@ def transpose_f32(t: torch.Tensor) -> torch.Tensor:
 
 # ---- INT8, W8A8 ---------------------------------------------------------------
 
-def i8_quantize_rows(x: torch.Tensor):
+def i8_quantize_rows(x: torch.Tensor, out=None):
+    """x f32 [rows, cols] -> (xq int8 [rows, cols], scale f32 [rows]); ``out`` = (xq, scale) to reuse buffers."""
     rows, cols = x.shape
-    xq = torch.empty((rows, cols), dtype=torch.int8, device=x.device)
-    s = torch.empty(rows, dtype=torch.float32, device=x.device)
+    if out is not None:
+        xq, s = out
+        if xq.shape != (rows, cols) or xq.dtype != torch.int8 or s.shape != (rows,) or s.dtype != torch.float32 \
+                or not (xq.is_cuda and s.is_cuda and xq.is_contiguous() and s.is_contiguous()):
+            raise ValueError("i8_quantize_rows: out must be (int8 [rows, cols], float32 [rows]) on the device")
+    else:
+        xq = torch.empty((rows, cols), dtype=torch.int8, device=x.device)
+        s = torch.empty(rows, dtype=torch.float32, device=x.device)
     call("rumus_hip_i8_quantize_rows", _dev(x, torch.float32, "x"), xq.data_ptr(), s.data_ptr(),
          rows, cols, _stream())
     return xq, s
@@ -362,3 +369,22 @@ def attention(q, k, v, causal: bool, out=None):
     call("rumus_hip_attention", q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), b, h, nq, nkv, d,
          strides, 1 if causal else 0, _stream())
     return o
+
+
+def kv_append(k_new, v_new, k_cache, v_cache, pos: int):
+    """Write the new tokens' keys / values ``[B, n, H, d]`` at positions ``pos .. pos+n-1`` of the
+    caches ``[B, T, H, d]`` (any strides with the last dim contiguous; a ``[B, H, T, d]`` cache is
+    passed as its ``transpose(1, 2)`` view), in one launch."""
+    import ctypes
+    b, n, h, d = k_new.shape
+    t_len = k_cache.shape[1]
+    for t, name in ((k_new, "k_new"), (v_new, "v_new"), (k_cache, "k_cache"), (v_cache, "v_cache")):
+        if t.dtype != torch.float32 or not t.is_cuda or t.stride(3) != 1:
+            raise ValueError(f"kv_append: {name} must be a float32 device tensor with a contiguous last dim")
+    if v_new.shape != k_new.shape or k_cache.shape != v_cache.shape or k_cache.shape[0] != b or \
+            k_cache.shape[2] != h or k_cache.shape[3] != d:
+        raise ValueError("kv_append: shapes of the new entries and the caches do not match")
+    strides = (ctypes.c_uint64 * 12)(*[s for t in (k_new, v_new, k_cache, v_cache)
+                                       for s in (t.stride(0), t.stride(2), t.stride(1))])
+    call("rumus_hip_kv_append", k_new.data_ptr(), v_new.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+         b, h, n, d, pos, t_len, strides, _stream())

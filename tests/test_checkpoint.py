@@ -100,3 +100,21 @@ def test_load_needs_a_gpu_device(tmp_path):
     ck.write_safetensors(path, {}, {"format": ck.FORMAT, "version": ck.VERSION})
     with pytest.raises(ValueError, match="cuda"):
         ck.load_w4(path, device="cpu")
+
+
+def test_perm_check_accepts_permutations_only():
+    rng = np.random.default_rng(3)
+    ck.check_perm(rng.permutation(300).astype(np.int32), 300, "perm")
+    ck.check_perm(np.zeros(0, np.int32), 0, "perm")
+    bad = np.arange(300, dtype=np.int32)
+    bad[7] = 300
+    with pytest.raises(ValueError, match="outside"):
+        ck.check_perm(bad, 300, "perm")
+    bad[7] = -1
+    with pytest.raises(ValueError, match="outside"):
+        ck.check_perm(bad, 300, "perm")
+    bad[7] = 8
+    with pytest.raises(ValueError, match="not a permutation"):
+        ck.check_perm(bad, 300, "perm")
+    with pytest.raises(ValueError, match="shape"):
+        ck.check_perm(np.arange(299, dtype=np.int32), 300, "perm")

@@ -118,6 +118,48 @@ def test_attention_rejects_bad_arguments(ops):
         ops.attention(q, q[:, :2], q[:, :2], True)         # more queries than keys
 
 
+@pytest.mark.parametrize("layout", ["token_major", "reference"])
+@pytest.mark.parametrize("b,h,n,pos,cache_len", [(1, 32, 1, 2047, 2048), (3, 2, 1, 0, 5), (2, 3, 20, 7, 40),
+                                                 (8, 4, 64, 0, 64)])
+def test_kv_append_is_an_exact_copy(ops, layout, b, h, n, pos, cache_len):
+    # the reference's cache is [batch, heads, cached_len, head_dim] (rumus-serve/src/model.rs:11-14); the
+    # block here keeps it token-major.  Both are the same call with other strides.  The new entries are
+    # the k and v slices of a fused q|k|v projection output, read in place.
+    say(f"kv_append {layout} b={b} h={h} n={n} pos={pos} T={cache_len}")
+    import torch
+    rng = np.random.default_rng(b * 100 + n + pos)
+    qkv = rng.normal(0, 1, (b, n, 3, h, 128)).astype(np.float32)
+    shape = (b, cache_len, h, 128) if layout == "token_major" else (b, h, cache_len, 128)
+    kc0 = rng.normal(0, 1, shape).astype(np.float32)
+    vc0 = rng.normal(0, 1, shape).astype(np.float32)
+    t, kc, vc = dev(qkv), dev(kc0), dev(vc0)
+    view = (lambda c: c) if layout == "token_major" else (lambda c: c.transpose(1, 2))
+    ops.kv_append(t[:, :, 1], t[:, :, 2], view(kc), view(vc), pos)
+    want_k, want_v = kc0.copy(), vc0.copy()
+    if layout == "token_major":
+        want_k[:, pos:pos + n], want_v[:, pos:pos + n] = qkv[:, :, 1], qkv[:, :, 2]
+    else:
+        want_k[:, :, pos:pos + n] = qkv[:, :, 1].transpose(0, 2, 1, 3)
+        want_v[:, :, pos:pos + n] = qkv[:, :, 2].transpose(0, 2, 1, 3)
+    np.testing.assert_array_equal(host(kc), want_k)          # new rows in place, every other entry untouched
+    np.testing.assert_array_equal(host(vc), want_v)
+    torch.cuda.synchronize()
+
+
+def test_kv_append_rejects_bad_arguments(ops):
+    import torch
+    from rumus_amd._lib import RumusError
+    new = torch.zeros((1, 2, 2, 128), device="cuda")
+    cache = torch.zeros((1, 8, 2, 128), device="cuda")
+    with pytest.raises(RumusError, match="do not fit"):
+        ops.kv_append(new, new, cache, cache, 7)               # positions 7..8 of a cache of 8
+    with pytest.raises(ValueError):
+        ops.kv_append(new, new, cache[:, :, :1], cache[:, :, :1], 0)   # head counts differ
+    odd = torch.zeros((1, 2, 2, 130), device="cuda")
+    with pytest.raises(RumusError, match="multiple of 4"):
+        ops.kv_append(odd, odd, torch.zeros((1, 8, 2, 130), device="cuda"), torch.zeros((1, 8, 2, 130), device="cuda"), 0)
+
+
 def _block(ops, dim, ffn, heads, g):
     import torch
     from rumus_amd import nn
@@ -175,4 +217,35 @@ def test_decoder_block_llama7b_shape(ops):
     err = np.abs(host(yp) - wantp).max()
     say(f"  prefill max abs err {err:.2e} (|y| max {np.abs(wantp).max():.2f})")
     close(host(yp), wantp, atol=1e-3)
+    torch.cuda.synchronize()
+
+
+def test_decoder_block_llama7b_full_prefill(ops):
+    # the benchmark's prefill at its full size: 8 sequences of 512 tokens, 4096 rows through every
+    # projection (other tile and round plans than a few hundred rows take), checked in full against
+    # the float64 block on the dequantized weights; then each sequence's last token is decoded again
+    # against the cache the prefill filled (kv_append at position 511) and must reproduce its row.
+    say("decoder block 4096/11008, prefill 8x512")
+    import torch
+    dim, ffn, heads, g = 4096, 11008, 32, 128
+    blk, wd = _block(ops, dim, ffn, heads, g)
+    xp, _, _ = workloads.decoder_block_inputs(8, 512, dim, seed=9)
+    yp, kp, vp = blk(dev(xp))
+    got, got_k, got_v = host(yp), host(kp), host(vp)
+    want, want_k, want_v = oracle.decoder_block(xp, wd, heads)
+    err = np.abs(got - want).max()
+    say(f"  prefill max abs err {err:.2e} (|y| max {np.abs(want).max():.2f})")
+    close(got, want, atol=1e-3)
+    close(got_k, want_k, atol=1e-3)
+    close(got_v, want_v, atol=1e-3)
+    # linearity in the batch: sequences do not see each other, so a block of two of them gives the same rows
+    y2, _, _ = blk(dev(xp[5:7]))
+    close(host(y2), got[5:7], atol=2e-4)
+    # decode of token 511 against the prefilled cache: same row as the prefill computed
+    kc = torch.zeros((8, 512, heads, 128), device="cuda")
+    vc = torch.zeros_like(kc)
+    ops.kv_append(kp[:, :511], vp[:, :511], kc, vc, 0)
+    yd, kc2, vc2 = blk(dev(xp[:, 511:512]), kc, vc, pos=511)
+    close(host(yd)[:, 0], want[:, 511], atol=1e-3)
+    close(host(kc2), want_k, atol=1e-3)
     torch.cuda.synchronize()

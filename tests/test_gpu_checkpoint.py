@@ -134,6 +134,13 @@ def test_inconsistent_files_are_refused(tmp_path):
         ({"l.qweight": q, "l.zeros": s}, base, "scales is missing"),
         ({"l.qweight": q, "l.scales": s, "l.zeros": s, "l.perm": np.arange(128, dtype=np.int32),
           "l.g_idx": np.zeros(128, np.int32)}, base, "both perm and g_idx"),
+        # gather indices are checked before any kernel reads through them
+        ({"l.qweight": q, "l.scales": s, "l.zeros": s, "l.perm": np.arange(1, 129, dtype=np.int32)}, base,
+         "entries outside"),
+        ({"l.qweight": q, "l.scales": s, "l.zeros": s, "l.perm": -np.arange(128, dtype=np.int32)}, base,
+         "entries outside"),
+        ({"l.qweight": q, "l.scales": s, "l.zeros": s, "l.perm": np.zeros(128, dtype=np.int32)}, base,
+         "not a permutation"),
     ]
     for tensors, meta, msg in cases:
         ck.write_safetensors(path, tensors, meta)

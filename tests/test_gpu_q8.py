@@ -135,6 +135,33 @@ def test_matmul_q8_vs_oracle(ops, m, k, n, bs):
     np.testing.assert_array_equal(deq.reshape(-1), oracle.q8_dequantize(words, k * n, bs))
 
 
+def test_matmul_q8_row_split_inside_on_a_fresh_stream(ops):
+    # 520 rows become 2080 rows of digit planes; the int8 GEMM inside splits them into 2048 rows of wide
+    # blocks and 32 rows that share K over workgroups, whose partial sums must fit behind this call's own
+    # buffers.  A stream that has never run anything has no workspace yet, so the reservation is exact.
+    import torch
+    from rumus_amd import nn
+    m, k, n, bs = 520, 4096, 11008, 4096
+    say(f"matmul_q8 m={m} k={k} n={n} bs={bs} on a fresh stream")
+    rng = np.random.default_rng(520)
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    a = rng.normal(0, 1, (m, k)).astype(np.float32)
+    wq = nn.quantize(dev(w), bs)
+    ad = dev(a)
+    torch.cuda.synchronize()
+    fresh = torch.cuda.Stream()
+    with torch.cuda.stream(fresh):
+        got = nn.matmul(ad, wq)
+    fresh.synchronize()
+    rows = [0, 1, 255, 511, 512, 513, 519]                  # both sides of the split at plane row 2048
+    words = host_u32(wq.buffer)
+    want = oracle.matmul_q8(a[rows], words, k, n, bs, threads=8)
+    assert_close(host(got)[rows], want)
+    # rows are independent: the whole product equals the product computed 104 rows at a time
+    parts = torch.cat([nn.matmul(ad[i:i + 104].contiguous(), wq) for i in range(0, m, 104)])
+    assert_close(host(got), host(parts))
+
+
 @pytest.mark.parametrize("bs,m", [(512, 64), (32, 64), (128, 64), (128, 100), (512, 400)])
 def test_matmul_q8_batch_accuracy_and_non_finite_rows(ops, bs, m):
     # batches: activations go through four 7-bit digit planes and the int8 matrix cores (block scales
