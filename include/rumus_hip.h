@@ -223,6 +223,29 @@ int rumus_hip_qmatmul_int4(const float* x, const uint32_t* packed,
                            uint32_t group_size, uint32_t num_groups,
                            rumus_hip_stream_t stream);
 
+/* rumus_hip_qmatmul_int4_perm for callers that cannot allocate (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No
+ * counterpart in the reference.  Same arguments, same kernels and the same
+ * bits as rumus_hip_qmatmul_int4_perm, but what that call parks in the
+ * stream's workspace between its kernels (activations in matrix-core order,
+ * partial tiles while K is shared over workgroups) lives in a static device
+ * array of rumus_hip_static_scratch_bytes() = 32 MiB that each GPU holds
+ * until the process ends; nothing is allocated or freed, on any call.
+ * EINVAL ("needs ... bytes of scratch memory") when the shape needs more than
+ * the array holds: with k = 4096, n = 11008 that is beyond about 300 rows;
+ * the need is the qmatmul_int4 line of the workspace bounds above.
+ * All calls on one GPU share the one array, whatever their stream: calls that
+ * overlap in time on one GPU race (calls on one stream do not overlap).
+ * Nothing in the array has to start at zero: every byte a kernel reads from
+ * it is written earlier in the same call. */
+int rumus_hip_qmatmul_int4_perm_static(const float* x, const uint32_t* packed_sorted,
+                                       const float* scales, const float* zero_points,
+                                       const float* bias, const int32_t* perm, float* y,
+                                       uint32_t m, uint32_t k, uint32_t n, uint32_t padded_k,
+                                       uint32_t group_size, uint32_t num_groups,
+                                       rumus_hip_stream_t stream);
+uint64_t rumus_hip_static_scratch_bytes(void);
+
 /* custom_forward(&QMatMulINT4TransposeOp, [grad_y, packed, scales, zp])
  * (quant.rs:262-317; kernel shaders/qmatmul_int4_transpose.wgsl:37-74):
  * out[m,k] = a[m,n] . dequant(W)^T. */

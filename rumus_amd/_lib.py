@@ -69,6 +69,8 @@ PROTOTYPES = {
     "rumus_hip_qmatmul_int4_t": (_i32, [_vp] * 5 + [_u32] * 6 + [_vp]),
     "rumus_hip_w4_actorder_prepare": (_i32, [_vp, _vp, _u32, _u32, _u32, _vp, _vp, _vp]),
     "rumus_hip_qmatmul_int4_perm": (_i32, [_vp] * 7 + [_u32] * 6 + [_vp]),
+    "rumus_hip_qmatmul_int4_perm_static": (_i32, [_vp] * 7 + [_u32] * 6 + [_vp]),
+    "rumus_hip_static_scratch_bytes": (_u64, []),
     "rumus_hip_rmsnorm": (_i32, [_vp, _vp, _vp, _u32, _u32, C.c_float, _vp]),
     "rumus_hip_add_rmsnorm": (_i32, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, C.c_float, _vp]),
     "rumus_hip_swiglu": (_i32, [_vp, _vp, _vp, _u64, _vp]),

@@ -47,6 +47,19 @@ struct WorkspaceNest {
     size_t prev_;
 };
 
+// While one of these lives on a thread, workspace_get on that thread hands out `ptr` (a caller-provided buffer
+// of `bytes`) instead of the stream's own buffer, and fails with EINVAL instead of allocating when a request
+// does not fit.  For entry points that must not allocate.
+struct WorkspaceFixed {
+    WorkspaceFixed(void* ptr, size_t bytes);
+    ~WorkspaceFixed();
+    WorkspaceFixed(const WorkspaceFixed&) = delete;
+    WorkspaceFixed& operator=(const WorkspaceFixed&) = delete;
+  private:
+    void* prev_ptr_;
+    size_t prev_bytes_;
+};
+
 // hipGetLastError() after a kernel launch.
 inline int check_launch(const char* kernel) { return check_hip(hipGetLastError(), kernel); }
 

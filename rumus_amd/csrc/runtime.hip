@@ -58,6 +58,17 @@ WorkspaceLease::~WorkspaceLease() {
     if (arena_) static_cast<Arena*>(arena_)->in_use.unlock();
 }
 
+static thread_local void* g_fixed_ptr = nullptr;
+static thread_local size_t g_fixed_bytes = 0;
+WorkspaceFixed::WorkspaceFixed(void* ptr, size_t bytes) : prev_ptr_(g_fixed_ptr), prev_bytes_(g_fixed_bytes) {
+    g_fixed_ptr = ptr;
+    g_fixed_bytes = bytes;
+}
+WorkspaceFixed::~WorkspaceFixed() {
+    g_fixed_ptr = prev_ptr_;
+    g_fixed_bytes = prev_bytes_;
+}
+
 int workspace_get(hipStream_t stream, size_t bytes, void** out, WorkspaceLease& lease) {
     int device = 0;
     if (int rc = check_hip(hipGetDevice(&device), "hipGetDevice")) return rc;
@@ -71,6 +82,14 @@ int workspace_get(hipStream_t stream, size_t bytes, void** out, WorkspaceLease& 
     found->in_use.lock();            // from here on this thread alone queues work that uses the buffer
     lease.arena_ = found;
     Arena& a = *found;
+    if (g_fixed_ptr) {               // a buffer of fixed size stands in for the stream's own: nothing is allocated
+        const size_t offset = g_nest_offset;
+        if (offset + bytes > g_fixed_bytes)
+            return set_error(RUMUS_HIP_EINVAL, "this call needs %zu bytes of scratch memory, the fixed buffer holds %zu",
+                             offset + bytes, g_fixed_bytes);
+        *out = static_cast<uint8_t*>(g_fixed_ptr) + offset;
+        return RUMUS_HIP_OK;
+    }
     if (const size_t offset = g_nest_offset) {
         if (a.bytes < offset + bytes)
             return set_error(RUMUS_HIP_EINVAL, "nested workspace of %zu bytes behind %zu does not fit the %zu reserved", bytes,

@@ -5,6 +5,8 @@
 //
 // Packed layout (rumus-vision/src/quant.rs:98-100): word (k/8)*N + col holds
 // rows 8*(k/8)..+7 of column col; scales / zero_points are f32 [groups, N].
+#include <mutex>
+
 #include "w4.h"
 
 namespace rumus {
@@ -345,6 +347,36 @@ static int dispatch(const W4Args& a, hipStream_t s) {
     return w4_launch_generic(a, s);
 }
 
+// ---- scratch memory of the entry point that allocates nothing -----------------------------------
+// rumus_hip_qmatmul_int4_perm_static keeps what the matrix-core path parks in memory between its
+// kernels (activations in matrix-core order, partial tiles of the K shares) in this array instead of
+// the stream's workspace.  Every GPU the library runs on holds its own copy, at its own address, until
+// the process ends.  In host code the array's name is only a handle for hipGetSymbolAddress: the
+// address the kernels get is the one looked up below, once per device.
+constexpr size_t kStaticScratchBytes = size_t(32) << 20;
+static __device__ __align__(256) uint8_t scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device.
+static int static_scratch(void** out) {
+    int device = 0;
+    if (int rc = check_hip(hipGetDevice(&device), "hipGetDevice")) return rc;
+    RUMUS_REQUIRE(device >= 0 && device < kMaxDevices, "static scratch: device %d beyond the %d supported", device,
+                  kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[device]) {
+        void* ptr = nullptr;
+        if (int rc = check_hip(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return rc;
+        RUMUS_REQUIRE(ptr != nullptr, "static scratch: no device address");
+        g_scratch_ptr[device] = ptr;
+    }
+    *out = g_scratch_ptr[device];
+    return RUMUS_HIP_OK;
+}
+
 }  // namespace rumus
 
 using namespace rumus;
@@ -434,6 +466,24 @@ int rumus_hip_qmatmul_int4_zp4(const float* x, const uint32_t* packed, const flo
     RUMUS_REQUIRE(!perm || k == padded_k, "qmatmul_int4_zp4: perm needs k == padded_k (%u vs %u)", k, padded_k);
     return dispatch(a, as_stream(stream));
 }
+
+int rumus_hip_qmatmul_int4_perm_static(const float* x, const uint32_t* packed_sorted, const float* scales,
+                                       const float* zero_points, const float* bias, const int32_t* perm,
+                                       float* y, uint32_t m, uint32_t k, uint32_t n, uint32_t padded_k,
+                                       uint32_t group_size, uint32_t num_groups, rumus_hip_stream_t stream) {
+    W4Args a{x, packed_sorted, scales, zero_points, bias, nullptr, perm, y, m, k, n, padded_k, group_size, num_groups};
+    if (int rc = validate(a, "qmatmul_int4_perm_static")) return rc;
+    RUMUS_REQUIRE(!perm || k == padded_k, "qmatmul_int4_perm_static: perm needs k == padded_k (%u vs %u)", k,
+                  padded_k);
+    void* ptr = nullptr;
+    if (int rc = static_scratch(&ptr)) return rc;
+    // every workspace request below is served from the array (or refused): same kernels, same order of
+    // the sums, and every byte a kernel reads from the array has been written earlier in this call
+    WorkspaceFixed fixed(ptr, kStaticScratchBytes);
+    return dispatch(a, as_stream(stream));
+}
+
+uint64_t rumus_hip_static_scratch_bytes(void) { return kStaticScratchBytes; }
 
 int rumus_hip_qmatmul_int4_t(const float* a, const uint32_t* packed, const float* scales,
                              const float* zero_points, float* out, uint32_t m, uint32_t k,

@@ -285,6 +285,14 @@ def qmatmul_int4_perm(x, packed_sorted, scales, zp, k, group_size, bias=None, pe
                     group_size, out)
 
 
+def qmatmul_int4_perm_static(x, packed_sorted, scales, zp, k, group_size, bias=None, perm=None, out=None):
+    """``qmatmul_int4_perm`` through the entry point that allocates nothing: temporaries live in the
+    library's static 32 MiB device array; shapes that need more raise ``RumusError``.  Pass ``out``
+    to keep this wrapper from allocating the result either."""
+    return _w4_call("rumus_hip_qmatmul_int4_perm_static", x, packed_sorted, scales, zp, bias, perm, k,
+                    group_size, out)
+
+
 def qmatmul_int4_t(a, packed, scales, zp, k, group_size, out=None):
     m, n = a.shape
     if packed.shape[1] != n:
