@@ -1,0 +1,434 @@
+// INT4 dequant-matmul for small batches (a few to about a hundred rows) on the int8 matrix cores.
+//
+//   y[m,n] = sum_g scale[g,n] * ( sum_{k in g} x[m,k] q[k,n]  -  zp[g,n] * sum_{k in g} x[m,k] )
+//
+// Inside a group only x and the raw nibbles meet, and a nibble is already an int8 operand: a packed
+// word becomes two operand registers with three instructions (w & 0x0f0f0f0f, (w >> 4) & 0x0f0f0f0f),
+// where the f16 path spends nine per word.  The f32 activations cannot enter an integer MFMA, so a
+// small kernel first writes them as fixed point: X = rint(x * 2^e) with |X| <= 2^20 relative to the
+// largest magnitude of the row's eighth of K (the part one wave of the matmul multiplies), split into
+// three signed digits X = d0 + 128 d1 + 16384 d2, one int8 plane each, stored in the order the MFMA's A
+// operand wants, plus the sum of X over every chunk of 64 or 128 k; a gather through `perm` (act-order)
+// happens there too.  Every product and every sum over a chunk is then an exact integer
+// (v_mfma_i32_16x16x64_i8, three per weight fragment); the three i32 tiles are put together with two
+// shift-adds and leave the integer domain once per chunk: one conversion and one multiply-add with the
+// group's scale.  The zero-point term is a small matrix product of its own, chunk sums of X times
+// -scale * zero-point, on v_mfma_f32_16x16x4_f32 once per round of chunks.
+//
+// A workgroup owns 16*Q columns over all of K for one block of 16*RT rows; its eight waves take an
+// eighth of K each and meet in LDS at the end, so nothing crosses workgroups: no partial sums in
+// memory, no atomics, the same bits on every run.  Lane (c = lane % 16, b = lane / 16) reads Q
+// adjacent columns of packed word rows 8*step + 2b and + 2b+1 with one load each (the 16 lanes of a
+// k block read 64*Q contiguous bytes); word j of those loads is the B operand of MFMA j, whose 16
+// columns are therefore n0 + Q*c + j: the output tile comes out with the Q columns of a lane side
+// by side.  Weights go global -> registers -> MFMA, a wave's whole share in flight when it is four
+// chunks or fewer; the activation planes come out of the L2 (every workgroup reads all of them, 3 bytes
+// per element).
+#include "w4.h"
+
+namespace rumus {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef uint32_t u3a4 __attribute__((ext_vector_type(3), aligned(4)));
+
+constexpr int kI8WK = 8;                   // waves of a workgroup = shares of K
+constexpr uint32_t kI8MaxRows = 128;       // beyond, the f16 tile kernel's larger tiles win
+
+struct W4I8Args {
+    const uint32_t* packed;
+    const float* scales;
+    const float* zp;
+    const uint32_t* zp4;
+    const float* bias;
+    const uint8_t* planes;    // [row tile][step][digit][64 lanes x 16 bytes]
+    const float* rscale;      // [row tile][share][16 rows]: 2^-e (NaN: that part of the row holds a NaN or an infinity)
+    const int32_t* csum;      // [row tile][chunk][16 rows]: sum of the chunk's X
+    float* y;
+    uint32_t m, n, steps, chunks, steps_per_group, per;   // per: chunks per share
+};
+
+#ifdef W4I8_TIMERS
+// instrumented build only (-DW4I8_TIMERS): wall-clock stamps (10 ns ticks) of every wave at fixed points
+constexpr uint32_t kStampWorkgroups = 512;                       // the first so many workgroups of a launch are recorded
+__device__ unsigned long long g_w4i8_stamps[kStampWorkgroups * 8 * 8];
+extern "C" int rumus_dbg_w4i8_stamps(unsigned long long* host, size_t count) {
+    if (count > kStampWorkgroups * 8 * 8) return 1;
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_w4i8_stamps), count * 8);
+}
+#define STAMP(i) do { const uint32_t wg_ = blockIdx.y * gridDim.x + blockIdx.x;                           \
+        if (lane == 0 && wg_ < kStampWorkgroups) g_w4i8_stamps[(wg_ * 8 + wk) * 8 + (i)] = wall_clock64(); } while (0)
+#else
+#define STAMP(i)
+#endif
+
+// low bytes of a, b, c, d -> one word
+__device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
+    const uint32_t lo = __builtin_amdgcn_perm((uint32_t)b, (uint32_t)a, 0x0c0c0400u);
+    const uint32_t hi = __builtin_amdgcn_perm((uint32_t)d, (uint32_t)c, 0x0c0c0400u);
+    return __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+}
+
+// ---- activations -> digit planes ------------------------------------------------------------------
+// One wave per (row, share of K); a lane takes 8 consecutive k at a time: half of a lane's operand bytes of
+// one step (its even elements fill one word - a packed word's even nibbles -, its odd elements the next).
+// f = 2^e; 1.5 * 2^23 + x * f has rint(x * f) in its low mantissa bits (round to nearest even by the addition
+// itself).  Rows past m are written as zeros: the matmul reads whole row tiles.  The first four groups of a
+// lane (shares up to 2048 k) stay in registers between the pass that finds the maximum and the pass that
+// writes the digits.
+template <int CS, bool VEC>
+__global__ __launch_bounds__(64) void w4_i8_prepare_kernel(const float* __restrict__ x, const int32_t* __restrict__ perm,
+                                                           uint8_t* __restrict__ planes, float* __restrict__ rscale,
+                                                           int32_t* __restrict__ csum, uint32_t m, uint32_t k,
+                                                           uint32_t steps, uint32_t chunks, uint32_t per) {
+    constexpr int CACHE = 4;
+    constexpr uint32_t SUBS = 8 * CS;                               // lanes per chunk
+    const uint32_t lane = threadIdx.x, share = blockIdx.x, row = blockIdx.y, rt = row >> 4, row_l = row & 15;
+    const uint32_t k_begin = min(share * per, chunks) * CS * 64, k_end = min((share + 1) * per, chunks) * CS * 64;
+    const bool live = row < m;
+    const float* xr = x + (uint64_t)(live ? row : 0) * k;
+
+    auto load8 = [&](uint32_t k0, float (&v)[8]) {
+#pragma unroll
+        for (int j4 = 0; j4 < 2; j4++) {
+            const uint32_t kk = k0 + 4 * j4;
+            if (VEC) {                                             // k % 4 == 0: a float4 is all in or all out
+                float4 f = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                if (live && k0 < k_end && kk < k) f = *reinterpret_cast<const float4*>(xr + kk);
+                v[4 * j4] = f.x; v[4 * j4 + 1] = f.y; v[4 * j4 + 2] = f.z; v[4 * j4 + 3] = f.w;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const bool in = live && k0 < k_end && kk + j < k;
+                    const uint32_t src = in ? (perm ? (uint32_t)perm[kk + j] : kk + j) : 0;
+                    const float f = xr[src];
+                    v[4 * j4 + j] = in ? f : 0.0f;
+                }
+            }
+        }
+    };
+    auto max_bits = [](const float (&v)[8]) {
+        uint32_t mb = 0;
+#pragma unroll
+        for (int j = 0; j < 8; j++) mb = max(mb, __float_as_uint(v[j]) & 0x7fffffffu);
+        return mb;
+    };
+
+    // pass 1: the largest magnitude, on the bit patterns: a NaN or an infinity sorts highest
+    float cache[CACHE][8];
+    uint32_t mb = 0;
+#pragma unroll
+    for (int i = 0; i < CACHE; i++) {
+        load8(k_begin + (lane + 64 * i) * 8, cache[i]);
+        mb = max(mb, max_bits(cache[i]));
+    }
+    for (uint32_t k0 = k_begin + (lane + 64 * CACHE) * 8; k0 < k_end; k0 += 512) {
+        float v[8];
+        load8(k0, v);
+        mb = max(mb, max_bits(v));
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mb = max(mb, (uint32_t)__shfl_xor((int)mb, o));
+    // 2^e with max * 2^e in [2^19, 2^20); tiny values stop at 2^100 (their products vanish in f32 anyway).  A
+    // non-finite activation poisons its row: the scale becomes NaN (the digits are then whatever the
+    // conversion gives; they only ever meet the NaN)
+    const bool finite = mb < 0x7f800000u;
+    int e = 19 - ((int)(mb >> 23) - 127);
+    e = mb == 0 ? 0 : min(e, 100);
+    const float f = finite ? __uint_as_float((uint32_t)(e + 127) << 23) : 0.0f;
+    if (lane == 0)
+        rscale[((uint64_t)rt * kI8WK + share) * 16 + row_l] =
+            finite ? __uint_as_float((uint32_t)(127 - e) << 23) : __uint_as_float(0x7fc00000u);
+
+    // pass 2: digits and chunk sums
+    auto emit = [&](uint32_t k0, const float (&v)[8]) {
+        int d[3][8], sum = 0;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int X = (int)__float_as_uint(fmaf(v[j], f, 12582912.0f)) - 0x4b400000;   // |X| <= 2^20
+            const int X1 = (X + 64) >> 7;
+            d[0][j] = __builtin_amdgcn_sbfe(X, 0, 7);              // X - 128 * X1
+            d[1][j] = __builtin_amdgcn_sbfe(X1, 0, 7);             // X1 - 128 * d2
+            d[2][j] = (X1 + 64) >> 7;                              // |d2| <= 64
+            sum += X;
+        }
+#pragma unroll
+        for (uint32_t o = 1; o < SUBS; o <<= 1) sum += __shfl_xor(sum, (int)o);   // whole chunks are in or out together
+        const uint32_t piece = k0 >> 4, step = piece >> 2, b = piece & 3, half = (k0 >> 3) & 1;
+#pragma unroll
+        for (int p = 0; p < 3; p++)
+            *reinterpret_cast<uint2*>(planes + (((uint64_t)rt * steps + step) * 3 + p) * 1024 + (b * 16 + row_l) * 16 + half * 8) =
+                make_uint2(pack4(d[p][0], d[p][2], d[p][4], d[p][6]), pack4(d[p][1], d[p][3], d[p][5], d[p][7]));
+        if ((k0 >> 3) % SUBS == 0) csum[((uint64_t)rt * chunks + (k0 >> 3) / SUBS) * 16 + row_l] = sum;
+    };
+#pragma unroll
+    for (int i = 0; i < CACHE; i++) {
+        const uint32_t k0 = k_begin + (lane + 64 * i) * 8;
+        if (k0 < k_end) emit(k0, cache[i]);
+    }
+    for (uint32_t k0 = k_begin + (lane + 64 * CACHE) * 8; k0 < k_end; k0 += 512) {
+        float v[8];
+        load8(k0, v);
+        emit(k0, v);
+    }
+}
+
+// ---- the matmul -------------------------------------------------------------------------------------
+template <int Q>
+__device__ __forceinline__ void load_q(const uint32_t* p, uint32_t (&o)[Q]) {
+    if constexpr (Q == 4) {
+        const uint4 v = *reinterpret_cast<const uint4*>(p);
+        o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+    } else if constexpr (Q == 3) {
+        const u3a4 v = *reinterpret_cast<const u3a4*>(p);
+        o[0] = v.x; o[1] = v.y; o[2] = v.z;
+    } else if constexpr (Q == 2) {
+        const uint2 v = *reinterpret_cast<const uint2*>(p);
+        o[0] = v.x; o[1] = v.y;
+    } else {
+        o[0] = *p;
+    }
+}
+
+// Q: columns per lane (16*Q per workgroup).  RT: row tiles of 16 per workgroup.  CS: steps of 64 k per
+// chunk (1 or 2).  U: chunks per round = chunks of weight loads in flight per lane.
+template <int Q, int RT, int CS, int U, bool ZP4>
+__global__ __launch_bounds__(512) void w4_gemm_i8_kernel(W4I8Args a) {
+    constexpr int WK = kI8WK;
+    static_assert((U * RT) % 2 == 0, "the two activation slots alternate with a fixed phase per unrolled position");
+    static_assert(U <= 4, "a round's chunks are the four k slots of the zero-point MFMA");
+    __shared__ float red[WK][RT * Q * 4][64];
+    const uint32_t lane = threadIdx.x & 63, wk = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t c = lane & 15, b = lane >> 4;
+    const uint32_t n0 = xcd_contiguous(blockIdx.x, gridDim.x) * (16 * Q), rb = blockIdx.y;
+    // past the edge: the last Q columns again (computed twice, stored twice with the same values)
+    const uint32_t colc = min(n0 + Q * c, a.n - Q);
+    const uint32_t f0 = min(wk * a.per, a.chunks), f1 = min(f0 + a.per, a.chunks);
+    const uint32_t flast = f1 > f0 ? f1 - 1 : f0 ? f0 - 1 : 0;
+    const uint32_t lane_w = 2 * b * a.n + colc;                    // lane part of a packed-word address
+
+    STAMP(0);
+    uint32_t braw[U][CS][2][Q], msc[U][Q], mzp[U][Q];
+    auto fetch_b = [&](int slot, uint32_t chunk) {
+        const uint32_t fc = min(chunk, flast);                       // past the wave's share: fetched again, adds 0
+#pragma unroll
+        for (int s = 0; s < CS; s++)
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+                load_q<Q>(a.packed + (uint64_t)((fc * CS + s) * 8 + h) * a.n + lane_w, braw[slot][s][h]);
+        const uint32_t g = fc * CS / a.steps_per_group;
+        load_q<Q>(reinterpret_cast<const uint32_t*>(a.scales) + (uint64_t)g * a.n + colc, msc[slot]);
+        if (ZP4) mzp[slot][0] = a.zp4[(uint64_t)g * (a.n / 8) + colc / 8];
+        else load_q<Q>(reinterpret_cast<const uint32_t*>(a.zp) + (uint64_t)g * a.n + colc, mzp[slot]);
+    };
+    v4i afr[2][CS][3];
+    auto fetch_a = [&](int slot, uint32_t chunk, uint32_t rt) {
+        const uint32_t fc = min(chunk, flast), rtg = rb * RT + rt;
+#pragma unroll
+        for (int s = 0; s < CS; s++)
+#pragma unroll
+            for (int p = 0; p < 3; p++)
+                afr[slot][s][p] = *reinterpret_cast<const v4i*>(
+                    a.planes + (((uint64_t)rtg * a.steps + fc * CS + s) * 3 + p) * 1024 + lane * 16);
+    };
+
+    v4f accf[RT][Q];
+#pragma unroll
+    for (int t = 0; t < RT; t++)
+#pragma unroll
+        for (int q = 0; q < Q; q++) accf[t][q] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // Loads retire in order, so what is issued last is waited for last: activation fragments (needed
+    // first, they come out of the L2) always go ahead of the weight loads that are needed later.
+    fetch_a(0, f0, 0);
+#pragma unroll
+    for (int u = 0; u < U; u++) fetch_b(u, f0 + u);
+    STAMP(1);
+
+    // Whole rounds of U chunks, straight-line code: a chunk past the wave's share is computed on the last
+    // chunk's data again (addresses are clamped) with its scale and zero-point set to 0, so it adds 0.
+    for (uint32_t base = f0; base < f1; base += U) {
+        // chunk sums of the round for the zero-point product: lane (row c, k slot b) holds chunk base + b
+        float sm[RT];
+#pragma unroll
+        for (int t = 0; t < RT; t++)
+            sm[t] = (float)a.csum[((uint64_t)(rb * RT + t) * a.chunks + min(base + b, flast)) * 16 + c];
+        float szq[Q];
+#pragma unroll
+        for (int q = 0; q < Q; q++) szq[q] = 0.0f;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint32_t chunk = base + u;
+            const bool alive = chunk < f1;                             // wave-uniform
+            v4i bf[CS][Q];
+#pragma unroll
+            for (int s = 0; s < CS; s++)
+#pragma unroll
+                for (int q = 0; q < Q; q++) {
+                    const uint32_t w0 = braw[u][s][0][q], w1 = braw[u][s][1][q];
+                    bf[s][q] = v4i{(int)(w0 & 0x0f0f0f0fu), (int)((w0 >> 4) & 0x0f0f0f0fu),
+                                   (int)(w1 & 0x0f0f0f0fu), (int)((w1 >> 4) & 0x0f0f0f0fu)};
+                }
+            float sc[Q];
+#pragma unroll
+            for (int q = 0; q < Q; q++) {
+                sc[q] = alive ? __uint_as_float(msc[u][q]) : 0.0f;
+                const float zq = ZP4 ? (float)((mzp[u][0] >> (4 * ((colc & 7u) + q))) & 15u) : __uint_as_float(mzp[u][q]);
+                // this chunk is k slot u of the round's zero-point product: -(scale * zp), 0 for a dead chunk
+                szq[q] = (alive && b == (uint32_t)u) ? -(sc[q] * zq) : szq[q];
+            }
+#pragma unroll
+            for (int t = 0; t < RT; t++) {
+                const int cur = (u * RT + t) & 1;
+                if (t + 1 < RT) {
+                    fetch_a(cur ^ 1, chunk, t + 1);
+                } else {
+                    fetch_a(cur ^ 1, chunk + 1, 0);
+                    fetch_b(u, chunk + U);                             // this slot's words are in bf by now
+                }
+                // the prefetches stay here: the scheduler would sink them to their first use to save registers
+                __builtin_amdgcn_sched_barrier(0);
+                v4i acc[Q][3];
+#pragma unroll
+                for (int q = 0; q < Q; q++)
+#pragma unroll
+                    for (int p = 0; p < 3; p++) acc[q][p] = v4i{0, 0, 0, 0};
+#pragma unroll
+                for (int s = 0; s < CS; s++)
+#pragma unroll
+                    for (int q = 0; q < Q; q++)
+#pragma unroll
+                        for (int p = 0; p < 3; p++)
+                            acc[q][p] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afr[cur][s][p], bf[s][q], acc[q][p], 0, 0, 0);
+#pragma unroll
+                for (int q = 0; q < Q; q++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        // exact: |d2 part| <= 128*64*15 * 2^14 < 2^31 - the rest
+                        int low = (acc[q][1][i] << 7) + acc[q][0][i];
+                        asm("" : "+v"(low));              // two shift-adds, not two shifts and a three-way add
+                        const int tot = (acc[q][2][i] << 14) + low;
+                        accf[t][q][i] = fmaf(sc[q], (float)tot, accf[t][q][i]);
+                    }
+            }
+#ifdef W4I8_TIMERS
+            if (base == f0 && u == 0) { __builtin_amdgcn_sched_barrier(0); if (accf[0][0][0] != 1e30f) STAMP(2); }
+#endif
+        }
+        // - scale * zp * (sum of X over the chunk), the round's chunks at once: [16 rows x 4 chunks] x [4 chunks x 16 columns]
+#pragma unroll
+        for (int t = 0; t < RT; t++)
+#pragma unroll
+            for (int q = 0; q < Q; q++) accf[t][q] = __builtin_amdgcn_mfma_f32_16x16x4f32(sm[t], szq[q], accf[t][q], 0, 0, 0);
+    }
+    STAMP(3);
+
+    // back to the activations' scale (this wave's share of K has its own), then the eight shares meet in LDS;
+    // wave w adds them up, in a fixed order, for rows 4b + w % 4 of row tile w / 4 and stores
+#pragma unroll
+    for (int t = 0; t < RT; t++) {
+        const float4 rs = *reinterpret_cast<const float4*>(a.rscale + ((uint64_t)(rb * RT + t) * WK + wk) * 16 + 4 * b);
+        const float r4[4] = {rs.x, rs.y, rs.z, rs.w};
+#pragma unroll
+        for (int q = 0; q < Q; q++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) red[wk][(t * Q + q) * 4 + i][lane] = f1 > f0 ? accf[t][q][i] * r4[i] : 0.0f;
+    }
+    __syncthreads();
+    STAMP(4);
+    if (wk >= RT * 4) return;
+    const uint32_t t = wk >> 2, i = wk & 3;
+    const uint32_t row = (rb * RT + t) * 16 + 4 * b + i;
+    if (row >= a.m) return;
+    float* dst = a.y + (uint64_t)row * a.n + colc;
+    float o[Q];
+#pragma unroll
+    for (int q = 0; q < Q; q++) {
+        float v = red[0][(t * Q + q) * 4 + i][lane];
+#pragma unroll
+        for (int w = 1; w < WK; w++) v += red[w][(t * Q + q) * 4 + i][lane];
+        if (a.bias) v += a.bias[colc + q];
+        o[q] = v;
+    }
+    if constexpr (Q == 4) *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+    else if constexpr (Q == 2) *reinterpret_cast<float2*>(dst) = make_float2(o[0], o[1]);
+    else {
+#pragma unroll
+        for (int q = 0; q < Q; q++) dst[q] = o[q];
+    }
+}
+
+bool w4_gemm_i8_supported(const W4Args& a) {
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(a.packed) | reinterpret_cast<uintptr_t>(a.scales) |
+                           reinterpret_cast<uintptr_t>(a.zp) | reinterpret_cast<uintptr_t>(a.y) |
+                           (a.bias ? reinterpret_cast<uintptr_t>(a.bias) : 0);
+    return a.m > 0 && a.m <= kI8MaxRows && a.group_size % 64 == 0 && a.n % 4 == 0 && a.n >= 4 && (bits & 15) == 0 &&
+           !a.g_idx && !a.tiled && !a.glu && (!a.zp4 || a.n % 8 == 0);
+}
+
+template <int Q, int RT, int CS, int U>
+static int launch_i8(const W4I8Args& k, bool zp4, uint32_t row_blocks, hipStream_t s) {
+    const dim3 grid(ceil_div(k.n, 16 * Q), row_blocks);
+    if (zp4) hipLaunchKernelGGL((w4_gemm_i8_kernel<Q, RT, CS, U, true>), grid, dim3(512), 0, s, k);
+    else hipLaunchKernelGGL((w4_gemm_i8_kernel<Q, RT, CS, U, false>), grid, dim3(512), 0, s, k);
+    return check_launch("w4_gemm_i8_kernel");
+}
+
+// Columns per lane.  Workgroups run one per compute unit, in rounds of 256, and a workgroup's time grows
+// with its columns on top of a fixed part (its share of the activation planes): the cheapest
+// rounds * (Q + 1.5) wins.  u4 zero-points come eight to a word: Q = 3 would straddle words.
+static int pick_q(uint32_t n, uint32_t row_blocks, bool zp4) {
+    int best = 4;
+    double best_cost = 1e30;
+    for (int q = 4; q >= 1; q--) {
+        if (q == 3 && zp4) continue;
+        const uint64_t wgs = (uint64_t)ceil_div(n, 16 * q) * row_blocks;
+        const double cost = (double)((wgs + 255) / 256) * (q + 1.5);
+        if (cost < best_cost) { best_cost = cost; best = q; }
+    }
+    return best;
+}
+
+template <int RT, int CS, int U>
+static int launch_i8_q(const W4I8Args& k, bool zp4, uint32_t row_blocks, hipStream_t s) {
+    switch (pick_q(k.n, row_blocks, zp4)) {
+        case 4: return launch_i8<4, RT, CS, U>(k, zp4, row_blocks, s);
+        case 3: return launch_i8<3, RT, CS, U>(k, zp4, row_blocks, s);
+        case 2: return launch_i8<2, RT, CS, U>(k, zp4, row_blocks, s);
+        default: return launch_i8<1, RT, CS, U>(k, zp4, row_blocks, s);
+    }
+}
+
+int w4_launch_gemm_i8(const W4Args& a, hipStream_t s) {
+    const uint32_t cs = a.group_size % 128 == 0 ? 2 : 1;             // chunk = 128 or 64 k: never across a group end
+    const uint32_t steps = a.padded_k / 64, chunks = steps / cs, per = ceil_div(chunks, (uint32_t)kI8WK);
+    const uint32_t rt_per = a.m <= 16 ? 1 : 2, row_blocks = ceil_div(a.m, 16 * rt_per), rts = row_blocks * rt_per;
+    RUMUS_REQUIRE(row_blocks <= 65535, "qmatmul_int4: m %u is beyond the grid limit", a.m);
+    auto up = [](size_t v) { return (v + 255) & ~size_t(255); };
+    const size_t planes_bytes = (size_t)rts * steps * 3 * 1024;
+    const size_t csum_bytes = up((size_t)rts * chunks * 16 * sizeof(int32_t)), rscale_bytes = (size_t)rts * kI8WK * 16 * sizeof(float);
+    void* ws = nullptr;
+    WorkspaceLease lease;                                            // until both kernels are queued
+    if (int rc = workspace_get(s, planes_bytes + csum_bytes + rscale_bytes, &ws, lease)) return rc;
+    uint8_t* planes = static_cast<uint8_t*>(ws);
+    int32_t* csum = reinterpret_cast<int32_t*>(planes + planes_bytes);
+    float* rscale = reinterpret_cast<float*>(planes + planes_bytes + csum_bytes);
+    const bool vec = !a.perm && a.k % 4 == 0 && (reinterpret_cast<uintptr_t>(a.x) & 15) == 0;
+    const dim3 pgrid(kI8WK, rts * 16);
+    if (cs == 2) {
+        if (vec) hipLaunchKernelGGL((w4_i8_prepare_kernel<2, true>), pgrid, dim3(64), 0, s, a.x, a.perm, planes, rscale, csum, a.m, a.k, steps, chunks, per);
+        else hipLaunchKernelGGL((w4_i8_prepare_kernel<2, false>), pgrid, dim3(64), 0, s, a.x, a.perm, planes, rscale, csum, a.m, a.k, steps, chunks, per);
+    } else {
+        if (vec) hipLaunchKernelGGL((w4_i8_prepare_kernel<1, true>), pgrid, dim3(64), 0, s, a.x, a.perm, planes, rscale, csum, a.m, a.k, steps, chunks, per);
+        else hipLaunchKernelGGL((w4_i8_prepare_kernel<1, false>), pgrid, dim3(64), 0, s, a.x, a.perm, planes, rscale, csum, a.m, a.k, steps, chunks, per);
+    }
+    if (int rc = check_launch("w4_i8_prepare_kernel")) return rc;
+    const W4I8Args k{a.packed, a.scales, a.zp, a.zp4, a.bias, planes, rscale, csum, a.y,
+                     a.m, a.n, steps, chunks, a.group_size / 64, per};
+    const bool zp4 = a.zp4 != nullptr;
+    // a wave's whole share in flight when it is up to four chunks (two for two row tiles: registers)
+    if (rt_per == 1) return cs == 2 ? launch_i8_q<1, 2, 4>(k, zp4, row_blocks, s) : launch_i8_q<1, 1, 4>(k, zp4, row_blocks, s);
+    return cs == 2 ? launch_i8_q<2, 2, 2>(k, zp4, row_blocks, s) : launch_i8_q<2, 1, 2>(k, zp4, row_blocks, s);
+}
+
+}  // namespace rumus

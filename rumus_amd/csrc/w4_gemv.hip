@@ -326,6 +326,7 @@ static int dispatch(const W4Args& a, hipStream_t s) {
     const bool few_rows = a.m <= w4_decode_max_rows(a.padded_k, a.n) || !w4_gemm_supported(a);
     if (few_rows && w4_gemv_dot8_supported(a)) return w4_launch_gemv_dot8(a, s);
     if (few_rows && w4_gemv_supported(a)) return w4_launch_gemv(a, s);
+    if (w4_gemm_i8_supported(a)) return w4_launch_gemm_i8(a, s);
     if (w4_gemm_supported(a)) return w4_launch_gemm(a, s);
     // Batches the matrix-core kernel does not take (group sizes that are no multiple of 32): the
     // decode kernel, a few rows at a time, is far ahead of the reference-order kernel
