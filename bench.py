@@ -406,6 +406,20 @@ def bench_q8_matmul(torch, ops, replays=10, warmup=2):
             rows.append({"workload": f"matmul_q8_{m}x4096x11008_bs{bs}", "ms_per_call": sec * 1e3,
                          "tflops": 2.0 * m * k * n / sec / 1e12,
                          "weight_gbs": (k * n + 4 * n * (k // bs)) / sec / 1e9})
+        if bs >= k:                                        # per output channel: also against a dense copy made once
+            wq, sw = ops.q8_dense_layout(words, k, n, bs)
+            for m in (512, 2048):
+                a = torch.randn((m, k), generator=gen, device=dev)
+                c = torch.empty((m, n), dtype=torch.float32, device=dev)
+
+                def burst():
+                    for _ in range(4):
+                        ops.matmul_q8_dense(a, wq, sw, out=c)
+
+                sec = time_graph(torch, burst, 4, replays, warmup)["median"]
+                rows.append({"workload": f"matmul_q8_dense_{m}x4096x11008", "ms_per_call": sec * 1e3,
+                             "tflops": 2.0 * m * k * n / sec / 1e12, "weight_gbs": (k * n + 4 * n) / sec / 1e9})
+            del wq, sw
         del words
     return rows
 

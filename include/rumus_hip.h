@@ -120,6 +120,22 @@ int rumus_hip_matmul_q8(const float* a, const uint32_t* b, float* c, uint32_t m,
                         uint32_t k, uint32_t n, uint32_t block_size,
                         rumus_hip_stream_t stream);
 
+/* The per-output-channel case of matmul_q8_dispatch (compute.rs:2021-2060 with
+ * block_size >= k, one block per column) for a weight that is multiplied more
+ * than once: rumus_hip_q8_dense_layout copies the Q8 buffer once into a dense
+ * int8 matrix wq [n, k] (row j = the k quantized values of column j) and its n
+ * block scales sw (the f16 header of block j, widened), and
+ * rumus_hip_matmul_q8_dense multiplies against that copy without touching the
+ * Q8 buffer: c[m,n] = a[m,k] x (wq, sw), bit for bit what rumus_hip_matmul_q8
+ * returns on its matrix-core route for the same tensor (m >= 384 there; here
+ * any m).  k % 16 == 0; a, wq, c 16-byte aligned; n <= 65535 for the layout
+ * call.  Workspace of the stream: 4 bytes per element of a (+ 16 per row), and
+ * below about a thousand rows also 16 bytes per element of c. */
+int rumus_hip_q8_dense_layout(const uint32_t* b_q8, uint32_t k, uint32_t n, uint32_t block_size,
+                              int8_t* wq, float* sw, rumus_hip_stream_t stream);
+int rumus_hip_matmul_q8_dense(const float* a, const int8_t* wq, const float* sw, float* c,
+                              uint32_t m, uint32_t k, uint32_t n, rumus_hip_stream_t stream);
+
 /* Tensor::add_bias (rumus/src/tensor/ops.rs:885-931, shaders/bias.wgsl:18-25):
  * out[i,j] = mat[i,j] + bias[j].  out may alias mat. */
 int rumus_hip_add_bias(const float* mat, const float* bias, float* out,

@@ -271,6 +271,31 @@ inline DeviceBuffer<float> matmul(const DeviceBuffer<float>& a, uint32_t m, cons
     return c;
 }
 
+// A per-output-channel Q8 weight (block_size >= k) in the layout the matrix cores read: made once with
+// prepare_dense, multiplied many times.  Same results as matmul() on the Q8 tensor from 384 rows on.
+struct Q8Dense {
+    DeviceBuffer<int8_t> wq;     // [n, k]
+    DeviceBuffer<float> sw;      // [n]
+    uint32_t k = 0, n = 0;
+};
+
+inline Q8Dense prepare_dense(const Q8Tensor& q, hipStream_t stream = nullptr) {
+    Q8Dense d;
+    d.k = q.k; d.n = q.n;
+    d.wq = DeviceBuffer<int8_t>((size_t)q.n * q.k);
+    d.sw = DeviceBuffer<float>(q.n);
+    check(rumus_hip_q8_dense_layout(q.buffer.data(), q.k, q.n, q.block_size, d.wq.data(), d.sw.data(), stream));
+    return d;
+}
+
+inline DeviceBuffer<float> matmul(const DeviceBuffer<float>& a, uint32_t m, const Q8Dense& b,
+                                  hipStream_t stream = nullptr) {
+    require(a.size() == (size_t)m * b.k, "matmul: inner dimension mismatch");
+    DeviceBuffer<float> c((size_t)m * b.n);
+    check(rumus_hip_matmul_q8_dense(a.data(), b.wq.data(), b.sw.data(), c.data(), m, b.k, b.n, stream));
+    return c;
+}
+
 // ---- INT8, W8A8 --------------------------------------------------------------------
 
 // Per-output-channel int8 weights, dynamic per-row int8 activations, i32 accumulate.

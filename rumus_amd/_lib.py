@@ -48,6 +48,8 @@ PROTOTYPES = {
     "rumus_hip_q8_dequantize": (_i32, [_vp, _vp, _u32, _u32, _vp]),
     "rumus_hip_q8_dequantize_kn": (_i32, [_vp, _vp, _u32, _u32, _u32, _vp]),
     "rumus_hip_matmul_q8": (_i32, [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
+    "rumus_hip_q8_dense_layout": (_i32, [_vp, _u32, _u32, _u32, _vp, _vp, _vp]),
+    "rumus_hip_matmul_q8_dense": (_i32, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _vp]),
     "rumus_hip_add_bias": (_i32, [_vp, _vp, _vp, _u32, _u32, _vp]),
     "rumus_hip_transpose_f32": (_i32, [_vp, _vp, _u32, _u32, _vp]),
     "rumus_hip_i8_quantize_rows": (_i32, [_vp, _vp, _vp, _u32, _u32, _vp]),

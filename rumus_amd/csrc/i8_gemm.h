@@ -17,10 +17,17 @@ typedef void __attribute__((address_space(3)))* lptr_t;
 // s_waitcnt with only vmcnt set (gfx9 encoding: vmcnt[3:0] | expcnt 7 | lgkmcnt 15 | vmcnt[5:4] << 14)
 #define RUMUS_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | 0x70 | 0xF00)
 
-// Wide-block kernel (i8_gemm_wide.hip): 256 x 32*tn blocks, tn = 8..12.
+// Wide-block kernel (i8_gemm_wide.hip): 256 x 32*tn blocks, tn = 8..12.  fold4: see i8_epilogue.
 int i8_gemm_launch_wide(int tn, const int8_t* A, const int8_t* B, const float* sx, const float* sw,
                         const float* bias, int32_t* acc, float* y, uint32_t M, uint32_t K, uint32_t N,
-                        hipStream_t s);
+                        hipStream_t s, bool fold4 = false);
+
+// The W8A8 GEMM on four interleaved digit planes per activation row with the planes added in the epilogue
+// (i8_epilogue, FOLD4): m4 = 4 * rows, y [m4 / 4, n].  Only the kernels of large shapes have that epilogue:
+// i8_gemm_fold4 returns EINVAL where i8_gemm_fold4_supported says no.
+bool i8_gemm_fold4_supported(uint32_t m4, uint32_t k, uint32_t n);
+int i8_gemm_fold4(const int8_t* planes, const int8_t* wq, const float* sx4, const float* sw, const float* bias,
+                  float* y, uint32_t m4, uint32_t k, uint32_t n, hipStream_t s);
 
 // Workspace bytes rumus_hip_i8_gemm takes for an m x k x n product (i32 partial sums where K is shared over
 // workgroups); replays the dispatch, no device call.
@@ -45,7 +52,10 @@ __device__ __forceinline__ uint32_t row_swizzle(uint32_t row) {
 // branch-free path: the row scales of the lane are fetched up front as float4
 // (four consecutive rows per register quad) and y is written with
 // non-temporal stores (it is not read again by this kernel).
-template <int TM, int TN, int BM, int BN>
+// FOLD4: the rows are the four digit planes of M / 4 activation rows, interleaved (row 4 r + p is plane p
+// of activation row r, sx[4 r + p] its weight): the four registers of a quad are the four planes of one output,
+// y[r, col] = sum over p, in order, of (f32(acc) * sx[4 r + p]) * sw[col] (+ bias), and y has M / 4 rows.
+template <int TM, int TN, int BM, int BN, bool FOLD4 = false>
 __device__ __forceinline__ void i8_epilogue(const v16i (&acc)[TM][TN], const float* __restrict__ sx,
                                             const float* __restrict__ sw,
                                             const float* __restrict__ bias,
@@ -53,6 +63,31 @@ __device__ __forceinline__ void i8_epilogue(const v16i (&acc)[TM][TN], const flo
                                             uint32_t M, uint32_t N, uint32_t m0, uint32_t n0,
                                             uint32_t wm, uint32_t wn, uint32_t lane) {
     const uint32_t col_l = lane & 31, row_l = (lane >> 5) * 4;
+    if constexpr (FOLD4) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const uint32_t col = n0 + (wn * TN + j) * 32 + col_l;
+            if (col >= N) continue;
+            const float swc = sw[col];
+            const float bc = bias ? bias[col] : 0.0f;
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const uint32_t row = m0 + (wm * TM + i) * 32 + 8 * g + row_l;    // a multiple of 4, as is M
+                    if (row >= M) continue;
+                    const float4 s4 = *reinterpret_cast<const float4*>(sx + row);
+                    float v = __fmul_rn(__fmul_rn((float)acc[i][j][4 * g], s4.x), swc);
+                    v = __fadd_rn(v, __fmul_rn(__fmul_rn((float)acc[i][j][4 * g + 1], s4.y), swc));
+                    v = __fadd_rn(v, __fmul_rn(__fmul_rn((float)acc[i][j][4 * g + 2], s4.z), swc));
+                    v = __fadd_rn(v, __fmul_rn(__fmul_rn((float)acc[i][j][4 * g + 3], s4.w), swc));
+                    if (bias) v = __fadd_rn(v, bc);
+                    __builtin_nontemporal_store(v, y + (uint64_t)(row / 4) * N + col);
+                }
+            }
+        }
+        return;
+    }
     // whole 32-column MFMA tiles are in or out when N % 32 == 0, so the fast path
     // only needs all rows of the block inside M
     const bool interior = m0 + BM <= M && N % 32 == 0 && ((reinterpret_cast<uintptr_t>(sx) & 15) == 0);

@@ -146,7 +146,7 @@ __global__ __launch_bounds__(256, OCC) void i8_gemm_kernel(
 // ~350 cycles that do not hide under the MFMAs (~910 cycles per step in all).
 // ---------------------------------------------------------------------------
 // WM x WN waves, each owning a (32*TM) x (32*TN) part of the block tile.
-template <int TM, int TN, int WM, int WN, int NS>
+template <int TM, int TN, int WM, int WN, int NS, bool FOLD4 = false>
 __global__ __launch_bounds__(64 * WM * WN) void i8_gemm_dma_kernel(
     const int8_t* __restrict__ A, const int8_t* __restrict__ B, const float* __restrict__ sx,
     const float* __restrict__ sw, const float* __restrict__ bias, int32_t* __restrict__ acc_out,
@@ -303,7 +303,7 @@ __global__ __launch_bounds__(64 * WM * WN) void i8_gemm_dma_kernel(
     RUMUS_WAIT_VMCNT(0);         // no LDS-DMA write may outlive the workgroup
 
     if (gridDim.y > 1) acc_out += (uint64_t)blockIdx.y * M * N;
-    i8_epilogue<TM, TN, BM, BN>(acc, sx, sw, bias, acc_out, y, M, N, m0, n0, wm, wn, lane);
+    i8_epilogue<TM, TN, BM, BN, FOLD4>(acc, sx, sw, bias, acc_out, y, M, N, m0, n0, wm, wn, lane);
 }
 
 // Sum of the K shares' i32 accumulators (exact, any order), then the rescale and bias of the epilogue.
@@ -323,7 +323,7 @@ __global__ __launch_bounds__(256) void i8_splitk_finish_kernel(const int32_t* __
     }
 }
 
-template <int TM, int TN, int WM, int WN, int NS>
+template <int TM, int TN, int WM, int WN, int NS, bool FOLD4 = false>
 static int launch_dma(const int8_t* A, const int8_t* B, const float* sx, const float* sw,
                       const float* bias, int32_t* acc, float* y, uint32_t M, uint32_t K, uint32_t N,
                       hipStream_t s) {
@@ -332,13 +332,13 @@ static int launch_dma(const int8_t* A, const int8_t* B, const float* sx, const f
     static bool attr_set = false;   // benign race: setting the attribute is idempotent
     if (!attr_set && lds_bytes > 64 * 1024) {
         if (int rc = check_hip(hipFuncSetAttribute(
-                reinterpret_cast<const void*>(&i8_gemm_dma_kernel<TM, TN, WM, WN, NS>),
+                reinterpret_cast<const void*>(&i8_gemm_dma_kernel<TM, TN, WM, WN, NS, FOLD4>),
                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes), "hipFuncSetAttribute"))
             return rc;
         attr_set = true;
     }
     uint32_t tm = ceil_div(M, BM), tn = ceil_div(N, BN);
-    hipLaunchKernelGGL((i8_gemm_dma_kernel<TM, TN, WM, WN, NS>), dim3(tm * tn), dim3(64 * WM * WN),
+    hipLaunchKernelGGL((i8_gemm_dma_kernel<TM, TN, WM, WN, NS, FOLD4>), dim3(tm * tn), dim3(64 * WM * WN),
                        lds_bytes, s, A, B, sx, sw, bias, acc, y, M, K, N, tm, tn, K / kBK);
     return check_launch("i8_gemm_dma_kernel");
 }
@@ -522,6 +522,36 @@ size_t i8_gemm_workspace_need(uint32_t m, uint32_t k, uint32_t n) {
         default: break;
     }
     return shares > 1 ? (size_t)shares * m * n * sizeof(int32_t) : 0;
+}
+
+// Routes whose kernels have the plane-adding epilogue: the two kernels of large shapes, and row splits into them.
+bool i8_gemm_fold4_supported(uint32_t m4, uint32_t k, uint32_t n) {
+    if (m4 == 0 || m4 % 4 != 0 || n == 0 || k == 0 || k % 16 != 0) return false;
+    const I8Choice c = i8_choose(m4, k, n);
+    switch (c.route) {
+        case I8Route::Wide:
+        case I8Route::Dma256: return true;
+        case I8Route::SplitRows:
+            return c.split_rows % 4 == 0 && i8_gemm_fold4_supported(c.split_rows, k, n) &&
+                   i8_gemm_fold4_supported(m4 - c.split_rows, k, n);
+        default: return false;
+    }
+}
+
+int i8_gemm_fold4(const int8_t* planes, const int8_t* wq, const float* sx4, const float* sw, const float* bias,
+                  float* y, uint32_t m4, uint32_t k, uint32_t n, hipStream_t s) {
+    RUMUS_REQUIRE(i8_gemm_fold4_supported(m4, k, n), "i8 gemm: no plane-adding kernel for %u x %u x %u", m4, k, n);
+    RUMUS_REQUIRE((reinterpret_cast<uintptr_t>(sx4) & 15) == 0, "i8 gemm: plane weights must be 16-byte aligned");
+    const I8Choice c = i8_choose(m4, k, n);
+    switch (c.route) {
+        case I8Route::SplitRows: {
+            const uint32_t m1 = c.split_rows;
+            if (int rc = i8_gemm_fold4(planes, wq, sx4, sw, bias, y, m1, k, n, s)) return rc;
+            return i8_gemm_fold4(planes + (uint64_t)m1 * k, wq, sx4 + m1, sw, bias, y + (uint64_t)(m1 / 4) * n, m4 - m1, k, n, s);
+        }
+        case I8Route::Wide: return i8_gemm_launch_wide(c.wide, planes, wq, sx4, sw, bias, nullptr, y, m4, k, n, s, true);
+        default: return launch_dma<2, 2, 4, 2, 5, true>(planes, wq, sx4, sw, bias, nullptr, y, m4, k, n, s);
+    }
 }
 
 }  // namespace rumus

@@ -46,7 +46,7 @@ struct WideLoads {
 // The K loop and the epilogue of one wave: rows [64*wm, 64*wm+64), column tiles
 // [ct0, ct0+TN) of the block.  Both kinds of waves of a workgroup (TN differs)
 // run the same number of barriers and issue the same number of loads per step.
-template <int TN, int W, int LOADS>
+template <int TN, int W, int LOADS, bool FOLD4>
 __device__ __forceinline__ void wide_wave(const WideLoads<LOADS>& ld, int8_t* lds, const float* __restrict__ sx,
                                           const float* __restrict__ sw, const float* __restrict__ bias,
                                           int32_t* __restrict__ acc_out, float* __restrict__ y, uint32_t M,
@@ -154,10 +154,10 @@ __device__ __forceinline__ void wide_wave(const WideLoads<LOADS>& ld, int8_t* ld
     step(ld.ksteps - 1, cur, std::true_type{});
     RUMUS_WAIT_VMCNT(0);         // no LDS-DMA write may outlive the workgroup
 
-    i8_epilogue<TM, TN, kWideBM, 32 * W>(acc, sx, sw, bias, acc_out, y, M, N, m0, n0 + ct0 * 32, wm, 0, lane);
+    i8_epilogue<TM, TN, kWideBM, 32 * W, FOLD4>(acc, sx, sw, bias, acc_out, y, M, N, m0, n0 + ct0 * 32, wm, 0, lane);
 }
 
-template <int W>
+template <int W, bool FOLD4>
 __global__ __launch_bounds__(64 * kWideWaves, 1) void i8_gemm_wide_kernel(
     const int8_t* __restrict__ A, const int8_t* __restrict__ B, const float* __restrict__ sx,
     const float* __restrict__ sw, const float* __restrict__ bias, int32_t* __restrict__ acc_out,
@@ -196,40 +196,48 @@ __global__ __launch_bounds__(64 * kWideWaves, 1) void i8_gemm_wide_kernel(
     ld.ksteps = K / kBK;
 
     const uint32_t wm = wave % kWideWM;
-    if (wave < kWideWM) wide_wave<TN0, W, LOADS>(ld, lds, sx, sw, bias, acc_out, y, M, N, m0, n0, wm, 0, lane);
-    else wide_wave<TN1, W, LOADS>(ld, lds, sx, sw, bias, acc_out, y, M, N, m0, n0, wm, TN0, lane);
+    if (wave < kWideWM) wide_wave<TN0, W, LOADS, FOLD4>(ld, lds, sx, sw, bias, acc_out, y, M, N, m0, n0, wm, 0, lane);
+    else wide_wave<TN1, W, LOADS, FOLD4>(ld, lds, sx, sw, bias, acc_out, y, M, N, m0, n0, wm, TN0, lane);
 }
 
-template <int W>
+template <int W, bool FOLD4>
 static int launch_wide(const int8_t* A, const int8_t* B, const float* sx, const float* sw, const float* bias,
                        int32_t* acc, float* y, uint32_t M, uint32_t K, uint32_t N, hipStream_t s) {
     constexpr size_t lds_bytes = (size_t)kWideStages * (kWideBM + 32 * W) * kBK;
     static_assert(lds_bytes <= 160 * 1024, "stages do not fit the 160 KB LDS");
     static bool attr_set = false;   // benign race: setting the attribute is idempotent
     if (!attr_set) {
-        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&i8_gemm_wide_kernel<W>),
+        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&i8_gemm_wide_kernel<W, FOLD4>),
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes),
                                "hipFuncSetAttribute"))
             return rc;
         attr_set = true;
     }
     const uint32_t tm = ceil_div(M, kWideBM), tn = ceil_div(N, 32 * W);
-    hipLaunchKernelGGL(i8_gemm_wide_kernel<W>, dim3(tm * tn), dim3(64 * kWideWaves), lds_bytes, s, A, B, sx, sw,
+    hipLaunchKernelGGL((i8_gemm_wide_kernel<W, FOLD4>), dim3(tm * tn), dim3(64 * kWideWaves), lds_bytes, s, A, B, sx, sw,
                        bias, acc, y, M, K, N, tm, tn);
     return check_launch("i8_gemm_wide_kernel");
 }
 
-int i8_gemm_launch_wide(int w, const int8_t* A, const int8_t* B, const float* sx, const float* sw,
-                        const float* bias, int32_t* acc, float* y, uint32_t M, uint32_t K, uint32_t N,
-                        hipStream_t s) {
+template <bool FOLD4>
+static int launch_wide_w(int w, const int8_t* A, const int8_t* B, const float* sx, const float* sw,
+                         const float* bias, int32_t* acc, float* y, uint32_t M, uint32_t K, uint32_t N,
+                         hipStream_t s) {
     switch (w) {
-        case 8: return launch_wide<8>(A, B, sx, sw, bias, acc, y, M, K, N, s);
-        case 9: return launch_wide<9>(A, B, sx, sw, bias, acc, y, M, K, N, s);
-        case 10: return launch_wide<10>(A, B, sx, sw, bias, acc, y, M, K, N, s);
-        case 11: return launch_wide<11>(A, B, sx, sw, bias, acc, y, M, K, N, s);
-        case 12: return launch_wide<12>(A, B, sx, sw, bias, acc, y, M, K, N, s);
+        case 8: return launch_wide<8, FOLD4>(A, B, sx, sw, bias, acc, y, M, K, N, s);
+        case 9: return launch_wide<9, FOLD4>(A, B, sx, sw, bias, acc, y, M, K, N, s);
+        case 10: return launch_wide<10, FOLD4>(A, B, sx, sw, bias, acc, y, M, K, N, s);
+        case 11: return launch_wide<11, FOLD4>(A, B, sx, sw, bias, acc, y, M, K, N, s);
+        case 12: return launch_wide<12, FOLD4>(A, B, sx, sw, bias, acc, y, M, K, N, s);
     }
     return set_error(RUMUS_HIP_EINVAL, "i8 gemm: no wide kernel for width %d", w);
+}
+
+int i8_gemm_launch_wide(int w, const int8_t* A, const int8_t* B, const float* sx, const float* sw,
+                        const float* bias, int32_t* acc, float* y, uint32_t M, uint32_t K, uint32_t N,
+                        hipStream_t s, bool fold4) {
+    return fold4 ? launch_wide_w<true>(w, A, B, sx, sw, bias, acc, y, M, K, N, s)
+                 : launch_wide_w<false>(w, A, B, sx, sw, bias, acc, y, M, K, N, s);
 }
 
 }  // namespace rumus

@@ -415,6 +415,9 @@ __device__ __forceinline__ uint32_t q8_row_amax(const float* __restrict__ ar, ui
     return max(max(red[0], red[1]), max(red[2], red[3]));
 }
 
+// INTERLEAVED: plane p of row r is row 4 r + p of `planes` and sxp[4 r + p] its weight (the order the plane-adding
+// epilogue of the int8 GEMM wants); otherwise the planes are stacked, row p m + r and sxp[p m + r].
+template <bool INTERLEAVED>
 __global__ __launch_bounds__(256) void q8_split_rows_kernel(const float* __restrict__ a, int8_t* __restrict__ planes,
                                                             float* __restrict__ sxp, uint32_t m, uint32_t k) {
     __shared__ uint32_t red[4];
@@ -430,7 +433,7 @@ __global__ __launch_bounds__(256) void q8_split_rows_kernel(const float* __restr
     if (tid < kQ8Planes) {
         float s = inv_bits ? __uint_as_float((inv_bits + 7u * tid) << 23) : 0.0f;
         if (ebits == 255) s = __uint_as_float(0x7FC00000u);    // inf / nan in the row: poison it
-        sxp[tid * m + row] = s;
+        sxp[INTERLEAVED ? kQ8Planes * row + tid : tid * m + row] = s;
     }
     const bool poisoned = ebits == 255;
     auto emit = [&](uint32_t j, const float4& v) {
@@ -448,7 +451,8 @@ __global__ __launch_bounds__(256) void q8_split_rows_kernel(const float* __restr
         }
 #pragma unroll
         for (int p = 0; p < kQ8Planes; p++)
-            *reinterpret_cast<uint32_t*>(planes + ((uint64_t)p * m + row) * k + j) = word[p];
+            *reinterpret_cast<uint32_t*>(planes + (INTERLEAVED ? (uint64_t)kQ8Planes * row + p : (uint64_t)p * m + row) * k + j) =
+                word[p];
     };
     if (cached) {
 #pragma unroll
@@ -485,35 +489,56 @@ __global__ __launch_bounds__(256) void q8_add_planes_kernel(const float* __restr
 
 static size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
 
-static int matmul_q8_mfma(const float* a, const uint32_t* b, float* c, uint32_t m, uint32_t k, uint32_t n,
-                          uint32_t stride, hipStream_t s) {
-    RUMUS_REQUIRE((uint64_t)kQ8Planes * m < (1ull << 31), "matmul_q8: m %u is beyond the grid limit", m);
-    const size_t planes_bytes = align256((size_t)kQ8Planes * m * k), sx_bytes = align256((size_t)kQ8Planes * m * sizeof(float));
-    const size_t wq_bytes = align256((size_t)n * k), sw_bytes = align256((size_t)n * sizeof(float));
-    const size_t y_bytes = (size_t)kQ8Planes * m * n * sizeof(float);
-    // the int8 GEMM below shares K over workgroups on small outputs and keeps the partial sums in the workspace
-    // too: room for them behind this call's own buffers
-    const size_t own_bytes = align256(planes_bytes + sx_bytes + wq_bytes + sw_bytes + y_bytes);
-    const size_t gemm_bytes = i8_gemm_workspace_need(kQ8Planes * m, k, n);
-    void* ws = nullptr;
-    WorkspaceLease lease;                                    // until the last kernel of this call is queued
-    if (int rc = workspace_get(s, own_bytes + gemm_bytes, &ws, lease)) return rc;
-    WorkspaceNest nest(own_bytes);
-    uint8_t* base = static_cast<uint8_t*>(ws);
+// c = a x (wq, sw): wq dense int8 [n, k], sw [n].  The planes are added in the GEMM's epilogue where the shape
+// has such a kernel (large ones), by a pass over the four partial outputs otherwise; both give the same bits.
+// `ws` holds q8_dense_workspace(m, k, n) bytes, the int8 GEMM's own partial sums behind `own` of them.
+struct Q8DenseWs { size_t planes, sx, y, own, total; bool fold; };
+
+static Q8DenseWs q8_dense_workspace(uint32_t m, uint32_t k, uint32_t n) {
+    Q8DenseWs w;
+    w.fold = i8_gemm_fold4_supported(kQ8Planes * m, k, n);
+    w.planes = align256((size_t)kQ8Planes * m * k);
+    w.sx = align256((size_t)kQ8Planes * m * sizeof(float));
+    w.y = w.fold ? 0 : align256((size_t)kQ8Planes * m * n * sizeof(float));
+    w.own = w.planes + w.sx + w.y;
+    w.total = w.own + (w.fold ? 0 : i8_gemm_workspace_need(kQ8Planes * m, k, n));
+    return w;
+}
+
+static int matmul_q8_planes(const float* a, const int8_t* wq, const float* sw, float* c, uint32_t m, uint32_t k,
+                            uint32_t n, const Q8DenseWs& w, uint8_t* base, hipStream_t s) {
     int8_t* planes = reinterpret_cast<int8_t*>(base);
-    float* sxp = reinterpret_cast<float*>(base + planes_bytes);
-    int8_t* wq = reinterpret_cast<int8_t*>(base + planes_bytes + sx_bytes);
-    float* sw = reinterpret_cast<float*>(base + planes_bytes + sx_bytes + wq_bytes);
-    float* yp = reinterpret_cast<float*>(base + planes_bytes + sx_bytes + wq_bytes + sw_bytes);
-    hipLaunchKernelGGL(q8_split_rows_kernel, dim3(m), dim3(256), 0, s, a, planes, sxp, m, k);
+    float* sxp = reinterpret_cast<float*>(base + w.planes);
+    if (w.fold) {
+        hipLaunchKernelGGL(q8_split_rows_kernel<true>, dim3(m), dim3(256), 0, s, a, planes, sxp, m, k);
+        if (int rc = check_launch("q8_split_rows_kernel")) return rc;
+        return i8_gemm_fold4(planes, wq, sxp, sw, nullptr, c, kQ8Planes * m, k, n, s);
+    }
+    float* yp = reinterpret_cast<float*>(base + w.planes + w.sx);
+    hipLaunchKernelGGL(q8_split_rows_kernel<false>, dim3(m), dim3(256), 0, s, a, planes, sxp, m, k);
     if (int rc = check_launch("q8_split_rows_kernel")) return rc;
-    hipLaunchKernelGGL(q8_unpack_channels_kernel, dim3(ceil_div(k / 4, 256), n), dim3(256), 0, s, b,
-                       reinterpret_cast<uint32_t*>(wq), sw, k / 4, stride);
-    if (int rc = check_launch("q8_unpack_channels_kernel")) return rc;
     if (int rc = rumus_hip_i8_gemm(planes, wq, sxp, sw, nullptr, nullptr, yp, kQ8Planes * m, k, n, s)) return rc;
     const uint64_t count = (uint64_t)m * n;
     hipLaunchKernelGGL(q8_add_planes_kernel, dim3((uint32_t)((count + 255) / 256)), dim3(256), 0, s, yp, c, count);
     return check_launch("q8_add_planes_kernel");
+}
+
+static int matmul_q8_mfma(const float* a, const uint32_t* b, float* c, uint32_t m, uint32_t k, uint32_t n,
+                          uint32_t stride, hipStream_t s) {
+    RUMUS_REQUIRE((uint64_t)kQ8Planes * m < (1ull << 31), "matmul_q8: m %u is beyond the grid limit", m);
+    const Q8DenseWs w = q8_dense_workspace(m, k, n);
+    const size_t wq_bytes = align256((size_t)n * k), sw_bytes = align256((size_t)n * sizeof(float));
+    void* ws = nullptr;
+    WorkspaceLease lease;                                    // until the last kernel of this call is queued
+    if (int rc = workspace_get(s, wq_bytes + sw_bytes + w.total, &ws, lease)) return rc;
+    WorkspaceNest nest(wq_bytes + sw_bytes + w.own);
+    uint8_t* base = static_cast<uint8_t*>(ws);
+    int8_t* wq = reinterpret_cast<int8_t*>(base);
+    float* sw = reinterpret_cast<float*>(base + wq_bytes);
+    hipLaunchKernelGGL(q8_unpack_channels_kernel, dim3(ceil_div(k / 4, 256), n), dim3(256), 0, s, b,
+                       reinterpret_cast<uint32_t*>(wq), sw, k / 4, stride);
+    if (int rc = check_launch("q8_unpack_channels_kernel")) return rc;
+    return matmul_q8_planes(a, wq, sw, c, m, k, n, w, base + wq_bytes + sw_bytes, s);
 }
 
 // Activations for the f16 variant of the block-scale kernel: x f = hi + lo, two f16 planes [2][m][k]
@@ -586,7 +611,7 @@ static int matmul_q8_mfma_blocks(const float* a, const uint32_t* b, float* c, ui
         if (int rc = check_launch("q8_split_rows_f16_kernel")) return rc;
         return q8_gemm_blocks_f16(halves, sxp, b, c, m, k, n, bs, stride, bpc, part, max_shares, s);
     }
-    hipLaunchKernelGGL(q8_split_rows_kernel, dim3(m), dim3(256), 0, s, a, planes, sxp, m, k);
+    hipLaunchKernelGGL(q8_split_rows_kernel<false>, dim3(m), dim3(256), 0, s, a, planes, sxp, m, k);
     if (int rc = check_launch("q8_split_rows_kernel")) return rc;
     return q8_gemm_blocks(planes, sxp, b, c, m, k, n, bs, stride, bpc, part, max_shares, s);   // sxp[0 .. m): the rows' 1 / f
 }
@@ -791,6 +816,38 @@ int rumus_hip_matmul_q8(const float* a, const uint32_t* b, float* c, uint32_t m,
     hipLaunchKernelGGL(matmul_q8_naive_kernel, grid, dim3(256), 0, as_stream(stream), a, b, c, m,
                        k, n, block_size, stride, blocks_per_col);
     return check_launch("matmul_q8_naive_kernel");
+}
+
+int rumus_hip_q8_dense_layout(const uint32_t* b_q8, uint32_t k, uint32_t n, uint32_t block_size, int8_t* wq,
+                              float* sw, rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE(b_q8 && wq && sw, "q8_dense_layout: null buffer");
+    RUMUS_REQUIRE(block_size > 0 && block_size % 4 == 0,
+                  "q8_dense_layout: block_size must be > 0 and divisible by 4 (got %u)", block_size);
+    RUMUS_REQUIRE(k > 0 && k % 4 == 0 && block_size >= k,
+                  "q8_dense_layout: one block per column wanted (k %u, a multiple of 4, block_size %u >= k)", k, block_size);
+    RUMUS_REQUIRE((reinterpret_cast<uintptr_t>(wq) & 3) == 0, "q8_dense_layout: wq must be 4-byte aligned");
+    if (n == 0) return RUMUS_HIP_OK;
+    RUMUS_REQUIRE(n <= 65535, "q8_dense_layout: n %u is beyond the grid limit", n);
+    hipLaunchKernelGGL(q8_unpack_channels_kernel, dim3(ceil_div(k / 4, 256), n), dim3(256), 0, as_stream(stream), b_q8,
+                       reinterpret_cast<uint32_t*>(wq), sw, k / 4, (4 + block_size + 3) / 4);
+    return check_launch("q8_unpack_channels_kernel");
+}
+
+int rumus_hip_matmul_q8_dense(const float* a, const int8_t* wq, const float* sw, float* c, uint32_t m, uint32_t k,
+                              uint32_t n, rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE(a && wq && sw && c, "matmul_q8_dense: null buffer");
+    if (m == 0 || n == 0) return RUMUS_HIP_OK;
+    RUMUS_REQUIRE(k > 0 && k % 16 == 0, "matmul_q8_dense: k must be a positive multiple of 16 (got %u)", k);
+    RUMUS_REQUIRE(((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(c) | reinterpret_cast<uintptr_t>(wq)) & 15) == 0,
+                  "matmul_q8_dense: a, wq and c must be 16-byte aligned");
+    RUMUS_REQUIRE((uint64_t)kQ8Planes * m < (1ull << 31), "matmul_q8_dense: m %u is beyond the grid limit", m);
+    hipStream_t s = as_stream(stream);
+    const Q8DenseWs w = q8_dense_workspace(m, k, n);
+    void* ws = nullptr;
+    WorkspaceLease lease;                                    // until the last kernel of this call is queued
+    if (int rc = workspace_get(s, w.total, &ws, lease)) return rc;
+    WorkspaceNest nest(w.own);
+    return matmul_q8_planes(a, wq, sw, c, m, k, n, w, static_cast<uint8_t*>(ws), s);
 }
 
 int rumus_hip_add_bias(const float* mat, const float* bias, float* out, uint32_t m, uint32_t n,

@@ -137,6 +137,17 @@ class Q8Tensor:
     def numel(self) -> int:
         return self.shape[0] * self.shape[1]
 
+    def prepare(self) -> "Q8Tensor":
+        """For a weight with one block per column that meets batches of hundreds of rows more than once: keep a
+        dense int8 copy beside the buffer (as many bytes again), which :func:`matmul` then multiplies against
+        instead of unpacking the buffer on every call.  Same results, bit for bit."""
+        k, n = self.shape
+        if self.block_size < k or k % 16 != 0 or n > 65535:
+            raise ValueError("prepare: wants one block per column (block_size >= k), k % 16 == 0 and n <= 65535")
+        if getattr(self, "_dense", None) is None:
+            object.__setattr__(self, "_dense", ops.q8_dense_layout(self.buffer, k, n, self.block_size))
+        return self
+
     def data(self):
         """``Tensor::data()`` on a Q8 tensor (core.rs:612-691): dequantize on the GPU, download the
         f32 values (buffer order, as the reference does) and keep the host copy for later calls."""
@@ -185,7 +196,14 @@ def matmul(lhs: torch.Tensor, rhs) -> torch.Tensor:
         raise ValueError("matmul: this path handles Q8 weights only")
     if lhs.dim() != 2 or lhs.shape[1] != rhs.shape[0]:
         raise ValueError("matmul: inner dimension mismatch")
+    dense = getattr(rhs, "_dense", None)
+    if dense is not None and lhs.shape[0] >= Q8_DENSE_MIN_ROWS:
+        return ops.matmul_q8_dense(lhs.contiguous(), *dense)
     return ops.matmul_q8(lhs.contiguous(), rhs.buffer, rhs.shape[0], rhs.shape[1], rhs.block_size)
+
+
+# below this many rows the kernels that read the Q8 buffer directly are the faster ones
+Q8_DENSE_MIN_ROWS = 384
 
 
 def linear_forward(linear: Linear, x: torch.Tensor, weight_q8: Q8Tensor) -> torch.Tensor:

@@ -13,7 +13,7 @@ from . import _lib
 from ._lib import RumusError, call
 
 __all__ = [
-    "q8_buf_size", "q8_quantize", "q8_dequantize", "q8_dequantize_kn", "matmul_q8", "add_bias", "transpose_f32",
+    "q8_buf_size", "q8_quantize", "q8_dequantize", "q8_dequantize_kn", "matmul_q8", "q8_dense_layout", "matmul_q8_dense", "add_bias", "transpose_f32",
     "i8_quantize_rows", "i8_quantize_cols_t", "i8_gemm", "w4_quantize_pack", "qmatmul_int4",
     "qmatmul_int4_t", "w4_actorder_prepare", "qmatmul_int4_perm", "w4_geometry", "RumusError",
 ]
@@ -81,6 +81,32 @@ def matmul_q8(a: torch.Tensor, words: torch.Tensor, k: int, n: int, block_size: 
         raise ValueError("matmul: out must be a contiguous f32 [m, n] tensor")
     call("rumus_hip_matmul_q8", _dev(a, torch.float32, "a"), _dev(words, torch.int32, "b"),
          c.data_ptr(), m, k, n, block_size, _stream())
+    return c
+
+
+def q8_dense_layout(words: torch.Tensor, k: int, n: int, block_size: int):
+    """A Q8 buffer with one block per column (``block_size >= k``) as dense int8 ``[n, k]`` plus the ``n`` block
+    scales: the operands of :func:`matmul_q8_dense`, made once per weight."""
+    wq = torch.empty((n, k), dtype=torch.int8, device=words.device)
+    sw = torch.empty(n, dtype=torch.float32, device=words.device)
+    call("rumus_hip_q8_dense_layout", _dev(words, torch.int32, "b"), k, n, block_size, wq.data_ptr(), sw.data_ptr(),
+         _stream())
+    return wq, sw
+
+
+def matmul_q8_dense(a: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor, out=None) -> torch.Tensor:
+    """``a @ W`` for a per-output-channel Q8 weight in the layout of :func:`q8_dense_layout`."""
+    n, k = wq.shape
+    m = a.shape[0]
+    if a.dim() != 2 or a.shape[1] != k:
+        raise ValueError("matmul: inner dimension mismatch")
+    if sw.numel() != n:
+        raise ValueError("matmul: one scale per output channel wanted")
+    c = torch.empty((m, n), dtype=torch.float32, device=a.device) if out is None else out
+    if c.shape != (m, n) or c.dtype != torch.float32 or not c.is_contiguous():
+        raise ValueError("matmul: out must be a contiguous f32 [m, n] tensor")
+    call("rumus_hip_matmul_q8_dense", _dev(a, torch.float32, "a"), _dev(wq, torch.int8, "wq"),
+         _dev(sw, torch.float32, "sw"), c.data_ptr(), m, k, n, _stream())
     return c
 
 

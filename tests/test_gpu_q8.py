@@ -162,6 +162,60 @@ def test_matmul_q8_row_split_inside_on_a_fresh_stream(ops):
     assert_close(host(got), host(parts))
 
 
+@pytest.mark.parametrize("m,k,n", [(1024, 256, 2048),     # planes added in the epilogue of the 256 x 256 blocks
+                                   (1501, 192, 2801),     # ... of the wide blocks, ragged on both sides
+                                   (1536, 128, 4096),     # ... rows split over two launches of those kernels
+                                   (3000, 64, 2050),      # rows split with a part on kernels without that epilogue:
+                                   (400, 512, 96),        # ... those and small shapes add the planes in a pass
+                                   (100, 1024, 300), (8, 48, 20), (1, 16, 5)])
+def test_matmul_q8_dense_copy(ops, m, k, n):
+    # a per-output-channel weight prepared once (Q8Tensor.prepare) against the same weight unpacked on every call
+    say(f"matmul_q8_dense m={m} k={k} n={n}")
+    from rumus_amd import nn
+    rng = np.random.default_rng(m * 3 + k + n)
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    a = rng.normal(0, 1, (m, k)).astype(np.float32)
+    a[m // 2, 3] = 2.0e4
+    if m > 4:
+        a[4] = 0.0
+    words = oracle.tensor_quantize(w, k)
+    wq, sw = ops.q8_dense_layout(dev(words), k, n, k)
+    blocks = words.reshape(n, 1 + k // 4)                  # a header word, then k / 4 data words per column
+    np.testing.assert_array_equal(host(wq).view(np.uint8), np.ascontiguousarray(blocks[:, 1:]).view(np.uint8))
+    np.testing.assert_array_equal(host(sw), (blocks[:, 0] & 0xFFFF).astype(np.uint16).view(np.float16).astype(np.float32))
+    got = host(ops.matmul_q8_dense(dev(a), wq, sw))
+    want = oracle.matmul_q8(a, words, k, n, k, threads=8)
+    assert_close(got, want)
+    if m > 4:
+        np.testing.assert_array_equal(got[4], np.zeros(n, np.float32))
+    if m >= 384:                                           # there matmul_q8 takes the same route on a copy it makes itself
+        np.testing.assert_array_equal(got, host(ops.matmul_q8(dev(a), dev(words), k, n, k)))
+    q = nn.Q8Tensor(dev(words), (k, n), k).prepare()
+    via_nn = host(nn.matmul(dev(a), q))
+    if m >= nn.Q8_DENSE_MIN_ROWS:
+        np.testing.assert_array_equal(via_nn, got)
+    else:
+        assert_close(via_nn, want)
+    ab = a.copy()
+    ab[m - 1, 7] = np.float32(np.inf)                      # poisons its own row only
+    gb = host(ops.matmul_q8_dense(dev(ab), wq, sw))
+    assert np.isnan(gb[m - 1]).all()
+    np.testing.assert_array_equal(gb[:m - 1], got[:m - 1])
+
+
+def test_q8_dense_rejects(ops):
+    say("q8 dense rejects")
+    import torch
+    words = dev(oracle.tensor_quantize(np.ones((64, 8), np.float32), 32))
+    with pytest.raises(ops.RumusError):                    # two blocks per column
+        ops.q8_dense_layout(words, 64, 8, 32)
+    wq = torch.zeros((8, 24), dtype=torch.int8, device="cuda")
+    with pytest.raises(ops.RumusError):                    # k % 16
+        ops.matmul_q8_dense(torch.zeros((4, 24), device="cuda"), wq, torch.ones(8, device="cuda"))
+    with pytest.raises(ValueError):
+        ops.matmul_q8_dense(torch.zeros((4, 32), device="cuda"), wq, torch.ones(8, device="cuda"))
+
+
 @pytest.mark.parametrize("bs,m", [(512, 64), (32, 64), (128, 64), (128, 100), (512, 400)])
 def test_matmul_q8_batch_accuracy_and_non_finite_rows(ops, bs, m):
     # batches: activations go through four 7-bit digit planes and the int8 matrix cores (block scales
