@@ -58,8 +58,19 @@ extern "C" int rumus_dbg_w4i8_stamps(unsigned long long* host, size_t count) {
 }
 #define STAMP(i) do { const uint32_t wg_ = blockIdx.y * gridDim.x + blockIdx.x;                           \
         if (lane == 0 && wg_ < kStampWorkgroups) g_w4i8_stamps[(wg_ * 8 + wk) * 8 + (i)] = wall_clock64(); } while (0)
+// the same for the kernel that prepares the activations: [workgroup][wave][stamp]
+constexpr uint32_t kPrepStampWorkgroups = 256;
+__device__ unsigned long long g_w4i8_prep_stamps[kPrepStampWorkgroups * 8 * 8];
+extern "C" int rumus_dbg_w4i8_prep_stamps(unsigned long long* host, size_t count) {
+    if (count > kPrepStampWorkgroups * 8 * 8) return 1;
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_w4i8_prep_stamps), count * 8);
+}
+#define PSTAMP(i) do { const uint32_t wg_ = blockIdx.y * gridDim.x + blockIdx.x;                          \
+        if (lane == 0 && wg_ < kPrepStampWorkgroups)                                                      \
+            g_w4i8_prep_stamps[(wg_ * 8 + (threadIdx.x >> 6)) * 8 + (i)] = wall_clock64(); } while (0)
 #else
 #define STAMP(i)
+#define PSTAMP(i)
 #endif
 
 // low bytes of a, b, c, d -> one word
@@ -76,17 +87,64 @@ __device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
 // itself).  Rows past m are written as zeros: the matmul reads whole row tiles.  The first four groups of a
 // lane (shares up to 2048 k) stay in registers between the pass that finds the maximum and the pass that
 // writes the digits.
-template <int CS, bool VEC>
-__global__ __launch_bounds__(64) void w4_i8_prepare_kernel(const float* __restrict__ x, const int32_t* __restrict__ perm,
-                                                           uint8_t* __restrict__ planes, float* __restrict__ rscale,
-                                                           int32_t* __restrict__ csum, uint32_t m, uint32_t k,
-                                                           uint32_t steps, uint32_t chunks, uint32_t per) {
+// STAGED (act-order, x[row][perm[j]]): the eight waves of a row are one workgroup that first copies the row
+// into LDS (k floats of dynamic LDS) with contiguous reads and gathers from there; gathered from global
+// memory a wave instruction touches 64 cache lines for 256 bytes, behind the load of perm itself.
+template <int CS, bool VEC, bool STAGED>
+__global__ __launch_bounds__(STAGED ? 64 * kI8WK : 64) void w4_i8_prepare_kernel(
+    const float* __restrict__ x, const int32_t* __restrict__ perm, uint8_t* __restrict__ planes,
+    float* __restrict__ rscale, int32_t* __restrict__ csum, uint32_t m, uint32_t k, uint32_t steps, uint32_t chunks,
+    uint32_t per) {
+    static_assert(!(VEC && STAGED), "staging is for the gather");
+    extern __shared__ __attribute__((aligned(16))) float lds_row[];
     constexpr int CACHE = 4;
     constexpr uint32_t SUBS = 8 * CS;                               // lanes per chunk
-    const uint32_t lane = threadIdx.x, share = blockIdx.x, row = blockIdx.y, rt = row >> 4, row_l = row & 15;
+    const uint32_t lane = threadIdx.x & 63, share = STAGED ? threadIdx.x >> 6 : blockIdx.x;
+    const uint32_t row = STAGED ? blockIdx.x : blockIdx.y, rt = row >> 4, row_l = row & 15;
     const uint32_t k_begin = min(share * per, chunks) * CS * 64, k_end = min((share + 1) * per, chunks) * CS * 64;
     const bool live = row < m;
     const float* xr = x + (uint64_t)(live ? row : 0) * k;
+    PSTAMP(0);
+    // STAGED (the launcher sends k % 8 == 0 and 16-byte aligned x and perm here): where a lane's 8 values come
+    // from, then the values themselves.  Straight-line code with clamped addresses: a load under a branch
+    // would make the wave wait for it at the end of the branch, one trip to memory after the other.
+    auto index8 = [&](uint32_t k0, int4 (&ix)[2]) {
+        const bool in = live && k0 < k_end && k0 < k;              // whole groups of 8 are in or out
+        const int4* src = reinterpret_cast<const int4*>(perm + (in ? k0 : 0));
+        ix[0] = src[0];
+        ix[1] = src[1];
+        return in;
+    };
+    auto gather8 = [&](const int4 (&ix)[2], bool in, float (&v)[8]) {
+        const uint32_t j[8] = {(uint32_t)ix[0].x, (uint32_t)ix[0].y, (uint32_t)ix[0].z, (uint32_t)ix[0].w,
+                               (uint32_t)ix[1].x, (uint32_t)ix[1].y, (uint32_t)ix[1].z, (uint32_t)ix[1].w};
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const float f = lds_row[j[e]];
+            v[e] = in ? f : 0.0f;
+        }
+    };
+    // the indices of the groups kept in registers are fetched while the row is on its way into LDS
+    int4 cix[STAGED ? CACHE : 1][2];
+    bool cin[STAGED ? CACHE : 1];
+    if (STAGED) {
+#pragma unroll
+        for (int i = 0; i < CACHE; i++) cin[i] = index8(k_begin + (lane + 64 * i) * 8, cix[i]);
+        constexpr uint32_t T = 64 * kI8WK;
+        const uint32_t vecs = k / 4;
+        const float4* src = reinterpret_cast<const float4*>(xr);
+        for (uint32_t i0 = threadIdx.x; i0 < vecs; i0 += 4 * T) {      // four loads in flight: one trip up to 8192 k
+            float4 t[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) t[u] = src[min(i0 + u * T, vecs - 1)];
+            __builtin_amdgcn_sched_barrier(0);                     // all issued before the first is waited for
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                if (i0 + u * T < vecs) reinterpret_cast<float4*>(lds_row)[i0 + u * T] = t[u];
+        }
+        __syncthreads();
+    }
+    PSTAMP(1);
 
     auto load8 = [&](uint32_t k0, float (&v)[8]) {
 #pragma unroll
@@ -96,6 +154,12 @@ __global__ __launch_bounds__(64) void w4_i8_prepare_kernel(const float* __restri
                 float4 f = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
                 if (live && k0 < k_end && kk < k) f = *reinterpret_cast<const float4*>(xr + kk);
                 v[4 * j4] = f.x; v[4 * j4 + 1] = f.y; v[4 * j4 + 2] = f.z; v[4 * j4 + 3] = f.w;
+            } else if (STAGED) {
+                if (j4 == 0) {
+                    int4 ix[2];
+                    const bool in = index8(k0, ix);
+                    gather8(ix, in, v);
+                }
             } else {
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
@@ -119,7 +183,8 @@ __global__ __launch_bounds__(64) void w4_i8_prepare_kernel(const float* __restri
     uint32_t mb = 0;
 #pragma unroll
     for (int i = 0; i < CACHE; i++) {
-        load8(k_begin + (lane + 64 * i) * 8, cache[i]);
+        if (STAGED) gather8(cix[i], cin[i], cache[i]);
+        else load8(k_begin + (lane + 64 * i) * 8, cache[i]);
         mb = max(mb, max_bits(cache[i]));
     }
     for (uint32_t k0 = k_begin + (lane + 64 * CACHE) * 8; k0 < k_end; k0 += 512) {
@@ -132,6 +197,7 @@ __global__ __launch_bounds__(64) void w4_i8_prepare_kernel(const float* __restri
     // 2^e with max * 2^e in [2^19, 2^20); tiny values stop at 2^100 (their products vanish in f32 anyway).  A
     // non-finite activation poisons its row: the scale becomes NaN (the digits are then whatever the
     // conversion gives; they only ever meet the NaN)
+    PSTAMP(2);
     const bool finite = mb < 0x7f800000u;
     int e = 19 - ((int)(mb >> 23) - 127);
     e = mb == 0 ? 0 : min(e, 100);
@@ -171,6 +237,7 @@ __global__ __launch_bounds__(64) void w4_i8_prepare_kernel(const float* __restri
         load8(k0, v);
         emit(k0, v);
     }
+    PSTAMP(3);
 }
 
 // ---- the matmul -------------------------------------------------------------------------------------
@@ -414,14 +481,25 @@ int w4_launch_gemm_i8(const W4Args& a, hipStream_t s) {
     int32_t* csum = reinterpret_cast<int32_t*>(planes + planes_bytes);
     float* rscale = reinterpret_cast<float*>(planes + planes_bytes + csum_bytes);
     const bool vec = !a.perm && a.k % 4 == 0 && (reinterpret_cast<uintptr_t>(a.x) & 15) == 0;
+    const bool staged = a.perm && (size_t)a.k * sizeof(float) <= 64 * 1024 && a.k % 8 == 0 &&
+                        ((reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.perm)) & 15) == 0;
     const dim3 pgrid(kI8WK, rts * 16);
-    if (cs == 2) {
-        if (vec) hipLaunchKernelGGL((w4_i8_prepare_kernel<2, true>), pgrid, dim3(64), 0, s, a.x, a.perm, planes, rscale, csum, a.m, a.k, steps, chunks, per);
-        else hipLaunchKernelGGL((w4_i8_prepare_kernel<2, false>), pgrid, dim3(64), 0, s, a.x, a.perm, planes, rscale, csum, a.m, a.k, steps, chunks, per);
-    } else {
-        if (vec) hipLaunchKernelGGL((w4_i8_prepare_kernel<1, true>), pgrid, dim3(64), 0, s, a.x, a.perm, planes, rscale, csum, a.m, a.k, steps, chunks, per);
-        else hipLaunchKernelGGL((w4_i8_prepare_kernel<1, false>), pgrid, dim3(64), 0, s, a.x, a.perm, planes, rscale, csum, a.m, a.k, steps, chunks, per);
-    }
+    const size_t row_bytes = (size_t)a.k * sizeof(float);
+#define RUMUS_I8_PREPARE(CS)                                                                                           \
+    do {                                                                                                               \
+        if (staged)                                                                                                    \
+            hipLaunchKernelGGL((w4_i8_prepare_kernel<CS, false, true>), dim3(rts * 16), dim3(64 * kI8WK), row_bytes, s, \
+                               a.x, a.perm, planes, rscale, csum, a.m, a.k, steps, chunks, per);                       \
+        else if (vec)                                                                                                  \
+            hipLaunchKernelGGL((w4_i8_prepare_kernel<CS, true, false>), pgrid, dim3(64), 0, s, a.x, a.perm, planes,    \
+                               rscale, csum, a.m, a.k, steps, chunks, per);                                            \
+        else                                                                                                           \
+            hipLaunchKernelGGL((w4_i8_prepare_kernel<CS, false, false>), pgrid, dim3(64), 0, s, a.x, a.perm, planes,   \
+                               rscale, csum, a.m, a.k, steps, chunks, per);                                            \
+    } while (0)
+    if (cs == 2) RUMUS_I8_PREPARE(2);
+    else RUMUS_I8_PREPARE(1);
+#undef RUMUS_I8_PREPARE
     if (int rc = check_launch("w4_i8_prepare_kernel")) return rc;
     const W4I8Args k{a.packed, a.scales, a.zp, a.zp4, a.bias, planes, rscale, csum, a.y,
                      a.m, a.n, steps, chunks, a.group_size / 64, per};

@@ -551,6 +551,79 @@ __global__ __launch_bounds__(256) void w4_convert_x_kernel(const float* __restri
     if (kb == 0) xs[blk * 32 + row] = sum;
 }
 
+// The same planes for act-order weights (x[row][perm[j]]).  Gathered from global memory a wave instruction
+// touches 64 cache lines for 256 bytes; here a workgroup copies `rows` whole rows of x into LDS with
+// contiguous reads and gathers from there.  Thread = (row, MFMA step): 16 values, both k blocks of the step.
+// Dynamic LDS: rows * kpad floats, kpad = k rounded up to 4.
+__global__ __launch_bounds__(256) void w4_convert_x_perm_kernel(const float* __restrict__ x,
+                                                                const int32_t* __restrict__ perm,
+                                                                uint8_t* __restrict__ xh, uint8_t* __restrict__ xl,
+                                                                float* __restrict__ xs, uint32_t m, uint32_t k,
+                                                                uint32_t xsteps, uint32_t rows, uint32_t kpad) {
+    extern __shared__ __attribute__((aligned(16))) float lds_rows[];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t row0 = blockIdx.x * rows;                  // rows divides 32: a workgroup stays inside a row tile
+    const uint32_t live = row0 < m ? min(rows, m - row0) : 0;
+    const float* src = x + (uint64_t)row0 * k;
+    if ((k % 4 == 0) && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+        const uint32_t vec = live * (k / 4);                  // the live rows are one contiguous run, and kpad == k
+        for (uint32_t i = tid; i < vec; i += 256)
+            reinterpret_cast<float4*>(lds_rows)[i] = reinterpret_cast<const float4*>(src)[i];
+    } else {
+        for (uint32_t r = 0; r < live; r++)
+            for (uint32_t i = tid; i < k; i += 256) lds_rows[r * kpad + i] = src[(uint64_t)r * k + i];
+    }
+    __syncthreads();
+    const uint32_t r = tid % rows, grow = row0 + r, tile = grow / 32, row = grow % 32;
+    const float* lr = lds_rows + r * kpad;
+    for (uint32_t step = tid / rows; step < xsteps; step += 256 / rows) {
+        const uint32_t k0 = step * 16;
+        float xv[16];
+        if (grow < m && k0 + 16 <= k && (reinterpret_cast<uintptr_t>(perm) & 15) == 0) {
+            int4 pj[4];
+#pragma unroll
+            for (int q = 0; q < 4; q++) pj[q] = *reinterpret_cast<const int4*>(perm + k0 + 4 * q);
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                xv[4 * q] = lr[(uint32_t)pj[q].x]; xv[4 * q + 1] = lr[(uint32_t)pj[q].y];
+                xv[4 * q + 2] = lr[(uint32_t)pj[q].z]; xv[4 * q + 3] = lr[(uint32_t)pj[q].w];
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 16; j++) {
+                const bool in = grow < m && k0 + j < k;
+                const float v = lr[in ? (uint32_t)perm[k0 + j] : 0];
+                xv[j] = in ? v : 0.0f;
+            }
+        }
+        const uint64_t blk = (uint64_t)tile * xsteps + step;
+        float sum[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+            v8h hi, lo;
+            sum[kb] = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const int j = (e >> 1) + 4 * (e & 1);            // fragment element e holds k offset j
+                const float v = xv[8 * kb + j];
+                const _Float16 h = (_Float16)v;
+                hi[e] = h;
+                lo[e] = (_Float16)(v - (float)h);
+                sum[kb] += v;
+            }
+            *reinterpret_cast<v8h*>(xh + (blk * 64 + kb * 32 + row) * 16) = hi;
+            *reinterpret_cast<v8h*>(xl + (blk * 64 + kb * 32 + row) * 16) = lo;
+        }
+        xs[blk * 32 + row] = sum[0] + sum[1];                 // the order of w4_convert_x_kernel: eight and eight
+    }
+}
+
+// rows of x per workgroup of w4_convert_x_perm_kernel (a power of two up to 8), 0: k too long for LDS
+static uint32_t convert_perm_rows(uint32_t kpad) {
+    const uint32_t fit = (64u * 1024) / (kpad * 4);
+    return fit >= 8 ? 8 : fit >= 4 ? 4 : fit >= 2 ? 2 : fit;
+}
+
 template <int RT, int WM, int TN, int WAVES, int DEPTH, int FOLD>
 static int launch_tile(const W4Args& a_in, hipStream_t s) {
     W4Args a = a_in;
@@ -582,8 +655,13 @@ static int launch_tile(const W4Args& a_in, hipStream_t s) {
             const bool vec = !a.perm && a.k % 8 == 0 && (reinterpret_cast<uintptr_t>(a.x) & 15) == 0;
             const dim3 grid(xsteps / 4, xtiles);
             float* sums = reinterpret_cast<float*>(base + 2 * plane_bytes);
-            if (vec) hipLaunchKernelGGL(w4_convert_x_kernel<true>, grid, dim3(256), 0, s, a.x, a.perm, base,
-                                        base + plane_bytes, sums, a.m, a.k, xsteps);
+            const uint32_t perm_rows = a.perm ? convert_perm_rows(k4) : 0;
+            if (perm_rows)
+                hipLaunchKernelGGL(w4_convert_x_perm_kernel, dim3(xtiles * 32 / perm_rows), dim3(256),
+                                   (size_t)perm_rows * k4 * sizeof(float), s, a.x, a.perm, base, base + plane_bytes, sums,
+                                   a.m, a.k, xsteps, perm_rows, k4);
+            else if (vec) hipLaunchKernelGGL(w4_convert_x_kernel<true>, grid, dim3(256), 0, s, a.x, a.perm, base,
+                                             base + plane_bytes, sums, a.m, a.k, xsteps);
             else hipLaunchKernelGGL(w4_convert_x_kernel<false>, grid, dim3(256), 0, s, a.x, a.perm, base,
                                     base + plane_bytes, sums, a.m, a.k, xsteps);
             if (int rc = check_launch("w4_convert_x_kernel")) return rc;
