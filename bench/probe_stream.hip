@@ -3,7 +3,7 @@
 // loads in flight per lane.  The decode-size kernels of the library read 9 to 50 MB per launch, where
 // dispatch, first-byte latency and the depth of the memory pipeline decide, not the HBM peak.
 //
-//   probe_stream <MiB per launch> [buffers]
+//   probe_stream <MiB per launch> [buffers] [row bytes of the strip shape, a multiple of 256]
 //
 // Every variant reads the same bytes (rotating over `buffers` distinct buffers so that no cache serves
 // them), 16 bytes per lane per load, and folds them into a value it never stores.  Shapes:
@@ -102,11 +102,13 @@ struct Timer {
 
 int main(int argc, char** argv) {
     const double mib = argc > 1 ? atof(argv[1]) : 22.0;
-    const int buffers = argc > 2 ? atoi(argv[2]) : (int)(640.0 / mib) + 1;
+    const int buffers = argc > 2 && atoi(argv[2]) > 0 ? atoi(argv[2]) : (int)(640.0 / mib) + 1;
     // a matrix of 1024-byte-per-wave-instruction pieces: rows of `row_bytes` for the strip shape
-    const uint32_t row_bytes = 44032;                       // 11008 packed words
+    const uint32_t row_bytes = argc > 3 ? (uint32_t)atoi(argv[3]) / 256 * 256 : 44032;   // 11008 packed words
     const size_t want = (size_t)(mib * 1048576.0);
-    const size_t rows = want / row_bytes / 512 * 512, bytes = rows * row_bytes;   // whole strips of 512 rows
+    size_t rows = want / row_bytes / 64 * 64;               // whole strips of 64 rows: every shape below divides them
+    if (rows == 0) rows = 64;
+    const size_t bytes = rows * row_bytes;
     std::vector<uint4*> bufs(buffers);
     for (auto& b : bufs) { CHECK(hipMalloc(&b, bytes + 65536)); CHECK(hipMemset(b, 1, bytes + 65536)); }
     uint32_t* sink;
@@ -124,25 +126,25 @@ int main(int argc, char** argv) {
     printf("one-wave kernel: %.2f us per launch\n", empty);
 
 #define FLAT(L, T) do { const uint32_t wgs = (uint32_t)(bytes / ((size_t)(L) * (T) * 16)); \
-        report("flat", wgs, T, L, 1, t.per_launch_us(buffers, [&](int i, hipStream_t s) { \
+        if (wgs >= 1 && (size_t)wgs * (L) * (T) * 16 == bytes) report("flat", wgs, T, L, 1, t.per_launch_us(buffers, [&](int i, hipStream_t s) { \
             hipLaunchKernelGGL(flat_kernel<L>, dim3(wgs), dim3(T), 0, s, bufs[i], sink); })); } while (0)
     FLAT(1, 256); FLAT(2, 256); FLAT(4, 256); FLAT(8, 256);
     FLAT(1, 512); FLAT(2, 512); FLAT(4, 512); FLAT(8, 512); FLAT(16, 512);
 
 #define DEEP(L, T, WGS) do { const uint32_t waves = (WGS) * ((T) / 64); \
         const uint32_t rounds = (uint32_t)(bytes / ((size_t)waves * (L) * 1024)); \
-        if (rounds >= 1) report("deep", WGS, T, L, rounds, t.per_launch_us(buffers, [&](int i, hipStream_t s) { \
+        if (rounds >= 1 && (size_t)rounds * waves * (L) * 1024 == bytes) report("deep", WGS, T, L, rounds, t.per_launch_us(buffers, [&](int i, hipStream_t s) { \
             hipLaunchKernelGGL((deep_kernel<L, false>), dim3(WGS), dim3(T), 0, s, bufs[i], sink, rounds, 0u); })); } while (0)
     DEEP(2, 512, 256); DEEP(4, 512, 256); DEEP(8, 512, 256); DEEP(16, 512, 256);
     DEEP(2, 512, 512); DEEP(4, 512, 512); DEEP(8, 512, 512);
     DEEP(2, 512, 1024); DEEP(4, 512, 1024);
-    DEEP(4, 256, 512); DEEP(4, 256, 1024); DEEP(8, 1024, 256);
+    DEEP(4, 256, 512); DEEP(4, 256, 1024);
 
     // strips: row_bytes / 256 workgroups, each a 256-byte column strip over all rows
 #define STRIPS(L, T) do { const uint32_t wgs = row_bytes / 256, waves = (T) / 64; \
         const uint32_t rounds = (uint32_t)(rows / ((size_t)waves * (L) * 4)); \
-        report("strip", wgs, T, L, rounds, t.per_launch_us(buffers, [&](int i, hipStream_t s) { \
+        if (rounds >= 1 && (size_t)rounds * waves * (L) * 4 == rows) report("strip", wgs, T, L, rounds, t.per_launch_us(buffers, [&](int i, hipStream_t s) { \
             hipLaunchKernelGGL((deep_kernel<L, true>), dim3(wgs), dim3(T), 0, s, bufs[i], sink, rounds, row_bytes / 16); })); } while (0)
-    STRIPS(2, 512); STRIPS(4, 512); STRIPS(8, 512); STRIPS(4, 1024); STRIPS(2, 1024);
+    STRIPS(1, 256); STRIPS(2, 256); STRIPS(1, 512); STRIPS(2, 512); STRIPS(4, 512); STRIPS(8, 512);
     return 0;
 }

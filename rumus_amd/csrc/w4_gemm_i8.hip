@@ -48,8 +48,8 @@ struct W4I8Args {
     uint32_t m, n, steps, chunks, steps_per_group, per;   // per: chunks per share
 };
 
-#ifdef W4I8_TIMERS
-// instrumented build only (-DW4I8_TIMERS): wall-clock stamps (10 ns ticks) of every wave at fixed points
+#ifdef RUMUS_TIMERS
+// instrumented build only (-DRUMUS_TIMERS): wall-clock stamps (10 ns ticks) of every wave at fixed points
 constexpr uint32_t kStampWorkgroups = 512;                       // the first so many workgroups of a launch are recorded
 __device__ unsigned long long g_w4i8_stamps[kStampWorkgroups * 8 * 8];
 extern "C" int rumus_dbg_w4i8_stamps(unsigned long long* host, size_t count) {
@@ -378,7 +378,7 @@ __global__ __launch_bounds__(512) void w4_gemm_i8_kernel(W4I8Args a) {
                         accf[t][q][i] = fmaf(sc[q], (float)tot, accf[t][q][i]);
                     }
             }
-#ifdef W4I8_TIMERS
+#ifdef RUMUS_TIMERS
             if (base == f0 && u == 0) { __builtin_amdgcn_sched_barrier(0); if (accf[0][0][0] != 1e30f) STAMP(2); }
 #endif
         }

@@ -60,10 +60,33 @@ template <int Q> __device__ __forceinline__ uint32_t quad_bcast(uint32_t v) {
 __device__ __forceinline__ float reduce_row_lanes(float v) {
     v += RUMUS_DPP_F(v, kDppRowShr4);   // out-of-row reads give 0
     v += RUMUS_DPP_F(v, kDppRowShr8);
-    v += __shfl_xor(v, 16);
-    v += __shfl_xor(v, 32);
+    // rows 0 + 1 and 2 + 3, then the halves: register swaps between lanes (v_permlane16_swap, v_permlane32_swap)
+    // instead of two trips through the LDS crossbar; the same sums as v += shfl_xor(v, 16); v += shfl_xor(v, 32)
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    const auto h = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(h[0]) + __uint_as_float(h[1]);
     return v;
 }
+
+#ifdef RUMUS_TIMERS
+// instrumented build only (-DRUMUS_TIMERS): wall-clock stamps (10 ns ticks) of every wave of the first 256
+// workgroups at fixed points, [workgroup][wave][stamp].  A stamp is taken once `after` is known (the branch
+// on its bits makes the clock read depend on it).
+constexpr uint32_t kD8StampWorkgroups = 256;
+__device__ unsigned long long g_d8_stamps[kD8StampWorkgroups * 8 * 8];
+extern "C" int rumus_dbg_d8_stamps(unsigned long long* host, size_t count) {
+    if (count > kD8StampWorkgroups * 8 * 8) return 1;
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_d8_stamps), count * 8);
+}
+#define D8_STAMP(i, after) do { __builtin_amdgcn_sched_barrier(0);                                         \
+        if ((threadIdx.x & 63) == 0 && blockIdx.x < kD8StampWorkgroups && (threadIdx.x >> 6) < 8 &&        \
+            __float_as_uint(after) != 0x7fabcdefu)                                                         \
+            g_d8_stamps[(blockIdx.x * 8 + (threadIdx.x >> 6)) * 8 + (i)] = wall_clock64();                 \
+        __builtin_amdgcn_sched_barrier(0); } while (0)
+#else
+#define D8_STAMP(i, after)
+#endif
 
 // Kernel arguments are passed flat, hottest first: the first 16 dwords are
 // preloaded into SGPRs by the command processor (see the build flags), which
@@ -105,6 +128,7 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
     for (int m = 0; m < M; m++)
 #pragma unroll
         for (int c = 0; c < 4; c++) acc[m][c] = 0.0f;
+    D8_STAMP(0, acc[0][0]);
 
     // every quad runs the same number of sweeps; a dead quad carries scale 0
     for (uint32_t base = 0; base < nchunks; base += RL) {
@@ -117,7 +141,17 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
         // the nibble planes are then built while the weight loads are in flight.
         // Branch-free (clamped addresses, values zeroed by select) so that the
         // wait before the plane build covers x only.
+        // The eight waves of a workgroup start together and the memory pipeline of the compute unit
+        // takes their requests, and returns their data, in order: without help the oldest wave issues
+        // all of its loads first and the activations of the other waves come back behind its weights
+        // (measured: planes built 0.7 us after the start in wave 0, 1.3 us in waves 1-3, 1.9 us in
+        // waves 4-7).  Raised priority while a wave asks for its activations puts the x requests of
+        // the waves that start together ahead of their weight requests (planes at 0.8 us in waves
+        // 0-3, 1.5 us in 4-7, which start 40 ns later; 0.03 to 0.2 us per launch by the machine).
+        // With packed zero-points the same change costs 0.3 to 0.5 us, so it stays off there.
+        constexpr bool kPrioX = !ZP4;
         float xv[M][OPL][8];
+        if (kPrioX && base == 0) __builtin_amdgcn_s_setprio(3);
         const uint32_t k0 = (ch * OCT + cq * OPL) * 8;   // first row this lane prepares
 #pragma unroll
         for (int m = 0; m < M; m++) {
@@ -154,21 +188,30 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
                 }
             }
         }
+        if (kPrioX && base == 0) {
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_setprio(0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        const uint32_t g = (ch * 8 * OCT) / group_size;
+        const uint64_t mo = TILED ? ((uint64_t)cchunk * (padded_k / group_size) + g) * kD8Cols + 4 * cq
+                                  : (uint64_t)g * n + col_c;
         uint4 w[OCT];
         const uint32_t* p = TILED ? packed + ((uint64_t)cchunk * (padded_k / 8) + (uint64_t)ch * OCT) * kD8Cols + 4 * cq
                                   : packed + (uint64_t)ch * OCT * n + col_c;
         const uint64_t wstride = TILED ? kD8Cols : n;
+        float4 sc, zp;
+        auto load_meta = [&]() __attribute__((always_inline)) {
+            sc = *reinterpret_cast<const float4*>(scales + mo);
+            // ZP4 + TILED: the two zero-point words of a tile's 16 columns sit side by side per group
+            zp = !ZP4 ? *reinterpret_cast<const float4*>(zps + mo)
+                 : TILED ? w4_zp4_unpack4(reinterpret_cast<const uint32_t*>(zps)[
+                               ((uint64_t)cchunk * (padded_k / group_size) + g) * 2 + (cq >> 1)] >> ((cq & 1) * 16))
+                         : w4_zp4_load4(reinterpret_cast<const uint32_t*>(zps), g, n, col_c);
+        };
 #pragma unroll
         for (int u = 0; u < OCT; u++) w[u] = *reinterpret_cast<const uint4*>(p + (uint64_t)u * wstride);
-        const uint32_t g = (ch * 8 * OCT) / group_size;
-        const uint64_t mo = TILED ? ((uint64_t)cchunk * (padded_k / group_size) + g) * kD8Cols + 4 * cq
-                                  : (uint64_t)g * n + col_c;
-        float4 sc = *reinterpret_cast<const float4*>(scales + mo);
-        // ZP4 + TILED: the two zero-point words of a tile's 16 columns sit side by side per group
-        const float4 zp = !ZP4 ? *reinterpret_cast<const float4*>(zps + mo)
-                          : TILED ? w4_zp4_unpack4(reinterpret_cast<const uint32_t*>(zps)[
-                                        ((uint64_t)cchunk * (padded_k / group_size) + g) * 2 + (cq >> 1)] >> ((cq & 1) * 16))
-                                  : w4_zp4_load4(reinterpret_cast<const uint32_t*>(zps), g, n, col_c);
+        load_meta();
         if (!(live && col_ok)) sc = make_float4(0, 0, 0, 0);
 
         uint32_t wv[OCT][4];
@@ -246,26 +289,38 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
                     pl[3 * OPL + t][i] = quad_bcast<3>(own[t][i]);
                 }
 
+            D8_STAMP(1, __uint_as_float(pl[OCT - 1][4]));      // planes built (last sweep, last row of x)
             // ---- 3. dot products -------------------------------------------------
+            // word row by word row, in the order the loads were issued and retire: the rows that have
+            // arrived are multiplied while the later ones are still on their way, and only the last
+            // row's 24 instructions follow the last byte
+            uint32_t d[4][5], qsum[4];
 #pragma unroll
             for (int c = 0; c < 4; c++) {
-                uint32_t d[5] = {0, 0, 0, 0, 0};
-                uint32_t qsum = 0;
+                qsum[c] = 0;
 #pragma unroll
-                for (int u = 0; u < OCT; u++) {
-                    qsum = udot8(wv[u][c], 0x11111111u, qsum);
+                for (int i = 0; i < 5; i++) d[c][i] = 0;
+            }
 #pragma unroll
-                    for (int i = 0; i < 5; i++) d[i] = udot8(wv[u][c], pl[u][i], d[i]);
+            for (int u = 0; u < OCT; u++)
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    qsum[c] = udot8(wv[u][c], 0x11111111u, qsum[c]);
+#pragma unroll
+                    for (int i = 0; i < 5; i++) d[c][i] = udot8(wv[u][c], pl[u][i], d[c][i]);
                 }
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
                 // D < 2^31: 8*OCT*225 * (16^5 - 1) / 15
-                const uint32_t D = d[0] + 16u * (d[1] + 16u * (d[2] + 16u * (d[3] + 16u * d[4])));
-                const int I = (int)D - (int)(qsum << 19);
+                const uint32_t D = d[c][0] + 16u * (d[c][1] + 16u * (d[c][2] + 16u * (d[c][3] + 16u * d[c][4])));
+                const int I = (int)D - (int)(qsum[c] << 19);
                 const float part = (float)I * finv;
                 acc[m][c] = fmaf(scv[c], fmaf(-zv[c], xs, part), acc[m][c]);
             }
         }
     }
 
+    D8_STAMP(2, acc[M - 1][3]);                                // every weight arrived and multiplied
     // ---- 4. reduce over the quads of a wave, then over the waves -----------------
     const uint32_t lane = tid & 63, wave = tid >> 6;
 #pragma unroll
@@ -278,7 +333,9 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
 #pragma unroll
             for (int c = 0; c < 4; c++) red[wave][m][(lane - 12) * 4 + c] = acc[m][c];
     }
+    D8_STAMP(3, acc[M - 1][3]);                                // reduced over the wave, written to LDS
     __syncthreads();
+    D8_STAMP(4, acc[M - 1][3]);                                // barrier passed
     if (tid < M * kD8Cols) {
         const uint32_t m = tid / kD8Cols, c = tid % kD8Cols;
         const uint32_t oc = cchunk * kD8Cols + c;
@@ -290,6 +347,7 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
             yout[(uint64_t)m * n + oc] = v;
         }
     }
+    D8_STAMP(5, acc[M - 1][3]);                                // result stored (the waves that store: issued)
 }
 
 // Launch geometry: threads per workgroup and word rows per quad.
