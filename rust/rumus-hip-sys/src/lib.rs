@@ -75,6 +75,19 @@ extern "C" {
     pub fn rumus_hip_attention(q: *const f32, k: *const f32, v: *const f32, out: *mut f32, batch: u32,
                                heads: u32, q_len: u32, kv_len: u32, head_dim: u32, strides: *const u64,
                                causal: c_int, s: Stream) -> c_int;
+    pub fn rumus_hip_kv_append(k_new: *const f32, v_new: *const f32, k_cache: *mut f32, v_cache: *mut f32, batch: u32,
+                               heads: u32, rows: u32, head_dim: u32, pos: u32, cache_len: u32, strides: *const u64,
+                               s: Stream) -> c_int;
+    pub fn rumus_hip_q8_dense_layout(b_q8: *const u32, k: u32, n: u32, block_size: u32, wq: *mut i8, sw: *mut f32,
+                                     s: Stream) -> c_int;
+    pub fn rumus_hip_matmul_q8_dense(a: *const f32, wq: *const i8, sw: *const f32, c: *mut f32, m: u32, k: u32,
+                                     n: u32, s: Stream) -> c_int;
+    pub fn rumus_hip_i8_gemm_workspace_size(m: u32, k: u32, n: u32) -> u64;
+    pub fn rumus_hip_qmatmul_int4_perm_static(x: *const f32, packed_sorted: *const u32, scales: *const f32,
+                                              zp: *const f32, bias: *const f32, perm: *const i32, y: *mut f32,
+                                              m: u32, k: u32, n: u32, padded_k: u32, group_size: u32,
+                                              num_groups: u32, s: Stream) -> c_int;
+    pub fn rumus_hip_static_scratch_bytes() -> u64;
     pub fn rumus_hip_qmatmul_int4_zp4(x: *const f32, packed: *const u32, scales: *const f32, qzeros: *const u32,
                                       bias: *const f32, perm: *const i32, y: *mut f32, m: u32, k: u32, n: u32,
                                       padded_k: u32, group_size: u32, num_groups: u32, s: Stream) -> c_int;
