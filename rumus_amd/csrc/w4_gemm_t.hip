@@ -98,10 +98,14 @@ __global__ __launch_bounds__(256) void w4t_prepare_kernel(const float* __restric
 // is converted into the A-fragment buffer (double-buffered) while the MFMAs of step t run; one barrier
 // per step.
 constexpr int kTRawGy = 64 * 128, kTRawW = 16 * 128, kTRawSz = 256, kTRawZo = 256;   // 64 bytes of zero-point integers used
-constexpr int kTRaw = kTRawGy + kTRawW + kTRawSz + kTRawZo;   // bytes of one raw stage
+constexpr int kTRawWt = kTRawW + kTRawSz + kTRawZo;           // weights and tables of one step
 constexpr int kTAbuf = 2 * 64 * 64;                           // hi, lo planes
 constexpr int kTSlots = 12;                                   // wave-wide loads per step: 8 grad_y, 1-2 weights, 2 tables
-constexpr size_t w4t_lds_bytes(int stages) { return (size_t)stages * kTRaw + 2 * kTAbuf + 64 * sizeof(float); }
+// The raw tile of grad_y of step t is dead once it has been converted (during step t - 1), the weights and tables of
+// step t are read during step t: one slot fewer for grad_y than for the rest, at the same depth of loads in flight.
+constexpr size_t w4t_lds_bytes(int stages) {
+    return (size_t)(stages - 1) * kTRawGy + (size_t)stages * kTRawWt + 2 * kTAbuf + 64 * sizeof(float);
+}
 
 // KW = waves per workgroup = 32-column slices of k per tile: 4 when groups are multiples of 128, 2 for
 // groups of 64, 1 for groups of 32 (a tile must lie inside one group, since the activations are re-scaled
@@ -113,8 +117,9 @@ __global__ __launch_bounds__(64 * KW, 2) void w4t_gemm_kernel(
     const float* __restrict__ sgrp, float* __restrict__ out, uint32_t m, uint32_t k, uint32_t n, uint32_t gs,
     uint32_t steps_per) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    uint8_t* const raw = lds;                                  // [kTStages][kTRaw]
-    uint8_t* const abuf = lds + kTStages * kTRaw;              // [2][kTAbuf]
+    uint8_t* const raw_gy = lds;                               // [kTStages - 1][kTRawGy]
+    uint8_t* const raw_wt = lds + (kTStages - 1) * kTRawGy;    // [kTStages][kTRawWt]
+    uint8_t* const abuf = raw_wt + kTStages * kTRawWt;         // [2][kTAbuf]
     float* const lds_c = reinterpret_cast<float*>(abuf + 2 * kTAbuf);
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -135,10 +140,11 @@ __global__ __launch_bounds__(64 * KW, 2) void w4t_gemm_kernel(
     const uint32_t l8 = lane >> 3, p8 = lane & 7;
     const uint8_t* src[kTLoads];
     uint32_t dst[kTLoads], colw[kTLoads], esz[kTLoads];        // colw: the lane's first column inside a step
-    bool wide[kTLoads];
+    bool wide[kTLoads], is_gy[kTLoads];                        // dst: offset inside the slot of its kind
 #pragma unroll
     for (int i = 0; i < kTLoads; i++) {
         const uint32_t q = KW * i + wave;
+        is_gy[i] = q < 8;
         if (q < 8) {
             const uint32_t row = min(m0 + 8 * q + l8, m - 1);
             src[i] = reinterpret_cast<const uint8_t*>(gy + (uint64_t)row * n);
@@ -148,21 +154,23 @@ __global__ __launch_bounds__(64 * KW, 2) void w4t_gemm_kernel(
             // fetch its last row again, into room the stage keeps for that
             const uint32_t wr = k0 / 8 + min(8 * (q - 8) + l8, 4u * KW - 1);
             src[i] = reinterpret_cast<const uint8_t*>(packed + (uint64_t)wr * n);
-            dst[i] = kTRawGy + (q - 8) * 1024; colw[i] = 4 * p8; wide[i] = true; esz[i] = 4;
+            dst[i] = (q - 8) * 1024; colw[i] = 4 * p8; wide[i] = true; esz[i] = 4;
         } else if (q == 8 + WS) {
             src[i] = reinterpret_cast<const uint8_t*>((lane < 32 ? sp : zf) + (uint64_t)g * n);
-            dst[i] = kTRawGy + kTRawW; colw[i] = lane & 31; wide[i] = false; esz[i] = 4;
+            dst[i] = kTRawW; colw[i] = lane & 31; wide[i] = false; esz[i] = 4;
         } else {
             src[i] = reinterpret_cast<const uint8_t*>(zo + (uint64_t)g * n);
-            dst[i] = kTRawGy + kTRawW + kTRawSz; colw[i] = 2 * (lane & 15); wide[i] = false; esz[i] = 2;
+            dst[i] = kTRawW + kTRawSz; colw[i] = 2 * (lane & 15); wide[i] = false; esz[i] = 2;
         }
     }
     // columns past n are fetched from column 0: the conversion turns them into zeros
-    auto issue = [&](uint32_t st, uint32_t stage) {
-        uint8_t* base = raw + stage * kTRaw;
+    auto issue = [&](uint32_t st, uint32_t gslot, uint32_t wslot) {
+        uint8_t* const gbase = raw_gy + gslot * kTRawGy;
+        uint8_t* const wbase = raw_wt + wslot * kTRawWt;
         const uint32_t c0 = min(st, st1 - 1) * 32;
 #pragma unroll
         for (int i = 0; i < kTLoads; i++) {
+            uint8_t* const base = is_gy[i] ? gbase : wbase;
             const uint32_t col = c0 + colw[i] < n ? c0 + colw[i] : 0;
             if (wide[i])
                 __builtin_amdgcn_global_load_lds((gptr_t)(src[i] + (uint64_t)col * esz[i]), (lptr_t)(base + dst[i]), 16, 0, 0);
@@ -177,15 +185,16 @@ __global__ __launch_bounds__(64 * KW, 2) void w4t_gemm_kernel(
     const float frow_raw = rowf[min(m0 + s_row, m - 1)];
     const float frow = frow_raw != frow_raw ? 0.0f : frow_raw; // inf / nan in the row: NaN times 0 poisons it below
     float csum = 0.0f;
-    auto convert_chunk = [&](uint32_t st, uint32_t stage, int buf, uint32_t s_ch) {
+    auto convert_chunk = [&](uint32_t st, uint32_t gslot, uint32_t wslot, int buf, uint32_t s_ch) {
         const uint32_t s_lds = s_row * 64 + ((s_ch ^ row_swizzle(s_row)) & 3) * 16;
-        const uint8_t* base = raw + stage * kTRaw;
-        const float4 g0 = *reinterpret_cast<const float4*>(base + s_row * 128 + s_ch * 32);
-        const float4 g1 = *reinterpret_cast<const float4*>(base + s_row * 128 + s_ch * 32 + 16);
-        const float4 s0 = *reinterpret_cast<const float4*>(base + kTRawGy + kTRawW + s_ch * 32);
-        const float4 s1 = *reinterpret_cast<const float4*>(base + kTRawGy + kTRawW + s_ch * 32 + 16);
-        const float4 z0 = *reinterpret_cast<const float4*>(base + kTRawGy + kTRawW + 128 + s_ch * 32);
-        const float4 z1 = *reinterpret_cast<const float4*>(base + kTRawGy + kTRawW + 128 + s_ch * 32 + 16);
+        const uint8_t* gbase = raw_gy + gslot * kTRawGy;
+        const uint8_t* tbase = raw_wt + wslot * kTRawWt + kTRawW;
+        const float4 g0 = *reinterpret_cast<const float4*>(gbase + s_row * 128 + s_ch * 32);
+        const float4 g1 = *reinterpret_cast<const float4*>(gbase + s_row * 128 + s_ch * 32 + 16);
+        const float4 s0 = *reinterpret_cast<const float4*>(tbase + s_ch * 32);
+        const float4 s1 = *reinterpret_cast<const float4*>(tbase + s_ch * 32 + 16);
+        const float4 z0 = *reinterpret_cast<const float4*>(tbase + 128 + s_ch * 32);
+        const float4 z1 = *reinterpret_cast<const float4*>(tbase + 128 + s_ch * 32 + 16);
         const uint32_t c0 = st * 32 + s_ch * 8;
         // n % 4 == 0: four columns are all-in or all-out; the columns past n hold values of column 0
         const float f0 = c0 < n ? frow : 0.0f, f1 = c0 + 4 < n ? frow : 0.0f;
@@ -211,20 +220,20 @@ __global__ __launch_bounds__(64 * KW, 2) void w4t_gemm_kernel(
         *reinterpret_cast<uint4*>(ab + s_lds) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
         *reinterpret_cast<uint4*>(ab + 64 * 64 + s_lds) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
     };
-    auto convert = [&](uint32_t st, uint32_t stage, int buf) {
+    auto convert = [&](uint32_t st, uint32_t gslot, uint32_t wslot, int buf) {
 #pragma unroll
-        for (int cc = 0; cc < CPT; cc++) convert_chunk(st, stage, buf, s_ch0 + cc);
+        for (int cc = 0; cc < CPT; cc++) convert_chunk(st, gslot, wslot, buf, s_ch0 + cc);
     };
 
     // ---- B role: lane (k = 32 wave + lane % 32, half = lane / 32): 8 words of word row 4 wave + k / 8 ----
     const uint32_t bc = lane & 31, bh = lane >> 5;
     const uint32_t shift = 4 * (bc & 7);
-    const uint32_t b_off = kTRawGy + (4 * wave + (bc >> 3)) * 128 + bh * 32;
-    auto b_frag = [&](int t, uint32_t stage) {
-        const uint8_t* sb = raw + stage * kTRaw;
+    const uint32_t b_off = (4 * wave + (bc >> 3)) * 128 + bh * 32;
+    auto b_frag = [&](int t, uint32_t wslot) {
+        const uint8_t* sb = raw_wt + wslot * kTRawWt;
         const uint4 w0 = *reinterpret_cast<const uint4*>(sb + b_off + t * 64), w1 = *reinterpret_cast<const uint4*>(sb + b_off + t * 64 + 16);
         const uint32_t w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
-        const t8h off = *reinterpret_cast<const t8h*>(sb + kTRawGy + kTRawW + kTRawSz + 32 * t + 16 * bh);   // 1024 + z0
+        const t8h off = *reinterpret_cast<const t8h*>(sb + kTRawW + kTRawSz + 32 * t + 16 * bh);   // 1024 + z0
         t2h h[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -250,19 +259,21 @@ __global__ __launch_bounds__(64 * KW, 2) void w4t_gemm_kernel(
     // Every step issues exactly kTLoads loads per wave, also past the end (the last step again, into a
     // stage nobody reads any more), so the counter arithmetic has no tail cases.
 #pragma unroll
-    for (int s = 0; s < kTStages - 1; s++) issue(st0 + s, s);
+    for (int s = 0; s < kTStages - 1; s++) issue(st0 + s, s, s);
     RUMUS_WAIT_VMCNT((kTStages - 2) * kTLoads);               // step st0 has landed
     __builtin_amdgcn_s_barrier();
-    convert(st0, 0, 0);
-    uint32_t cur = 0;                                          // raw stage of step st
+    convert(st0, 0, 0, 0);
+    uint32_t cur = 0, gcur = 0;                                // slots of step st: weights and tables, grad_y
     for (uint32_t st = st0; st < st1; st++) {
         const int ab = (st - st0) & 1;
         const uint32_t nxt = cur + 1 == kTStages ? 0 : cur + 1, prv = cur == 0 ? kTStages - 1 : cur - 1;
+        const uint32_t gnxt = gcur + 1 == kTStages - 1 ? 0 : gcur + 1;
         // step st+1 has landed once only the kTStages-3 younger steps are outstanding; past the barrier
-        // the A fragments of step st are visible and the stage of step st-1 is free
+        // the A fragments of step st are visible, the weight slot of step st-1 is free and so is the grad_y
+        // slot of step st itself (converted during step st-1)
         RUMUS_WAIT_VMCNT((kTStages - 3) * kTLoads);
         __builtin_amdgcn_s_barrier();
-        issue(st + (kTStages - 1), prv);
+        issue(st + (kTStages - 1), gcur, prv);
         const t8h b0 = b_frag(0, cur), b1 = b_frag(1, cur);
         const uint8_t* abp = abuf + ab * kTAbuf;
 #pragma unroll
@@ -274,8 +285,9 @@ __global__ __launch_bounds__(64 * KW, 2) void w4t_gemm_kernel(
             acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const t8h*>(hi + a_off[1]), b1, acc[i], 0, 0, 0);
             acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const t8h*>(lo + a_off[1]), b1, acc[i], 0, 0, 0);
         }
-        if (st + 1 < st1) convert(st + 1, nxt, ab ^ 1);
+        if (st + 1 < st1) convert(st + 1, gnxt, nxt, ab ^ 1);
         cur = nxt;
+        gcur = gnxt;
     }
     RUMUS_WAIT_VMCNT(0);         // no direct-to-LDS write may outlive the workgroup
 
@@ -386,27 +398,11 @@ int w4_launch_gemm_t(const float* gy, const uint32_t* packed, const float* scale
     hipLaunchKernelGGL(w4t_prepare_kernel, dim3(m + num_groups), dim3(256), 0, s, gy, scales, zp, rowf, sgrp, sp, zf, zo, m,
                        n);
     if (int rc = check_launch("w4t_prepare_kernel")) return rc;
-    // stages of loads in flight: the step rate does not depend on them (3 to 5 measured within 4 %: the
-    // vector ALU work of the conversion sets the pace), so the count follows occupancy: four stages leave
-    // LDS for two workgroups per compute unit, three stages for three.  Workgroups run in rounds of that many
-    // per CU and a round lasts the same whether it is full or not (544 workgroups: 678 us with four stages,
-    // 437 us with three), so the cheaper of the two by the measured round times (us at 4096 x 11008, g128; only
-    // their ratios matter) is taken.
-    auto rounds_cost = [](uint64_t wgs, uint32_t per_cu, const uint32_t* round_us) {
-        const uint64_t slots = 256ull * per_cu, rest = wgs % slots;
-        return (wgs / slots) * round_us[per_cu] + round_us[(rest + 255) / 256];
-    };
-    static const uint32_t us4[3] = {0, 225, 350}, us3[4] = {0, 260, 383, 465};   // by workgroups per CU in the round
-    const int ns = rounds_cost(tiles * shares, 3, us3) < rounds_cost(tiles * shares, 2, us4) ? 3 : 4;
-    int rc;
-    switch (ns) {
-        case 4:
-            rc = kw == 4 ? RUMUS_W4T_LAUNCH(4, 4) : kw == 2 ? RUMUS_W4T_LAUNCH(4, 2) : RUMUS_W4T_LAUNCH(4, 1);
-            break;
-        default:
-            rc = kw == 4 ? RUMUS_W4T_LAUNCH(3, 4) : kw == 2 ? RUMUS_W4T_LAUNCH(3, 2) : RUMUS_W4T_LAUNCH(3, 1);
-            break;
-    }
+    // Three weight slots and two grad_y slots: 39.75 KB of LDS, four workgroups per compute unit.  Workgroups run in
+    // rounds of that many per CU and a round lasts almost the same whether it is full or not, so what matters is how
+    // many fit: with four stages (three per CU) 2048 rows x 4096 took 0.70 ms for 1024 workgroups on 768 places, with
+    // three stages 0.57 ms on 1024 places, and the four-stage form was faster for no batch from 256 to 4096 rows.
+    const int rc = kw == 4 ? RUMUS_W4T_LAUNCH(3, 4) : kw == 2 ? RUMUS_W4T_LAUNCH(3, 2) : RUMUS_W4T_LAUNCH(3, 1);
     if (rc) return rc;
     if (shares == 1) return RUMUS_HIP_OK;
     const uint32_t count4 = (uint32_t)((uint64_t)m * k / 4);
