@@ -69,11 +69,7 @@ bool w4_gemm_supported(const W4Args& a);
 uint32_t w4_decode_max_rows(uint32_t padded_k, uint32_t n);   // w4_gemv.hip
 int w4_launch_gemm(const W4Args& a, hipStream_t s);
 
-// Sum of partial results laid out like y, in order, plus bias (w4_gemm_tile.hip).
-int w4_launch_reduce(const float* part, const float* bias, float* y, uint32_t m, uint32_t n, uint32_t splits,
-                     hipStream_t s);
-
-// int8 matrix cores for up to 16 rows (w4_gemm_i8.hip): group_size % 64 == 0, n % 4 == 0, 16-byte aligned
+// int8 matrix cores for up to 128 rows (w4_gemm_i8.hip): group_size % 64 == 0, n % 4 == 0, 16-byte aligned
 // buffers, no g_idx.
 bool w4_gemm_i8_supported(const W4Args& a);
 int w4_launch_gemm_i8(const W4Args& a, hipStream_t s);

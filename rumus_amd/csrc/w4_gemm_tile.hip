@@ -461,16 +461,6 @@ __global__ __launch_bounds__(256) void w4_gemm_reduce_kernel(const float4* __res
     y[idx] = s;
 }
 
-// y = part[0] + ... + part[splits - 1] (+ bias), part in the layout of y; m * n % 4 == 0, splits <= kMaxSplits
-int w4_launch_reduce(const float* part, const float* bias, float* y, uint32_t m, uint32_t n, uint32_t splits,
-                     hipStream_t s) {
-    RUMUS_REQUIRE(splits >= 1 && splits <= (uint32_t)kMaxSplits, "w4 reduce: %u partial results", splits);
-    const uint32_t count4 = (uint32_t)((uint64_t)m * n / 4);
-    hipLaunchKernelGGL(w4_gemm_reduce_kernel, dim3(ceil_div(count4, 256)), dim3(256), 0, s,
-                       reinterpret_cast<const float4*>(part), bias, reinterpret_cast<float4*>(y), count4, n / 4, splits);
-    return check_launch("w4_gemm_reduce_kernel");
-}
-
 bool w4_gemm_supported(const W4Args& a) {
     const uintptr_t bits = reinterpret_cast<uintptr_t>(a.packed) | reinterpret_cast<uintptr_t>(a.scales) |
                            reinterpret_cast<uintptr_t>(a.zp) | reinterpret_cast<uintptr_t>(a.y) |

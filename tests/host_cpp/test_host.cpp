@@ -10,6 +10,7 @@
 #include <vector>
 
 #include "rumus_hip.hpp"
+#include "rumus_hip_block.hpp"
 #include "rumus_hip_file.hpp"
 #include "rumus_oracle.h"
 
@@ -224,6 +225,39 @@ static void test_file(const std::string& dir) {
     }
 }
 
+// The decoder block on layers the Python side stored (block.safetensors: q, k, v, o, gate, up, down; block_x.bin:
+// [batch, n, dim] f32): a prefill that fills the caches, then one decode step at position n on block_x1.bin
+// ([batch, 1, dim]).  Outputs go back as files; the Python test compares them bit for bit with its own block.
+static void test_block(const std::string& dir) {
+    const auto px = slurp(dir + "/block_x.bin"), px1 = slurp(dir + "/block_x1.bin"), cfg = slurp(dir + "/block_cfg.txt");
+    if (px.empty() || px1.empty() || cfg.empty()) return;
+    uint32_t batch = 0, n = 0, heads = 0, cache_len = 0;
+    CHECK(sscanf(std::string(cfg.begin(), cfg.end()).c_str(), "%u %u %u %u", &batch, &n, &heads, &cache_len) == 4,
+          "block_cfg.txt: batch n heads cache_len");
+    printf("[host-cpp] decoder block: batch %u, %u tokens, %u heads\n", batch, n, heads);
+    fflush(stdout);
+    auto layers = load_w4(dir + "/block.safetensors");
+    const uint32_t dim = heads * 128;
+    std::vector<float> ones(dim, 1.0f);
+    DecoderBlockW4 blk = DecoderBlockW4::from_layers(layers, ones, ones, heads);
+    std::vector<float> hx(px.size() / 4), hx1(px1.size() / 4);
+    memcpy(hx.data(), px.data(), px.size());
+    memcpy(hx1.data(), px1.data(), px1.size());
+    CHECK(hx.size() == (size_t)batch * n * dim && hx1.size() == (size_t)batch * dim, "block input sizes");
+    DeviceBuffer<float> x(hx), x1(hx1), y(hx.size()), y1(hx1.size());
+    DeviceBuffer<float> kc(std::vector<float>((size_t)batch * cache_len * dim, 0.0f)),
+        vc(std::vector<float>((size_t)batch * cache_len * dim, 0.0f));
+    blk.forward(x.data(), batch, n, y.data(), kc.data(), vc.data(), cache_len, 0);
+    blk.forward(x1.data(), batch, 1, y1.data(), kc.data(), vc.data(), cache_len, n);
+    const auto hy = y.download(), hy1 = y1.download(), hk = kc.download();
+    spill(dir + "/block_y.bin", hy.data(), hy.size() * 4);
+    spill(dir + "/block_y1.bin", hy1.data(), hy1.size() * 4);
+    spill(dir + "/block_k.bin", hk.data(), hk.size() * 4);
+    bool threw = false;
+    try { blk.forward(x.data(), batch, n, y.data(), kc.data(), vc.data(), cache_len, 1); } catch (const Error& e) { threw = e.code == RUMUS_HIP_EINVAL; }
+    CHECK(threw, "several tokens at pos > 0 must be rejected");
+}
+
 static void test_errors() {
     printf("[host-cpp] preconditions\n");
     fflush(stdout);
@@ -250,6 +284,7 @@ int main(int argc, char** argv) {
     test_int8_linear(300, 1024, 260);
     test_errors();
     test_file(argc > 1 ? argv[1] : "/tmp");
+    test_block(argc > 1 ? argv[1] : "/tmp");
     printf(g_fail ? "host-cpp: %d FAILED\n" : "host-cpp: all passed\n", g_fail);
     return g_fail ? 1 : 0;
 }

@@ -36,6 +36,22 @@ def test_cpp_host_mirror_matches_oracle(tmp_path):
     x = rng.standard_normal((m, k)).astype(np.float32)
     x.tofile(tmp_path / "py_x.bin")
 
+    # a decoder block for the C++ mirror of DecoderBlockW4: seven stored layers, a prefill input and one
+    # decode token; small enough for a test, large enough for the matrix-core attention (64 rows or more)
+    from rumus_amd import nn
+    heads, ffn, gs, batch, ntok, cache_len = 2, 512, 64, 2, 70, 96
+    dim = heads * 128
+    shapes = {"q": (dim, dim), "k": (dim, dim), "v": (dim, dim), "o": (dim, dim), "gate": (dim, ffn),
+              "up": (dim, ffn), "down": (ffn, dim)}
+    wts = {name: dev((rng.standard_normal(sh) * 0.05).astype(np.float32)) for name, sh in shapes.items()}
+    blk = nn.DecoderBlockW4.from_f32(wts, gs, heads)
+    ck.save_w4(str(tmp_path / "block.safetensors"), blk.proj)
+    bx = rng.standard_normal((batch, ntok, dim)).astype(np.float32)
+    bx1 = rng.standard_normal((batch, 1, dim)).astype(np.float32)
+    bx.tofile(tmp_path / "block_x.bin")
+    bx1.tofile(tmp_path / "block_x1.bin")
+    (tmp_path / "block_cfg.txt").write_text(f"{batch} {ntok} {heads} {cache_len}\n")
+
     out = subprocess.run([BIN, str(tmp_path)], capture_output=True, text=True, timeout=300)
     print(out.stdout)
     print(out.stderr)
@@ -59,3 +75,17 @@ def test_cpp_host_mirror_matches_oracle(tmp_path):
     np.testing.assert_array_equal(host(plain(dev(xc))), yc)
     assert layers["blk.act_order"].weight.perm is not None
     assert torch.equal(layers["blk.act_order"].weight.scales_tensor, plain.weight.scales_tensor)
+
+    # the C++ decoder block on the stored layers: the bits of the Python block, prefill and decode step
+    y_py, k_py, v_py = blk(dev(bx))
+    kc = torch.zeros((batch, cache_len, heads, 128), dtype=torch.float32, device="cuda")
+    vc = torch.zeros_like(kc)
+    kc[:, :ntok] = k_py
+    vc[:, :ntok] = v_py
+    y1_py, kc, vc = blk(dev(bx1), kc, vc, pos=ntok)
+    y_cpp = np.fromfile(tmp_path / "block_y.bin", dtype=np.float32).reshape(batch, ntok, dim)
+    y1_cpp = np.fromfile(tmp_path / "block_y1.bin", dtype=np.float32).reshape(batch, 1, dim)
+    k_cpp = np.fromfile(tmp_path / "block_k.bin", dtype=np.float32).reshape(batch, cache_len, heads, 128)
+    np.testing.assert_array_equal(y_cpp, host(y_py))
+    np.testing.assert_array_equal(k_cpp, host(kc))
+    np.testing.assert_array_equal(y1_cpp, host(y1_py))
