@@ -148,7 +148,9 @@ __global__ __launch_bounds__(64 * KW, 2) void w4t_gemm_kernel(
         if (q < 8) {
             const uint32_t row = min(m0 + 8 * q + l8, m - 1);
             src[i] = reinterpret_cast<const uint8_t*>(gy + (uint64_t)row * n);
-            dst[i] = q * 1024; colw[i] = 4 * p8; wide[i] = true; esz[i] = 4;
+            // rows two apart would put the conversion's 128-bit reads two to a bank: every other pair of rows
+            // holds its 16-byte pieces swapped in twos (LDS piece p of row r = piece p ^ (r / 2 % 2) of the tile)
+            dst[i] = q * 1024; colw[i] = 4 * (p8 ^ ((l8 >> 1) & 1)); wide[i] = true; esz[i] = 4;
         } else if (q < 8 + WS) {
             // the tile's 4 KW word rows (< padded_k / 8: whole groups exist in the arrays); lanes past them
             // fetch its last row again, into room the stage keeps for that
@@ -189,8 +191,9 @@ __global__ __launch_bounds__(64 * KW, 2) void w4t_gemm_kernel(
         const uint32_t s_lds = s_row * 64 + ((s_ch ^ row_swizzle(s_row)) & 3) * 16;
         const uint8_t* gbase = raw_gy + gslot * kTRawGy;
         const uint8_t* tbase = raw_wt + wslot * kTRawWt + kTRawW;
-        const float4 g0 = *reinterpret_cast<const float4*>(gbase + s_row * 128 + s_ch * 32);
-        const float4 g1 = *reinterpret_cast<const float4*>(gbase + s_row * 128 + s_ch * 32 + 16);
+        const uint32_t sw = (s_row >> 1) & 1;                  // see the loads: pieces swapped in twos
+        const float4 g0 = *reinterpret_cast<const float4*>(gbase + s_row * 128 + ((2 * s_ch) ^ sw) * 16);
+        const float4 g1 = *reinterpret_cast<const float4*>(gbase + s_row * 128 + ((2 * s_ch + 1) ^ sw) * 16);
         const float4 s0 = *reinterpret_cast<const float4*>(tbase + s_ch * 32);
         const float4 s1 = *reinterpret_cast<const float4*>(tbase + s_ch * 32 + 16);
         const float4 z0 = *reinterpret_cast<const float4*>(tbase + 128 + s_ch * 32);
