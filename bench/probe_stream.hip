@@ -12,6 +12,7 @@
 //             next round's loads issued before the current round is consumed
 //   strip   : as deep, but a wave instruction reads four 256-byte segments `row_bytes` apart (a column
 //             strip of a row-major matrix) instead of 1 KB contiguous
+//   -nt     : the same with the non-temporal hint on every load
 // Times are per launch, replayed from a HIP graph of `buffers` launches.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -24,13 +25,24 @@
 
 __device__ __forceinline__ uint32_t fold(uint4 v) { return v.x ^ v.y ^ v.z ^ v.w; }
 
+// NT: the load carries the non-temporal hint (data used once)
+typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+template <bool NT>
+__device__ __forceinline__ uint4 ld(const uint4* p) {
+    if (NT) {
+        const u4v v = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(p));
+        return make_uint4(v.x, v.y, v.z, v.w);
+    }
+    return *p;
+}
+
 // flat: workgroup b reads LOADS * threads * 16 contiguous bytes
-template <int LOADS>
+template <int LOADS, bool NT = false>
 __global__ __launch_bounds__(512) void flat_kernel(const uint4* __restrict__ p, uint32_t* sink) {
     const uint4* q = p + (size_t)blockIdx.x * LOADS * blockDim.x + threadIdx.x;
     uint4 v[LOADS];
 #pragma unroll
-    for (int i = 0; i < LOADS; i++) v[i] = q[(size_t)i * blockDim.x];
+    for (int i = 0; i < LOADS; i++) v[i] = ld<NT>(q + (size_t)i * blockDim.x);
     uint32_t s = 0;
 #pragma unroll
     for (int i = 0; i < LOADS; i++) s |= fold(v[i]);
@@ -38,7 +50,7 @@ __global__ __launch_bounds__(512) void flat_kernel(const uint4* __restrict__ p, 
 }
 
 // deep: a wave owns rounds * LOADS KB, contiguous; double-buffered rounds
-template <int LOADS, bool STRIP>
+template <int LOADS, bool STRIP, bool NT = false>
 __global__ __launch_bounds__(512) void deep_kernel(const uint4* __restrict__ p, uint32_t* sink, uint32_t rounds,
                                                    uint32_t row_vec /* uint4 per matrix row, strip only */) {
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
@@ -51,9 +63,9 @@ __global__ __launch_bounds__(512) void deep_kernel(const uint4* __restrict__ p, 
                 // workgroup = a strip of 16 uint4 (256 bytes) columns; wave = rounds * LOADS * 4 rows of it;
                 // lane (c = lane % 16, b = lane / 16) reads row 4 * (r * LOADS + i) + b
                 const size_t row = (size_t)wave * rounds * LOADS * 4 + (size_t)(r * LOADS + i) * 4 + (lane >> 4);
-                v[slot][i] = p[row * row_vec + (size_t)blockIdx.x * 16 + (lane & 15)];
+                v[slot][i] = ld<NT>(p + row * row_vec + (size_t)blockIdx.x * 16 + (lane & 15));
             } else {
-                v[slot][i] = p[(wave_id * rounds + r) * LOADS * 64 + (size_t)i * 64 + lane];
+                v[slot][i] = ld<NT>(p + (wave_id * rounds + r) * LOADS * 64 + (size_t)i * 64 + lane);
             }
         }
     };
@@ -130,6 +142,10 @@ int main(int argc, char** argv) {
             hipLaunchKernelGGL(flat_kernel<L>, dim3(wgs), dim3(T), 0, s, bufs[i], sink); })); } while (0)
     FLAT(1, 256); FLAT(2, 256); FLAT(4, 256); FLAT(8, 256);
     FLAT(1, 512); FLAT(2, 512); FLAT(4, 512); FLAT(8, 512); FLAT(16, 512);
+#define FLAT_NT(L, T) do { const uint32_t wgs = (uint32_t)(bytes / ((size_t)(L) * (T) * 16)); \
+        if (wgs >= 1 && (size_t)wgs * (L) * (T) * 16 == bytes) report("flat-nt", wgs, T, L, 1, t.per_launch_us(buffers, [&](int i, hipStream_t s) { \
+            hipLaunchKernelGGL((flat_kernel<L, true>), dim3(wgs), dim3(T), 0, s, bufs[i], sink); })); } while (0)
+    FLAT_NT(1, 512); FLAT_NT(4, 512); FLAT_NT(8, 512);
 
 #define DEEP(L, T, WGS) do { const uint32_t waves = (WGS) * ((T) / 64); \
         const uint32_t rounds = (uint32_t)(bytes / ((size_t)waves * (L) * 1024)); \
@@ -146,5 +162,10 @@ int main(int argc, char** argv) {
         if (rounds >= 1 && (size_t)rounds * waves * (L) * 4 == rows) report("strip", wgs, T, L, rounds, t.per_launch_us(buffers, [&](int i, hipStream_t s) { \
             hipLaunchKernelGGL((deep_kernel<L, true>), dim3(wgs), dim3(T), 0, s, bufs[i], sink, rounds, row_bytes / 16); })); } while (0)
     STRIPS(1, 256); STRIPS(2, 256); STRIPS(1, 512); STRIPS(2, 512); STRIPS(4, 512); STRIPS(8, 512);
+#define STRIPS_NT(L, T) do { const uint32_t wgs = row_bytes / 256, waves = (T) / 64; \
+        const uint32_t rounds = (uint32_t)(rows / ((size_t)waves * (L) * 4)); \
+        if (rounds >= 1 && (size_t)rounds * waves * (L) * 4 == rows) report("strip-nt", wgs, T, L, rounds, t.per_launch_us(buffers, [&](int i, hipStream_t s) { \
+            hipLaunchKernelGGL((deep_kernel<L, true, true>), dim3(wgs), dim3(T), 0, s, bufs[i], sink, rounds, row_bytes / 16); })); } while (0)
+    STRIPS_NT(4, 512); STRIPS_NT(8, 512);
     return 0;
 }
