@@ -80,6 +80,36 @@ __device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
     return __builtin_amdgcn_perm(hi, lo, 0x05040100u);
 }
 
+// ---- lane exchanges without a trip through the LDS crossbar (integers: any order of the operands) --------
+// value of the lane's partner under the DPP pattern `ctrl`
+template <int CTRL>
+__device__ __forceinline__ int dpp_move(int v) { return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true); }
+constexpr int kDppQuadXor1 = 0xB1, kDppQuadXor2 = 0x4E;        // quad_perm [1,0,3,2], [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141, kDppRowMirror = 0x140;   // lane i <-> 7 - i of its 8, 15 - i of its 16
+
+// sum over aligned groups of LANES = 8 or 16 lanes, in every lane of the group
+template <uint32_t LANES>
+__device__ __forceinline__ int group_sum(int v) {
+    static_assert(LANES == 8 || LANES == 16, "half a row or a row of lanes");
+    v += dpp_move<kDppQuadXor1>(v);
+    v += dpp_move<kDppQuadXor2>(v);
+    v += dpp_move<kDppHalfMirror>(v);          // the other quad of the 8
+    if (LANES == 16) v += dpp_move<kDppRowMirror>(v);   // the other 8 of the row
+    return v;
+}
+
+// maximum over the 64 lanes of a wave, in every lane
+__device__ __forceinline__ uint32_t wave_max(uint32_t v) {
+    v = max(v, (uint32_t)dpp_move<kDppQuadXor1>((int)v));
+    v = max(v, (uint32_t)dpp_move<kDppQuadXor2>((int)v));
+    v = max(v, (uint32_t)dpp_move<kDppHalfMirror>((int)v));
+    v = max(v, (uint32_t)dpp_move<kDppRowMirror>((int)v));
+    const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);     // rows 0 | 1, 2 | 3
+    v = max(r[0], r[1]);
+    const auto h = __builtin_amdgcn_permlane32_swap(v, v, false, false);     // the halves
+    return max(h[0], h[1]);
+}
+
 // ---- activations -> digit planes ------------------------------------------------------------------
 // One wave per (row, share of K); a lane takes 8 consecutive k at a time: half of a lane's operand bytes of
 // one step (its even elements fill one word - a packed word's even nibbles -, its odd elements the next).
@@ -192,8 +222,7 @@ __global__ __launch_bounds__(STAGED ? 64 * kI8WK : 64) void w4_i8_prepare_kernel
         load8(k0, v);
         mb = max(mb, max_bits(v));
     }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) mb = max(mb, (uint32_t)__shfl_xor((int)mb, o));
+    mb = wave_max(mb);
     // 2^e with max * 2^e in [2^19, 2^20); tiny values stop at 2^100 (their products vanish in f32 anyway).  A
     // non-finite activation poisons its row: the scale becomes NaN (the digits are then whatever the
     // conversion gives; they only ever meet the NaN)
@@ -218,8 +247,7 @@ __global__ __launch_bounds__(STAGED ? 64 * kI8WK : 64) void w4_i8_prepare_kernel
             d[2][j] = (X1 + 64) >> 7;                              // |d2| <= 64
             sum += X;
         }
-#pragma unroll
-        for (uint32_t o = 1; o < SUBS; o <<= 1) sum += __shfl_xor(sum, (int)o);   // whole chunks are in or out together
+        sum = group_sum<SUBS>(sum);                                  // whole chunks are in or out together
         const uint32_t piece = k0 >> 4, step = piece >> 2, b = piece & 3, half = (k0 >> 3) & 1;
 #pragma unroll
         for (int p = 0; p < 3; p++)
