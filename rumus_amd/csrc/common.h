@@ -70,6 +70,35 @@ constexpr int kXcds = 8;        // MI355X: 8 accelerator dies, each with its own
 
 inline uint32_t ceil_div(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
 
+// Reductions over the 64 lanes of a wave, the result in every lane, without a trip through the LDS crossbar
+// (__shfl_xor is ds_bpermute): four DPP exchanges inside the rows of 16 lanes, then v_permlane16_swap and
+// v_permlane32_swap across them.  The pairs that meet are those of the xor butterfly with offsets 1, 2, 4, 8,
+// 16, 32 (lane i meets 7 - i and 15 - i instead of i ^ 4 and i ^ 8, which hold the same partial results), so a
+// commutative `op` gives the same bits as that butterfly, in every lane.
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_lane(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
+}
+template <typename T, typename F>
+__device__ __forceinline__ T wave_all_reduce(T value, F op) {
+    static_assert(sizeof(T) == 4, "32-bit values");
+    auto bits = [](T t) { return __builtin_bit_cast(uint32_t, t); };
+    auto val = [](uint32_t u) { return __builtin_bit_cast(T, u); };
+    T v = value;
+    v = op(v, val(dpp_lane<0xB1>(bits(v))));       // quad_perm [1,0,3,2]
+    v = op(v, val(dpp_lane<0x4E>(bits(v))));       // quad_perm [2,3,0,1]
+    v = op(v, val(dpp_lane<0x141>(bits(v))));      // row_half_mirror: the other quad of the 8
+    v = op(v, val(dpp_lane<0x140>(bits(v))));      // row_mirror: the other 8 of the row
+    const auto r = __builtin_amdgcn_permlane16_swap(bits(v), bits(v), false, false);   // rows 0 | 1, 2 | 3
+    v = op(val(r[0]), val(r[1]));
+    const auto h = __builtin_amdgcn_permlane32_swap(bits(v), bits(v), false, false);   // the halves
+    return op(val(h[0]), val(h[1]));
+}
+__device__ __forceinline__ float wave_sum(float v) { return wave_all_reduce(v, [](float a, float b) { return a + b; }); }
+__device__ __forceinline__ int32_t wave_sum(int32_t v) { return wave_all_reduce(v, [](int32_t a, int32_t b) { return a + b; }); }
+__device__ __forceinline__ float wave_max(float v) { return wave_all_reduce(v, [](float a, float b) { return fmaxf(a, b); }); }
+__device__ __forceinline__ uint32_t wave_max(uint32_t v) { return wave_all_reduce(v, [](uint32_t a, uint32_t b) { return a > b ? a : b; }); }
+
 // Workgroups are handed to the 8 XCDs round-robin (workgroup b runs on XCD
 // b % 8).  This maps b to a logical tile index so that each XCD owns one
 // contiguous range of tiles: neighbouring tiles then share an L2.

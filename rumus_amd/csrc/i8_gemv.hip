@@ -65,10 +65,7 @@ __global__ __launch_bounds__(64 * kGemvWaves) void i8_gemv_kernel(
     for (int r = 0; r < M; r++)
 #pragma unroll
         for (int j = 0; j < kGemvCols; j++) {
-            int32_t v = acc[r][j];
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
-            acc[r][j] = v;
+            acc[r][j] = wave_sum(acc[r][j]);
         }
     // lane j of the first kCols lanes writes column n0 + j of every row
     if (lane < kGemvCols && n0 + lane < N) {

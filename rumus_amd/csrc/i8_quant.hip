@@ -7,11 +7,7 @@
 
 namespace rumus {
 
-__device__ __forceinline__ float wave_max64(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
-    return v;
-}
+__device__ __forceinline__ float wave_max64(float v) { return wave_max(v); }
 
 __device__ __forceinline__ int q_i8(float v, float inv) {
     float t = rintf(__fmul_rn(v, inv));

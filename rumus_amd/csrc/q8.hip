@@ -10,12 +10,6 @@
 
 namespace rumus {
 
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
-    return v;
-}
-
 __device__ __forceinline__ int quant_i8(float v, float inv) {
     // quantize.wgsl:93: clamp(i32(round(v*inv)), -128, 127), round = half-even.
     float t = rintf(__fmul_rn(v, inv));
@@ -323,9 +317,7 @@ __global__ __launch_bounds__(512) void matmul_q8_rows_kernel(
     for (int cc = 0; cc < CW; cc++)
 #pragma unroll
         for (int r = 0; r < M; r++) {
-            float v = acc[cc][r];
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+            const float v = wave_sum(acc[cc][r]);
             if (lane == 0 && col0 + cc < n) c[(uint64_t)r * n + col0 + cc] = v;
         }
 }
@@ -408,8 +400,7 @@ __device__ __forceinline__ uint32_t q8_row_amax(const float* __restrict__ ar, ui
                        max(__float_as_uint(t.z) & 0x7FFFFFFFu, __float_as_uint(t.w) & 0x7FFFFFFFu));
         }
     }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) amax = max(amax, (uint32_t)__shfl_xor((int)amax, off));
+    amax = wave_max(amax);
     if ((tid & 63) == 0) red[tid >> 6] = amax;
     __syncthreads();
     return max(max(red[0], red[1]), max(red[2], red[3]));

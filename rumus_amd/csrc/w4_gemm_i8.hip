@@ -98,18 +98,6 @@ __device__ __forceinline__ int group_sum(int v) {
     return v;
 }
 
-// maximum over the 64 lanes of a wave, in every lane
-__device__ __forceinline__ uint32_t wave_max(uint32_t v) {
-    v = max(v, (uint32_t)dpp_move<kDppQuadXor1>((int)v));
-    v = max(v, (uint32_t)dpp_move<kDppQuadXor2>((int)v));
-    v = max(v, (uint32_t)dpp_move<kDppHalfMirror>((int)v));
-    v = max(v, (uint32_t)dpp_move<kDppRowMirror>((int)v));
-    const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);     // rows 0 | 1, 2 | 3
-    v = max(r[0], r[1]);
-    const auto h = __builtin_amdgcn_permlane32_swap(v, v, false, false);     // the halves
-    return max(h[0], h[1]);
-}
-
 // ---- activations -> digit planes ------------------------------------------------------------------
 // One wave per (row, share of K); a lane takes 8 consecutive k at a time: half of a lane's operand bytes of
 // one step (its even elements fill one word - a packed word's even nibbles -, its odd elements the next).

@@ -57,8 +57,7 @@ __global__ __launch_bounds__(256) void w4t_prepare_kernel(const float* __restric
         amax = max(max(amax, max(__float_as_uint(t.x) & 0x7FFFFFFFu, __float_as_uint(t.y) & 0x7FFFFFFFu)),
                    max(__float_as_uint(t.z) & 0x7FFFFFFFu, __float_as_uint(t.w) & 0x7FFFFFFFu));
     }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) amax = max(amax, (uint32_t)__shfl_xor((int)amax, off));
+    amax = wave_max(amax);
     if ((tid & 63) == 0) red[tid >> 6] = amax;
     __syncthreads();
     amax = max(max(red[0], red[1]), max(red[2], red[3]));

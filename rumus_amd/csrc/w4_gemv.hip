@@ -280,9 +280,7 @@ __global__ __launch_bounds__(256) void w4_transpose_kernel(
         for (int r = 0; r < MR; r++)
 #pragma unroll
             for (int j = 0; j < 8; j++) {
-                float v = acc[q][r][j];
-#pragma unroll
-                for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+                const float v = wave_sum(acc[q][r][j]);
                 if ((tid & 63) == 0) red[tid >> 6][q][r][j] = v;
             }
     __syncthreads();
