@@ -245,7 +245,10 @@ __global__ __launch_bounds__(256) void matmul_q8_tiled_kernel(
 // 0 stands for one run per block.
 struct __attribute__((packed, aligned(4))) Q8Words4 { uint32_t x, y, z, w; };
 
-template <int M>
+// ONCE: one block per column.  The bytes of a column are then one unbroken run behind a single header and the
+// loads carry the non-temporal hint (1 x 4096 x 11008 from HBM: 14.5 -> 13.2 us; with smaller blocks the same
+// hint costs 0.4 to 1.2 us).
+template <int M, bool ONCE>
 __global__ __launch_bounds__(512) void matmul_q8_rows_kernel(
     const float* __restrict__ a, const uint32_t* __restrict__ b, float* __restrict__ c, uint32_t k,
     uint32_t n, uint32_t stride, uint32_t blocks_per_col, uint32_t kpad, uint32_t runs_per_block,
@@ -279,7 +282,13 @@ __global__ __launch_bounds__(512) void matmul_q8_rows_kernel(
 #pragma unroll
         for (int cc = 0; cc < CW; cc++) {
             hdr[cc] = colbase[cc][off];
-            w4[cc] = *reinterpret_cast<const Q8Words4*>(colbase[cc] + off + 1 + in_blk * 4);
+            if constexpr (ONCE) {
+                typedef uint32_t q8_u4 __attribute__((ext_vector_type(4), aligned(4)));
+                const q8_u4 t = __builtin_nontemporal_load(reinterpret_cast<const q8_u4*>(colbase[cc] + off + 1 + in_blk * 4));
+                w4[cc] = Q8Words4{t.x, t.y, t.z, t.w};
+            } else {
+                w4[cc] = *reinterpret_cast<const Q8Words4*>(colbase[cc] + off + 1 + in_blk * 4);
+            }
         }
         float part[CW][M];
 #pragma unroll
@@ -327,8 +336,12 @@ static int launch_q8_rows(const float* a, const uint32_t* b, float* c, uint32_t 
                           uint32_t stride, uint32_t blocks_per_col, uint32_t kpad, hipStream_t s) {
     const uint32_t runs_per_block = bs / 16;
     const uint32_t run_magic = runs_per_block == 1 ? 0u : (uint32_t)((0x100000000ull + runs_per_block - 1) / runs_per_block);
-    hipLaunchKernelGGL(matmul_q8_rows_kernel<M>, dim3(ceil_div(n, 32)), dim3(512), (size_t)M * kpad * sizeof(float), s,
-                       a, b, c, k, n, stride, blocks_per_col, kpad, runs_per_block, run_magic);
+    if (blocks_per_col == 1)
+        hipLaunchKernelGGL((matmul_q8_rows_kernel<M, true>), dim3(ceil_div(n, 32)), dim3(512), (size_t)M * kpad * sizeof(float), s,
+                           a, b, c, k, n, stride, blocks_per_col, kpad, runs_per_block, run_magic);
+    else
+        hipLaunchKernelGGL((matmul_q8_rows_kernel<M, false>), dim3(ceil_div(n, 32)), dim3(512), (size_t)M * kpad * sizeof(float), s,
+                           a, b, c, k, n, stride, blocks_per_col, kpad, runs_per_block, run_magic);
     return check_launch("matmul_q8_rows_kernel");
 }
 
