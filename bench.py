@@ -186,8 +186,34 @@ def bench_i8_gemm(torch, ops, replays=12, warmup=3):
         vendor = ops_per / time_graph(torch, burst_vendor, per_graph, replays, warmup)["median"] / 1e12
     except Exception as exc:   # informational only
         log(f"[bench] vendor int8 GEMM not timed: {exc}")
+    # The same kernel on operands without bit activity (all ones: every product and sum is still computed, the
+    # instruction stream and the memory traffic are those of the timed run above): what the kernel's schedule
+    # reaches when the board's power management does not hold the shader clock down.  Not a throughput claim.
+    quiet = None
+    try:
+        xq1, wq1 = torch.ones_like(xq), torch.ones_like(wq)
+
+        def burst_quiet():
+            for _ in range(per_graph):
+                ops.i8_gemm(xq1, wq1, sx, sw, None, out=y)
+
+        tq = time_graph(torch, burst_quiet, per_graph, replays, warmup)["median"]
+        quiet = {"operands": "all ones", "ms_per_launch": tq * 1e3, "tops": ops_per / tq / 1e12,
+                 "frac": ops_per / tq / 1e12 / I8_PEAK_TOPS}
+        wt1 = wq1.t()
+
+        def burst_vendor_quiet():
+            for _ in range(per_graph):
+                torch._int_mm(xq1, wt1)
+
+        quiet["vendor_int_mm_tops"] = ops_per / time_graph(torch, burst_vendor_quiet, per_graph, replays, warmup)["median"] / 1e12
+        del xq1, wq1, wt1
+    except Exception as exc:   # informational only
+        log(f"[bench] constant-operand run not timed: {exc}")
     return {
         "workload": "int8_gemm_2048x4096x11008", "ms_per_launch": sec * 1e3, "tops": tops, "hip_graph": t["graph"],
+        "operands": "int8 from absmax-quantized normal samples (random bits)",
+        "same_kernel_constant_operands": quiet,
         "timing": spread(t),
         "roofline": {"bound": "mfma", "achieved": tops, "peak": I8_PEAK_TOPS, "unit": "TOP/s",
                      "frac": tops / I8_PEAK_TOPS, "traffic": None},
