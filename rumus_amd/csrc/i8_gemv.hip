@@ -115,29 +115,37 @@ int i8_launch_gemv(const int8_t* xq, const int8_t* wq, const float* sx, const fl
 // 64 of weight row c as the B operand and of activation row c as the A operand (the activations come
 // out of the caches: every wave reads all of them).  No LDS on the way in, eight K steps of loads in
 // flight per lane; the four partial 16 x 16 tiles meet in LDS at the end.  Exact i32 sums.
-template <int RT>
+// TN: column tiles of 16 per workgroup.  Every workgroup reads all of the activations, so two column tiles halve
+// that traffic per weight byte; it pays where the launch still has several workgroups per compute unit (from HBM,
+// 4096 x 22016: 16 rows 31.7 -> 27.7 us, 8 rows 26.9 -> 25.8 us; 4096 x 11008, 688 -> 344 workgroups: 15.3 -> 18.1 us).
+template <int RT, int TN>
 __global__ __launch_bounds__(256) void i8_stream_kernel(
     const int8_t* __restrict__ xq, const int8_t* __restrict__ wq, const float* __restrict__ sx,
     const float* __restrict__ sw, const float* __restrict__ bias, int32_t* __restrict__ acc_out,
     float* __restrict__ y, uint32_t M, uint32_t K, uint32_t N) {
-    __shared__ int32_t part[3][RT][4][64];                     // waves 1..3: [row tile][register][lane]
+    __shared__ int32_t part[3][RT * TN][4][64];                // waves 1..3: [row tile, column tile][register][lane]
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t c = lane & 15, q = lane >> 4;
-    const uint32_t n0 = blockIdx.x * 16;
+    const uint32_t n0 = blockIdx.x * 16 * TN;
     const uint32_t kq = K / 4;                                 // K % 256 == 0: a quarter is whole K steps of 64
-    const int8_t* bp = wq + (uint64_t)min(n0 + c, N - 1) * K + wave * kq + 16 * q;
+    const int8_t* bp[TN];
+#pragma unroll
+    for (int j = 0; j < TN; j++) bp[j] = wq + (uint64_t)min(n0 + 16 * j + c, N - 1) * K + wave * kq + 16 * q;
     const int8_t* ap[RT];
 #pragma unroll
     for (int t = 0; t < RT; t++) ap[t] = xq + (uint64_t)min(16 * t + c, M - 1) * K + wave * kq + 16 * q;
-    v4i acc[RT];
+    v4i acc[RT][TN];
 #pragma unroll
-    for (int t = 0; t < RT; t++) acc[t] = v4i{0, 0, 0, 0};
+    for (int t = 0; t < RT; t++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) acc[t][j] = v4i{0, 0, 0, 0};
     for (uint32_t k0 = 0; k0 < kq; k0 += 512) {                // 8 K steps per round, the last round maybe shorter
-        v4i b[8], a[8][RT];
+        v4i b[8][TN], a[8][RT];
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             const uint32_t kk = min(k0 + 64 * i, kq - 64);     // past the end: the last step again, not multiplied
-            b[i] = *reinterpret_cast<const v4i*>(bp + kk);
+#pragma unroll
+            for (int j = 0; j < TN; j++) b[i][j] = *reinterpret_cast<const v4i*>(bp[j] + kk);
 #pragma unroll
             for (int t = 0; t < RT; t++) a[i][t] = *reinterpret_cast<const v4i*>(ap[t] + kk);
         }
@@ -145,7 +153,10 @@ __global__ __launch_bounds__(256) void i8_stream_kernel(
         for (int i = 0; i < 8; i++) {
             if (k0 + 64 * i < kq) {
 #pragma unroll
-                for (int t = 0; t < RT; t++) acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i][t], b[i], acc[t], 0, 0, 0);
+                for (int t = 0; t < RT; t++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+                        acc[t][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i][t], b[i][j], acc[t][j], 0, 0, 0);
             }
         }
     }
@@ -153,38 +164,47 @@ __global__ __launch_bounds__(256) void i8_stream_kernel(
 #pragma unroll
         for (int t = 0; t < RT; t++)
 #pragma unroll
-            for (int r = 0; r < 4; r++) part[wave - 1][t][r][lane] = acc[t][r];
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) part[wave - 1][t * TN + j][r][lane] = acc[t][j][r];
     }
     __syncthreads();
     if (wave > 0) return;
     // register r of lane l: row 4 (l / 16) + r, column l % 16 of the 16 x 16 tile
-    const uint32_t col = n0 + c;
-    if (col >= N) return;
-    const float swc = y ? sw[col] : 0.0f, bc = (y && bias) ? bias[col] : 0.0f;
 #pragma unroll
-    for (int t = 0; t < RT; t++)
+    for (int j = 0; j < TN; j++) {
+        const uint32_t col = n0 + 16 * j + c;
+        if (col >= N) continue;
+        const float swc = y ? sw[col] : 0.0f, bc = (y && bias) ? bias[col] : 0.0f;
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const uint32_t row = 16 * t + 4 * q + r;
-            if (row >= M) continue;
-            const int32_t v = acc[t][r] + part[0][t][r][lane] + part[1][t][r][lane] + part[2][t][r][lane];
-            const uint64_t o = (uint64_t)row * N + col;
-            if (acc_out) acc_out[o] = v;
-            if (y) {
-                float f = __fmul_rn(__fmul_rn((float)v, sx[row]), swc);
-                if (bias) f = __fadd_rn(f, bc);
-                y[o] = f;
+        for (int t = 0; t < RT; t++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const uint32_t row = 16 * t + 4 * q + r;
+                if (row >= M) continue;
+                const int u = t * TN + j;
+                const int32_t v = acc[t][j][r] + part[0][u][r][lane] + part[1][u][r][lane] + part[2][u][r][lane];
+                const uint64_t o = (uint64_t)row * N + col;
+                if (acc_out) acc_out[o] = v;
+                if (y) {
+                    float f = __fmul_rn(__fmul_rn((float)v, sx[row]), swc);
+                    if (bias) f = __fadd_rn(f, bc);
+                    y[o] = f;
+                }
             }
-        }
+    }
 }
 
 // 5 <= m <= 32, k % 256 == 0, 16-byte aligned operands
 int i8_launch_stream(const int8_t* xq, const int8_t* wq, const float* sx, const float* sw, const float* bias, int32_t* acc,
                      float* y, uint32_t m, uint32_t k, uint32_t n, hipStream_t s) {
-    if (m <= 16)
-        hipLaunchKernelGGL(i8_stream_kernel<1>, dim3(ceil_div(n, 16)), dim3(256), 0, s, xq, wq, sx, sw, bias, acc, y, m, k, n);
+    const bool two = m >= 8 && m <= 16 && ceil_div(n, 16) >= 1280;    // five workgroups per compute unit or more
+    if (two)
+        hipLaunchKernelGGL((i8_stream_kernel<1, 2>), dim3(ceil_div(n, 32)), dim3(256), 0, s, xq, wq, sx, sw, bias, acc, y, m, k, n);
+    else if (m <= 16)
+        hipLaunchKernelGGL((i8_stream_kernel<1, 1>), dim3(ceil_div(n, 16)), dim3(256), 0, s, xq, wq, sx, sw, bias, acc, y, m, k, n);
     else
-        hipLaunchKernelGGL(i8_stream_kernel<2>, dim3(ceil_div(n, 16)), dim3(256), 0, s, xq, wq, sx, sw, bias, acc, y, m, k, n);
+        hipLaunchKernelGGL((i8_stream_kernel<2, 1>), dim3(ceil_div(n, 16)), dim3(256), 0, s, xq, wq, sx, sw, bias, acc, y, m, k, n);
     return check_launch("i8_stream_kernel");
 }
 

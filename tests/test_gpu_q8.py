@@ -323,6 +323,7 @@ def test_i8_quantize_cols_t_bit_exact(ops, k, n):
                                    (6, 4096, 64), (128, 1088, 70),   # 17 K steps in two shares of 9 and 8
                                    # 5 to 32 rows, K % 256 == 0: MFMA tiles fed straight from global memory
                                    (5, 256, 16), (16, 1024, 100), (17, 1024, 40), (32, 2816, 70), (9, 11008, 30),
+                                   (12, 256, 20490), (8, 512, 22016),   # the same with two column tiles per workgroup
                                    # up to 4 rows: the dot4 decode kernel
                                    (1, 4096, 1100), (2, 11008, 130), (3, 5008, 67), (4, 4096, 260), (4, 48, 5),
                                    (5, 576, 200),             # 9 steps: a single share
