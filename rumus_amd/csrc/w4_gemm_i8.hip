@@ -304,6 +304,15 @@ __global__ __launch_bounds__(512) void w4_gemm_i8_kernel(W4I8Args a) {
         if (ZP4) mzp[slot][0] = a.zp4[(uint64_t)g * (a.n / 8) + colc / 8];
         else load_q<Q>(reinterpret_cast<const uint32_t*>(a.zp) + (uint64_t)g * a.n + colc, mzp[slot]);
     };
+    // A lane of a row past m reads the last real row's fragment instead of its own zeros (the same address as
+    // that row's lane: no extra traffic); what it computes is never stored.  With 8 of a tile's 16 rows real the
+    // planes cost half the bytes out of L2.
+    uint32_t a_lane[RT];
+#pragma unroll
+    for (int t = 0; t < RT; t++) {
+        const uint32_t first = (rb * RT + t) * 16, real = a.m > first ? min(a.m - first, 16u) : 1u;
+        a_lane[t] = (b * 16 + min(c, real - 1)) * 16;
+    }
     v4i afr[2][CS][3];
     auto fetch_a = [&](int slot, uint32_t chunk, uint32_t rt) {
         const uint32_t fc = min(chunk, flast), rtg = rb * RT + rt;
@@ -312,7 +321,7 @@ __global__ __launch_bounds__(512) void w4_gemm_i8_kernel(W4I8Args a) {
 #pragma unroll
             for (int p = 0; p < 3; p++)
                 afr[slot][s][p] = *reinterpret_cast<const v4i*>(
-                    a.planes + (((uint64_t)rtg * a.steps + fc * CS + s) * 3 + p) * 1024 + lane * 16);
+                    a.planes + (((uint64_t)rtg * a.steps + fc * CS + s) * 3 + p) * 1024 + a_lane[rt]);
     };
 
     v4f accf[RT][Q];
