@@ -263,6 +263,28 @@ def probe_mfma_ceiling():
     return {"tops": tops.value, "shader_mhz": mhz.value}
 
 
+def probe_f16_mfma_ceiling():
+    """f16 TFLOP/s of v_mfma_f32_32x32x16_f16 issued back to back from registers (bench/probe_mfma.hip): with
+    random f16 operands, with random activations against small-integer weights (what the W4 kernels multiply),
+    and with ones; or None."""
+    import ctypes
+    path = os.path.join(ROOT, "bench", "librumus_probe.so")
+    if not os.path.exists(path):
+        return None
+    lib = ctypes.CDLL(path)
+    if not hasattr(lib, "rumus_probe_f16_mfma"):
+        return None
+    lib.rumus_probe_f16_mfma.restype = ctypes.c_int
+    lib.rumus_probe_f16_mfma.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
+    out = {}
+    for name, mode in (("random_operands", 1), ("random_times_nibbles", 2), ("ones", 0)):
+        tf, mhz = ctypes.c_double(), ctypes.c_double()
+        if lib.rumus_probe_f16_mfma(mode, ctypes.byref(tf), ctypes.byref(mhz)) != 0:
+            return None
+        out[name] = {"tflops": tf.value, "shader_mhz": mhz.value}
+    return out
+
+
 def bench_gemv_shapes(torch, ops, replays=10, warmup=2):
     """The same decode kernel on the wider projections of a Llama-7B block (q|k|v, gate|up, down),
     each rotating over enough weight sets (> 600 MB) to defeat the Infinity Cache.  The longer a
@@ -683,6 +705,7 @@ def main():
         out["w4_gemv_wider"] = bench_gemv_shapes(torch, ops)
         out["w4_gemm"] = [bench_w4_gemm(torch, ops, 16), bench_w4_gemm(torch, ops, 128),
                           bench_w4_gemm(torch, ops, 1024), bench_w4_gemm(torch, ops, 2048)]
+        out["f16_mfma_only"] = probe_f16_mfma_ceiling()
         out["q8_matmul"] = bench_q8_matmul(torch, ops)
         out["w4_grad_x"] = bench_grad_x(torch, ops)
         out["int8_decode"] = bench_i8_small(torch, ops)

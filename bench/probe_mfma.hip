@@ -80,6 +80,81 @@ extern "C" int rumus_probe_i8_mfma(int random_bits, double* tops, double* mhz) {
     return 0;
 }
 
+// The same for the f16 matrix instruction of the W4 GEMM kernels, v_mfma_f32_32x32x16_f16.  random_bits = 1: both
+// operands random f16 values of magnitude 2^-3 .. 2^4 (random sign and mantissa); 2: A random like that, B small
+// integers 0..15 (what a packed nibble becomes); 0: ones.
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+__global__ __launch_bounds__(256) void probe_f16_mfma_kernel(float* out, long long* ticks, int iters, int random_bits) {
+    v8h a, b;
+    for (int q = 0; q < 8; q++) { a[q] = (_Float16)1.0f; b[q] = (_Float16)1.0f; }
+    if (random_bits) {
+        const uint32_t t = threadIdx.x * 977u + blockIdx.x * 131071u;
+        for (int q = 0; q < 8; q++) {
+            const uint32_t ra = mix(t + q), rb = mix(t + 29 + q);
+            // sign | exponent 12..19 (2^-3 .. 2^4) | 10 mantissa bits
+            const uint16_t ha = (uint16_t)(((ra >> 16) & 0x8000u) | ((12u + (ra & 7u)) << 10) | ((ra >> 3) & 0x3ffu));
+            const uint16_t hb = (uint16_t)(((rb >> 16) & 0x8000u) | ((12u + (rb & 7u)) << 10) | ((rb >> 3) & 0x3ffu));
+            a[q] = __builtin_bit_cast(_Float16, ha);
+            b[q] = random_bits == 2 ? (_Float16)(float)(rb & 15u) : __builtin_bit_cast(_Float16, hb);
+        }
+    }
+    v16f c0 = {0}, c1 = {0}, c2 = {0}, c3 = {0};
+    const long long t0 = clock64(), w0 = wall_clock64();
+    for (int i = 0; i < iters; i++) {
+        c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c0, 0, 0, 0);
+        c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c1, 0, 0, 0);
+        c2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c2, 0, 0, 0);
+        c3 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c3, 0, 0, 0);
+    }
+    const long long t1 = clock64(), w1 = wall_clock64();
+    if (threadIdx.x == 0 && blockIdx.x == 0) { ticks[0] = t1 - t0; ticks[1] = w1 - w0; }
+    float s = 0;
+    for (int r = 0; r < 16; r++) s += c0[r] + c1[r] + c2[r] + c3[r];
+    out[blockIdx.x * 256 + threadIdx.x] = s;
+}
+
+// Returns 0 on success.  tflops: f16 TFLOP/s over the whole device (2 flop per multiply-add); mhz as above.
+extern "C" int rumus_probe_f16_mfma(int random_bits, double* tflops, double* mhz) {
+    hipDeviceProp_t prop;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 1;
+    const int wgs = prop.multiProcessorCount * 2;      // 8 waves per CU, 2 per SIMD
+    const int iters = 20000;
+    float* out = nullptr;
+    long long* ticks = nullptr;
+    if (hipMalloc(&out, (size_t)wgs * 256 * 4) != hipSuccess) return 1;
+    if (hipMalloc(&ticks, 16) != hipSuccess) { (void)hipFree(out); return 1; }
+    hipEvent_t e0, e1;
+    (void)hipEventCreate(&e0);
+    (void)hipEventCreate(&e1);
+    float best_ms = 1e30f;
+    long long h[2] = {0, 1};
+    for (int rep = 0; rep < 4; rep++) {                 // the first run ramps the clock
+        (void)hipEventRecord(e0, 0);
+        hipLaunchKernelGGL(probe_f16_mfma_kernel, dim3(wgs), dim3(256), 0, 0, out, ticks, iters, random_bits);
+        (void)hipEventRecord(e1, 0);
+        if (hipEventSynchronize(e1) != hipSuccess) { best_ms = -1; break; }
+        float ms = 0;
+        (void)hipEventElapsedTime(&ms, e0, e1);
+        if (rep > 0 && ms < best_ms) {
+            best_ms = ms;
+            (void)hipMemcpy(h, ticks, 16, hipMemcpyDeviceToHost);
+        }
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    (void)hipFree(out);
+    (void)hipFree(ticks);
+    if (best_ms <= 0) return 1;
+    // 4 waves per workgroup, 4 MFMAs per iteration, 32*32*16 multiply-adds each
+    const double flop = (double)wgs * 4 * iters * 4 * 2.0 * 16384.0;
+    *tflops = flop / (best_ms * 1e-3) / 1e12;
+    *mhz = (double)h[0] / (double)h[1] * 100.0;
+    return 0;
+}
+
 // ---- what one small memory-bound launch can reach -----------------------------------------
 // A kernel that only reads `bytes` (64 bytes per thread, four 128-bit loads issued at once,
 // one XCD-contiguous slab per workgroup) and folds them into a value it never stores, launched
