@@ -88,9 +88,11 @@ extern "C" int rumus_dbg_d8_stamps(unsigned long long* host, size_t count) {
 #define D8_STAMP(i, after)
 #endif
 
-// Kernel arguments are passed flat, hottest first: the first 16 dwords are
-// preloaded into SGPRs by the command processor (see the build flags), which
-// takes the kernel-argument fetch off the critical path.
+// Kernel arguments are passed flat.  This file is built with the first two
+// arguments (the pointers to the packed words and the scales) preloaded into
+// SGPRs at wave launch and the rest fetched by the wave: preloading more
+// slows the launch of each of the 2048 waves by more than the fetch costs
+// (the numbers are with the build flags).
 //
 // T threads = T/4 quads; a quad owns OCT consecutive word rows per sweep and
 // each of its lanes prepares OPL = OCT/4 of them.  FASTX: activations are
