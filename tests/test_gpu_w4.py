@@ -520,7 +520,9 @@ def test_decode_layout_is_bit_identical(ops, m, k, n, g):
         np.testing.assert_array_equal(got, host(ops.qmatmul_int4(dev(x), *d, k, g, bias=dev(b))))
 
 
-@pytest.mark.parametrize("m,k,n,g", [(1, 4096, 4096, 128), (3, 1000, 48, 64), (8, 512, 11008, 32), (5, 256, 16, 256)])
+@pytest.mark.parametrize("m,k,n,g", [(1, 4096, 4096, 128), (3, 1000, 48, 64), (8, 512, 11008, 32), (5, 256, 16, 256),
+                                     # one row: 256-thread workgroups, 64 rows per quad (groups of 64 and up)
+                                     (1, 1000, 48, 64), (1, 11008, 272, 128), (1, 520, 16, 256), (1, 512, 64, 32)])
 def test_decode_layout_u4_zero_points(ops, m, k, n, g):
     say(f"qmatmul_int4_decode_zp4 m={m} k={k} n={n} g={g}")
     rng = np.random.default_rng(m + k + n + 1)
@@ -536,7 +538,9 @@ def test_decode_layout_u4_zero_points(ops, m, k, n, g):
     got = host(ops.qmatmul_int4_decode_zp4(dev(x), pt, st, qt, k, g, bias=dev(b)))
     zp = oracle.w4_qzeros_unpack(qzeros, n)
     assert_close(got, oracle.qmatmul_int4(x, packed, scales, zp, k, g, bias=b, threads=8))
-    if m <= ops.qmatmul_int4_decode_max_rows(packed.shape[0] * 8, n):   # the row-major entry point runs the same kernel arithmetic then
+    # the row-major entry point runs the same kernel arithmetic then (one row on groups of 64 and up takes 64 rows
+    # per quad on the tile-major copy: another fixed-point scale per chunk, so close but not the same bits)
+    if m <= ops.qmatmul_int4_decode_max_rows(packed.shape[0] * 8, n) and not (m == 1 and g % 64 == 0):
         np.testing.assert_array_equal(got, host(ops.qmatmul_int4_zp4(dev(x), *d, k, g, bias=dev(b))))
     # act-order on top
     if k % g == 0:
