@@ -292,6 +292,98 @@ __global__ __launch_bounds__(256) void w4_transpose_kernel(
     }
 }
 
+// The same product for a few rows on vector loads (n % 4 == 0, 16-byte aligned arrays, KR word rows inside one
+// group): out[m, k] = sum_n t[m, n] q[k, n] - sum_n t[m, n] zp[g, n] with t = a * scale[g], so the scale and the
+// zero-point are applied once per column and row of a instead of once per nibble, a nibble costs one byte-to-float
+// conversion and one multiply-add, and every thread reads four columns per load.  4096 x 11008 from HBM: one row
+// 17.3 -> 11.9 us, four rows 57 -> 19.5 us against the scalar-load kernel above, which remains for other shapes.
+template <int MR, int KR>
+__global__ __launch_bounds__(256) void w4_transpose_vec_kernel(
+    const float* __restrict__ a, const uint32_t* __restrict__ packed,
+    const float* __restrict__ scales, const float* __restrict__ zp, float* __restrict__ out,
+    uint32_t m, uint32_t k, uint32_t n, uint32_t gs, uint32_t word_rows) {
+    __shared__ float red[4][MR][KR * 8 + 1];
+    const uint32_t kr0 = blockIdx.x * KR, row0 = blockIdx.y * MR, tid = threadIdx.x;
+    const uint32_t nv = n / 4, g = (kr0 * 8) / gs;
+    const float4* a4 = reinterpret_cast<const float4*>(a);
+    const float4* sc4 = reinterpret_cast<const float4*>(scales) + (uint64_t)g * nv;
+    const float4* zp4 = reinterpret_cast<const float4*>(zp) + (uint64_t)g * nv;
+    const uint4* w4[KR];
+#pragma unroll
+    for (int q = 0; q < KR; q++)            // past the end: the last row again, not stored
+        w4[q] = reinterpret_cast<const uint4*>(packed) + (uint64_t)min(kr0 + q, word_rows - 1) * nv;
+    float acc[MR][KR][8], u[MR];
+#pragma unroll
+    for (int r = 0; r < MR; r++) {
+        u[r] = 0.0f;
+#pragma unroll
+        for (int q = 0; q < KR; q++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) acc[r][q][j] = 0.0f;
+    }
+#pragma unroll 2
+    for (uint32_t v = tid; v < nv; v += 256) {
+        const float4 s4 = sc4[v], z4 = zp4[v];
+        uint4 w[KR];
+#pragma unroll
+        for (int q = 0; q < KR; q++) w[q] = w4[q][v];
+        float4 av[MR];
+#pragma unroll
+        for (int r = 0; r < MR; r++) {
+            av[r] = a4[(uint64_t)min(row0 + r, m - 1) * nv + v];
+            if (row0 + r >= m) av[r] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
+        const float sc[4] = {s4.x, s4.y, s4.z, s4.w}, z[4] = {z4.x, z4.y, z4.z, z4.w};
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            float t[MR];
+#pragma unroll
+            for (int r = 0; r < MR; r++) {
+                const float ar = c == 0 ? av[r].x : c == 1 ? av[r].y : c == 2 ? av[r].z : av[r].w;
+                t[r] = ar * sc[c];
+                u[r] = fmaf(t[r], z[c], u[r]);
+            }
+#pragma unroll
+            for (int q = 0; q < KR; q++) {
+                const uint32_t word = c == 0 ? w[q].x : c == 1 ? w[q].y : c == 2 ? w[q].z : w[q].w;
+                const uint32_t lo = word & 0x0f0f0f0fu, hi = (word >> 4) & 0x0f0f0f0fu;   // nibbles 0,2,4,6 | 1,3,5,7
+                // (float)((x >> 8 i) & 0xff) is one v_cvt_f32_ubyte<i>
+                const float f[8] = {(float)(lo & 0xffu), (float)(hi & 0xffu),
+                                    (float)((lo >> 8) & 0xffu), (float)((hi >> 8) & 0xffu),
+                                    (float)((lo >> 16) & 0xffu), (float)((hi >> 16) & 0xffu),
+                                    (float)(lo >> 24), (float)(hi >> 24)};
+#pragma unroll
+                for (int j = 0; j < 8; j++)
+#pragma unroll
+                    for (int r = 0; r < MR; r++) acc[r][q][j] = fmaf(t[r], f[j], acc[r][q][j]);
+            }
+        }
+    }
+    const uint32_t wave = tid >> 6;
+#pragma unroll
+    for (int r = 0; r < MR; r++) {
+#pragma unroll
+        for (int q = 0; q < KR; q++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const float s = wave_sum(acc[r][q][j]);
+                if ((tid & 63) == 0) red[wave][r][q * 8 + j] = s;
+            }
+        const float su = wave_sum(u[r]);
+        if ((tid & 63) == 0) red[wave][r][KR * 8] = su;
+    }
+    __syncthreads();
+    for (uint32_t e = tid; e < MR * KR * 8; e += 256) {
+        const uint32_t r = e / (KR * 8), i = e % (KR * 8);
+        const uint32_t kk = kr0 * 8 + i;
+        if (row0 + r < m && kk < k && kr0 + i / 8 < word_rows) {
+            const float dot = (red[0][r][i] + red[1][r][i]) + (red[2][r][i] + red[3][r][i]);
+            const float zs = (red[0][r][KR * 8] + red[1][r][KR * 8]) + (red[2][r][KR * 8] + red[3][r][KR * 8]);
+            out[(uint64_t)(row0 + r) * k + kk] = dot - zs;
+        }
+    }
+}
+
 static int validate(const W4Args& a, const char* who) {
     RUMUS_REQUIRE(a.group_size > 0 && a.group_size % 8 == 0,
                   "%s: group_size must be a multiple of 8 (got %u)", who, a.group_size);
@@ -491,16 +583,38 @@ int rumus_hip_qmatmul_int4_t(const float* a, const uint32_t* packed, const float
     W4Args v{a, packed, scales, zero_points, nullptr, nullptr, nullptr, out, m, k, n, padded_k, group_size, num_groups};
     if (int rc = validate(v, "qmatmul_int4_t")) return rc;
     if (m == 0 || k == 0) return RUMUS_HIP_OK;
-    // tile of a workgroup: 4 rows x 32 outputs from 3 rows on (each value of a is then read once per
-    // 32 outputs, each word once per 4 rows); single rows keep one word row per workgroup for
-    // the sake of parallelism
     hipStream_t s = as_stream(stream);
-    // where the matrix-core kernel is ahead of the one below (4096 x 11008: 45 us for up to 64 rows with groups
-    // of 128, 85 us with 64, 176 us with 32, against 67 us per 8 rows)
-    const uint32_t mfma_from = group_size % 128 == 0 ? 8 : group_size == 64 ? 12 : 24;
+    // where the matrix-core kernel is ahead of the vector kernel below, which takes four rows per pass (from HBM,
+    // us, vector at 8 / 12 / 16 / 24 / 32 / 48 rows against the matrix cores at any of them: 4096 x 11008 g128
+    // 30 / 31 / 40 / 53 / 65 / 97 against 49-51, g64 against 59-61, g32 against 105-110; 11008 x 4096 32 / 39 / 46 / 65 /
+    // 83 / 120 against 37-42, 56-60, 139-143; 4096 x 4096 17 / 15 / 20 / 26 / 33 / 46 against 31-34, 38-41, 45-50)
+    const uint32_t mfma_from = group_size % 128 == 0 ? 13 : group_size == 64 ? 21 : 49;
     if (m >= mfma_from && w4_gemm_t_supported(m, k, n, group_size, a, packed, scales, zero_points, out))
         return w4_launch_gemm_t(a, packed, scales, zero_points, out, m, k, n, padded_k, group_size, num_groups, s);
     const uint32_t word_rows = padded_k / 8;
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(packed) |
+                           reinterpret_cast<uintptr_t>(scales) | reinterpret_cast<uintptr_t>(zero_points);
+    if (n % 4 == 0 && (bits & 15) == 0 && group_size % 16 == 0) {
+        // two word rows per workgroup (they share scale and zero-point), one while that leaves fewer than 256 workgroups
+        const bool two = word_rows >= 512;
+        const uint32_t mr = m <= 2 ? m : 4;           // rows per pass (eight at once: 34 us against 26 in two passes)
+        const dim3 grid(two ? ceil_div(word_rows, 2) : word_rows, ceil_div(m, mr));
+#define RUMUS_W4T_VEC(MR)                                                                                              \
+        do {                                                                                                           \
+            if (two) hipLaunchKernelGGL((w4_transpose_vec_kernel<MR, 2>), grid, dim3(256), 0, s, a, packed, scales,    \
+                                        zero_points, out, m, k, n, group_size, word_rows);                             \
+            else hipLaunchKernelGGL((w4_transpose_vec_kernel<MR, 1>), grid, dim3(256), 0, s, a, packed, scales,        \
+                                    zero_points, out, m, k, n, group_size, word_rows);                                 \
+        } while (0)
+        if (mr == 1) RUMUS_W4T_VEC(1);
+        else if (mr == 2) RUMUS_W4T_VEC(2);
+        else RUMUS_W4T_VEC(4);
+#undef RUMUS_W4T_VEC
+        return check_launch("w4_transpose_vec_kernel");
+    }
+    // other shapes (n % 4 != 0, unaligned arrays, odd group sizes): 4 rows x 32 outputs per workgroup from 3 rows on
+    // (each value of a is then read once per 32 outputs, each word once per 4 rows); single rows keep one word
+    // row per workgroup for the sake of parallelism
     if (m >= 3)
         hipLaunchKernelGGL((w4_transpose_kernel<4, 4>), dim3(ceil_div(word_rows, 4), ceil_div(m, 4)), dim3(256), 0, s, a,
                            packed, scales, zero_points, out, m, k, n, group_size, word_rows);

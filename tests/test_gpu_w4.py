@@ -282,7 +282,10 @@ def test_act_order_rejects_unbalanced_groups(ops):
                                      (40, 512, 300, 64),        # groups of 64: two waves per workgroup
                                      (70, 256, 132, 32),        # groups of 32: one
                                      (300, 200, 64, 32),        # k ends inside a group of 32
-                                     (9, 96, 40, 16)])          # other group sizes keep the vector kernel
+                                     (9, 96, 40, 16),           # other group sizes: the vector kernel, four rows per pass
+                                     (1, 4096, 1100, 128), (2, 1000, 68, 64), (4, 11008, 260, 128),   # two word rows per workgroup
+                                     (7, 520, 36, 32), (12, 4104, 64, 128),   # k ends inside the last word row pair
+                                     (5, 72, 22, 8), (3, 256, 50, 128)])    # n % 4 != 0, groups of 8: scalar loads
 def test_qmatmul_int4_transpose(ops, m, k, n, g):
     say(f"qmatmul_int4_t m={m} k={k} n={n} g={g}")
     rng = np.random.default_rng(k + n)
@@ -328,6 +331,16 @@ def test_qmatmul_int4_transpose_scaling_and_non_finite_rows(ops):
         out = host(ops.qmatmul_int4_t(dev(gb), *d, k, g))
         assert np.isnan(out[9]).all()
         np.testing.assert_array_equal(np.delete(out, 9, axis=0), np.delete(got, 9, axis=0))
+    # the same rows, few enough for the vector kernel (scale and zero-point applied per column: sum t q - sum t zp)
+    few = host(ops.qmatmul_int4_t(dev(gy[:6]), *d, k, g))
+    assert (np.abs(few - exact[:6]) / terms[:6]).max() < 2e-6
+    np.testing.assert_array_equal(few[4], np.zeros(k, np.float32))
+    for bad in (np.float32(np.nan), np.float32(np.inf)):
+        gb = gy[:6].copy()
+        gb[2, 33] = bad
+        out = host(ops.qmatmul_int4_t(dev(gb), *d, k, g))
+        assert np.isnan(out[2]).all()
+        np.testing.assert_array_equal(np.delete(out, 2, axis=0), np.delete(few, 2, axis=0))
 
 
 def test_gptq_actorder_config_full_size(ops):
