@@ -296,7 +296,7 @@ __global__ __launch_bounds__(256) void w4_transpose_kernel(
 // group): out[m, k] = sum_n t[m, n] q[k, n] - sum_n t[m, n] zp[g, n] with t = a * scale[g], so the scale and the
 // zero-point are applied once per column and row of a instead of once per nibble, a nibble costs one byte-to-float
 // conversion and one multiply-add, and every thread reads four columns per load.  4096 x 11008 from HBM: one row
-// 17.3 -> 11.9 us, four rows 57 -> 19.5 us against the scalar-load kernel above, which remains for other shapes.
+// 17.3 -> 11.2 us, four rows 57 -> 16.7 us against the scalar-load kernel above, which remains for other shapes.
 template <int MR, int KR>
 __global__ __launch_bounds__(256) void w4_transpose_vec_kernel(
     const float* __restrict__ a, const uint32_t* __restrict__ packed,
@@ -595,9 +595,11 @@ int rumus_hip_qmatmul_int4_t(const float* a, const uint32_t* packed, const float
     const uintptr_t bits = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(packed) |
                            reinterpret_cast<uintptr_t>(scales) | reinterpret_cast<uintptr_t>(zero_points);
     if (n % 4 == 0 && (bits & 15) == 0 && group_size % 16 == 0) {
-        // two word rows per workgroup (they share scale and zero-point), one while that leaves fewer than 256 workgroups
-        const bool two = word_rows >= 512;
         const uint32_t mr = m <= 2 ? m : 4;           // rows per pass (eight at once: 34 us against 26 in two passes)
+        // two word rows per workgroup (they share scale and zero-point) once the passes over the rows multiply the
+        // workgroups; a single pass wants the workgroups (4096 x 11008: 4 rows 19.9 -> 16.7 us with one word row
+        // each, 8 rows 22.7 -> 25.4 us)
+        const bool two = m > 4 && word_rows >= 512;
         const dim3 grid(two ? ceil_div(word_rows, 2) : word_rows, ceil_div(m, mr));
 #define RUMUS_W4T_VEC(MR)                                                                                              \
         do {                                                                                                           \
