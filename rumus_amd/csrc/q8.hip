@@ -259,26 +259,18 @@ __global__ __launch_bounds__(512) void matmul_q8_rows_kernel(
     extern __shared__ float xs[];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t nruns = kpad / 16;
-    for (uint32_t r = 0; r < M; r++)
-        for (uint32_t kk = tid; kk < kpad; kk += 512)
-            xs[((r * 4 + (kk % 16) / 4) * nruns + kk / 16) * 4 + kk % 4] = kk < k ? a[(uint64_t)r * k + kk] : 0.0f;
-    __syncthreads();
     const uint32_t col0 = blockIdx.x * 32 + wave * CW;
     const uint32_t* colbase[CW];
 #pragma unroll
     for (int cc = 0; cc < CW; cc++)
         colbase[cc] = b + (uint64_t)min(col0 + cc, n - 1) * blocks_per_col * stride;   // past n: re-reads the last column
-    float acc[CW][M];
-#pragma unroll
-    for (int cc = 0; cc < CW; cc++)
-#pragma unroll
-        for (int r = 0; r < M; r++) acc[cc][r] = 0.0f;
-    for (uint32_t run = lane; run < nruns; run += 64) {
-        const uint32_t blk = run_magic ? __umulhi(run, run_magic) : run;   // magic 0: one run per block
-        const uint32_t in_blk = run - blk * runs_per_block;
+    // Weights of one run (16 k) of the wave's four columns.  Branch-free: a run past the end reads the last one
+    // again (and is not multiplied), so that no wait for memory sits at the end of a branch.
+    auto fetch = [&](uint32_t run, Q8Words4 (&w4)[CW], uint32_t (&hdr)[CW]) {
+        const uint32_t rc = min(run, nruns - 1);
+        const uint32_t blk = run_magic ? __umulhi(rc, run_magic) : rc;   // magic 0: one run per block
+        const uint32_t in_blk = rc - blk * runs_per_block;
         const uint32_t off = blk * stride;                   // header word of the block; data follows
-        Q8Words4 w4[CW];
-        uint32_t hdr[CW];
 #pragma unroll
         for (int cc = 0; cc < CW; cc++) {
             hdr[cc] = colbase[cc][off];
@@ -290,6 +282,27 @@ __global__ __launch_bounds__(512) void matmul_q8_rows_kernel(
                 w4[cc] = *reinterpret_cast<const Q8Words4*>(colbase[cc] + off + 1 + in_blk * 4);
             }
         }
+    };
+    // Blocks smaller than a column: the first two runs of every lane are on their way while the activations are
+    // staged, and two stay in flight (1 x 4096 x 11008 from HBM, blocks of 32: 16.8 -> 16.0 us, of 128: 16.1 -> 15.4).
+    // One block per column streams with the non-temporal hint and is faster in the plain loop (13.3 against 14.9 us).
+    Q8Words4 wa[CW], wb[CW];
+    uint32_t ha[CW], hb[CW];
+    if constexpr (!ONCE) {
+        fetch(lane, wa, ha);
+        fetch(lane + 64, wb, hb);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    for (uint32_t r = 0; r < M; r++)
+        for (uint32_t kk = tid; kk < kpad; kk += 512)
+            xs[((r * 4 + (kk % 16) / 4) * nruns + kk / 16) * 4 + kk % 4] = kk < k ? a[(uint64_t)r * k + kk] : 0.0f;
+    __syncthreads();
+    float acc[CW][M];
+#pragma unroll
+    for (int cc = 0; cc < CW; cc++)
+#pragma unroll
+        for (int r = 0; r < M; r++) acc[cc][r] = 0.0f;
+    auto multiply = [&](uint32_t run, const Q8Words4 (&w4)[CW], const uint32_t (&hdr)[CW]) {
         float part[CW][M];
 #pragma unroll
         for (int cc = 0; cc < CW; cc++)
@@ -321,6 +334,29 @@ __global__ __launch_bounds__(512) void matmul_q8_rows_kernel(
 #pragma unroll
             for (int r = 0; r < M; r++) acc[cc][r] = fmaf(part[cc][r], sc, acc[cc][r]);
         }
+    };
+    if constexpr (ONCE) {
+        for (uint32_t run = lane; run < nruns; run += 64) {
+            fetch(run, wa, ha);
+            multiply(run, wa, ha);
+        }
+    }
+    // two runs per lane in flight: the slot just multiplied is refilled two runs ahead
+    for (uint32_t run = lane; !ONCE && run < nruns; run += 128) {
+        Q8Words4 w0[CW];
+        uint32_t h0[CW];
+#pragma unroll
+        for (int cc = 0; cc < CW; cc++) { w0[cc] = wa[cc]; h0[cc] = ha[cc]; }
+        fetch(run + 128, wa, ha);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(run, w0, h0);
+        Q8Words4 w1[CW];
+        uint32_t h1[CW];
+#pragma unroll
+        for (int cc = 0; cc < CW; cc++) { w1[cc] = wb[cc]; h1[cc] = hb[cc]; }
+        fetch(run + 192, wb, hb);                            // outside the branch: a load under one is waited for at its end
+        __builtin_amdgcn_sched_barrier(0);
+        if (run + 64 < nruns) multiply(run + 64, w1, h1);
     }
 #pragma unroll
     for (int cc = 0; cc < CW; cc++)
