@@ -322,7 +322,9 @@ uint32_t rumus_hip_qmatmul_int4_decode_max_rows(uint32_t padded_k, uint32_t n);
  * rumus_hip_w4_decode_layout; qzeros_t[(c*num_groups + g)*2 + h] =
  * qzeros[g*(n/8) + 2*c + h], the two zero-point words of tile c's 16 columns.
  * Same bits as rumus_hip_qmatmul_int4_zp4 on the row-major arrays while m is
- * within rumus_hip_qmatmul_int4_decode_max_rows.
+ * within rumus_hip_qmatmul_int4_decode_max_rows, except for one row with
+ * group_size % 64 == 0: that case fixes the point of x per 64 rows instead of
+ * 32 here (same tolerance, other bits).
  * EINVAL as for the f32 zero-point forms.  No counterpart in the reference. */
 int rumus_hip_w4_decode_layout_zp4(const uint32_t* packed, const float* scales,
                                    const uint32_t* qzeros, uint32_t padded_k, uint32_t n,
