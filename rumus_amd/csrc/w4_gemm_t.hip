@@ -50,13 +50,29 @@ __global__ __launch_bounds__(256) void w4t_prepare_kernel(const float* __restric
     const uint32_t tid = threadIdx.x;
     const bool is_row = blockIdx.x < m;
     const float* r = is_row ? gy + (uint64_t)blockIdx.x * n : scales + (uint64_t)(blockIdx.x - m) * n;   // n % 4 == 0, aligned
-    uint32_t amax = 0;
-#pragma unroll 4
-    for (uint32_t j = 4 * tid; j < n; j += 1024) {
-        const float4 t = *reinterpret_cast<const float4*>(r + j);
-        amax = max(max(amax, max(__float_as_uint(t.x) & 0x7FFFFFFFu, __float_as_uint(t.y) & 0x7FFFFFFFu)),
-                   max(__float_as_uint(t.z) & 0x7FFFFFFFu, __float_as_uint(t.w) & 0x7FFFFFFFu));
+    // The first kPrepCache steps of a thread (n up to 12288) stay in registers between the pass that finds the maximum
+    // and the pass that writes the tables, and the zero-points are asked for together with them: one trip to memory
+    // instead of one per four steps and pass.
+    constexpr int kPrepCache = 12;
+    const uint32_t g = is_row ? 0 : blockIdx.x - m;
+    const float* zr = zp + (uint64_t)g * n;
+    float4 cs[kPrepCache], cz[kPrepCache];
+#pragma unroll
+    for (int i = 0; i < kPrepCache; i++) {
+        const uint32_t j = min(4 * tid + 1024 * i, n - 4);      // clamped: no load under a branch
+        cs[i] = *reinterpret_cast<const float4*>(r + j);
+        cz[i] = *reinterpret_cast<const float4*>(zr + j);       // a row's workgroup reads group 0's and drops them
     }
+    auto max4 = [](uint32_t a, const float4& t) {
+        return max(max(a, max(__float_as_uint(t.x) & 0x7FFFFFFFu, __float_as_uint(t.y) & 0x7FFFFFFFu)),
+                   max(__float_as_uint(t.z) & 0x7FFFFFFFu, __float_as_uint(t.w) & 0x7FFFFFFFu));
+    };
+    uint32_t amax = 0;
+#pragma unroll
+    for (int i = 0; i < kPrepCache; i++)
+        if (4 * tid + 1024 * i < n) amax = max4(amax, cs[i]);
+#pragma unroll 4
+    for (uint32_t j = 4 * tid + 1024 * kPrepCache; j < n; j += 1024) amax = max4(amax, *reinterpret_cast<const float4*>(r + j));
     amax = wave_max(amax);
     if ((tid & 63) == 0) red[tid >> 6] = amax;
     __syncthreads();
@@ -67,16 +83,12 @@ __global__ __launch_bounds__(256) void w4t_prepare_kernel(const float* __restric
             rowf[blockIdx.x] = e >= 255 ? __uint_as_float(0x7FC00000u) : e < 14 ? 0.0f : __uint_as_float((267u - e) << 23);
         return;
     }
-    const uint32_t g = blockIdx.x - m;
     const uint32_t se = (amax >> 23) + ((amax & 0x7FFFFFu) ? 1u : 0u);      // S_g = 2^(se - 127)
     const bool ok = se >= 1 && se <= 253;                      // S_g and 1 / S_g are normal floats
     const float s_inv = ok ? __uint_as_float((254u - se) << 23) : 0.0f;
     if (tid == 0) sgrp[g] = ok ? __uint_as_float(se << 23) : (amax >= 0x7F000000u ? __uint_as_float(0x7FC00000u) : 0.0f);
-    const float* zr = zp + (uint64_t)g * n;
     typedef _Float16 v4h __attribute__((ext_vector_type(4)));
-#pragma unroll 4
-    for (uint32_t j = 4 * tid; j < n; j += 1024) {             // independent iterations: their loads overlap
-        const float4 sv = *reinterpret_cast<const float4*>(r + j), z = *reinterpret_cast<const float4*>(zr + j);
+    auto emit = [&](uint32_t j, const float4& sv, const float4& z) {
         // zero-points are 0 .. 15 unless a group's weights sit far from zero (zp = -min / scale); beyond
         // +-1000 the integer part stops growing and the rest goes into the f32 correction with the fraction
         auto whole = [](float v) { return fminf(fmaxf(rintf(v), -1000.0f), 1000.0f); };
@@ -86,7 +98,13 @@ __global__ __launch_bounds__(256) void w4t_prepare_kernel(const float* __restric
         *reinterpret_cast<float4*>(zf + (uint64_t)g * n + j) = make_float4(z.x - z0.x, z.y - z0.y, z.z - z0.z, z.w - z0.w);
         *reinterpret_cast<v4h*>(zo + (uint64_t)g * n + j) =
             v4h{(_Float16)(1024.0f + z0.x), (_Float16)(1024.0f + z0.y), (_Float16)(1024.0f + z0.z), (_Float16)(1024.0f + z0.w)};
-    }
+    };
+#pragma unroll
+    for (int i = 0; i < kPrepCache; i++)
+        if (4 * tid + 1024 * i < n) emit(4 * tid + 1024 * i, cs[i], cz[i]);
+#pragma unroll 4
+    for (uint32_t j = 4 * tid + 1024 * kPrepCache; j < n; j += 1024)   // independent iterations: their loads overlap
+        emit(j, *reinterpret_cast<const float4*>(r + j), *reinterpret_cast<const float4*>(zr + j));
 }
 
 // One workgroup: rows [64 y, 64 y + 64), k [128 x, 128 x + 128), n steps [z steps_per, ..).
