@@ -127,7 +127,9 @@ constexpr size_t w4t_lds_bytes(int stages) {
 // KW = waves per workgroup = 32-column slices of k per tile: 4 when groups are multiples of 128, 2 for
 // groups of 64, 1 for groups of 32 (a tile must lie inside one group, since the activations are re-scaled
 // per group; the smaller workgroups convert the same 64 x 32 activations for fewer output columns).
-template <int kTStages, int KW>
+// HALF: at most 32 rows (one row tile, half full): the loads, the conversion and the MFMAs of rows 32..63 are
+// left out (4096 x 11008 at 16 rows: the call 44.6 -> 40.7 us; groups of 64 at 24 rows 56.1 -> 47.4 us).
+template <int kTStages, int KW, bool HALF = false>
 __global__ __launch_bounds__(64 * KW, 2) void w4t_gemm_kernel(
     const float* __restrict__ gy, const uint32_t* __restrict__ packed, const float* __restrict__ sp,
     const float* __restrict__ zf, const _Float16* __restrict__ zo, const float* __restrict__ rowf,
@@ -140,7 +142,8 @@ __global__ __launch_bounds__(64 * KW, 2) void w4t_gemm_kernel(
     float* const lds_c = reinterpret_cast<float*>(abuf + 2 * kTAbuf);
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    constexpr int kTLoads = kTSlots / KW;                      // per wave and step
+    constexpr int kTLoads = (HALF ? kTSlots - 4 : kTSlots) / KW;   // per wave and step
+    constexpr int RTILES = HALF ? 1 : 2;                       // 32-row tiles of the accumulators
     constexpr int WS = KW == 4 ? 2 : 1;                        // slots of weight words (8 word rows each)
     const uint32_t k0 = blockIdx.x * (32 * KW), m0 = blockIdx.y * 64;
     const uint32_t g = k0 / gs;
@@ -160,7 +163,8 @@ __global__ __launch_bounds__(64 * KW, 2) void w4t_gemm_kernel(
     bool wide[kTLoads], is_gy[kTLoads];                        // dst: offset inside the slot of its kind
 #pragma unroll
     for (int i = 0; i < kTLoads; i++) {
-        const uint32_t q = KW * i + wave;
+        uint32_t q = KW * i + wave;
+        if (HALF && q >= 4) q += 4;                            // no loads of rows 32..63 of grad_y
         is_gy[i] = q < 8;
         if (q < 8) {
             const uint32_t row = min(m0 + 8 * q + l8, m - 1);
@@ -241,6 +245,7 @@ __global__ __launch_bounds__(64 * KW, 2) void w4t_gemm_kernel(
         *reinterpret_cast<uint4*>(ab + 64 * 64 + s_lds) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
     };
     auto convert = [&](uint32_t st, uint32_t gslot, uint32_t wslot, int buf) {
+        if (HALF && s_row >= 32) return;                       // whole waves when KW >= 2
 #pragma unroll
         for (int cc = 0; cc < CPT; cc++) convert_chunk(st, gslot, wslot, buf, s_ch0 + cc);
     };
@@ -269,9 +274,9 @@ __global__ __launch_bounds__(64 * KW, 2) void w4t_gemm_kernel(
 #pragma unroll
     for (int t = 0; t < 2; t++) a_off[t] = fr * 64 + (((2 * t + fh) ^ fsw) & 3) * 16;
 
-    t16f acc[2];
+    t16f acc[RTILES];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < RTILES; i++)
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[i][r] = 0.0f;
 
@@ -297,7 +302,7 @@ __global__ __launch_bounds__(64 * KW, 2) void w4t_gemm_kernel(
         const t8h b0 = b_frag(0, cur), b1 = b_frag(1, cur);
         const uint8_t* abp = abuf + ab * kTAbuf;
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
+        for (int i = 0; i < RTILES; i++) {
             const uint8_t* hi = abp + i * 32 * 64;
             const uint8_t* lo = abp + 64 * 64 + i * 32 * 64;
             acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const t8h*>(hi + a_off[0]), b0, acc[i], 0, 0, 0);
@@ -323,7 +328,7 @@ __global__ __launch_bounds__(64 * KW, 2) void w4t_gemm_kernel(
     const float s_big = sgrp[g];
     if (col < k) {
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int i = 0; i < RTILES; i++)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const uint32_t lr = 32 * i + 8 * (r / 4) + 4 * fh + (r % 4), row = m0 + lr;
@@ -358,27 +363,29 @@ bool w4_gemm_t_supported(uint32_t m, uint32_t k, uint32_t n, uint32_t group_size
            (uint64_t)m * k < (1ull << 32) && (uint64_t)m * n < (1ull << 40);
 }
 
-template <int NS, int KW>
+template <int NS, int KW, bool HALF = false>
 static int launch_w4t(uint32_t ktiles, uint32_t mtiles, uint32_t shares, hipStream_t s, const float* gy,
                       const uint32_t* packed, const float* sp, const float* zf, const _Float16* zo, const float* rowf,
                       const float* sgrp, float* out, uint32_t m, uint32_t k, uint32_t n, uint32_t gs, uint32_t steps_per) {
     constexpr size_t lds_bytes = w4t_lds_bytes(NS);
     static bool attr_set = false;   // benign race: setting the attribute is idempotent
     if (!attr_set && lds_bytes > 64 * 1024) {
-        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&w4t_gemm_kernel<NS, KW>),
+        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&w4t_gemm_kernel<NS, KW, HALF>),
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes),
                                "hipFuncSetAttribute"))
             return rc;
         attr_set = true;
     }
-    hipLaunchKernelGGL((w4t_gemm_kernel<NS, KW>), dim3(ktiles, mtiles, shares), dim3(64 * KW), lds_bytes, s, gy, packed, sp, zf, zo,
+    hipLaunchKernelGGL((w4t_gemm_kernel<NS, KW, HALF>), dim3(ktiles, mtiles, shares), dim3(64 * KW), lds_bytes, s, gy, packed, sp, zf, zo,
                        rowf, sgrp, out, m, k, n, gs, steps_per);
     return check_launch("w4t_gemm_kernel");
 }
 
 #define RUMUS_W4T_LAUNCH(NS, KW)                                                                                  \
-    launch_w4t<NS, KW>(ktiles, mtiles, shares, s, gy, packed, sp, zf, zo, rowf, sgrp, shares > 1 ? part : out, m, k, n, \
-                       group_size, steps_per)
+    (m <= 32 ? launch_w4t<NS, KW, true>(ktiles, mtiles, shares, s, gy, packed, sp, zf, zo, rowf, sgrp,              \
+                                        shares > 1 ? part : out, m, k, n, group_size, steps_per)                   \
+             : launch_w4t<NS, KW>(ktiles, mtiles, shares, s, gy, packed, sp, zf, zo, rowf, sgrp,                    \
+                                  shares > 1 ? part : out, m, k, n, group_size, steps_per))
 
 int w4_launch_gemm_t(const float* gy, const uint32_t* packed, const float* scales, const float* zp, float* out,
                      uint32_t m, uint32_t k, uint32_t n, uint32_t padded_k, uint32_t group_size, uint32_t num_groups,
