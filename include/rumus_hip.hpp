@@ -266,6 +266,11 @@ inline DeviceBuffer<float> dequantize_kn(const Q8Tensor& q, hipStream_t stream =
 inline DeviceBuffer<float> matmul(const DeviceBuffer<float>& a, uint32_t m, const Q8Tensor& b,
                                   hipStream_t stream = nullptr) {
     require(a.size() == (size_t)m * b.k, "matmul: inner dimension mismatch");
+    // the kernel, like matmul_q8.wgsl:47-52, reads ceil(k / block_size) whole blocks per column; Tensor::quantize
+    // blocks the flat transposed tensor, which is that many only when k % block_size == 0 (or one block holds it all)
+    require(b.block_size > 0 && b.buffer.size() >= (size_t)b.n * ((b.k + b.block_size - 1) / b.block_size) *
+                                                       ((4 + (size_t)b.block_size + 3) / 4),
+            "matmul: the Q8 buffer is shorter than n columns of whole blocks (k % block_size != 0?)");
     DeviceBuffer<float> c((size_t)m * b.n);
     check(rumus_hip_matmul_q8(a.data(), b.buffer.data(), c.data(), m, b.k, b.n, b.block_size, stream));
     return c;

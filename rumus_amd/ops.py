@@ -76,6 +76,10 @@ def matmul_q8(a: torch.Tensor, words: torch.Tensor, k: int, n: int, block_size: 
     m = a.shape[0]
     if a.dim() != 2 or a.shape[1] != k:
         raise ValueError("matmul: inner dimension mismatch")
+    # the kernel, like matmul_q8.wgsl:47-52, reads ceil(k / block_size) whole blocks per column; Tensor::quantize blocks
+    # the flat transposed tensor, which is that many only when k % block_size == 0 (or one block holds it all)
+    if block_size <= 0 or words.numel() < n * (-(-k // block_size)) * ((4 + block_size + 3) // 4):
+        raise ValueError("matmul: the Q8 buffer is shorter than n columns of whole blocks (k % block_size != 0?)")
     c = torch.empty((m, n), dtype=torch.float32, device=a.device) if out is None else out
     if c.shape != (m, n) or c.dtype != torch.float32 or not c.is_contiguous():
         raise ValueError("matmul: out must be a contiguous f32 [m, n] tensor")

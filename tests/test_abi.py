@@ -59,6 +59,24 @@ def test_preconditions_are_rejected_before_any_launch(library):
         _lib.call("rumus_hip_matmul_q8", None, None, None, 1, 8, 1, 3, None)
 
 
+def test_matmul_q8_refuses_a_buffer_without_whole_blocks_per_column():
+    # Tensor::quantize blocks the flat transposed tensor: with k % block_size != 0 the buffer holds fewer blocks than
+    # matmul_q8's addressing (ceil(k / block_size) per column) walks, and the kernel would read past its end
+    import torch
+    from rumus_amd import ops
+    k, n, bs = 1000, 100, 256
+    flat_words = library_free_q8_words(k * n, bs)
+    a = torch.zeros((2, k), dtype=torch.float32)
+    with pytest.raises(ValueError, match="whole blocks"):
+        ops.matmul_q8(a, torch.zeros(flat_words, dtype=torch.int32), k, n, bs)
+
+
+def library_free_q8_words(numel, bs):
+    """Words of a flat-blocked Q8 buffer (tensor/core.rs:87-98) without loading the library."""
+    blocks = -(-numel // bs)
+    return blocks * ((4 + bs + 3) // 4)
+
+
 def test_product_package_does_not_touch_the_oracle():
     pkg = os.path.join(ROOT, "rumus_amd")
     for dirpath, _, files in os.walk(pkg):
