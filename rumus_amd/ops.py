@@ -59,6 +59,8 @@ def q8_quantize(flat: torch.Tensor, block_size: int) -> torch.Tensor:
 
 
 def q8_dequantize(words: torch.Tensor, numel: int, block_size: int) -> torch.Tensor:
+    if block_size > 0 and block_size % 4 == 0 and words.numel() * 4 < q8_buf_size(numel, block_size):
+        raise ValueError("q8_dequantize: the buffer is shorter than numel elements in blocks of block_size")
     out = torch.empty(numel, dtype=torch.float32, device=words.device)
     call("rumus_hip_q8_dequantize", _dev(words, torch.int32, "in"), out.data_ptr(), numel,
          block_size, _stream())
@@ -67,6 +69,8 @@ def q8_dequantize(words: torch.Tensor, numel: int, block_size: int) -> torch.Ten
 
 def q8_dequantize_kn(words: torch.Tensor, k: int, n: int, block_size: int) -> torch.Tensor:
     """The dequantized weight in its own ``[k, n]`` order (the buffer holds the transposed tensor)."""
+    if block_size > 0 and block_size % 4 == 0 and words.numel() * 4 < q8_buf_size(k * n, block_size):
+        raise ValueError("q8_dequantize_kn: the buffer is shorter than k * n elements in blocks of block_size")
     out = torch.empty((k, n), dtype=torch.float32, device=words.device)
     call("rumus_hip_q8_dequantize_kn", _dev(words, torch.int32, "in"), out.data_ptr(), k, n, block_size, _stream())
     return out
@@ -162,8 +166,12 @@ def i8_quantize_cols_t(w: torch.Tensor):
 def i8_gemm(xq, wq, sx=None, sw=None, bias=None, want_acc=False, want_y=True, out=None):
     m, k = xq.shape
     n = wq.shape[0]
-    if wq.shape[1] != k:
+    if xq.dim() != 2 or wq.dim() != 2 or wq.shape[1] != k:
         raise ValueError("i8_gemm: inner dimension mismatch")
+    if (sx is not None and sx.numel() < m) or (sw is not None and sw.numel() < n) or (bias is not None and bias.numel() < n):
+        raise ValueError("i8_gemm: sx must hold m scales, sw and bias n values")
+    if out is not None and (tuple(out.shape) != (m, n) or out.dtype != torch.float32 or not out.is_contiguous()):
+        raise ValueError("i8_gemm: out must be a contiguous f32 [m, n] tensor")
     acc = torch.empty((m, n), dtype=torch.int32, device=xq.device) if want_acc else None
     y = None
     if want_y:
@@ -222,6 +230,7 @@ def w4_qzeros_unpack(qzeros, n):
 def w4_decode_layout(packed, scales, zp, group_size):
     """Tile-major copies (16 columns per tile) of the three arrays of an INT4 weight."""
     rows, n = packed.shape
+    _w4_sizes("w4_decode_layout", packed, scales, zp, rows * 8, group_size, 0)
     out = (torch.empty_like(packed), torch.empty_like(scales), torch.empty_like(zp))
     call("rumus_hip_w4_decode_layout", _dev(packed, torch.int32, "packed"), _dev(scales, torch.float32, "scales"),
          _dev(zp, torch.float32, "zero_points"), rows * 8, n, group_size, out[0].data_ptr(), out[1].data_ptr(),
@@ -242,6 +251,7 @@ def w4_decode_layout_zp4(packed, scales, qzeros, group_size):
     """Tile-major copies for AWQ storage: packed, scales as in w4_decode_layout, u4 zero-points with
     the two words of a tile side by side."""
     rows, n = packed.shape
+    _w4_sizes("w4_decode_layout_zp4", packed, scales, qzeros, rows * 8, group_size, 0, zp4=True)
     out = (torch.empty_like(packed), torch.empty_like(scales), torch.empty_like(qzeros))
     call("rumus_hip_w4_decode_layout_zp4", _dev(packed, torch.int32, "packed"), _dev(scales, torch.float32, "scales"),
          _dev(qzeros, torch.int32, "qzeros"), rows * 8, n, group_size, out[0].data_ptr(), out[1].data_ptr(),
@@ -254,6 +264,7 @@ def qmatmul_int4_decode_zp4(x, packed_t, scales_t, qzeros_t, k, group_size, bias
     n = packed_t.shape[1]
     if x.dim() != 2 or x.shape[1] != k:
         raise ValueError("qmatmul_int4_decode_zp4: x must be [m, k]")
+    _w4_sizes("qmatmul_int4_decode_zp4", packed_t, scales_t, qzeros_t, k, group_size, m, bias, perm, out, zp4=True)
     padded_k, groups = w4_geometry(k, group_size) if group_size > 0 else (k, 0)
     y = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=x.device)
     call("rumus_hip_qmatmul_int4_decode_zp4", _dev(x, torch.float32, "x"), _dev(packed_t, torch.int32, "packed_t"),
@@ -269,6 +280,7 @@ def qmatmul_int4_decode_swiglu(gate_up, packed_t, scales_t, zp_t, k, group_size,
     n = packed_t.shape[1]
     if gate_up.dim() != 2 or gate_up.shape[1] != 2 * k:
         raise ValueError("qmatmul_int4_decode_swiglu: gate_up must be [m, 2k]")
+    _w4_sizes("qmatmul_int4_decode_swiglu", packed_t, scales_t, zp_t, k, group_size, m, bias, None, out)
     padded_k, groups = w4_geometry(k, group_size) if group_size > 0 else (k, 0)
     y = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=gate_up.device)
     call("rumus_hip_qmatmul_int4_decode_swiglu", _dev(gate_up, torch.float32, "gate_up"),
@@ -283,6 +295,7 @@ def qmatmul_int4_zp4(x, packed, scales, qzeros, k, group_size, bias=None, perm=N
     n = packed.shape[1]
     if x.dim() != 2 or x.shape[1] != k:
         raise ValueError("qmatmul_int4_zp4: x must be [m, k]")
+    _w4_sizes("qmatmul_int4_zp4", packed, scales, qzeros, k, group_size, m, bias, perm, out, zp4=True)
     padded_k, groups = w4_geometry(k, group_size) if group_size > 0 else (k, 0)
     y = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=x.device)
     call("rumus_hip_qmatmul_int4_zp4", _dev(x, torch.float32, "x"), _dev(packed, torch.int32, "packed"),
@@ -292,11 +305,32 @@ def qmatmul_int4_zp4(x, packed, scales, qzeros, k, group_size, bias=None, perm=N
     return y
 
 
+def _w4_sizes(who, packed, scales, zp, k, group_size, rows, bias=None, index=None, out=None, out_cols=None, zp4=False):
+    """The kernels take raw pointers: a short array would be read past its end on the device.  Checks the element
+    counts the geometry implies (the library itself rejects a bad group size or alignment)."""
+    if group_size <= 0 or packed.dim() != 2:
+        return
+    n = packed.shape[1]
+    padded_k, groups = w4_geometry(k, group_size)
+    zp_need = groups * (n // 8) if zp4 else groups * n
+    if packed.numel() < max(padded_k // 8, 1) * n or scales.numel() < groups * n or zp.numel() < zp_need:
+        raise ValueError(f"{who}: packed / scales / zero-points are smaller than k={k}, n={n}, group_size={group_size} needs")
+    if bias is not None and bias.numel() < n:
+        raise ValueError(f"{who}: bias must hold n = {n} values")
+    if index is not None and index.numel() < k:
+        raise ValueError(f"{who}: g_idx / perm must hold k = {k} entries")
+    if out is not None:
+        cols = n if out_cols is None else out_cols
+        if tuple(out.shape) != (rows, cols) or out.dtype != torch.float32 or not out.is_contiguous():
+            raise ValueError(f"{who}: out must be a contiguous f32 [{rows}, {cols}] tensor")
+
+
 def _w4_call(name, x, packed, scales, zp, bias, extra, k, group_size, out=None):
     m = x.shape[0]
     n = packed.shape[1]
     if x.dim() != 2 or x.shape[1] != k:
         raise ValueError("qmatmul_int4: x must be [m, k]")
+    _w4_sizes(name, packed, scales, zp, k, group_size, m, bias, extra, out)
     padded_k, groups = w4_geometry(k, group_size) if group_size > 0 else (k, 0)
     y = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=x.device)
     call(name, _dev(x, torch.float32, "x"), _dev(packed, torch.int32, "packed"),
@@ -327,6 +361,7 @@ def qmatmul_int4_t(a, packed, scales, zp, k, group_size, out=None):
     m, n = a.shape
     if packed.shape[1] != n:
         raise ValueError("qmatmul_int4_t: a must be [m, n]")
+    _w4_sizes("qmatmul_int4_t", packed, scales, zp, k, group_size, m)
     padded_k, groups = w4_geometry(k, group_size)
     if out is None:
         out = torch.empty((m, k), dtype=torch.float32, device=a.device)

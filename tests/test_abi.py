@@ -71,6 +71,32 @@ def test_matmul_q8_refuses_a_buffer_without_whole_blocks_per_column():
         ops.matmul_q8(a, torch.zeros(flat_words, dtype=torch.int32), k, n, bs)
 
 
+def test_binding_refuses_arrays_shorter_than_the_geometry():
+    # raw pointers go to the device: a short array would be read past its end there
+    import torch
+    from rumus_amd import ops
+    k, n, g = 256, 64, 128
+    x = torch.zeros((2, k))
+    packed = torch.zeros((k // 8, n), dtype=torch.int32)
+    scales = torch.zeros((k // g, n))
+    with pytest.raises(ValueError, match="smaller than"):
+        ops.qmatmul_int4(x, packed[:-1], scales, scales, k, g)
+    with pytest.raises(ValueError, match="smaller than"):
+        ops.qmatmul_int4(x, packed, scales[:-1], scales, k, g)
+    with pytest.raises(ValueError, match="bias"):
+        ops.qmatmul_int4(x, packed, scales, scales, k, g, bias=torch.zeros(n - 1))
+    with pytest.raises(ValueError, match="perm"):
+        ops.qmatmul_int4_perm(x, packed, scales, scales, k, g, perm=torch.zeros(k - 1, dtype=torch.int32))
+    with pytest.raises(ValueError, match="out must be"):
+        ops.qmatmul_int4(x, packed, scales, scales, k, g, out=torch.zeros((2, n + 1)))
+    with pytest.raises(ValueError, match="smaller than"):
+        ops.qmatmul_int4_t(torch.zeros((2, n)), packed, scales, scales[:-1], k, g)
+    with pytest.raises(ValueError, match="sx must hold"):
+        ops.i8_gemm(torch.zeros((4, 32), dtype=torch.int8), torch.zeros((8, 32), dtype=torch.int8), torch.zeros(3), torch.zeros(8))
+    with pytest.raises(ValueError, match="shorter"):
+        ops.q8_dequantize(torch.zeros(10, dtype=torch.int32), 1024, 32)
+
+
 def library_free_q8_words(numel, bs):
     """Words of a flat-blocked Q8 buffer (tensor/core.rs:87-98) without loading the library."""
     blocks = -(-numel // bs)
