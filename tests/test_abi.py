@@ -24,6 +24,14 @@ def library():
     return _lib.lib()
 
 
+def test_header_is_plain_c(tmp_path):
+    # the boundary is a C ABI: the header must compile as C99 with nothing but itself
+    src = tmp_path / "c_abi.c"
+    src.write_text('#include "rumus_hip.h"\nint main(void) { return rumus_hip_version() ? 0 : 1; }\n')
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(ROOT, "include"),
+                    "-fsyntax-only", str(src)], check=True)
+
+
 def test_header_and_binding_agree():
     assert _declared() == sorted(_lib.PROTOTYPES)
 
