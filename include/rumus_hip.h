@@ -12,6 +12,10 @@
  *   - every pointer is a caller-owned DEVICE pointer (hipMalloc'd) unless it
  *     is said to be a host pointer; the library never frees caller memory and
  *     allocates nothing on the launch path;
+ *   - a call whose batch is empty (zero rows, zero elements) succeeds, queues
+ *     nothing and reads no array: the pointers of such a call may be NULL, as
+ *     the data pointer of an empty tensor is.  The scalar preconditions
+ *     (group and block sizes, divisibility) are checked all the same;
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
  *     launches are asynchronous on that stream, like wgpu's queue.submit
  *     (rumus/src/backend/gpu/compute.rs:1981);

@@ -500,7 +500,7 @@ extern "C" {
 
 int rumus_hip_rmsnorm(const float* x, const float* weight, float* y, uint32_t rows, uint32_t dim, float eps,
                       rumus_hip_stream_t stream) {
-    RUMUS_REQUIRE(x && weight && y, "rmsnorm: null buffer");
+    RUMUS_REQUIRE(rows == 0 || (x && weight && y), "rmsnorm: null buffer");
     RUMUS_REQUIRE(dim > 0, "rmsnorm: dim must be > 0");
     if (rows == 0) return RUMUS_HIP_OK;
     const bool vec = dim % 4 == 0 && dim <= 8192 &&
@@ -515,9 +515,9 @@ int rumus_hip_rmsnorm(const float* x, const float* weight, float* y, uint32_t ro
 
 int rumus_hip_add_rmsnorm(const float* x, const float* delta, const float* weight, float* sum, float* y,
                           uint32_t rows, uint32_t dim, float eps, rumus_hip_stream_t stream) {
-    RUMUS_REQUIRE(x && delta && weight && sum && y, "add_rmsnorm: null buffer");
+    RUMUS_REQUIRE(rows == 0 || (x && delta && weight && sum && y), "add_rmsnorm: null buffer");
     RUMUS_REQUIRE(dim > 0, "add_rmsnorm: dim must be positive");
-    RUMUS_REQUIRE(y != x && y != delta && y != sum, "add_rmsnorm: y must not alias x, delta or sum");
+    RUMUS_REQUIRE(rows == 0 || (y != x && y != delta && y != sum), "add_rmsnorm: y must not alias x, delta or sum");
     if (rows == 0) return RUMUS_HIP_OK;
     const bool vec = dim % 4 == 0 && dim <= 8192 &&
                      ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(delta) |
@@ -531,7 +531,7 @@ int rumus_hip_add_rmsnorm(const float* x, const float* delta, const float* weigh
 }
 
 int rumus_hip_swiglu(const float* gate, const float* up, float* out, uint64_t numel, rumus_hip_stream_t stream) {
-    RUMUS_REQUIRE(gate && up && out, "swiglu: null buffer");
+    RUMUS_REQUIRE(numel == 0 || (gate && up && out), "swiglu: null buffer");
     if (numel == 0) return RUMUS_HIP_OK;
     hipLaunchKernelGGL(swiglu_kernel, dim3((uint32_t)((numel + 255) / 256)), dim3(256), 0, as_stream(stream), gate,
                        up, out, numel);
@@ -539,7 +539,7 @@ int rumus_hip_swiglu(const float* gate, const float* up, float* out, uint64_t nu
 }
 
 int rumus_hip_swiglu_rows(const float* gate_up, float* out, uint32_t rows, uint32_t n, rumus_hip_stream_t stream) {
-    RUMUS_REQUIRE(gate_up && out, "swiglu_rows: null buffer");
+    RUMUS_REQUIRE(rows == 0 || n == 0 || (gate_up && out), "swiglu_rows: null buffer");
     RUMUS_REQUIRE(rows <= 65535, "swiglu_rows: rows %u beyond the grid limit", rows);
     if (rows == 0 || n == 0) return RUMUS_HIP_OK;
     hipLaunchKernelGGL(swiglu_rows_kernel, dim3(ceil_div(n, 256), rows), dim3(256), 0, as_stream(stream), gate_up, out,
@@ -548,7 +548,7 @@ int rumus_hip_swiglu_rows(const float* gate_up, float* out, uint32_t rows, uint3
 }
 
 int rumus_hip_add(const float* a, const float* b, float* out, uint64_t numel, rumus_hip_stream_t stream) {
-    RUMUS_REQUIRE(a && b && out, "add: null buffer");
+    RUMUS_REQUIRE(numel == 0 || (a && b && out), "add: null buffer");
     if (numel == 0) return RUMUS_HIP_OK;
     hipLaunchKernelGGL(add_kernel, dim3((uint32_t)((numel + 255) / 256)), dim3(256), 0, as_stream(stream), a, b, out,
                        numel);
@@ -558,7 +558,7 @@ int rumus_hip_add(const float* a, const float* b, float* out, uint64_t numel, ru
 int rumus_hip_attention(const float* q, const float* k, const float* v, float* out, uint32_t batch, uint32_t heads,
                         uint32_t q_len, uint32_t kv_len, uint32_t head_dim, const uint64_t* strides, int causal,
                         rumus_hip_stream_t stream) {
-    RUMUS_REQUIRE(q && k && v && out && strides, "attention: null buffer");
+    RUMUS_REQUIRE((batch == 0 || heads == 0 || q_len == 0) || (q && k && v && out && strides), "attention: null buffer");
     RUMUS_REQUIRE(head_dim == kHeadDim, "attention: head_dim must be %d (got %u)", kHeadDim, head_dim);
     RUMUS_REQUIRE(q_len <= kv_len, "attention: q_len %u exceeds kv_len %u", q_len, kv_len);
     if (batch == 0 || heads == 0 || q_len == 0) return RUMUS_HIP_OK;
@@ -596,7 +596,8 @@ int rumus_hip_attention(const float* q, const float* k, const float* v, float* o
 int rumus_hip_kv_append(const float* k_new, const float* v_new, float* k_cache, float* v_cache, uint32_t batch,
                         uint32_t heads, uint32_t rows, uint32_t head_dim, uint32_t pos, uint32_t cache_len,
                         const uint64_t* strides, rumus_hip_stream_t stream) {
-    RUMUS_REQUIRE(k_new && v_new && k_cache && v_cache && strides, "kv_append: null buffer");
+    RUMUS_REQUIRE((batch == 0 || heads == 0 || rows == 0) || (k_new && v_new && k_cache && v_cache && strides),
+                  "kv_append: null buffer");
     RUMUS_REQUIRE(head_dim > 0 && head_dim % 4 == 0, "kv_append: head_dim %u must be a positive multiple of 4", head_dim);
     RUMUS_REQUIRE((uint64_t)pos + rows <= cache_len, "kv_append: positions %u..%llu do not fit a cache of %u", pos,
                   (unsigned long long)pos + rows, cache_len);

@@ -561,13 +561,16 @@ using namespace rumus;
 extern "C" int rumus_hip_i8_gemm(const int8_t* xq, const int8_t* wq, const float* sx,
                                  const float* sw, const float* bias, int32_t* acc, float* y,
                                  uint32_t m, uint32_t k, uint32_t n, rumus_hip_stream_t stream) {
+    if (m == 0 || n == 0) {                                  // nothing to read or write: null pointers are fine
+        RUMUS_REQUIRE(k > 0 && k % 16 == 0, "i8_gemm: k must be a positive multiple of 16 (got %u)", k);
+        return RUMUS_HIP_OK;
+    }
     RUMUS_REQUIRE(xq && wq, "i8_gemm: null operand");
     RUMUS_REQUIRE(acc || y, "i8_gemm: both outputs are null");
     RUMUS_REQUIRE(!y || (sx && sw), "i8_gemm: y needs sx and sw");
     RUMUS_REQUIRE(k > 0 && k % 16 == 0, "i8_gemm: k must be a positive multiple of 16 (got %u)", k);
     RUMUS_REQUIRE(((reinterpret_cast<uintptr_t>(xq) | reinterpret_cast<uintptr_t>(wq)) & 15) == 0,
                   "i8_gemm: operands must be 16-byte aligned");
-    if (m == 0 || n == 0) return RUMUS_HIP_OK;
     hipStream_t s = as_stream(stream);
     const I8Choice c = i8_choose(m, k, n);
     switch (c.route) {

@@ -174,7 +174,7 @@ extern "C" {
 
 int rumus_hip_i8_quantize_rows(const float* x, int8_t* xq, float* scale, uint32_t rows,
                                uint32_t cols, rumus_hip_stream_t stream) {
-    RUMUS_REQUIRE(x && xq && scale, "i8_quantize_rows: null buffer");
+    RUMUS_REQUIRE(rows == 0 || (x && xq && scale), "i8_quantize_rows: null buffer");
     if (rows == 0) return RUMUS_HIP_OK;
     RUMUS_REQUIRE(cols > 0, "i8_quantize_rows: cols must be > 0");
     hipStream_t s = as_stream(stream);
@@ -191,7 +191,7 @@ int rumus_hip_i8_quantize_rows(const float* x, int8_t* xq, float* scale, uint32_
 
 int rumus_hip_i8_quantize_cols_t(const float* w, int8_t* wq, float* sw, uint32_t k, uint32_t n,
                                  rumus_hip_stream_t stream) {
-    RUMUS_REQUIRE(w && wq && sw, "i8_quantize_cols_t: null buffer");
+    RUMUS_REQUIRE(n == 0 || (w && wq && sw), "i8_quantize_cols_t: null buffer");
     if (n == 0) return RUMUS_HIP_OK;
     RUMUS_REQUIRE(k > 0, "i8_quantize_cols_t: k must be > 0");
     hipStream_t s = as_stream(stream);

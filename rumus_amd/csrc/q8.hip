@@ -751,7 +751,7 @@ int rumus_hip_q8_quantize(const float* in, uint32_t* out, uint32_t numel, uint32
                           rumus_hip_stream_t stream) {
     RUMUS_REQUIRE(block_size > 0 && block_size % 4 == 0,
                   "quantize: block_size must be > 0 and divisible by 4 (got %u)", block_size);
-    RUMUS_REQUIRE(in && out, "quantize: null buffer");
+    RUMUS_REQUIRE(numel == 0 || (in && out), "quantize: null buffer");
     if (numel == 0) return RUMUS_HIP_OK;
     uint32_t num_blocks = ceil_div(numel, block_size);
     uint32_t stride = (4 + block_size + 3) / 4;
@@ -778,7 +778,7 @@ int rumus_hip_q8_dequantize(const uint32_t* in, float* out, uint32_t numel, uint
                             rumus_hip_stream_t stream) {
     RUMUS_REQUIRE(block_size > 0 && block_size % 4 == 0,
                   "dequantize: block_size must be > 0 and divisible by 4 (got %u)", block_size);
-    RUMUS_REQUIRE(in && out, "dequantize: null buffer");
+    RUMUS_REQUIRE(numel == 0 || (in && out), "dequantize: null buffer");
     if (numel == 0) return RUMUS_HIP_OK;
     uint32_t stride = (4 + block_size + 3) / 4;
     uint32_t words = numel / 4 + (numel % 4 != 0);
@@ -791,7 +791,7 @@ int rumus_hip_q8_dequantize_kn(const uint32_t* in, float* out, uint32_t k, uint3
                                rumus_hip_stream_t stream) {
     RUMUS_REQUIRE(block_size > 0 && block_size % 4 == 0,
                   "dequantize: block_size must be > 0 and divisible by 4 (got %u)", block_size);
-    RUMUS_REQUIRE(in && out, "dequantize: null buffer");
+    RUMUS_REQUIRE(k == 0 || n == 0 || (in && out), "dequantize: null buffer");
     if (k == 0 || n == 0) return RUMUS_HIP_OK;
     RUMUS_REQUIRE(n <= 65535u * 32u, "dequantize: n %u is beyond the grid limit", n);
     const uint32_t stride = (4 + block_size + 3) / 4;
@@ -804,7 +804,7 @@ int rumus_hip_matmul_q8(const float* a, const uint32_t* b, float* c, uint32_t m,
                         uint32_t n, uint32_t block_size, rumus_hip_stream_t stream) {
     RUMUS_REQUIRE(block_size > 0 && block_size % 4 == 0,
                   "matmul_q8: block_size must be > 0 and divisible by 4 (got %u)", block_size);
-    RUMUS_REQUIRE(a && b && c, "matmul_q8: null buffer");
+    RUMUS_REQUIRE(m == 0 || n == 0 || (a && b && c), "matmul_q8: null buffer");
     if (m == 0 || n == 0) return RUMUS_HIP_OK;
     RUMUS_REQUIRE(k > 0, "matmul_q8: k must be > 0");
     uint32_t blocks_per_col = ceil_div(k, block_size);
@@ -860,7 +860,7 @@ int rumus_hip_matmul_q8(const float* a, const uint32_t* b, float* c, uint32_t m,
 
 int rumus_hip_q8_dense_layout(const uint32_t* b_q8, uint32_t k, uint32_t n, uint32_t block_size, int8_t* wq,
                               float* sw, rumus_hip_stream_t stream) {
-    RUMUS_REQUIRE(b_q8 && wq && sw, "q8_dense_layout: null buffer");
+    RUMUS_REQUIRE(n == 0 || (b_q8 && wq && sw), "q8_dense_layout: null buffer");
     RUMUS_REQUIRE(block_size > 0 && block_size % 4 == 0,
                   "q8_dense_layout: block_size must be > 0 and divisible by 4 (got %u)", block_size);
     RUMUS_REQUIRE(k > 0 && k % 4 == 0 && block_size >= k,
@@ -875,7 +875,7 @@ int rumus_hip_q8_dense_layout(const uint32_t* b_q8, uint32_t k, uint32_t n, uint
 
 int rumus_hip_matmul_q8_dense(const float* a, const int8_t* wq, const float* sw, float* c, uint32_t m, uint32_t k,
                               uint32_t n, rumus_hip_stream_t stream) {
-    RUMUS_REQUIRE(a && wq && sw && c, "matmul_q8_dense: null buffer");
+    RUMUS_REQUIRE(m == 0 || n == 0 || (a && wq && sw && c), "matmul_q8_dense: null buffer");
     if (m == 0 || n == 0) return RUMUS_HIP_OK;
     RUMUS_REQUIRE(k > 0 && k % 16 == 0, "matmul_q8_dense: k must be a positive multiple of 16 (got %u)", k);
     RUMUS_REQUIRE(((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(c) | reinterpret_cast<uintptr_t>(wq)) & 15) == 0,
@@ -892,7 +892,7 @@ int rumus_hip_matmul_q8_dense(const float* a, const int8_t* wq, const float* sw,
 
 int rumus_hip_add_bias(const float* mat, const float* bias, float* out, uint32_t m, uint32_t n,
                        rumus_hip_stream_t stream) {
-    RUMUS_REQUIRE(mat && bias && out, "add_bias: null buffer");
+    RUMUS_REQUIRE(m == 0 || n == 0 || (mat && bias && out), "add_bias: null buffer");
     uint64_t total = (uint64_t)m * n;
     if (total == 0) return RUMUS_HIP_OK;
     hipLaunchKernelGGL(add_bias_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0,
@@ -902,7 +902,7 @@ int rumus_hip_add_bias(const float* mat, const float* bias, float* out, uint32_t
 
 int rumus_hip_transpose_f32(const float* in, float* out, uint32_t rows, uint32_t cols,
                             rumus_hip_stream_t stream) {
-    RUMUS_REQUIRE(in && out, "transpose: null buffer");
+    RUMUS_REQUIRE(rows == 0 || cols == 0 || (in && out), "transpose: null buffer");
     if (rows == 0 || cols == 0) return RUMUS_HIP_OK;
     if (rows % 4 == 0 && cols % 4 == 0 &&
         ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {

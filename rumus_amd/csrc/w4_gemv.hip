@@ -393,7 +393,9 @@ static int validate(const W4Args& a, const char* who) {
     RUMUS_REQUIRE(a.k <= a.padded_k && a.padded_k < a.k + a.group_size,
                   "%s: padded_k %u does not pad k %u to group_size %u", who, a.padded_k, a.k,
                   a.group_size);
-    RUMUS_REQUIRE(a.x && a.packed && a.scales && (a.zp || a.zp4) && a.y, "%s: null buffer", who);
+    // a call without rows, columns or depth touches no array: null pointers are fine there (an empty tensor has none)
+    RUMUS_REQUIRE(a.m == 0 || a.n == 0 || a.k == 0 || (a.x && a.packed && a.scales && (a.zp || a.zp4) && a.y),
+                  "%s: null buffer", who);
     RUMUS_REQUIRE(!a.zp4 || a.n % 8 == 0, "%s: packed zero-points need n %% 8 == 0 (got %u)", who, a.n);
     return RUMUS_HIP_OK;
 }
@@ -583,6 +585,7 @@ int rumus_hip_qmatmul_int4_t(const float* a, const uint32_t* packed, const float
     W4Args v{a, packed, scales, zero_points, nullptr, nullptr, nullptr, out, m, k, n, padded_k, group_size, num_groups};
     if (int rc = validate(v, "qmatmul_int4_t")) return rc;
     if (m == 0 || k == 0) return RUMUS_HIP_OK;
+    RUMUS_REQUIRE(n > 0, "qmatmul_int4_t: n must be > 0");
     hipStream_t s = as_stream(stream);
     // where the matrix-core kernel is ahead of the vector kernel below, which takes four rows per pass (from HBM,
     // us, vector at 8 / 12 / 16 / 24 / 32 / 48 rows against the matrix cores at any of them: 4096 x 11008 g128

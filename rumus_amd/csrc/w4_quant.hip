@@ -204,7 +204,7 @@ template <bool SYM>
 static int quantize_pack(const float* w, uint32_t k, uint32_t n, uint32_t gs, uint32_t* packed,
                          float* scales, float* zps, hipStream_t s) {
     RUMUS_REQUIRE(gs > 0 && gs % 8 == 0, "group_size must be a multiple of 8 (got %u)", gs);
-    RUMUS_REQUIRE(w && packed && scales && (SYM || zps), "w4_quantize_pack: null buffer");
+    RUMUS_REQUIRE(n == 0 || k == 0 || (w && packed && scales && (SYM || zps)), "w4_quantize_pack: null buffer");
     if (n == 0 || k == 0) return RUMUS_HIP_OK;
     const uint32_t groups = ceil_div(k, gs);
     const dim3 grid(ceil_div(n, 256), groups);
@@ -305,7 +305,7 @@ int rumus_hip_w4_quantize_pack_awq(const float* w, uint32_t k, uint32_t n, uint3
     RUMUS_REQUIRE(group_size > 0 && group_size % 8 == 0,
                   "w4_quantize_pack_awq: group_size must be a multiple of 8 (got %u)", group_size);
     RUMUS_REQUIRE(n % 8 == 0, "w4_quantize_pack_awq: n must be a multiple of 8 (got %u)", n);
-    RUMUS_REQUIRE(w && packed && scales && qzeros, "w4_quantize_pack_awq: null buffer");
+    RUMUS_REQUIRE(n == 0 || k == 0 || (w && packed && scales && qzeros), "w4_quantize_pack_awq: null buffer");
     if (k == 0 || n == 0) return RUMUS_HIP_OK;
     const uint32_t groups = ceil_div(k, group_size);
     const dim3 grid(ceil_div(n, 256), groups);

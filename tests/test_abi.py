@@ -67,6 +67,38 @@ def test_preconditions_are_rejected_before_any_launch(library):
         _lib.call("rumus_hip_matmul_q8", None, None, None, 1, 8, 1, 3, None)
 
 
+def test_empty_calls_succeed_without_arrays_and_full_ones_need_them(library):
+    """A call with no rows queues nothing and reads no array, so it may come without pointers (an empty tensor has
+    none) and needs no GPU; the same call with rows is refused for its null pointers; scalar preconditions hold
+    either way."""
+    L = library
+    assert L.rumus_hip_qmatmul_int4(None, None, None, None, None, None, None, 0, 128, 64, 128, 64, 2, None) == 0
+    assert L.rumus_hip_qmatmul_int4(None, None, None, None, None, None, None, 2, 128, 64, 128, 64, 2, None) == _lib.EINVAL
+    assert b"null buffer" in L.rumus_hip_last_error()
+    assert L.rumus_hip_qmatmul_int4(None, None, None, None, None, None, None, 0, 128, 64, 128, 12, 2, None) == _lib.EINVAL
+    assert L.rumus_hip_qmatmul_int4_t(None, None, None, None, None, 0, 128, 64, 128, 64, 2, None) == 0
+    assert L.rumus_hip_qmatmul_int4_decode(None, None, None, None, None, None, None, 0, 128, 64, 128, 64, 2, None) == 0
+    assert L.rumus_hip_matmul_q8(None, None, None, 0, 64, 8, 32, None) == 0
+    assert L.rumus_hip_matmul_q8(None, None, None, 1, 64, 8, 32, None) == _lib.EINVAL
+    assert L.rumus_hip_matmul_q8(None, None, None, 0, 64, 8, 6, None) == _lib.EINVAL
+    assert L.rumus_hip_matmul_q8_dense(None, None, None, None, 0, 64, 8, None) == 0
+    assert L.rumus_hip_q8_quantize(None, None, 0, 32, None) == 0
+    assert L.rumus_hip_q8_dequantize(None, None, 0, 32, None) == 0
+    assert L.rumus_hip_i8_quantize_rows(None, None, None, 0, 64, None) == 0
+    assert L.rumus_hip_i8_quantize_rows(None, None, None, 3, 64, None) == _lib.EINVAL
+    assert L.rumus_hip_i8_gemm(None, None, None, None, None, None, None, 0, 64, 8, None) == 0
+    assert L.rumus_hip_i8_gemm(None, None, None, None, None, None, None, 0, 24, 8, None) == _lib.EINVAL
+    assert L.rumus_hip_add_bias(None, None, None, 0, 8, None) == 0
+    assert L.rumus_hip_transpose_f32(None, None, 0, 8, None) == 0
+    assert L.rumus_hip_rmsnorm(None, None, None, 0, 64, 1e-6, None) == 0
+    assert L.rumus_hip_rmsnorm(None, None, None, 2, 64, 1e-6, None) == _lib.EINVAL
+    assert L.rumus_hip_swiglu(None, None, None, 0, None) == 0
+    assert L.rumus_hip_add(None, None, None, 0, None) == 0
+    assert L.rumus_hip_attention(None, None, None, None, 1, 4, 0, 8, 128, None, 0, None) == 0
+    assert L.rumus_hip_kv_append(None, None, None, None, 1, 4, 0, 128, 3, 16, None, None) == 0
+    assert L.rumus_hip_kv_append(None, None, None, None, 1, 4, 0, 128, 17, 16, None, None) == _lib.EINVAL
+
+
 def test_matmul_q8_refuses_a_buffer_without_whole_blocks_per_column():
     # Tensor::quantize blocks the flat transposed tensor: with k % block_size != 0 the buffer holds fewer blocks than
     # matmul_q8's addressing (ceil(k / block_size) per column) walks, and the kernel would read past its end
