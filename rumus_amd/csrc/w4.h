@@ -33,6 +33,10 @@ struct W4Args {
     const uint8_t* xl = nullptr;
     const float* xs = nullptr;
     uint32_t xsteps = 0;
+    // w4_gemm_tile only (set by its launcher): a power of two per row that brings the row's largest magnitude into
+    // [2^14, 2^15) before the split into f16 planes (rinv), and its reciprocal for the results (rfac)
+    const float* rinv = nullptr;
+    const float* rfac = nullptr;
 };
 
 // zero-points of 4 (col % 4 == 0) or 2 (col % 2 == 0) adjacent columns from the packed form

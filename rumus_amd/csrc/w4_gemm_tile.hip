@@ -141,6 +141,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
     constexpr int PLANE = 8 * STEP;
     __shared__ __attribute__((aligned(16))) uint8_t lds_a[2][2][PLANE];   // [buffer][hi, lo]
     __shared__ __attribute__((aligned(16))) float lds_xs[2][8][BM];       // [buffer][k16 step][row]: sum of x
+    __shared__ float lds_rf[BM];                                          // the rows' factors for the results
 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t wm = wave / WN, wn = wave % WN;
@@ -154,6 +155,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
     const uint32_t st_end = min(nstages, st_begin + stages_per_split);
     const uint32_t word_rows = a.padded_k / 8;
     const uint32_t k_end = min(a.padded_k, st_end * kStageK);
+    if (tid < BM) lds_rf[tid] = a.rfac[min(m0 + tid, a.m - 1)];          // read after the stages' barriers
 
     // ---- staging role: thread t converts 16 consecutive k (MFMA step t%8) of row t/8 -----
     const uint32_t s_row = tid >> 3, s_step = tid & 7;
@@ -212,6 +214,9 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
     constexpr int PIECES = PRE ? 4 : 2 * NI;             // spread over the last steps of a stage: the
     static_assert(!PRE || NCH % 4 == 0, "chunks per piece"); // loads were issued at its first step
     float xsum[NI];
+    float s_rinv[NI];                                    // non-PRE: the factor of each row this thread converts
+#pragma unroll
+    for (int it = 0; it < NI; it++) s_rinv[it] = PRE ? 1.0f : a.rinv[min(m0 + s_row + RPP * it, a.m - 1)];
     auto stage_store_piece = [&](uint32_t st, uint32_t buf, int piece, int slot) __attribute__((always_inline)) {
         if constexpr (PRE) {                               // NCH/4 chunks per piece, the sums with the last
             if constexpr (NCH == 4) {
@@ -242,8 +247,9 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
         const bool row_ok = m0 + row < a.m;
         const float4 q0 = xraw[slot][it][2 * b], q1 = xraw[slot][it][2 * b + 1];
         const bool in0 = row_ok && kk < a.k, in1 = row_ok && kk + 4 < a.k;   // k % 4 == 0
-        const float xv[8] = {in0 ? q0.x : 0.0f, in0 ? q0.y : 0.0f, in0 ? q0.z : 0.0f, in0 ? q0.w : 0.0f,
-                             in1 ? q1.x : 0.0f, in1 ? q1.y : 0.0f, in1 ? q1.z : 0.0f, in1 ? q1.w : 0.0f};
+        const float rv = s_rinv[it];                       // exact: a power of two
+        const float xv[8] = {in0 ? q0.x * rv : 0.0f, in0 ? q0.y * rv : 0.0f, in0 ? q0.z * rv : 0.0f, in0 ? q0.w * rv : 0.0f,
+                             in1 ? q1.x * rv : 0.0f, in1 ? q1.y * rv : 0.0f, in1 ? q1.z * rv : 0.0f, in1 ? q1.w * rv : 0.0f};
         v8h hi, lo;
         float sum = b ? xsum[it] : 0.0f;
 #pragma unroll
@@ -429,9 +435,10 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
         for (int r = 0; r < 16; r++) {
             const uint32_t row = m0 + (wm * RT + i) * 32 + 8 * (r / 4) + 4 * kb + (r % 4);
             if (row >= a.m) continue;
+            const float rf = lds_rf[row - m0];             // back to the row's own scale: exact, a power of two
             float o[TN];
 #pragma unroll
-            for (int j = 0; j < TN; j++) o[j] = fmaf(acc[i][j][r], flt_of(sc_cur, j), bv[j]);
+            for (int j = 0; j < TN; j++) o[j] = fmaf(acc[i][j][r] * rf, flt_of(sc_cur, j), bv[j]);
             float* p = dst + (uint64_t)row * a.n + colbase;
             if (TN == 4) *reinterpret_cast<float4*>(p) = make_float4(o[0], o[1], o[2], o[TN - 1]);
             else *reinterpret_cast<float2*>(p) = make_float2(o[0], o[1]);
@@ -482,6 +489,46 @@ static uint32_t pick_splits(uint32_t tiles, uint32_t nstages, uint32_t* stages_p
 // xp[r][j] = x[r][perm[j]] (perm null: j) for j < k, 0 for k <= j < k4: the act-order column
 // gather done once per call instead of once per workgroup column, and the padding / alignment
 // of rows that the tile kernel's 128-bit loads need.
+// One workgroup per row of x: rinv[row] = 2^(141 - E) for a largest magnitude a * 2^(E - 127), 1 <= a < 2, so that
+// the scaled row lies in [2^14, 2^15) -- inside the range of f16 whatever the row's own size, and with its small
+// elements' low halves clear of f16's subnormals -- and rfac[row] = 1 / rinv[row].  Both are powers of two: scaling
+// by them is exact, so rows that needed none give the bits they gave without.  A row of zeros, or one that holds
+// an infinity or a NaN (which poisons the row's results, as it should), keeps the factor 1.
+// amax: bits of the row's largest magnitude.  2^(141 - E) has the biased exponent 268 - e; kept within [14, 240] so
+// that both factors are normal numbers (rows below 2^-99 are scaled by 2^113 only: they stay far inside f16's
+// range all the same).  Returns the bits of rinv; rfac has the biased exponent 254 minus that one.
+__device__ __forceinline__ uint32_t w4_row_factor_exponent(uint32_t amax) {
+    const uint32_t e = amax >> 23;                           // biased exponent of the largest magnitude
+    return e == 0 || e == 255 ? 127u : min(268u - e, 240u);
+}
+
+__global__ __launch_bounds__(256) void w4_row_factor_kernel(const float* __restrict__ x, uint32_t k,
+                                                            float* __restrict__ rinv, float* __restrict__ rfac) {
+    __shared__ uint32_t part[4];
+    const uint32_t tid = threadIdx.x, row = blockIdx.x;
+    const float* xr = x + (uint64_t)row * k;
+    uint32_t amax = 0;                                       // bit patterns of |x| order like the values; NaN sorts last
+    if (k % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+        for (uint32_t i = tid; i < k / 4; i += 256) {
+            const float4 v = reinterpret_cast<const float4*>(xr)[i];
+            amax = max(max(amax, __float_as_uint(v.x) & 0x7FFFFFFFu), __float_as_uint(v.y) & 0x7FFFFFFFu);
+            amax = max(max(amax, __float_as_uint(v.z) & 0x7FFFFFFFu), __float_as_uint(v.w) & 0x7FFFFFFFu);
+        }
+    } else {
+        for (uint32_t i = tid; i < k; i += 256) amax = max(amax, __float_as_uint(xr[i]) & 0x7FFFFFFFu);
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) amax = max(amax, (uint32_t)__shfl_xor((int)amax, o));
+    if ((tid & 63) == 0) part[tid >> 6] = amax;
+    __syncthreads();
+    if (tid == 0) {
+        amax = max(max(part[0], part[1]), max(part[2], part[3]));
+        const uint32_t b = w4_row_factor_exponent(amax);
+        rinv[row] = __uint_as_float(b << 23);
+        rfac[row] = __uint_as_float((254u - b) << 23);
+    }
+}
+
 __global__ __launch_bounds__(256) void w4_prepare_x_kernel(const float* __restrict__ x,
                                                            const int32_t* __restrict__ perm,
                                                            float* __restrict__ xp, uint32_t k, uint32_t k4) {
@@ -503,7 +550,7 @@ __global__ __launch_bounds__(256) void w4_convert_x_kernel(const float* __restri
                                                            const int32_t* __restrict__ perm,
                                                            uint8_t* __restrict__ xh, uint8_t* __restrict__ xl,
                                                            float* __restrict__ xs, uint32_t m, uint32_t k,
-                                                           uint32_t xsteps) {
+                                                           uint32_t xsteps, const float* __restrict__ rinv) {
     const uint32_t tid = threadIdx.x, row = tid >> 3, kblk = tid & 7;
     const uint32_t tile = blockIdx.y, step = blockIdx.x * 4 + (kblk >> 1), kb = kblk & 1;
     const uint32_t grow = tile * 32 + row, k0 = step * 16 + kb * 8;
@@ -525,10 +572,11 @@ __global__ __launch_bounds__(256) void w4_convert_x_kernel(const float* __restri
     }
     v8h hi, lo;
     float sum = 0.0f;
+    const float rv = rinv[min(grow, m - 1)];                 // exact: a power of two
 #pragma unroll
     for (int e = 0; e < 8; e++) {
         const int j = (e >> 1) + 4 * (e & 1);                // fragment element e holds k offset j
-        const float v = xv[j];
+        const float v = xv[j] * rv;
         const _Float16 h = (_Float16)v;
         hi[e] = h;
         lo[e] = (_Float16)(v - (float)h);                    // hi + lo equals v to 2^-22 |v|
@@ -541,17 +589,21 @@ __global__ __launch_bounds__(256) void w4_convert_x_kernel(const float* __restri
     if (kb == 0) xs[blk * 32 + row] = sum;
 }
 
-// The same planes for act-order weights (x[row][perm[j]]).  Gathered from global memory a wave instruction
-// touches 64 cache lines for 256 bytes; here a workgroup copies `rows` whole rows of x into LDS with
-// contiguous reads and gathers from there.  Thread = (row, MFMA step): 16 values, both k blocks of the step.
+// The same planes from whole rows: a workgroup copies `rows` rows of x into LDS with contiguous reads, finds each
+// row's factor there (no pass of its own over x, no launch of its own) and converts from LDS.  With act-order
+// weights (x[row][perm[j]]) the gather happens in LDS too: from global memory a wave instruction would touch 64
+// cache lines for 256 bytes.  Thread = (row, MFMA step): 16 values, both k blocks of the step.
 // Dynamic LDS: rows * kpad floats, kpad = k rounded up to 4.
-__global__ __launch_bounds__(256) void w4_convert_x_perm_kernel(const float* __restrict__ x,
+__global__ __launch_bounds__(256) void w4_convert_x_rows_kernel(const float* __restrict__ x,
                                                                 const int32_t* __restrict__ perm,
                                                                 uint8_t* __restrict__ xh, uint8_t* __restrict__ xl,
                                                                 float* __restrict__ xs, uint32_t m, uint32_t k,
-                                                                uint32_t xsteps, uint32_t rows, uint32_t kpad) {
+                                                                uint32_t xsteps, uint32_t rows, uint32_t kpad,
+                                                                float* __restrict__ rfac) {
     extern __shared__ __attribute__((aligned(16))) float lds_rows[];
+    __shared__ uint32_t rowmax[8];
     const uint32_t tid = threadIdx.x;
+    if (tid < 8) rowmax[tid] = 0;
     const uint32_t row0 = blockIdx.x * rows;                  // rows divides 32: a workgroup stays inside a row tile
     const uint32_t live = row0 < m ? min(rows, m - row0) : 0;
     const float* src = x + (uint64_t)row0 * k;
@@ -566,10 +618,27 @@ __global__ __launch_bounds__(256) void w4_convert_x_perm_kernel(const float* __r
     __syncthreads();
     const uint32_t r = tid % rows, grow = row0 + r, tile = grow / 32, row = grow % 32;
     const float* lr = lds_rows + r * kpad;
+    // the row's factor (w4_row_factor_kernel's), from the copy in LDS
+    {
+        uint32_t am = 0;
+        if (grow < m)
+            for (uint32_t i = tid / rows; i < k; i += 256 / rows) am = max(am, __float_as_uint(lr[i]) & 0x7FFFFFFFu);
+        atomicMax(&rowmax[r], am);
+    }
+    __syncthreads();
+    const uint32_t fb = w4_row_factor_exponent(rowmax[r]);
+    const float rv = __uint_as_float(fb << 23);               // exact: a power of two
+    if (tid < rows && grow < m) rfac[grow] = __uint_as_float((254u - fb) << 23);
     for (uint32_t step = tid / rows; step < xsteps; step += 256 / rows) {
         const uint32_t k0 = step * 16;
         float xv[16];
-        if (grow < m && k0 + 16 <= k && (reinterpret_cast<uintptr_t>(perm) & 15) == 0) {
+        if (!perm && grow < m && k0 + 16 <= k) {             // plain order: kpad % 4 == 0, so the row is aligned
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const float4 v = *reinterpret_cast<const float4*>(lr + k0 + 4 * q);
+                xv[4 * q] = v.x; xv[4 * q + 1] = v.y; xv[4 * q + 2] = v.z; xv[4 * q + 3] = v.w;
+            }
+        } else if (perm && grow < m && k0 + 16 <= k && (reinterpret_cast<uintptr_t>(perm) & 15) == 0) {
             int4 pj[4];
 #pragma unroll
             for (int q = 0; q < 4; q++) pj[q] = *reinterpret_cast<const int4*>(perm + k0 + 4 * q);
@@ -582,7 +651,7 @@ __global__ __launch_bounds__(256) void w4_convert_x_perm_kernel(const float* __r
 #pragma unroll
             for (int j = 0; j < 16; j++) {
                 const bool in = grow < m && k0 + j < k;
-                const float v = lr[in ? (uint32_t)perm[k0 + j] : 0];
+                const float v = lr[in ? (perm ? (uint32_t)perm[k0 + j] : k0 + j) : 0];
                 xv[j] = in ? v : 0.0f;
             }
         }
@@ -595,7 +664,7 @@ __global__ __launch_bounds__(256) void w4_convert_x_perm_kernel(const float* __r
 #pragma unroll
             for (int e = 0; e < 8; e++) {
                 const int j = (e >> 1) + 4 * (e & 1);            // fragment element e holds k offset j
-                const float v = xv[8 * kb + j];
+                const float v = xv[8 * kb + j] * rv;
                 const _Float16 h = (_Float16)v;
                 hi[e] = h;
                 lo[e] = (_Float16)(v - (float)h);
@@ -608,7 +677,7 @@ __global__ __launch_bounds__(256) void w4_convert_x_perm_kernel(const float* __r
     }
 }
 
-// rows of x per workgroup of w4_convert_x_perm_kernel (a power of two up to 8), 0: k too long for LDS
+// rows of x per workgroup of w4_convert_x_rows_kernel (a power of two up to 8), 0: k too long for LDS
 static uint32_t convert_perm_rows(uint32_t kpad) {
     const uint32_t fit = (64u * 1024) / (kpad * 4);
     return fit >= 8 ? 8 : fit >= 4 ? 4 : fit >= 2 ? 2 : fit;
@@ -635,25 +704,35 @@ static int launch_tile(const W4Args& a_in, hipStream_t s) {
     const size_t x_bytes = PRE ? 2 * plane_bytes + sums_bytes
                                : prepare ? (((size_t)a.m * k4 * sizeof(float) + 255) & ~size_t(255)) : 0;
     const size_t part_bytes = splits > 1 ? (size_t)splits * a.m * a.n * sizeof(float) : 0;
+    const size_t fac_bytes = ((size_t)2 * a.m * sizeof(float) + 255) & ~size_t(255);   // rinv[m], rfac[m]
     float* out = a.y;
     WorkspaceLease lease;                                    // until the last kernel of this call is queued
-    if (x_bytes + part_bytes) {
+    {
         void* ws = nullptr;
-        if (int rc = workspace_get(s, x_bytes + part_bytes, &ws, lease)) return rc;
+        if (int rc = workspace_get(s, fac_bytes + x_bytes + part_bytes, &ws, lease)) return rc;
+        float* fac = static_cast<float*>(ws);
+        ws = static_cast<uint8_t*>(ws) + fac_bytes;
+        a.rinv = fac;
+        a.rfac = fac + a.m;
+        // the pre-converting kernel that holds whole rows in LDS finds the factors itself
+        if (!(PRE && a.perm && convert_perm_rows(k4))) {
+            hipLaunchKernelGGL(w4_row_factor_kernel, dim3(a.m), dim3(256), 0, s, a.x, a.k, fac, fac + a.m);
+            if (int rc = check_launch("w4_row_factor_kernel")) return rc;
+        }
         if (PRE) {
             uint8_t* base = static_cast<uint8_t*>(ws);
             const bool vec = !a.perm && a.k % 8 == 0 && (reinterpret_cast<uintptr_t>(a.x) & 15) == 0;
             const dim3 grid(xsteps / 4, xtiles);
             float* sums = reinterpret_cast<float*>(base + 2 * plane_bytes);
-            const uint32_t perm_rows = a.perm ? convert_perm_rows(k4) : 0;
+            const uint32_t perm_rows = a.perm ? convert_perm_rows(k4) : 0;   // 0: a row does not fit LDS
             if (perm_rows)
-                hipLaunchKernelGGL(w4_convert_x_perm_kernel, dim3(xtiles * 32 / perm_rows), dim3(256),
+                hipLaunchKernelGGL(w4_convert_x_rows_kernel, dim3(xtiles * 32 / perm_rows), dim3(256),
                                    (size_t)perm_rows * k4 * sizeof(float), s, a.x, a.perm, base, base + plane_bytes, sums,
-                                   a.m, a.k, xsteps, perm_rows, k4);
+                                   a.m, a.k, xsteps, perm_rows, k4, fac + a.m);
             else if (vec) hipLaunchKernelGGL(w4_convert_x_kernel<true>, grid, dim3(256), 0, s, a.x, a.perm, base,
-                                             base + plane_bytes, sums, a.m, a.k, xsteps);
+                                             base + plane_bytes, sums, a.m, a.k, xsteps, a.rinv);
             else hipLaunchKernelGGL(w4_convert_x_kernel<false>, grid, dim3(256), 0, s, a.x, a.perm, base,
-                                    base + plane_bytes, sums, a.m, a.k, xsteps);
+                                    base + plane_bytes, sums, a.m, a.k, xsteps, a.rinv);
             if (int rc = check_launch("w4_convert_x_kernel")) return rc;
             a.xh = base;
             a.xl = base + plane_bytes;
