@@ -211,13 +211,14 @@ __global__ __launch_bounds__(STAGED ? 64 * kI8WK : 64) void w4_i8_prepare_kernel
         mb = max(mb, max_bits(v));
     }
     mb = wave_max(mb);
-    // 2^e with max * 2^e in [2^19, 2^20); tiny values stop at 2^100 (their products vanish in f32 anyway).  A
+    // 2^e with max * 2^e in [2^19, 2^20); e stops at 126, where 2^-e is the smallest normal number, so parts whose
+    // largest magnitude lies below 2^-107 keep fewer than 20 bits.  A
     // non-finite activation poisons its row: the scale becomes NaN (the digits are then whatever the
     // conversion gives; they only ever meet the NaN)
     PSTAMP(2);
     const bool finite = mb < 0x7f800000u;
     int e = 19 - ((int)(mb >> 23) - 127);
-    e = mb == 0 ? 0 : min(e, 100);
+    e = mb == 0 ? 0 : min(e, 126);
     const float f = finite ? __uint_as_float((uint32_t)(e + 127) << 23) : 0.0f;
     if (lane == 0)
         rscale[((uint64_t)rt * kI8WK + share) * 16 + row_l] =

@@ -80,3 +80,81 @@ def test_rows_of_any_magnitude(ops, m, k, n, g, act_order):
         out = host(call(dev(xb)))
         assert np.isnan(out[9]).all()
         np.testing.assert_array_equal(np.delete(out, 9, axis=0), np.delete(got, 9, axis=0))
+
+
+@pytest.mark.parametrize("m", [1, 4, 8, 16, 64, 128])
+@pytest.mark.parametrize("act_order", [False, True])
+def test_few_rows_of_any_magnitude(ops, m, act_order):
+    """Up to 128 rows the kernels turn x into fixed point, 20 bits below the largest magnitude of a part of the row
+    (32 consecutive k for up to 8 rows, an eighth of K beyond): uniformly scaled rows, 1e-30 to 3e33, are as
+    accurate as ordinary ones; in a part that one element dominates the others are rounded to that element's
+    2^-20, so the error there is bounded by max|x| 2^-19 sum|w| rather than by the summed terms."""
+    say(f"w4 forward row scaling m={m} act_order={act_order}")
+    k, n, g = 1024, 1024, 128
+    rng = np.random.default_rng(100 + m)
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    x = rng.normal(0, 1, (8 * m, k)).astype(np.float32)[:m]
+    scale = np.ones(m, np.float32)
+    for r, f in ((1, 1e-12), (2, 1e9), (5, 1e-30), (6, 3e33)):
+        if r < m:
+            scale[r] = f
+    if m == 1:
+        scale[0] = 1e-30
+    x *= scale[:, None]
+    dominated = 3 if m > 3 else None
+    if dominated is not None:
+        x[dominated, 7] = 2.0e5
+    packed, scales, zp = oracle.w4_from_f32(w, g)
+    d = [dev(a) for a in (packed, scales, zp)]
+    if act_order:
+        perm_np = rng.permutation(k).astype(np.int32)
+        perm = dev(perm_np)
+        xs = x[:, perm_np]
+        got = host(ops.qmatmul_int4_perm(dev(x), *d, k, g, perm=perm))
+    else:
+        xs = x
+        got = host(ops.qmatmul_int4(dev(x), *d, k, g))
+    deq = oracle.w4_dequant(packed, scales, zp, k, g).astype(np.float64)
+    exact = xs.astype(np.float64) @ deq
+    terms = np.abs(xs).astype(np.float64) @ np.abs(deq) + 1e-300
+    assert np.isfinite(got).all()
+    rel = np.abs(got - exact) / terms
+    plain = [r for r in range(m) if r != dominated]
+    assert rel[plain].max() < 2e-6, rel[plain].max(axis=1)
+    if dominated is not None:
+        q = oracle.w4_unpack(packed, k).astype(np.float64)
+        rows_of_group = np.repeat(np.arange(scales.shape[0]), g)[:k]
+        factored = np.abs(xs[dominated]).astype(np.float64) @ ((q + np.abs(zp[rows_of_group])) * scales[rows_of_group])
+        bound = 2.0e5 * 2.0 ** -19 * np.abs(deq).sum(axis=0) + 2e-6 * factored
+        assert (np.abs(got[dominated] - exact[dominated]) <= bound).all()
+
+
+@pytest.mark.parametrize("m", [1, 4, 8, 64, 512])
+@pytest.mark.parametrize("bs", [32, 128, 1024])
+def test_q8_matmul_rows_of_any_magnitude(ops, m, bs):
+    """f32 x Q8 (matmul_q8.wgsl:37-98) through every route (vector kernels, digit planes on the int8 matrix cores,
+    f16 matrix cores per block): rows from 1e-30 to 3e33 and a row with one element of 2e5, in units of the summed
+    terms."""
+    say(f"matmul_q8 row scaling m={m} bs={bs}")
+    k, n = 1024, 1024
+    rng = np.random.default_rng(200 + m + bs)
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    x = rng.normal(0, 1, (8 * m, k)).astype(np.float32)[:m]
+    for r, f in ((1, 1e-12), (2, 1e9), (5, 1e-30), (6, 3e33)):
+        if r < m:
+            x[r] *= np.float32(f)
+    if m == 1:
+        x[0] *= np.float32(1e-30)
+    if m > 3:
+        x[3, 7] = 2.0e5
+    words = ops.q8_quantize(ops.transpose_f32(dev(w)).reshape(-1), bs)
+    wd = host(ops.q8_dequantize_kn(words, k, n, bs)).astype(np.float64)
+    got = host(ops.matmul_q8(dev(x), words, k, n, bs))
+    exact = x.astype(np.float64) @ wd
+    terms = np.abs(x).astype(np.float64) @ np.abs(wd) + 1e-300
+    assert np.isfinite(got).all()
+    rel = np.abs(got - exact) / terms
+    plain = [r for r in range(m) if r != 3]
+    assert rel[plain].max() < 2e-6
+    if m > 3:                                            # the dominated row: digit planes below the row part's maximum
+        assert rel[3].max() < 2e-4
