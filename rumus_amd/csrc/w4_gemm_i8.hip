@@ -5,14 +5,15 @@
 // Inside a group only x and the raw nibbles meet, and a nibble is already an int8 operand: a packed
 // word becomes two operand registers with three instructions (w & 0x0f0f0f0f, (w >> 4) & 0x0f0f0f0f),
 // where the f16 path spends nine per word.  The f32 activations cannot enter an integer MFMA, so a
-// small kernel first writes them as fixed point: X = rint(x * 2^e) with |X| <= 2^20 relative to the
+// small kernel first writes them as fixed point: X = rint(x * 2^e) with |X| < 2^22 relative to the
 // largest magnitude of the row's eighth of K (the part one wave of the matmul multiplies), split into
-// three signed digits X = d0 + 128 d1 + 16384 d2, one int8 plane each, stored in the order the MFMA's A
-// operand wants, plus the sum of X over every chunk of 64 or 128 k; a gather through `perm` (act-order)
-// happens there too.  Every product and every sum over a chunk is then an exact integer
-// (v_mfma_i32_16x16x64_i8, three per weight fragment); the three i32 tiles are put together with two
-// shift-adds and leave the integer domain once per chunk: one conversion and one multiply-add with the
-// group's scale.  The zero-point term is a small matrix product of its own, chunk sums of X times
+// three signed digits X = d0 + 256 d1 + 65536 d2 (|d0|, |d1| <= 128, |d2| <= 64), one int8 plane each,
+// stored in the order the MFMA's A operand wants, plus the sum of X over every chunk of 64 or 128 k; a
+// gather through `perm` (act-order) happens there too.  Every product and every sum over a chunk is then
+// an exact integer (v_mfma_i32_16x16x64_i8, three per weight fragment); the two low tiles are put
+// together with a shift-add (below 2^26), the high one joins them in f32 (its weight, 2^16 times up to
+// 64 * 15 * 128, does not fit 32 bits) -- one rounding of 2^-24 of the chunk's sum -- and one
+// multiply-add applies the group's scale.  The zero-point term is a small matrix product of its own, chunk sums of X times
 // -scale * zero-point, on v_mfma_f32_16x16x4_f32 once per round of chunks.
 //
 // A workgroup owns 16*Q columns over all of K for one block of 16*RT rows; its eight waves take an
@@ -211,13 +212,13 @@ __global__ __launch_bounds__(STAGED ? 64 * kI8WK : 64) void w4_i8_prepare_kernel
         mb = max(mb, max_bits(v));
     }
     mb = wave_max(mb);
-    // 2^e with max * 2^e in [2^19, 2^20); e stops at 126, where 2^-e is the smallest normal number, so parts whose
+    // 2^e with max * 2^e in [2^21, 2^22); e stops at 126, where 2^-e is the smallest normal number, so parts whose
     // largest magnitude lies below 2^-107 keep fewer than 20 bits.  A
     // non-finite activation poisons its row: the scale becomes NaN (the digits are then whatever the
     // conversion gives; they only ever meet the NaN)
     PSTAMP(2);
     const bool finite = mb < 0x7f800000u;
-    int e = 19 - ((int)(mb >> 23) - 127);
+    int e = 21 - ((int)(mb >> 23) - 127);
     e = mb == 0 ? 0 : min(e, 126);
     const float f = finite ? __uint_as_float((uint32_t)(e + 127) << 23) : 0.0f;
     if (lane == 0)
@@ -229,11 +230,11 @@ __global__ __launch_bounds__(STAGED ? 64 * kI8WK : 64) void w4_i8_prepare_kernel
         int d[3][8], sum = 0;
 #pragma unroll
         for (int j = 0; j < 8; j++) {
-            const int X = (int)__float_as_uint(fmaf(v[j], f, 12582912.0f)) - 0x4b400000;   // |X| <= 2^20
-            const int X1 = (X + 64) >> 7;
-            d[0][j] = __builtin_amdgcn_sbfe(X, 0, 7);              // X - 128 * X1
-            d[1][j] = __builtin_amdgcn_sbfe(X1, 0, 7);             // X1 - 128 * d2
-            d[2][j] = (X1 + 64) >> 7;                              // |d2| <= 64
+            const int X = (int)__float_as_uint(fmaf(v[j], f, 12582912.0f)) - 0x4b400000;   // |X| < 2^22
+            const int X1 = (X + 128) >> 8;
+            d[0][j] = __builtin_amdgcn_sbfe(X, 0, 8);              // X - 256 * X1
+            d[1][j] = __builtin_amdgcn_sbfe(X1, 0, 8);             // X1 - 256 * d2
+            d[2][j] = (X1 + 128) >> 8;                             // |d2| <= 64
             sum += X;
         }
         sum = group_sum<SUBS>(sum);                                  // whole chunks are in or out together
@@ -397,11 +398,11 @@ __global__ __launch_bounds__(512) void w4_gemm_i8_kernel(W4I8Args a) {
                 for (int q = 0; q < Q; q++)
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
-                        // exact: |d2 part| <= 128*64*15 * 2^14 < 2^31 - the rest
-                        int low = (acc[q][1][i] << 7) + acc[q][0][i];
-                        asm("" : "+v"(low));              // two shift-adds, not two shifts and a three-way add
-                        const int tot = (acc[q][2][i] << 14) + low;
-                        accf[t][q][i] = fmaf(sc[q], (float)tot, accf[t][q][i]);
+                        // |low| <= 128 * 15 * 128 * 257 < 2^26 is exact; the high digits' tile times 2^16 passes 2^31,
+                        // so it joins in f32: exact by itself, one rounding in the sum
+                        const int low = (acc[q][1][i] << 8) + acc[q][0][i];
+                        const float tot = fmaf((float)acc[q][2][i], 65536.0f, (float)low);
+                        accf[t][q][i] = fmaf(sc[q], tot, accf[t][q][i]);
                     }
             }
 #ifdef RUMUS_TIMERS
