@@ -677,6 +677,72 @@ __global__ __launch_bounds__(256) void w4_convert_x_rows_kernel(const float* __r
     }
 }
 
+// The same planes for plain x (no gather, k % 8 == 0, 16-byte aligned rows) in one pass over x and no launch for the
+// factors: a workgroup takes four rows, thread (row t % 4, step t / 4 + 64 i) keeps its ITER steps of 16 values in
+// registers between finding the row's largest magnitude and writing the planes.  ITER = ceil(xsteps / 64) up to 16
+// (K up to 16384).
+template <int ITER>
+__global__ __launch_bounds__(256) void w4_convert_x_regs_kernel(const float* __restrict__ x, uint8_t* __restrict__ xh,
+                                                                uint8_t* __restrict__ xl, float* __restrict__ xs,
+                                                                float* __restrict__ rfac, uint32_t m, uint32_t k,
+                                                                uint32_t xsteps) {
+    __shared__ uint32_t rowmax[4];
+    const uint32_t tid = threadIdx.x, r = tid & 3, s0 = tid >> 2;
+    const uint32_t grow = blockIdx.x * 4 + r, tile = grow >> 5, row = grow & 31;
+    const bool live = grow < m;
+    const float* xr = x + (uint64_t)(live ? grow : 0) * k;
+    if (tid < 4) rowmax[tid] = 0;
+    float4 v[ITER][4];
+    uint32_t am = 0;
+#pragma unroll
+    for (int i = 0; i < ITER; i++) {
+        const uint32_t k0 = (s0 + 64 * i) * 16;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const uint32_t kk = k0 + 4 * q;
+            const bool in = live && kk < k;                  // k % 4 == 0: a float4 is all in or all out
+            const float4 f = *reinterpret_cast<const float4*>(xr + (in ? kk : 0));
+            v[i][q] = in ? f : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            am = max(max(am, __float_as_uint(v[i][q].x) & 0x7FFFFFFFu), __float_as_uint(v[i][q].y) & 0x7FFFFFFFu);
+            am = max(max(am, __float_as_uint(v[i][q].z) & 0x7FFFFFFFu), __float_as_uint(v[i][q].w) & 0x7FFFFFFFu);
+        }
+    }
+#pragma unroll
+    for (int o = 4; o <= 32; o <<= 1) am = max(am, (uint32_t)__shfl_xor((int)am, o));   // the lanes of this row
+    __syncthreads();                                         // rowmax is zeroed
+    if ((tid & 63) < 4) atomicMax(&rowmax[r], am);
+    __syncthreads();
+    const uint32_t fb = w4_row_factor_exponent(rowmax[r]);
+    const float rv = __uint_as_float(fb << 23);              // exact: a power of two
+    if (tid < 4 && live) rfac[grow] = __uint_as_float((254u - fb) << 23);
+#pragma unroll
+    for (int i = 0; i < ITER; i++) {
+        const uint32_t step = s0 + 64 * i;
+        if (step >= xsteps) break;
+        const uint64_t blk = (uint64_t)tile * xsteps + step;
+        const float xv[16] = {v[i][0].x, v[i][0].y, v[i][0].z, v[i][0].w, v[i][1].x, v[i][1].y, v[i][1].z, v[i][1].w,
+                              v[i][2].x, v[i][2].y, v[i][2].z, v[i][2].w, v[i][3].x, v[i][3].y, v[i][3].z, v[i][3].w};
+        float sum[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+            v8h hi, lo;
+            sum[kb] = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const int j = (e >> 1) + 4 * (e & 1);        // fragment element e holds k offset j
+                const float t = xv[8 * kb + j] * rv;
+                const _Float16 h = (_Float16)t;
+                hi[e] = h;
+                lo[e] = (_Float16)(t - (float)h);
+                sum[kb] += t;
+            }
+            *reinterpret_cast<v8h*>(xh + (blk * 64 + kb * 32 + row) * 16) = hi;
+            *reinterpret_cast<v8h*>(xl + (blk * 64 + kb * 32 + row) * 16) = lo;
+        }
+        xs[blk * 32 + row] = sum[0] + sum[1];                // the order of w4_convert_x_kernel: eight and eight
+    }
+}
+
 // rows of x per workgroup of w4_convert_x_rows_kernel (a power of two up to 8), 0: k too long for LDS
 static uint32_t convert_perm_rows(uint32_t kpad) {
     const uint32_t fit = (64u * 1024) / (kpad * 4);
@@ -714,8 +780,12 @@ static int launch_tile(const W4Args& a_in, hipStream_t s) {
         ws = static_cast<uint8_t*>(ws) + fac_bytes;
         a.rinv = fac;
         a.rfac = fac + a.m;
-        // the pre-converting kernel that holds whole rows in LDS finds the factors itself
-        if (!(PRE && a.perm && convert_perm_rows(k4))) {
+        // the pre-converting kernels that hold whole rows (in LDS for the gather, in registers for plain x) find
+        // the factors themselves
+        const bool vec8 = !a.perm && a.k % 8 == 0 && (reinterpret_cast<uintptr_t>(a.x) & 15) == 0;
+        const uint32_t regs_iter = PRE && vec8 ? ceil_div(xsteps, 64u) : 0;   // steps of 16 k per thread
+        const bool in_regs = regs_iter >= 1 && regs_iter <= 16;
+        if (!(PRE && ((a.perm && convert_perm_rows(k4)) || in_regs))) {
             hipLaunchKernelGGL(w4_row_factor_kernel, dim3(a.m), dim3(256), 0, s, a.x, a.k, fac, fac + a.m);
             if (int rc = check_launch("w4_row_factor_kernel")) return rc;
         }
@@ -725,7 +795,16 @@ static int launch_tile(const W4Args& a_in, hipStream_t s) {
             const dim3 grid(xsteps / 4, xtiles);
             float* sums = reinterpret_cast<float*>(base + 2 * plane_bytes);
             const uint32_t perm_rows = a.perm ? convert_perm_rows(k4) : 0;   // 0: a row does not fit LDS
-            if (perm_rows)
+            if (in_regs) {
+                const dim3 g4(xtiles * 8);                   // four rows each
+#define RUMUS_W4_REGS(N) hipLaunchKernelGGL(w4_convert_x_regs_kernel<N>, g4, dim3(256), 0, s, a.x, base, base + plane_bytes, \
+                                            sums, fac + a.m, a.m, a.k, xsteps)
+                if (regs_iter <= 4) RUMUS_W4_REGS(4);
+                else if (regs_iter <= 8) RUMUS_W4_REGS(8);
+                else if (regs_iter <= 11) RUMUS_W4_REGS(11);
+                else RUMUS_W4_REGS(16);
+#undef RUMUS_W4_REGS
+            } else if (perm_rows)
                 hipLaunchKernelGGL(w4_convert_x_rows_kernel, dim3(xtiles * 32 / perm_rows), dim3(256),
                                    (size_t)perm_rows * k4 * sizeof(float), s, a.x, a.perm, base, base + plane_bytes, sums,
                                    a.m, a.k, xsteps, perm_rows, k4, fac + a.m);

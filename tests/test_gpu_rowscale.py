@@ -17,11 +17,12 @@ def ops():
 
 # the workgroup shapes of the f16 kernel: 32-row tiles that convert x themselves (plain, through the gathered copy,
 # ragged), 64-row tiles on pre-converted planes (gathered through LDS, 128-bit reads, element-wise reads), and their
-# four-wave form
+# four-wave form; the last two: more steps of K per thread of the kernel that converts plain x from registers
 @pytest.mark.parametrize("m,k,n,g,act_order", [(160, 512, 1024, 128, False), (520, 1024, 1536, 128, False),
                                                (300, 512, 512, 64, True), (136, 520, 516, 32, False),
                                                (600, 1024, 2048, 128, True), (600, 1024, 2048, 128, False),
-                                               (600, 1028, 2048, 128, False), (1024, 256, 11008, 128, False)])
+                                               (600, 1028, 2048, 128, False), (1024, 256, 11008, 128, False),
+                                               (600, 8192, 2048, 128, False), (600, 14336, 2048, 128, False)])
 def test_rows_of_any_magnitude(ops, m, k, n, g, act_order):
     """Batches beyond 128 rows split x into two f16 planes: every row is first scaled by a power of two into
     f16's range, so rows of 1e-12, rows of 1e9 and a row with one element of 2e5 (beyond f16's 65504) come
