@@ -354,6 +354,25 @@ int rumus_hip_qmatmul_int4_decode_swiglu(const float* gate_up, const uint32_t* p
                                          uint32_t n, uint32_t padded_k, uint32_t group_size,
                                          uint32_t num_groups, rumus_hip_stream_t stream);
 
+/* EXTENSION: the decode projection with the neighbouring operators of a
+ * pre-norm decoder block folded in, so that a decode step launches no kernel
+ * for them:
+ *   norm_weight non-NULL: x [m, k] goes through RMSNorm first,
+ *       x * rsqrt(mean(x^2) + eps) * norm_weight (what rumus_hip_rmsnorm computes);
+ *   swiglu != 0: x is gate_up [m, 2k] as in rumus_hip_qmatmul_int4_decode_swiglu
+ *       (norm_weight must be NULL);
+ *   residual non-NULL: residual [m, n] is added to the result (it may be y).
+ * With none of the three it is rumus_hip_qmatmul_int4_decode without perm.
+ * EINVAL unless m <= 8, n % 16 == 0, k % 8 == 0, group_size % 32 == 0, 16-byte
+ * aligned buffers and y != x.  No counterpart in the reference. */
+int rumus_hip_qmatmul_int4_decode_block(const float* x, const float* norm_weight, float eps,
+                                        int swiglu, const uint32_t* packed_t,
+                                        const float* scales_t, const float* zero_points_t,
+                                        const float* bias, const float* residual, float* y,
+                                        uint32_t m, uint32_t k, uint32_t n, uint32_t padded_k,
+                                        uint32_t group_size, uint32_t num_groups,
+                                        rumus_hip_stream_t stream);
+
 /* EXTENSION: qmatmul_int4_perm on AWQ storage: zero-points come as qzeros
  * (layout above) instead of f32.  perm may be NULL (plain k order).
  * EINVAL also unless n % 8 == 0. */

@@ -93,6 +93,12 @@ struct DecoderBlockW4 {
     // (may be null for a prefill that keeps no cache).  pos == 0: causal self-attention over the n tokens, whose
     // keys and values are also written to the caches at 0 .. n-1.  pos > 0: n must be 1; the token's key and value
     // are written at `pos` and it attends positions 0 .. pos.
+    static bool folds(const QLinear& lin, uint32_t rows) {
+        const QuantizedTensor& w = lin.weight;
+        return w.has_decode_layout() && w.perm.size() == 0 && w.k % 8 == 0 &&
+               rows <= rumus_hip_qmatmul_int4_decode_max_rows(w.padded_k, w.n);
+    }
+
     void forward(const float* x, uint32_t batch, uint32_t n, float* y, float* k_cache, float* v_cache,
                  uint32_t cache_len, uint32_t pos, hipStream_t stream = nullptr) const {
         require(batch > 0 && n > 0, "DecoderBlockW4: empty input");
@@ -102,8 +108,21 @@ struct DecoderBlockW4 {
         const uint64_t d = dim;
         DeviceBuffer<float> hn((size_t)rows * d), qkv_out((size_t)rows * 3 * d), att((size_t)rows * d),
             ob((size_t)rows * d), gu((size_t)rows * 2 * ffn), dn((size_t)rows * d);
-        check(rumus_hip_rmsnorm(x, norm1.data(), hn.data(), rows, dim, eps, stream));
-        qkv.forward(hn.data(), rows, qkv_out.data(), stream);
+        // a decode step whose rows suit every projection's decode kernel: the norms, the SwiGLU and the residual adds
+        // ride on the projections (rumus_hip_qmatmul_int4_decode_block), seven launches in all
+        const bool folded = pos != 0 && folds(qkv, rows) && folds(o, rows) && folds(gate_up, rows) && folds(down, rows);
+        auto project = [&](const QLinear& lin, const float* in, const float* norm_w, int swiglu, const float* resid,
+                           float* out) {
+            const QuantizedTensor& w = lin.weight;
+            check(rumus_hip_qmatmul_int4_decode_block(in, norm_w, eps, swiglu, w.packed_t.data(), w.scales_t.data(),
+                                                      w.zp_t.data(), lin.bias.size() ? lin.bias.data() : nullptr, resid,
+                                                      out, rows, w.k, w.n, w.padded_k, w.group_size, w.num_groups, stream));
+        };
+        if (folded) project(qkv, x, norm1.data(), 0, nullptr, qkv_out.data());
+        else {
+            check(rumus_hip_rmsnorm(x, norm1.data(), hn.data(), rows, dim, eps, stream));
+            qkv.forward(hn.data(), rows, qkv_out.data(), stream);
+        }
         const float* q = qkv_out.data();
         const float* k = q + d;
         const float* v = q + 2 * d;
@@ -119,6 +138,13 @@ struct DecoderBlockW4 {
         } else {
             const uint64_t st[12] = {pb, 128, pr, cb, 128, cr, cb, 128, cr, (uint64_t)n * d, 128, d};
             check(rumus_hip_attention(q, k_cache, v_cache, att.data(), batch, h, 1, pos + 1, 128, st, 0, stream));
+        }
+        if (folded) {
+            project(o, att.data(), nullptr, 0, x, ob.data());                   // x1 = x + o
+            project(gate_up, ob.data(), norm2.data(), 0, nullptr, gu.data());
+            project(down, gu.data(), nullptr, 1, ob.data(), y);                 // y = x1 + down(swiglu)
+            check(rumus_hip_sync(stream));   // the temporaries are released on return
+            return;
         }
         o.forward(att.data(), rows, ob.data(), stream);
         // x1 = x + o (kept in `ob`), h2 = rmsnorm(x1) (kept in `hn`)

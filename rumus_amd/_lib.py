@@ -66,6 +66,7 @@ PROTOTYPES = {
     "rumus_hip_w4_decode_layout_zp4": (_i32, [_vp, _vp, _vp, _u32, _u32, _u32, _vp, _vp, _vp, _vp]),
     "rumus_hip_qmatmul_int4_decode_zp4": (_i32, [_vp] * 7 + [_u32] * 6 + [_vp]),
     "rumus_hip_qmatmul_int4_decode_swiglu": (_i32, [_vp] * 6 + [_u32] * 6 + [_vp]),
+    "rumus_hip_qmatmul_int4_decode_block": (_i32, [_vp, _vp, C.c_float, _i32] + [_vp] * 6 + [_u32] * 6 + [_vp]),
     "rumus_hip_qmatmul_int4_zp4": (_i32, [_vp] * 7 + [_u32] * 6 + [_vp]),
     "rumus_hip_qmatmul_int4": (_i32, [_vp] * 7 + [_u32] * 6 + [_vp]),
     "rumus_hip_qmatmul_int4_t": (_i32, [_vp] * 5 + [_u32] * 6 + [_vp]),

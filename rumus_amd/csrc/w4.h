@@ -66,6 +66,9 @@ int w4_launch_gemv(const W4Args& a, hipStream_t s);
 // 16-byte aligned buffers, no g_idx); preferred over the f32 bandwidth kernel.
 bool w4_gemv_dot8_supported(const W4Args& a);
 int w4_launch_gemv_dot8(const W4Args& a, hipStream_t s);
+// the decoder block's forms (decode layout, f32 zero-points, no perm): input through RMSNorm with `norm_w` (or null),
+// or through SwiGLU (a.glu), `resid` (or null) added to the result
+int w4_launch_gemv_dot8_block(const W4Args& a, const float* norm_w, float eps, const float* resid, hipStream_t s);
 
 // f16 MFMA kernel for larger m (needs group_size 32, 64 or a multiple of 128,
 // n % 4 == 0, 16-byte aligned buffers, no g_idx).

@@ -550,6 +550,27 @@ int rumus_hip_qmatmul_int4_decode_swiglu(const float* gate_up, const uint32_t* p
     return w4_launch_gemv_dot8(a, as_stream(stream));
 }
 
+int rumus_hip_qmatmul_int4_decode_block(const float* x, const float* norm_weight, float eps, int swiglu,
+                                        const uint32_t* packed_t, const float* scales_t, const float* zero_points_t,
+                                        const float* bias, const float* residual, float* y, uint32_t m, uint32_t k,
+                                        uint32_t n, uint32_t padded_k, uint32_t group_size, uint32_t num_groups,
+                                        rumus_hip_stream_t stream) {
+    W4Args a{x, packed_t, scales_t, zero_points_t, bias, nullptr, nullptr, y, m, k, n, padded_k, group_size,
+             num_groups, nullptr, true, swiglu != 0};
+    if (int rc = validate(a, "qmatmul_int4_decode_block")) return rc;
+    RUMUS_REQUIRE(!(swiglu && norm_weight), "qmatmul_int4_decode_block: RMSNorm and SwiGLU inputs exclude each other");
+    RUMUS_REQUIRE(n % 16 == 0, "qmatmul_int4_decode_block: n must be a multiple of 16 (got %u)", n);
+    RUMUS_REQUIRE(m <= 8, "qmatmul_int4_decode_block: at most 8 rows (got %u)", m);
+    if (m == 0 || n == 0) return RUMUS_HIP_OK;
+    RUMUS_REQUIRE(k > 0 && k % 8 == 0, "qmatmul_int4_decode_block: k must be a positive multiple of 8 (got %u)", k);
+    RUMUS_REQUIRE(((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(norm_weight)) & 15) == 0,
+                  "qmatmul_int4_decode_block: x and norm_weight must be 16-byte aligned");
+    RUMUS_REQUIRE(y != x, "qmatmul_int4_decode_block: y must not be x (residual may be y)");
+    RUMUS_REQUIRE(w4_gemv_dot8_supported(a),
+                  "qmatmul_int4_decode_block: needs group_size %% 32 == 0 and 16-byte aligned buffers");
+    return w4_launch_gemv_dot8_block(a, norm_weight, eps, residual, as_stream(stream));
+}
+
 int rumus_hip_qmatmul_int4_zp4(const float* x, const uint32_t* packed, const float* scales,
                                const uint32_t* qzeros, const float* bias, const int32_t* perm, float* y,
                                uint32_t m, uint32_t k, uint32_t n, uint32_t padded_k, uint32_t group_size,

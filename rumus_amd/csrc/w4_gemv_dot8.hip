@@ -104,13 +104,30 @@ extern "C" int rumus_dbg_d8_stamps(unsigned long long* host, size_t count) {
 // GLU (with FASTX): `xin` holds rows of 2k floats, gate | up, and the activations are
 // silu(gate) * up computed on the way in: the SwiGLU between a fused gate|up projection and the
 // down projection costs no launch and no round trip of its own.
-template <int M, int T, int OCT, bool FASTX, bool ZP4, bool TILED, bool GLU = false>
+// LDS of the fused norm: the waves' sums of squares per row (only the kernels with the norm allocate it)
+template <int WAVES, int M>
+__device__ __forceinline__ float* d8_sq_lds() {
+    __shared__ float sq[WAVES * M];
+    return sq;
+}
+
+// NORM (with FASTX): the activations are RMSNorm(x) = x * rsqrt(mean(x^2) + eps) * norm_w, the norm folded into the
+// kernel that consumes it: the planes are built from x * norm_w, every lane adds the squares of the x it loads anyway
+// (a workgroup's lanes load each element of the row exactly once), the sums of squares travel with the wave sums
+// through LDS, and rsqrt(...) multiplies the result.  `resid` (or null): y = ... + resid[m][n], the residual add of
+// the decoder block, in the epilogue.
+// BLOCK: the kernel looks at norm_w / eps / resid at all; the plain kernels are launched with nulls there and
+// compile to what they were without these arguments.
+template <int M, int T, int OCT, bool FASTX, bool ZP4, bool TILED, bool GLU = false, bool NORM = false, bool BLOCK = false>
 __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
     const uint32_t* __restrict__ packed, const float* __restrict__ scales,
     const float* __restrict__ zps, const float* __restrict__ xin, float* __restrict__ yout,
     uint32_t n, uint32_t k, uint32_t padded_k, uint32_t group_size,
-    const float* __restrict__ bias, const int32_t* __restrict__ perm) {
+    const float* __restrict__ bias, const int32_t* __restrict__ perm,
+    const float* __restrict__ norm_w, float eps, const float* __restrict__ resid) {
+    static_assert(!NORM || BLOCK, "the norm is one of the block's forms");
     static_assert(OCT == 4 || OCT == 8, "a quad shares 4 or 8 word rows");
+    static_assert(!NORM || (FASTX && !GLU), "the fused norm reads plain rows with 128-bit loads");
     constexpr int RL = T / 4;      // quads per workgroup
     constexpr int WAVES = T / 64;
     constexpr int OPL = OCT / 4;   // word rows prepared per lane
@@ -130,6 +147,11 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
     for (int m = 0; m < M; m++)
 #pragma unroll
         for (int c = 0; c < 4; c++) acc[m][c] = 0.0f;
+    float ssq[NORM ? M : 1];                     // NORM: this lane's sum of squares per row
+    if constexpr (NORM) {
+#pragma unroll
+        for (int m = 0; m < M; m++) ssq[m] = 0.0f;
+    }
     D8_STAMP(0, acc[0][0]);
 
     // every quad runs the same number of sweeps; a dead quad carries scale 0
@@ -178,6 +200,17 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
                     xv[m][t][2] = in ? lo.z : 0.0f; xv[m][t][3] = in ? lo.w : 0.0f;
                     xv[m][t][4] = in ? hi.x : 0.0f; xv[m][t][5] = in ? hi.y : 0.0f;
                     xv[m][t][6] = in ? hi.z : 0.0f; xv[m][t][7] = in ? hi.w : 0.0f;
+                    if constexpr (NORM) {
+                        const float4 wl = *reinterpret_cast<const float4*>(norm_w + kc);
+                        const float4 wh = *reinterpret_cast<const float4*>(norm_w + kc + 4);
+                        const float nw[8] = {wl.x, wl.y, wl.z, wl.w, wh.x, wh.y, wh.z, wh.w};
+#pragma unroll
+                        for (int j = 0; j < 8; j++) {
+                            // a quad past the end of K multiplies chunk 0 again, with scale 0: its x is not the row's
+                            ssq[m] = live ? fmaf(xv[m][t][j], xv[m][t][j], ssq[m]) : ssq[m];
+                            xv[m][t][j] *= nw[j];
+                        }
+                    }
                 } else {
 #pragma unroll
                     for (int j = 0; j < 8; j++) {
@@ -335,6 +368,15 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
 #pragma unroll
             for (int c = 0; c < 4; c++) red[wave][m][(lane - 12) * 4 + c] = acc[m][c];
     }
+    if constexpr (NORM) {
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            float q = ssq[m];
+#pragma unroll
+            for (int o = 32; o >= 1; o >>= 1) q += __shfl_xor(q, o);
+            if (lane == 0) d8_sq_lds<WAVES, M>()[wave * M + m] = q;
+        }
+    }
     D8_STAMP(3, acc[M - 1][3]);                                // reduced over the wave, written to LDS
     __syncthreads();
     D8_STAMP(4, acc[M - 1][3]);                                // barrier passed
@@ -345,7 +387,16 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
             float v = 0.0f;
 #pragma unroll
             for (int wi = 0; wi < WAVES; wi++) v += red[wi][m][c];
+            if constexpr (NORM) {
+                float q = 0.0f;
+#pragma unroll
+                for (int wi = 0; wi < WAVES; wi++) q += d8_sq_lds<WAVES, M>()[wi * M + m];
+                v *= rsqrtf(q / (float)k + eps);
+            }
             if (bias) v += bias[oc];
+            if constexpr (BLOCK) {
+                if (resid) v += resid[(uint64_t)m * n + oc];
+            }
             yout[(uint64_t)m * n + oc] = v;
         }
     }
@@ -371,13 +422,13 @@ static void launch_variant(const W4Args& a, hipStream_t s) {
         if (a.group_size % 64 == 0) {
             hipLaunchKernelGGL((w4_gemv_dot8_kernel<1, 256, 8, true, true, true, false>), dim3(ceil_div(a.n, kD8Cols)),
                                dim3(256), 0, s, a.packed, a.scales, zps, a.x, a.y, a.n, a.k, a.padded_k, a.group_size,
-                               a.bias, a.perm);
+                               a.bias, a.perm, nullptr, 0.0f, nullptr);
             return;
         }
     }
     hipLaunchKernelGGL((w4_gemv_dot8_kernel<M, kD8Threads, kD8Oct, FASTX, ZP4, TILED, GLU>), dim3(ceil_div(a.n, kD8Cols)),
                        dim3(kD8Threads), 0, s, a.packed, a.scales, zps, a.x, a.y, a.n, a.k, a.padded_k,
-                       a.group_size, a.bias, a.perm);
+                       a.group_size, a.bias, a.perm, nullptr, 0.0f, nullptr);
 }
 
 template <int M>
@@ -414,6 +465,37 @@ int w4_launch_gemv_dot8(const W4Args& a, hipStream_t s) {
         case 6: return launch_m<6>(a, s);
         case 7: return launch_m<7>(a, s);
         case 8: return launch_m<8>(a, s);
+    }
+    return set_error(RUMUS_HIP_EINVAL, "w4 gemv: m = %u out of range", a.m);
+}
+
+template <int M>
+static int launch_block_m(const W4Args& a, const float* norm_w, float eps, const float* resid, hipStream_t s) {
+    const dim3 grid(ceil_div(a.n, kD8Cols)), block(kD8Threads);
+#define RUMUS_D8_BLOCK(GLU, NORM)                                                                                      \
+    hipLaunchKernelGGL((w4_gemv_dot8_kernel<M, kD8Threads, kD8Oct, true, false, true, GLU, NORM, true>), grid, block, 0, \
+                       s, a.packed, a.scales, a.zp, a.x, a.y, a.n, a.k, a.padded_k, a.group_size, a.bias,              \
+                       static_cast<const int32_t*>(nullptr), norm_w, eps, resid)
+    if (a.glu) RUMUS_D8_BLOCK(true, false);
+    else if (norm_w) RUMUS_D8_BLOCK(false, true);
+    else RUMUS_D8_BLOCK(false, false);
+#undef RUMUS_D8_BLOCK
+    return check_launch("w4_gemv_dot8_kernel");
+}
+
+// y = f(x) . dequant(W) + bias + resid on the decode layout with f32 zero-points: f = RMSNorm with `norm_w`
+// (a.glu false, norm_w non-null), SwiGLU of gate | up rows (a.glu), or nothing.  The caller has checked the
+// shapes (w4_gemv_dot8_supported, a.tiled, no packed zero-points, no perm, k % 8 == 0, 16-byte aligned x).
+int w4_launch_gemv_dot8_block(const W4Args& a, const float* norm_w, float eps, const float* resid, hipStream_t s) {
+    switch (a.m) {
+        case 1: return launch_block_m<1>(a, norm_w, eps, resid, s);
+        case 2: return launch_block_m<2>(a, norm_w, eps, resid, s);
+        case 3: return launch_block_m<3>(a, norm_w, eps, resid, s);
+        case 4: return launch_block_m<4>(a, norm_w, eps, resid, s);
+        case 5: return launch_block_m<5>(a, norm_w, eps, resid, s);
+        case 6: return launch_block_m<6>(a, norm_w, eps, resid, s);
+        case 7: return launch_block_m<7>(a, norm_w, eps, resid, s);
+        case 8: return launch_block_m<8>(a, norm_w, eps, resid, s);
     }
     return set_error(RUMUS_HIP_EINVAL, "w4 gemv: m = %u out of range", a.m);
 }

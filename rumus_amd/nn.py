@@ -290,6 +290,8 @@ class DecoderBlockW4:
         b, n, d = x.shape
         h = self.heads
         x2 = x.reshape(b * n, d)
+        if k_cache is not None and n == 1 and self._folds(b):
+            return self._decode_folded(x2, b, k_cache, v_cache, pos)
         hn = ops.rmsnorm(x2, self.norm1, self.eps)
         qkv = self.qkv(hn).view(b, n, 3, h, 128)
         q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
@@ -314,5 +316,30 @@ class DecoderBlockW4:
             down = dw(ops.swiglu_rows(gu))
         y = ops.add(x1, down, out=down)
         return y.view(b, n, d), k_out, v_out
+
+    def _folds(self, rows: int) -> bool:
+        """A decode step of few enough rows for every projection's decode kernel, plain weights: the norms, the
+        SwiGLU and the residual adds then ride on the projections (``qmatmul_int4_decode_block``)."""
+        layers = (self.qkv, self.proj["o"], self.gate_up, self.proj["down"])
+        return all(rows <= lin.weight.decode_rows and lin.weight.perm is None and lin.weight.k % 8 == 0
+                   for lin in layers)
+
+    def _decode_folded(self, x2, b, k_cache, v_cache, pos):
+        """The decode step in seven launches: q|k|v on RMSNorm(x), cache append, attention (two), o + x,
+        gate|up on RMSNorm of that, down on SwiGLU + the residual."""
+        h, d = self.heads, self.dim
+
+        def project(lin, x, **kw):
+            w = lin.weight
+            return ops.qmatmul_int4_decode_block(x, *w.decode, w.k, w.group_size, bias=lin.bias, **kw)
+
+        qkv = project(self.qkv, x2, norm_weight=self.norm1, eps=self.eps).view(b, 1, 3, h, 128)
+        q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
+        ops.kv_append(k, v, k_cache, v_cache, pos)
+        att = ops.attention(q, k_cache[:, :pos + 1], v_cache[:, :pos + 1], causal=False)
+        x1 = project(self.proj["o"], att.view(b, d), residual=x2)
+        gu = project(self.gate_up, x1, norm_weight=self.norm2, eps=self.eps)
+        y = project(self.proj["down"], gu, swiglu=True, residual=x1, out=x1)
+        return y.view(b, 1, d), k_cache, v_cache
 
     __call__ = forward

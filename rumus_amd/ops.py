@@ -290,6 +290,30 @@ def qmatmul_int4_decode_swiglu(gate_up, packed_t, scales_t, zp_t, k, group_size,
     return y
 
 
+def qmatmul_int4_decode_block(x, packed_t, scales_t, zp_t, k, group_size, norm_weight=None, eps: float = 1e-6,
+                              swiglu: bool = False, bias=None, residual=None, out=None):
+    """The decode projection with a decoder block's neighbours folded in: ``x`` through RMSNorm with
+    ``norm_weight`` (or, ``swiglu``, ``x`` = gate | up rows of ``2k``), ``residual`` ``[m, n]`` added to the result
+    (it may be ``out``); one launch."""
+    m = x.shape[0]
+    n = packed_t.shape[1]
+    if x.dim() != 2 or x.shape[1] != (2 * k if swiglu else k):
+        raise ValueError("qmatmul_int4_decode_block: x must be [m, k] (gate | up: [m, 2k])")
+    if norm_weight is not None and norm_weight.numel() < k:
+        raise ValueError("qmatmul_int4_decode_block: norm_weight must hold k values")
+    if residual is not None and (residual.dim() != 2 or tuple(residual.shape) != (m, n) or not residual.is_contiguous()):
+        raise ValueError("qmatmul_int4_decode_block: residual must be a contiguous [m, n] tensor")
+    _w4_sizes("qmatmul_int4_decode_block", packed_t, scales_t, zp_t, k, group_size, m, bias, None, out)
+    padded_k, groups = w4_geometry(k, group_size) if group_size > 0 else (k, 0)
+    y = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=x.device)
+    call("rumus_hip_qmatmul_int4_decode_block", _dev(x, torch.float32, "x"), _opt(norm_weight, torch.float32, "norm_weight"),
+         float(eps), 1 if swiglu else 0, _dev(packed_t, torch.int32, "packed_t"), _dev(scales_t, torch.float32, "scales_t"),
+         _dev(zp_t, torch.float32, "zero_points_t"), _opt(bias, torch.float32, "bias"),
+         _opt(residual, torch.float32, "residual"), _dev(y, torch.float32, "y"), m, k, n, padded_k, group_size, groups,
+         _stream())
+    return y
+
+
 def qmatmul_int4_zp4(x, packed, scales, qzeros, k, group_size, bias=None, perm=None, out=None):
     m = x.shape[0]
     n = packed.shape[1]

@@ -65,6 +65,11 @@ extern "C" {
                                                 zero_points_t: *const f32, bias: *const f32, y: *mut f32,
                                                 m: u32, k: u32, n: u32, padded_k: u32, group_size: u32,
                                                 num_groups: u32, s: Stream) -> c_int;
+    pub fn rumus_hip_qmatmul_int4_decode_block(x: *const f32, norm_weight: *const f32, eps: f32, swiglu: c_int,
+                                               packed_t: *const u32, scales_t: *const f32,
+                                               zero_points_t: *const f32, bias: *const f32, residual: *const f32,
+                                               y: *mut f32, m: u32, k: u32, n: u32, padded_k: u32, group_size: u32,
+                                               num_groups: u32, s: Stream) -> c_int;
     pub fn rumus_hip_add_rmsnorm(x: *const f32, delta: *const f32, weight: *const f32, sum: *mut f32, y: *mut f32,
                                  rows: u32, dim: u32, eps: f32, s: Stream) -> c_int;
     pub fn rumus_hip_rmsnorm(x: *const f32, weight: *const f32, y: *mut f32, rows: u32, dim: u32, eps: f32,

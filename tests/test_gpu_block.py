@@ -83,6 +83,48 @@ def test_decode_gemv_with_swiglu_input(ops, m, k, n, g):
         ops.qmatmul_int4_decode_swiglu(dev(gu[:, :k]), pt, st, zt, k, g)
 
 
+@pytest.mark.parametrize("m,k,n,g", [(1, 4096, 4096, 128), (1, 11008, 1024, 128), (3, 512, 48, 64), (5, 264, 16, 256),
+                                     (8, 1024, 272, 32), (2, 5120, 640, 128)])
+def test_decode_projection_with_the_block_folded_in(ops, m, k, n, g):
+    """qmatmul_int4_decode_block: RMSNorm or SwiGLU on the way in, residual on the way out, one launch; against
+    the operators one after the other (oracle), and against the separate kernels."""
+    say(f"qmatmul_int4_decode_block m={m} k={k} n={n} g={g}")
+    rng = np.random.default_rng(3 * m + k + n)
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    x = rng.normal(0, 2, (m, k)).astype(np.float32)
+    if m > 1:
+        x[1] *= 1e-3                                          # rows of different size: the norm is per row
+    nw = rng.normal(1, 0.2, k).astype(np.float32)
+    b = rng.normal(0, 0.01, n).astype(np.float32)
+    r = rng.normal(0, 1, (m, n)).astype(np.float32)
+    packed, scales, zp = oracle.w4_from_f32(w, g)
+    pt, st, zt = ops.w4_decode_layout(dev(packed), dev(scales), dev(zp), g)
+    # RMSNorm -> projection -> + bias + residual
+    hn = oracle.rmsnorm(x, nw, 1e-5).astype(np.float32)
+    want = oracle.qmatmul_int4(hn, packed, scales, zp, k, g, bias=b, threads=8) + r
+    got = host(ops.qmatmul_int4_decode_block(dev(x), pt, st, zt, k, g, norm_weight=dev(nw), eps=1e-5, bias=dev(b),
+                                             residual=dev(r)))
+    close(got, want)
+    # the norm alone, against the two kernels it replaces (the factor meets the sum instead of x: rounding only)
+    two = host(ops.qmatmul_int4_decode(ops.rmsnorm(dev(x), dev(nw), 1e-5), pt, st, zt, k, g))
+    one = host(ops.qmatmul_int4_decode_block(dev(x), pt, st, zt, k, g, norm_weight=dev(nw), eps=1e-5))
+    np.testing.assert_allclose(one, two, rtol=2e-5, atol=2e-5)
+    # SwiGLU -> projection -> residual accumulated in place
+    gu = rng.normal(0, 2, (m, 2 * k)).astype(np.float32)
+    acc = dev(r)
+    out = ops.qmatmul_int4_decode_block(dev(gu), pt, st, zt, k, g, swiglu=True, residual=acc, out=acc)
+    assert out.data_ptr() == acc.data_ptr()
+    plain = host(ops.qmatmul_int4_decode_swiglu(dev(gu), pt, st, zt, k, g))
+    np.testing.assert_array_equal(host(out), plain + r)       # one add per element: the same bits
+    # nothing folded in: the decode kernel itself
+    np.testing.assert_array_equal(host(ops.qmatmul_int4_decode_block(dev(x), pt, st, zt, k, g)),
+                                  host(ops.qmatmul_int4_decode(dev(x), pt, st, zt, k, g)))
+    with pytest.raises(Exception, match="exclude each other"):
+        ops.qmatmul_int4_decode_block(dev(gu), pt, st, zt, k, g, norm_weight=dev(nw), swiglu=True)
+    with pytest.raises(Exception, match="residual must be"):
+        ops.qmatmul_int4_decode_block(dev(x), pt, st, zt, k, g, residual=dev(r[:, :n - 1]))
+
+
 @pytest.mark.parametrize("b,h,nq,nkv,causal", [
     (1, 2, 64, 64, True), (2, 3, 100, 100, True), (1, 2, 70, 70, False), (1, 4, 33, 97, True),
     (2, 32, 1, 2048, False), (3, 2, 1, 1, False), (1, 2, 1, 300, True), (1, 1, 512, 512, True),
