@@ -78,6 +78,12 @@ def test_empty_calls_succeed_without_arrays_and_full_ones_need_them(library):
     assert L.rumus_hip_qmatmul_int4(None, None, None, None, None, None, None, 0, 128, 64, 128, 12, 2, None) == _lib.EINVAL
     assert L.rumus_hip_qmatmul_int4_t(None, None, None, None, None, 0, 128, 64, 128, 64, 2, None) == 0
     assert L.rumus_hip_qmatmul_int4_decode(None, None, None, None, None, None, None, 0, 128, 64, 128, 64, 2, None) == 0
+    assert L.rumus_hip_qmatmul_int4_decode_block(None, None, 1e-6, 0, None, None, None, None, None, None,
+                                                 0, 128, 64, 128, 64, 2, None) == 0
+    assert L.rumus_hip_qmatmul_int4_decode_block(None, None, 1e-6, 0, None, None, None, None, None, None,
+                                                 1, 128, 64, 128, 64, 2, None) == _lib.EINVAL
+    assert L.rumus_hip_qmatmul_int4_decode_block(None, None, 1e-6, 0, None, None, None, None, None, None,
+                                                 9, 128, 64, 128, 64, 2, None) == _lib.EINVAL
     assert L.rumus_hip_matmul_q8(None, None, None, 0, 64, 8, 32, None) == 0
     assert L.rumus_hip_matmul_q8(None, None, None, 1, 64, 8, 32, None) == _lib.EINVAL
     assert L.rumus_hip_matmul_q8(None, None, None, 0, 64, 8, 6, None) == _lib.EINVAL
