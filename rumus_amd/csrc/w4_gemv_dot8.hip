@@ -371,10 +371,12 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
     if constexpr (NORM) {
 #pragma unroll
         for (int m = 0; m < M; m++) {
+            // over the quad, then over the sixteen quads like the column sums: DPP and lane swaps, no LDS crossbar
             float q = ssq[m];
-#pragma unroll
-            for (int o = 32; o >= 1; o >>= 1) q += __shfl_xor(q, o);
-            if (lane == 0) d8_sq_lds<WAVES, M>()[wave * M + m] = q;
+            q += RUMUS_DPP_F(q, kDppXor1);
+            q += RUMUS_DPP_F(q, kDppXor2);
+            q = reduce_row_lanes(q);
+            if (lane == 15) d8_sq_lds<WAVES, M>()[wave * M + m] = q;
         }
     }
     D8_STAMP(3, acc[M - 1][3]);                                // reduced over the wave, written to LDS
