@@ -445,6 +445,23 @@ int rumus_hip_kv_append(const float* k_new, const float* v_new, float* k_cache, 
                         uint32_t pos, uint32_t cache_len, const uint64_t* strides,
                         rumus_hip_stream_t stream);
 
+/* EXTENSION: rumus_hip_kv_append of ONE new token at `pos` followed by
+ * rumus_hip_attention of its query (q_len 1) over positions 0 .. pos, without
+ * the launch for the append: the newest key and value are read from k_new /
+ * v_new and the kernel writes them into the caches on its way.  Same bits in
+ * `out` and in the caches as the two calls.
+ * strides: HOST array of 18 element strides (floats, multiples of 4), {batch,
+ * head, row} for q, k_new, v_new, k_cache, v_cache, out in that order (the row
+ * strides of q, k_new, v_new and out are not used: one row each).
+ * EINVAL unless head_dim == 128, pos < cache_len, 16-byte aligned operands.
+ * Uses the stream's workspace like rumus_hip_attention with q_len == 1
+ * (kv_len = pos + 1).  No counterpart in the reference. */
+int rumus_hip_attention_decode_append(const float* q, const float* k_new, const float* v_new,
+                                      float* k_cache, float* v_cache, float* out, uint32_t batch,
+                                      uint32_t heads, uint32_t head_dim, uint32_t pos,
+                                      uint32_t cache_len, const uint64_t* strides,
+                                      rumus_hip_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -109,7 +109,7 @@ struct DecoderBlockW4 {
         DeviceBuffer<float> hn((size_t)rows * d), qkv_out((size_t)rows * 3 * d), att((size_t)rows * d),
             ob((size_t)rows * d), gu((size_t)rows * 2 * ffn), dn((size_t)rows * d);
         // a decode step whose rows suit every projection's decode kernel: the norms, the SwiGLU and the residual adds
-        // ride on the projections (rumus_hip_qmatmul_int4_decode_block), seven launches in all
+        // ride on the projections (rumus_hip_qmatmul_int4_decode_block), six launches in all
         const bool folded = pos != 0 && folds(qkv, rows) && folds(o, rows) && folds(gate_up, rows) && folds(down, rows);
         auto project = [&](const QLinear& lin, const float* in, const float* norm_w, int swiglu, const float* resid,
                            float* out) {
@@ -128,7 +128,7 @@ struct DecoderBlockW4 {
         const float* v = q + 2 * d;
         const uint64_t pb = (uint64_t)n * 3 * d, pr = 3 * d;                 // fused projection output
         const uint64_t cb = (uint64_t)cache_len * h * 128, cr = (uint64_t)h * 128;   // token-major cache
-        if (k_cache && v_cache) {
+        if (k_cache && v_cache && pos == 0) {
             const uint64_t st[12] = {pb, 128, pr, pb, 128, pr, cb, 128, cr, cb, 128, cr};
             check(rumus_hip_kv_append(k, v, k_cache, v_cache, batch, h, n, 128, pos, cache_len, st, stream));
         }
@@ -136,8 +136,10 @@ struct DecoderBlockW4 {
             const uint64_t st[12] = {pb, 128, pr, pb, 128, pr, pb, 128, pr, (uint64_t)n * d, 128, d};
             check(rumus_hip_attention(q, k, v, att.data(), batch, h, n, n, 128, st, 1, stream));
         } else {
-            const uint64_t st[12] = {pb, 128, pr, cb, 128, cr, cb, 128, cr, (uint64_t)n * d, 128, d};
-            check(rumus_hip_attention(q, k_cache, v_cache, att.data(), batch, h, 1, pos + 1, 128, st, 0, stream));
+            // the cache write of the new token rides on the attention
+            const uint64_t st[18] = {pb, 128, pr, pb, 128, pr, pb, 128, pr, cb, 128, cr, cb, 128, cr, (uint64_t)n * d, 128, d};
+            check(rumus_hip_attention_decode_append(q, k, v, k_cache, v_cache, att.data(), batch, h, 128, pos, cache_len,
+                                                    st, stream));
         }
         if (folded) {
             project(o, att.data(), nullptr, 0, x, ob.data());                   // x1 = x + o

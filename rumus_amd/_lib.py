@@ -81,6 +81,7 @@ PROTOTYPES = {
     "rumus_hip_add": (_i32, [_vp, _vp, _vp, _u64, _vp]),
     "rumus_hip_i8_gemm_workspace_size": (_u64, [_u32, _u32, _u32]),
     "rumus_hip_kv_append": (_i32, [_vp] * 4 + [_u32] * 6 + [C.POINTER(C.c_uint64), _vp]),
+    "rumus_hip_attention_decode_append": (_i32, [_vp] * 6 + [_u32] * 5 + [C.POINTER(C.c_uint64), _vp]),
     "rumus_hip_attention": (_i32, [_vp] * 4 + [_u32] * 5 + [C.POINTER(C.c_uint64), _i32, _vp]),
 }
 

@@ -110,6 +110,12 @@ struct AttnArgs {
     uint32_t batch, heads, q_len, kv_len;
     float scale;
     int causal;
+    // decode with append (attention_decode_kernel only; null otherwise): the newest key / value, position kv_len - 1,
+    // are read from the projection output instead of the cache, and the workgroup of the last slice writes them
+    // into the cache (k, v above, which are writable then)
+    const float* k_new = nullptr;
+    const float* v_new = nullptr;
+    uint64_t kn_sb = 0, kn_sh = 0, vn_sb = 0, vn_sh = 0;
 };
 
 constexpr int kHeadDim = 128;
@@ -389,7 +395,9 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttnArgs a, float
 #pragma unroll
     for (int sweep = 0; sweep < kDecodeSlice / 64; sweep++) {
         const uint32_t jj = sweep * 64 + kq, key = j0 + jj;
-        const float* kp = kb + (uint64_t)min(key, a.kv_len - 1) * a.k_sr + lane4 * 32;
+        const uint32_t kc = min(key, a.kv_len - 1);
+        const float* kp = (a.k_new && kc == a.kv_len - 1) ? a.k_new + b * a.kn_sb + h * a.kn_sh + lane4 * 32
+                                                         : kb + (uint64_t)kc * a.k_sr + lane4 * 32;
         float d = 0.0f;
 #pragma unroll
         for (int i = 0; i < 8; i++) {
@@ -418,7 +426,10 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttnArgs a, float
 #pragma unroll
         for (int u = 0; u < 8; u++) {
             const uint32_t key = j0 + jj + 8 * u;
-            vv[u] = *reinterpret_cast<const float4*>(vb + (uint64_t)min(key, a.kv_len - 1) * a.v_sr + 4 * c4);
+            const uint32_t vc = min(key, a.kv_len - 1);
+            const float* vp = (a.v_new && vc == a.kv_len - 1) ? a.v_new + b * a.vn_sb + h * a.vn_sh
+                                                             : vb + (uint64_t)vc * a.v_sr;
+            vv[u] = *reinterpret_cast<const float4*>(vp + 4 * c4);
             p[u] = key < j1 ? expf(sc[jj + 8 * u] - m) : 0.0f;
         }
 #pragma unroll
@@ -430,6 +441,13 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttnArgs a, float
     }
     *reinterpret_cast<float4*>(&osum[kg][4 * c4]) = o;
     if (c4 == 0) lsum[kg] = l;
+    // the append: no workgroup reads position kv_len - 1 of the cache in this launch
+    if (a.k_new && blockIdx.x == gridDim.x - 1 && tid < 64) {
+        const bool is_v = tid >= 32;
+        const float* src = is_v ? a.v_new + b * a.vn_sb + h * a.vn_sh : a.k_new + b * a.kn_sb + h * a.kn_sh;
+        float* dstc = const_cast<float*>(is_v ? vb + (uint64_t)(a.kv_len - 1) * a.v_sr : kb + (uint64_t)(a.kv_len - 1) * a.k_sr);
+        reinterpret_cast<float4*>(dstc)[tid & 31] = reinterpret_cast<const float4*>(src)[tid & 31];
+    }
     __syncthreads();
     if (tid < kHeadDim) {
         float* dst = part + ((uint64_t)bh * gridDim.x + blockIdx.x) * (kHeadDim + 2);
@@ -617,6 +635,45 @@ int rumus_hip_kv_append(const float* k_new, const float* v_new, float* k_cache, 
     hipLaunchKernelGGL(kv_append_kernel, dim3((uint32_t)((per_batch + 255) / 256), batch, 2), dim3(256), 0,
                        as_stream(stream), a);
     return check_launch("kv_append_kernel");
+}
+
+// kv_append of one token at `pos` and attention of its query over positions 0 .. pos, in the two launches of
+// the decode attention: the newest key / value are read from k_new / v_new and stored by the last slice's workgroup.
+int rumus_hip_attention_decode_append(const float* q, const float* k_new, const float* v_new, float* k_cache,
+                                      float* v_cache, float* out, uint32_t batch, uint32_t heads, uint32_t head_dim,
+                                      uint32_t pos, uint32_t cache_len, const uint64_t* strides,
+                                      rumus_hip_stream_t stream) {
+    RUMUS_REQUIRE((batch == 0 || heads == 0) || (q && k_new && v_new && k_cache && v_cache && out && strides),
+                  "attention_decode_append: null buffer");
+    RUMUS_REQUIRE(head_dim == kHeadDim, "attention_decode_append: head_dim must be %d (got %u)", kHeadDim, head_dim);
+    RUMUS_REQUIRE(pos < cache_len, "attention_decode_append: position %u does not fit a cache of %u", pos, cache_len);
+    if (batch == 0 || heads == 0) return RUMUS_HIP_OK;
+    for (int i = 0; i < 18; i++)
+        RUMUS_REQUIRE(strides[i] % 4 == 0, "attention_decode_append: stride %d (%llu) must be a multiple of 4 floats", i,
+                      (unsigned long long)strides[i]);
+    RUMUS_REQUIRE(((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k_new) | reinterpret_cast<uintptr_t>(v_new) |
+                    reinterpret_cast<uintptr_t>(k_cache) | reinterpret_cast<uintptr_t>(v_cache) |
+                    reinterpret_cast<uintptr_t>(out)) & 15) == 0, "attention_decode_append: operands must be 16-byte aligned");
+    RUMUS_REQUIRE((uint64_t)batch * heads <= 65535, "attention_decode_append: batch * heads beyond the grid limit");
+    // strides: {q, k_new, v_new, k_cache, v_cache, out} x {batch, head, row}; the rows of q, k_new, v_new and out
+    // are single, their row strides unused
+    AttnArgs a{q, k_cache, v_cache, out, strides[0], strides[1], strides[2], strides[9], strides[10], strides[11],
+               strides[12], strides[13], strides[14], strides[15], strides[16], strides[17],
+               batch, heads, 1, pos + 1, 1.0f / sqrtf((float)head_dim), 0};
+    a.k_new = k_new;
+    a.v_new = v_new;
+    a.kn_sb = strides[3]; a.kn_sh = strides[4];
+    a.vn_sb = strides[6]; a.vn_sh = strides[7];
+    hipStream_t s = as_stream(stream);
+    const uint32_t slices = ceil_div(pos + 1, kDecodeSlice);
+    void* ws = nullptr;
+    WorkspaceLease lease;                                    // until both kernels are queued
+    if (int rc = workspace_get(s, (size_t)batch * heads * slices * (kHeadDim + 2) * sizeof(float), &ws, lease)) return rc;
+    hipLaunchKernelGGL(attention_decode_kernel, dim3(slices, batch * heads), dim3(256), 0, s, a, static_cast<float*>(ws));
+    if (int rc = check_launch("attention_decode_kernel")) return rc;
+    hipLaunchKernelGGL(attention_merge_kernel, dim3(batch * heads), dim3(kHeadDim), 0, s, a,
+                       static_cast<const float*>(ws), slices);
+    return check_launch("attention_merge_kernel");
 }
 
 }  // extern "C"

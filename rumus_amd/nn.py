@@ -301,8 +301,7 @@ class DecoderBlockW4:
         else:
             if n != 1:
                 raise ValueError("DecoderBlockW4: decode takes one token per sequence")
-            ops.kv_append(k, v, k_cache, v_cache, pos)
-            att = ops.attention(q, k_cache[:, :pos + 1], v_cache[:, :pos + 1], causal=False)
+            att = ops.attention_decode_append(q, k, v, k_cache, v_cache, pos)
             k_out, v_out = k_cache, v_cache
         o = self.proj["o"](att.view(b * n, d))
         x1, h2 = ops.add_rmsnorm(x2, o, self.norm2, self.eps, sum_out=o, out=hn)
@@ -325,7 +324,7 @@ class DecoderBlockW4:
                    for lin in layers)
 
     def _decode_folded(self, x2, b, k_cache, v_cache, pos):
-        """The decode step in seven launches: q|k|v on RMSNorm(x), cache append, attention (two), o + x,
+        """The decode step in six launches: q|k|v on RMSNorm(x), attention with the cache append (two), o + x,
         gate|up on RMSNorm of that, down on SwiGLU + the residual."""
         h, d = self.heads, self.dim
 
@@ -335,8 +334,7 @@ class DecoderBlockW4:
 
         qkv = project(self.qkv, x2, norm_weight=self.norm1, eps=self.eps).view(b, 1, 3, h, 128)
         q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
-        ops.kv_append(k, v, k_cache, v_cache, pos)
-        att = ops.attention(q, k_cache[:, :pos + 1], v_cache[:, :pos + 1], causal=False)
+        att = ops.attention_decode_append(q, k, v, k_cache, v_cache, pos)   # writes k, v at pos on its way
         x1 = project(self.proj["o"], att.view(b, d), residual=x2)
         gu = project(self.gate_up, x1, norm_weight=self.norm2, eps=self.eps)
         y = project(self.proj["down"], gu, swiglu=True, residual=x1, out=x1)

@@ -485,3 +485,24 @@ def kv_append(k_new, v_new, k_cache, v_cache, pos: int):
                                        for s in (t.stride(0), t.stride(2), t.stride(1))])
     call("rumus_hip_kv_append", k_new.data_ptr(), v_new.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
          b, h, n, d, pos, t_len, strides, _stream())
+
+
+def attention_decode_append(q, k_new, v_new, k_cache, v_cache, pos: int, out=None):
+    """``kv_append`` of one new token per sequence at ``pos`` and ``attention`` of its query over positions
+    ``0..pos``, without the launch for the append.  ``q``, ``k_new``, ``v_new`` ``[B, 1, H, 128]``, caches
+    ``[B, T, H, 128]`` (any strides with the last dim contiguous); returns ``[B, 1, H, 128]``."""
+    import ctypes
+    b, n, h, d = q.shape
+    if n != 1 or tuple(k_new.shape) != (b, 1, h, d) or tuple(v_new.shape) != (b, 1, h, d):
+        raise ValueError("attention_decode_append: q, k_new and v_new must be [B, 1, H, d]")
+    if k_cache.shape != v_cache.shape or k_cache.shape[0] != b or k_cache.shape[2] != h or k_cache.shape[3] != d:
+        raise ValueError("attention_decode_append: shapes of the new entries and the caches do not match")
+    o = out if out is not None else torch.empty((b, 1, h, d), dtype=torch.float32, device=q.device)
+    ts = (q, k_new, v_new, k_cache, v_cache, o)
+    for t, name in zip(ts, ("q", "k_new", "v_new", "k_cache", "v_cache", "out")):
+        if t.dtype != torch.float32 or not t.is_cuda or t.stride(3) != 1:
+            raise ValueError(f"attention_decode_append: {name} must be a float32 device tensor with a contiguous last dim")
+    strides = (ctypes.c_uint64 * 18)(*[s for t in ts for s in (t.stride(0), t.stride(2), t.stride(1))])
+    call("rumus_hip_attention_decode_append", q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), k_cache.data_ptr(),
+         v_cache.data_ptr(), o.data_ptr(), b, h, d, pos, k_cache.shape[1], strides, _stream())
+    return o

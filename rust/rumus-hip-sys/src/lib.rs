@@ -77,6 +77,9 @@ extern "C" {
     pub fn rumus_hip_swiglu(gate: *const f32, up: *const f32, out: *mut f32, numel: u64, s: Stream) -> c_int;
     pub fn rumus_hip_swiglu_rows(gate_up: *const f32, out: *mut f32, rows: u32, n: u32, s: Stream) -> c_int;
     pub fn rumus_hip_add(a: *const f32, b: *const f32, out: *mut f32, numel: u64, s: Stream) -> c_int;
+    pub fn rumus_hip_attention_decode_append(q: *const f32, k_new: *const f32, v_new: *const f32, k_cache: *mut f32,
+                                             v_cache: *mut f32, out: *mut f32, batch: u32, heads: u32, head_dim: u32,
+                                             pos: u32, cache_len: u32, strides: *const u64, s: Stream) -> c_int;
     pub fn rumus_hip_attention(q: *const f32, k: *const f32, v: *const f32, out: *mut f32, batch: u32,
                                heads: u32, q_len: u32, kv_len: u32, head_dim: u32, strides: *const u64,
                                causal: c_int, s: Stream) -> c_int;

@@ -188,6 +188,49 @@ def test_kv_append_is_an_exact_copy(ops, layout, b, h, n, pos, cache_len):
     torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("layout", ["token_major", "reference"])
+@pytest.mark.parametrize("b,h,pos,cache_len", [(1, 32, 2047, 2048), (3, 2, 0, 5), (2, 3, 255, 300), (2, 3, 256, 300),
+                                               (1, 4, 4, 5)])
+def test_attention_decode_append_is_append_then_attention(ops, layout, b, h, pos, cache_len):
+    """One call for the cache write of the newest token and the attention of its query: the same bits in the output
+    and in the caches as kv_append followed by attention, on both cache layouts, at the first and the last
+    position and across a slice boundary of the decode kernel (256 keys)."""
+    say(f"attention_decode_append {layout} b={b} h={h} pos={pos} T={cache_len}")
+    rng = np.random.default_rng(7 * b + h + pos)
+    qkv = rng.normal(0, 1, (b, 1, 3, h, 128)).astype(np.float32)
+    shape = (b, cache_len, h, 128) if layout == "token_major" else (b, h, cache_len, 128)
+    kc0 = rng.normal(0, 1, shape).astype(np.float32)
+    vc0 = rng.normal(0, 1, shape).astype(np.float32)
+    view = (lambda c: c) if layout == "token_major" else (lambda c: c.transpose(1, 2))
+    t = dev(qkv)
+    q, k, v = t[:, :, 0], t[:, :, 1], t[:, :, 2]
+    kc, vc = dev(kc0), dev(vc0)
+    ops.kv_append(k, v, view(kc), view(vc), pos)
+    want = host(ops.attention(q, view(kc)[:, :pos + 1], view(vc)[:, :pos + 1], causal=False))
+    kc2, vc2 = dev(kc0), dev(vc0)
+    got = host(ops.attention_decode_append(q, k, v, view(kc2), view(vc2), pos))
+    np.testing.assert_array_equal(got, want)
+    np.testing.assert_array_equal(host(kc2), host(kc))
+    np.testing.assert_array_equal(host(vc2), host(vc))
+    # against float64 as well
+    kk = host(view(kc))[:, :pos + 1]
+    vv = host(view(vc))[:, :pos + 1]
+    close(got, oracle.attention(qkv[:, :, 0], kk, vv, False), atol=2e-5)
+
+
+def test_attention_decode_append_rejects_bad_arguments(ops):
+    import torch
+    from rumus_amd._lib import RumusError
+    q = torch.zeros((1, 1, 2, 128), device="cuda")
+    cache = torch.zeros((1, 4, 2, 128), device="cuda")
+    with pytest.raises(RumusError, match="does not fit"):
+        ops.attention_decode_append(q, q, q, cache, cache.clone(), 4)
+    with pytest.raises(ValueError, match="must be"):
+        ops.attention_decode_append(torch.zeros((1, 2, 2, 128), device="cuda"), q, q, cache, cache.clone(), 0)
+    with pytest.raises(ValueError, match="do not match"):
+        ops.attention_decode_append(q, q, q, torch.zeros((1, 4, 3, 128), device="cuda"), cache, 0)
+
+
 def test_kv_append_rejects_bad_arguments(ops):
     import torch
     from rumus_amd._lib import RumusError
