@@ -381,6 +381,12 @@ def test_qlinear_module_mirror(ops):
     assert_close(host(ql.backward_input(dev(gy))), oracle.qmatmul_int4_t(gy, packed, scales, zp, k, g))
     with pytest.raises(ValueError):
         nn.QuantizedTensor.from_f32(dev(w), k, n, 12)
+    # without the second (tile-major) copy of the weight: the same rows through the reference's arrays, same bits
+    with_copy = host(ql.forward(dev(x)))
+    assert ql.weight.decode is not None
+    ql.weight.drop_decode_layout()
+    assert ql.weight.decode is None
+    np.testing.assert_array_equal(host(ql.forward(dev(x))), with_copy)
 
 
 def test_headline_shape_properties(ops):
