@@ -79,7 +79,7 @@ int rumus_hip_sync(rumus_hip_stream_t stream);
  *   matmul_q8, m >= 5: 4 * m * k * 4 (digit planes of a) + 4 * m * n * 4 + 32 MiB
  *       (partial sums of the int8 GEMM inside); with one block per column from
  *       384 rows on also k * n + 4 * n;
- *   attention with q_len == 1: batch * heads * ceil(kv_len / 256) * 520.
+ *   attention with q_len == 1: batch * heads * ceil(kv_len / 64) * 520.
  * rumus_hip_shutdown frees every workspace (no launch may be in flight). */
 int rumus_hip_workspace_reserve(rumus_hip_stream_t stream, uint64_t bytes);
 int rumus_hip_shutdown(void);

@@ -371,44 +371,67 @@ __global__ __launch_bounds__(256, 2) void attention_mfma_kernel(AttnArgs a) {
 
 // Decode case (q_len == 1): the keys of one (batch, head) are split over gridDim.x workgroups
 // so that the chip is covered; each writes (max, sum, unnormalised output) of its slice and
-// attention_merge_kernel combines the slices.  Within a workgroup: 4 lanes per key for the
-// scores (64 keys per sweep), then one thread per 4 output dims and key group for p.V.
-constexpr int kDecodeSlice = 256;   // keys per workgroup
+// attention_merge_kernel combines the slices.  Within a workgroup: 8 lanes per key for the
+// scores (32 keys per sweep), then one thread per 4 output dims and key group for p.V.
+constexpr int kDecodeSlice = 256;   // most keys per workgroup
 
+// lane exchanges inside 8 lanes without the LDS crossbar: quad_perm [1,0,3,2], [2,3,0,1], row_half_mirror
+__device__ __forceinline__ float dpp8_sum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));
+    return v;
+}
+
+// SLICE keys per workgroup (64, 128 or 256: the launcher takes the largest that still makes two workgroups per CU).
+// Scores: 8 lanes per key, lane l of them holding dims 32 i + 4 l .. + 3, so that a load instruction of a wave reads
+// whole 128-byte lines (8 keys x 128 bytes; with 4 lanes on 32 consecutive dims each it touched 64 lines for 16
+// bytes apiece and the lines did not survive in the L1 until their other pieces were asked for).
+template <int SLICE>
 __global__ __launch_bounds__(256) void attention_decode_kernel(AttnArgs a, float* __restrict__ part) {
-    __shared__ float sc[kDecodeSlice];
+    __shared__ float sc[SLICE];
     __shared__ float red[4], lsum[8];
     __shared__ __attribute__((aligned(16))) float osum[8][kHeadDim];
-    const uint32_t tid = threadIdx.x, lane4 = tid & 3, kq = tid >> 2;
+    const uint32_t tid = threadIdx.x, lane8 = tid & 7, kq = tid >> 3;
     const uint32_t bh = blockIdx.y, b = bh / a.heads, h = bh % a.heads;
-    const uint32_t j0 = blockIdx.x * kDecodeSlice, j1 = min(a.kv_len, j0 + kDecodeSlice);
-    const float* qp = a.q + b * a.q_sb + h * a.q_sh + lane4 * 32;
+    const uint32_t j0 = blockIdx.x * SLICE, j1 = min(a.kv_len, j0 + SLICE);
+    const float* qp = a.q + b * a.q_sb + h * a.q_sh + lane8 * 4;
     const float* kb = a.k + b * a.k_sb + h * a.k_sh;
     const float* vb = a.v + b * a.v_sb + h * a.v_sh;
-    float q[32];
+    float q[16];
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const float4 t = *reinterpret_cast<const float4*>(qp + 4 * i);
+    for (int i = 0; i < 4; i++) {
+        const float4 t = *reinterpret_cast<const float4*>(qp + 32 * i);
         q[4 * i] = t.x * a.scale; q[4 * i + 1] = t.y * a.scale; q[4 * i + 2] = t.z * a.scale; q[4 * i + 3] = t.w * a.scale;
     }
+    // p.V below: thread = (4 output dims, 1 of 8 key groups), eight 128-bit loads of V in flight
+    const uint32_t c4 = tid & 31, kg = tid >> 5;
+    auto load_v = [&](uint32_t jj, float4 (&vv)[8]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const uint32_t vc = min(j0 + jj + 8 * u, a.kv_len - 1);
+            const float* vp = (a.v_new && vc == a.kv_len - 1) ? a.v_new + b * a.vn_sb + h * a.vn_sh
+                                                             : vb + (uint64_t)vc * a.v_sr;
+            vv[u] = *reinterpret_cast<const float4*>(vp + 4 * c4);
+        }
+    };
     float mloc = -INFINITY;
 #pragma unroll
-    for (int sweep = 0; sweep < kDecodeSlice / 64; sweep++) {
-        const uint32_t jj = sweep * 64 + kq, key = j0 + jj;
+    for (int sweep = 0; sweep < SLICE / 32; sweep++) {
+        const uint32_t jj = sweep * 32 + kq, key = j0 + jj;
         const uint32_t kc = min(key, a.kv_len - 1);
-        const float* kp = (a.k_new && kc == a.kv_len - 1) ? a.k_new + b * a.kn_sb + h * a.kn_sh + lane4 * 32
-                                                         : kb + (uint64_t)kc * a.k_sr + lane4 * 32;
+        const float* kp = ((a.k_new && kc == a.kv_len - 1) ? a.k_new + b * a.kn_sb + h * a.kn_sh
+                                                          : kb + (uint64_t)kc * a.k_sr) + lane8 * 4;
         float d = 0.0f;
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const float4 kk = *reinterpret_cast<const float4*>(kp + 4 * i);
+        for (int i = 0; i < 4; i++) {
+            const float4 kk = *reinterpret_cast<const float4*>(kp + 32 * i);
             d = fmaf(q[4 * i], kk.x, d); d = fmaf(q[4 * i + 1], kk.y, d);
             d = fmaf(q[4 * i + 2], kk.z, d); d = fmaf(q[4 * i + 3], kk.w, d);
         }
-        d += __shfl_xor(d, 1);
-        d += __shfl_xor(d, 2);
+        d = dpp8_sum(d);
         d = key < j1 ? d : -INFINITY;
-        if (lane4 == 0) sc[jj] = d;
+        if (lane8 == 0) sc[jj] = d;
         mloc = fmaxf(mloc, d);
     }
 #pragma unroll
@@ -416,22 +439,16 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttnArgs a, float
     if ((tid & 63) == 0) red[tid >> 6] = mloc;
     __syncthreads();
     const float m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));   // finite: the slice is not empty
-    // p.V: thread = (4 output dims, 1 of 8 key groups), eight 128-bit loads of V in flight
-    const uint32_t c4 = tid & 31, kg = tid >> 5;
     float4 o = make_float4(0, 0, 0, 0);
     float l = 0.0f;
-    for (uint32_t jj = kg; jj < kDecodeSlice; jj += 64) {
+#pragma unroll
+    for (int it = 0; it < SLICE / 64; it++) {
+        const uint32_t jj = kg + 64 * it;
         float p[8];
         float4 vv[8];
+        load_v(jj, vv);
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
-            const uint32_t key = j0 + jj + 8 * u;
-            const uint32_t vc = min(key, a.kv_len - 1);
-            const float* vp = (a.v_new && vc == a.kv_len - 1) ? a.v_new + b * a.vn_sb + h * a.vn_sh
-                                                             : vb + (uint64_t)vc * a.v_sr;
-            vv[u] = *reinterpret_cast<const float4*>(vp + 4 * c4);
-            p[u] = key < j1 ? expf(sc[jj + 8 * u] - m) : 0.0f;
-        }
+        for (int u = 0; u < 8; u++) p[u] = j0 + jj + 8 * u < j1 ? expf(sc[jj + 8 * u] - m) : 0.0f;
 #pragma unroll
         for (int u = 0; u < 8; u++) {
             l += p[u];
@@ -469,7 +486,7 @@ __global__ __launch_bounds__(kHeadDim) void attention_merge_kernel(AttnArgs a, c
                                                                    uint32_t slices) {
     const uint32_t bh = blockIdx.x, b = bh / a.heads, h = bh % a.heads, dim = threadIdx.x;
     const float* src = part + (uint64_t)bh * slices * (kHeadDim + 2);
-    // slices is small (kv_len / 256); the loads of a pass do not depend on each other
+    // slices is small (kv_len / 64 at most); the loads of a pass do not depend on each other
     float m = -INFINITY;
 #pragma unroll 8
     for (uint32_t s = 0; s < slices; s++) m = fmaxf(m, src[s * (kHeadDim + 2)]);
@@ -511,6 +528,25 @@ __global__ __launch_bounds__(256) void kv_append_kernel(KvAppendArgs a) {
 }
 
 }  // namespace rumus
+
+// One query row per (batch, head): slices of 256 keys, or of 128 or 64 while that is what it takes to put two
+// workgroups on every CU (32 heads at 2048 keys: 512 workgroups of 128 keys), merged by a second kernel.
+static int launch_attention_decode(const rumus::AttnArgs& a, hipStream_t s) {
+    using namespace rumus;
+    const uint32_t bh = a.batch * a.heads;
+    const uint32_t slice = (uint64_t)bh * ceil_div(a.kv_len, 256u) >= 512 ? 256 : (uint64_t)bh * ceil_div(a.kv_len, 128u) >= 512 ? 128 : 64;
+    const uint32_t slices = ceil_div(a.kv_len, slice);
+    void* ws = nullptr;
+    WorkspaceLease lease;                                    // until both kernels are queued
+    if (int rc = workspace_get(s, (size_t)bh * slices * (kHeadDim + 2) * sizeof(float), &ws, lease)) return rc;
+    const dim3 grid(slices, bh);
+    if (slice == 256) hipLaunchKernelGGL(attention_decode_kernel<256>, grid, dim3(256), 0, s, a, static_cast<float*>(ws));
+    else if (slice == 128) hipLaunchKernelGGL(attention_decode_kernel<128>, grid, dim3(256), 0, s, a, static_cast<float*>(ws));
+    else hipLaunchKernelGGL(attention_decode_kernel<64>, grid, dim3(256), 0, s, a, static_cast<float*>(ws));
+    if (int rc = check_launch("attention_decode_kernel")) return rc;
+    hipLaunchKernelGGL(attention_merge_kernel, dim3(bh), dim3(kHeadDim), 0, s, a, static_cast<const float*>(ws), slices);
+    return check_launch("attention_merge_kernel");
+}
 
 using namespace rumus;
 
@@ -590,18 +626,7 @@ int rumus_hip_attention(const float* q, const float* k, const float* v, float* o
                strides[6], strides[7], strides[8], strides[9], strides[10], strides[11],
                batch, heads, q_len, kv_len, 1.0f / sqrtf((float)head_dim), causal};
     hipStream_t s = as_stream(stream);
-    if (q_len == 1) {
-        const uint32_t slices = ceil_div(kv_len, kDecodeSlice);
-        void* ws = nullptr;
-        WorkspaceLease lease;                                // until both kernels are queued
-        if (int rc = workspace_get(s, (size_t)batch * heads * slices * (kHeadDim + 2) * sizeof(float), &ws, lease)) return rc;
-        hipLaunchKernelGGL(attention_decode_kernel, dim3(slices, batch * heads), dim3(256), 0, s, a,
-                           static_cast<float*>(ws));
-        if (int rc = check_launch("attention_decode_kernel")) return rc;
-        hipLaunchKernelGGL(attention_merge_kernel, dim3(batch * heads), dim3(kHeadDim), 0, s, a,
-                           static_cast<const float*>(ws), slices);
-        return check_launch("attention_merge_kernel");
-    }
+    if (q_len == 1) return launch_attention_decode(a, s);
     if (q_len >= 64) {                                       // enough rows to fill 32-row matrix-core tiles
         RUMUS_REQUIRE(ceil_div(q_len, 128) <= 65535, "attention: q_len %u beyond the grid limit", q_len);
         hipLaunchKernelGGL(attention_mfma_kernel, dim3(batch * heads, ceil_div(q_len, 128)), dim3(256), 0, s, a);
@@ -664,16 +689,7 @@ int rumus_hip_attention_decode_append(const float* q, const float* k_new, const 
     a.v_new = v_new;
     a.kn_sb = strides[3]; a.kn_sh = strides[4];
     a.vn_sb = strides[6]; a.vn_sh = strides[7];
-    hipStream_t s = as_stream(stream);
-    const uint32_t slices = ceil_div(pos + 1, kDecodeSlice);
-    void* ws = nullptr;
-    WorkspaceLease lease;                                    // until both kernels are queued
-    if (int rc = workspace_get(s, (size_t)batch * heads * slices * (kHeadDim + 2) * sizeof(float), &ws, lease)) return rc;
-    hipLaunchKernelGGL(attention_decode_kernel, dim3(slices, batch * heads), dim3(256), 0, s, a, static_cast<float*>(ws));
-    if (int rc = check_launch("attention_decode_kernel")) return rc;
-    hipLaunchKernelGGL(attention_merge_kernel, dim3(batch * heads), dim3(kHeadDim), 0, s, a,
-                       static_cast<const float*>(ws), slices);
-    return check_launch("attention_merge_kernel");
+    return launch_attention_decode(a, as_stream(stream));
 }
 
 }  // extern "C"
