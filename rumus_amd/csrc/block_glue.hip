@@ -415,24 +415,39 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttnArgs a, float
             vv[u] = *reinterpret_cast<const float4*>(vp + 4 * c4);
         }
     };
+    // All of the slice.s key loads are issued before the first is used; behind the last
+    // group's loads goes the first batch of V (memory returns in order: asked for ahead of the keys it would hold
+    // up the scores), so that its trip to memory overlaps the scores, the reduction and the barrier.
+    constexpr int SWEEPS = SLICE / 32, GROUP = SWEEPS;
     float mloc = -INFINITY;
+    float4 vfirst[8];
 #pragma unroll
-    for (int sweep = 0; sweep < SLICE / 32; sweep++) {
-        const uint32_t jj = sweep * 32 + kq, key = j0 + jj;
-        const uint32_t kc = min(key, a.kv_len - 1);
-        const float* kp = ((a.k_new && kc == a.kv_len - 1) ? a.k_new + b * a.kn_sb + h * a.kn_sh
-                                                          : kb + (uint64_t)kc * a.k_sr) + lane8 * 4;
-        float d = 0.0f;
+    for (int g0 = 0; g0 < SWEEPS; g0 += GROUP) {
+        float4 kk[GROUP][4];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const float4 kk = *reinterpret_cast<const float4*>(kp + 32 * i);
-            d = fmaf(q[4 * i], kk.x, d); d = fmaf(q[4 * i + 1], kk.y, d);
-            d = fmaf(q[4 * i + 2], kk.z, d); d = fmaf(q[4 * i + 3], kk.w, d);
+        for (int s = 0; s < GROUP; s++) {
+            const uint32_t kc = min(j0 + (g0 + s) * 32 + kq, a.kv_len - 1);
+            const float* kp = ((a.k_new && kc == a.kv_len - 1) ? a.k_new + b * a.kn_sb + h * a.kn_sh
+                                                              : kb + (uint64_t)kc * a.k_sr) + lane8 * 4;
+#pragma unroll
+            for (int i = 0; i < 4; i++) kk[s][i] = *reinterpret_cast<const float4*>(kp + 32 * i);
         }
-        d = dpp8_sum(d);
-        d = key < j1 ? d : -INFINITY;
-        if (lane8 == 0) sc[jj] = d;
-        mloc = fmaxf(mloc, d);
+        if (g0 + GROUP >= SWEEPS) load_v(kg, vfirst);
+        __builtin_amdgcn_sched_barrier(0);                 // the loads stay ahead of the arithmetic
+#pragma unroll
+        for (int s = 0; s < GROUP; s++) {
+            const uint32_t jj = (g0 + s) * 32 + kq, key = j0 + jj;
+            float d = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                d = fmaf(q[4 * i], kk[s][i].x, d); d = fmaf(q[4 * i + 1], kk[s][i].y, d);
+                d = fmaf(q[4 * i + 2], kk[s][i].z, d); d = fmaf(q[4 * i + 3], kk[s][i].w, d);
+            }
+            d = dpp8_sum(d);
+            d = key < j1 ? d : -INFINITY;
+            if (lane8 == 0) sc[jj] = d;
+            mloc = fmaxf(mloc, d);
+        }
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) mloc = fmaxf(mloc, __shfl_xor(mloc, o));
@@ -446,7 +461,12 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttnArgs a, float
         const uint32_t jj = kg + 64 * it;
         float p[8];
         float4 vv[8];
-        load_v(jj, vv);
+        if (it == 0) {
+#pragma unroll
+            for (int u = 0; u < 8; u++) vv[u] = vfirst[u];
+        } else {
+            load_v(jj, vv);
+        }
 #pragma unroll
         for (int u = 0; u < 8; u++) p[u] = j0 + jj + 8 * u < j1 ? expf(sc[jj + 8 * u] - m) : 0.0f;
 #pragma unroll
