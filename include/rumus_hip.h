@@ -252,8 +252,11 @@ int rumus_hip_qmatmul_int4(const float* x, const uint32_t* packed,
  * array of rumus_hip_static_scratch_bytes() = 32 MiB that each GPU holds
  * until the process ends; nothing is allocated or freed, on any call.
  * EINVAL ("needs ... bytes of scratch memory") when the shape needs more than
- * the array holds: with k = 4096, n = 11008 that is beyond about 300 rows;
- * the need is the qmatmul_int4 line of the workspace bounds above.
+ * the array holds; the need is the qmatmul_int4 line of the workspace bounds
+ * above and does not grow evenly with m: with k = 4096, n = 11008 calls of
+ * 318 to 512 rows are refused (their partial sums, kept while the output has
+ * few tiles, do not fit), calls of up to 317 rows and of 513 to about 1900
+ * rows run.
  * All calls on one GPU share the one array, whatever their stream: calls that
  * overlap in time on one GPU race (calls on one stream do not overlap).
  * Nothing in the array has to start at zero: every byte a kernel reads from

@@ -292,6 +292,9 @@ struct Q8Dense {
 };
 
 inline Q8Dense prepare_dense(const Q8Tensor& q, hipStream_t stream = nullptr) {
+    require(q.block_size > 0 && q.block_size >= q.k, "prepare_dense: one block per column wanted (block_size >= k)");
+    require(q.buffer.size() >= (size_t)q.n * ((4 + (size_t)q.block_size + 3) / 4),
+            "prepare_dense: the Q8 buffer is shorter than n blocks");
     Q8Dense d;
     d.k = q.k; d.n = q.n;
     d.wq = DeviceBuffer<int8_t>((size_t)q.n * q.k);

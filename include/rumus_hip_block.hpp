@@ -99,15 +99,49 @@ struct DecoderBlockW4 {
                rows <= rumus_hip_qmatmul_int4_decode_max_rows(w.padded_k, w.n);
     }
 
+    // The block's temporaries, [rows, ...] each.  A caller that runs many steps keeps one, sized once for its
+    // largest batch * n: forward() on it allocates nothing, frees nothing and does not wait for the stream (so a
+    // decode step can be queued behind the previous one, or captured into a HIP graph once the stream's workspace
+    // is reserved).  Calls that share a Scratch must be ordered on one stream.
+    struct Scratch {
+        DeviceBuffer<float> hn, qkv_out, att, ob, gu, dn, sw;
+        uint32_t rows = 0;
+        Scratch() = default;
+        Scratch(const DecoderBlockW4& b, uint32_t max_rows) { reserve(b, max_rows); }
+        void reserve(const DecoderBlockW4& b, uint32_t max_rows) {
+            if (max_rows <= rows) return;
+            const size_t r = max_rows, d = b.dim, f = b.ffn;
+            hn = DeviceBuffer<float>(r * d);
+            qkv_out = DeviceBuffer<float>(r * 3 * d);
+            att = DeviceBuffer<float>(r * d);
+            ob = DeviceBuffer<float>(r * d);
+            gu = DeviceBuffer<float>(r * 2 * f);
+            dn = DeviceBuffer<float>(r * d);
+            sw = DeviceBuffer<float>(r * f);
+            rows = max_rows;
+        }
+    };
+
+    // One call with temporaries of its own: allocates them, waits for the stream and frees them.
     void forward(const float* x, uint32_t batch, uint32_t n, float* y, float* k_cache, float* v_cache,
                  uint32_t cache_len, uint32_t pos, hipStream_t stream = nullptr) const {
+        require(batch > 0 && n > 0, "DecoderBlockW4: empty input");
+        Scratch scratch(*this, batch * n);
+        forward(x, batch, n, y, k_cache, v_cache, cache_len, pos, scratch, stream);
+        check(rumus_hip_sync(stream));       // the temporaries are released on return
+    }
+
+    // The same on the caller's temporaries: asynchronous on `stream`, no allocation.
+    void forward(const float* x, uint32_t batch, uint32_t n, float* y, float* k_cache, float* v_cache,
+                 uint32_t cache_len, uint32_t pos, Scratch& scratch, hipStream_t stream = nullptr) const {
         require(batch > 0 && n > 0, "DecoderBlockW4: empty input");
         require(pos == 0 || n == 1, "DecoderBlockW4: decode takes one token per sequence");
         require(pos == 0 || (k_cache && v_cache), "DecoderBlockW4: decode needs the caches");
         const uint32_t rows = batch * n, h = heads;
         const uint64_t d = dim;
-        DeviceBuffer<float> hn((size_t)rows * d), qkv_out((size_t)rows * 3 * d), att((size_t)rows * d),
-            ob((size_t)rows * d), gu((size_t)rows * 2 * ffn), dn((size_t)rows * d);
+        require(rows <= scratch.rows, "DecoderBlockW4: the scratch holds fewer rows than batch * n");
+        DeviceBuffer<float>&hn = scratch.hn, &qkv_out = scratch.qkv_out, &att = scratch.att, &ob = scratch.ob,
+                           &gu = scratch.gu, &dn = scratch.dn, &sw = scratch.sw;
         // a decode step whose rows suit every projection's decode kernel: the norms, the SwiGLU and the residual adds
         // ride on the projections (rumus_hip_qmatmul_int4_decode_block), six launches in all
         const bool folded = pos != 0 && folds(qkv, rows) && folds(o, rows) && folds(gate_up, rows) && folds(down, rows);
@@ -145,7 +179,6 @@ struct DecoderBlockW4 {
             project(o, att.data(), nullptr, 0, x, ob.data());                   // x1 = x + o
             project(gate_up, ob.data(), norm2.data(), 0, nullptr, gu.data());
             project(down, gu.data(), nullptr, 1, ob.data(), y);                 // y = x1 + down(swiglu)
-            check(rumus_hip_sync(stream));   // the temporaries are released on return
             return;
         }
         o.forward(att.data(), rows, ob.data(), stream);
@@ -160,13 +193,10 @@ struct DecoderBlockW4 {
                                                        down.bias.size() ? down.bias.data() : nullptr, dn.data(), rows,
                                                        dw.k, dw.n, dw.padded_k, dw.group_size, dw.num_groups, stream));
         } else {
-            DeviceBuffer<float> sw((size_t)rows * ffn);
             check(rumus_hip_swiglu_rows(gu.data(), sw.data(), rows, ffn, stream));
             down.forward(sw.data(), rows, dn.data(), stream);
-            check(rumus_hip_sync(stream));   // `sw` is released on leaving this scope
         }
         check(rumus_hip_add(ob.data(), dn.data(), y, (uint64_t)rows * d, stream));
-        check(rumus_hip_sync(stream));       // the temporaries are released on return
     }
 };
 

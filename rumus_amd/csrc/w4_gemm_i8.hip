@@ -49,30 +49,6 @@ struct W4I8Args {
     uint32_t m, n, steps, chunks, steps_per_group, per;   // per: chunks per share
 };
 
-#ifdef RUMUS_TIMERS
-// instrumented build only (-DRUMUS_TIMERS): wall-clock stamps (10 ns ticks) of every wave at fixed points
-constexpr uint32_t kStampWorkgroups = 512;                       // the first so many workgroups of a launch are recorded
-__device__ unsigned long long g_w4i8_stamps[kStampWorkgroups * 8 * 8];
-extern "C" int rumus_dbg_w4i8_stamps(unsigned long long* host, size_t count) {
-    if (count > kStampWorkgroups * 8 * 8) return 1;
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_w4i8_stamps), count * 8);
-}
-#define STAMP(i) do { const uint32_t wg_ = blockIdx.y * gridDim.x + blockIdx.x;                           \
-        if (lane == 0 && wg_ < kStampWorkgroups) g_w4i8_stamps[(wg_ * 8 + wk) * 8 + (i)] = wall_clock64(); } while (0)
-// the same for the kernel that prepares the activations: [workgroup][wave][stamp]
-constexpr uint32_t kPrepStampWorkgroups = 256;
-__device__ unsigned long long g_w4i8_prep_stamps[kPrepStampWorkgroups * 8 * 8];
-extern "C" int rumus_dbg_w4i8_prep_stamps(unsigned long long* host, size_t count) {
-    if (count > kPrepStampWorkgroups * 8 * 8) return 1;
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_w4i8_prep_stamps), count * 8);
-}
-#define PSTAMP(i) do { const uint32_t wg_ = blockIdx.y * gridDim.x + blockIdx.x;                          \
-        if (lane == 0 && wg_ < kPrepStampWorkgroups)                                                      \
-            g_w4i8_prep_stamps[(wg_ * 8 + (threadIdx.x >> 6)) * 8 + (i)] = wall_clock64(); } while (0)
-#else
-#define STAMP(i)
-#define PSTAMP(i)
-#endif
 
 // low bytes of a, b, c, d -> one word
 __device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
@@ -123,7 +99,6 @@ __global__ __launch_bounds__(STAGED ? 64 * kI8WK : 64) void w4_i8_prepare_kernel
     const uint32_t k_begin = min(share * per, chunks) * CS * 64, k_end = min((share + 1) * per, chunks) * CS * 64;
     const bool live = row < m;
     const float* xr = x + (uint64_t)(live ? row : 0) * k;
-    PSTAMP(0);
     // STAGED (the launcher sends k % 8 == 0 and 16-byte aligned x and perm here): where a lane's 8 values come
     // from, then the values themselves.  Straight-line code with clamped addresses: a load under a branch
     // would make the wave wait for it at the end of the branch, one trip to memory after the other.
@@ -163,7 +138,6 @@ __global__ __launch_bounds__(STAGED ? 64 * kI8WK : 64) void w4_i8_prepare_kernel
         }
         __syncthreads();
     }
-    PSTAMP(1);
 
     auto load8 = [&](uint32_t k0, float (&v)[8]) {
 #pragma unroll
@@ -216,7 +190,6 @@ __global__ __launch_bounds__(STAGED ? 64 * kI8WK : 64) void w4_i8_prepare_kernel
     // largest magnitude lies below 2^-107 keep fewer than 20 bits.  A
     // non-finite activation poisons its row: the scale becomes NaN (the digits are then whatever the
     // conversion gives; they only ever meet the NaN)
-    PSTAMP(2);
     const bool finite = mb < 0x7f800000u;
     int e = 21 - ((int)(mb >> 23) - 127);
     e = mb == 0 ? 0 : min(e, 126);
@@ -255,7 +228,6 @@ __global__ __launch_bounds__(STAGED ? 64 * kI8WK : 64) void w4_i8_prepare_kernel
         load8(k0, v);
         emit(k0, v);
     }
-    PSTAMP(3);
 }
 
 // ---- the matmul -------------------------------------------------------------------------------------
@@ -292,7 +264,6 @@ __global__ __launch_bounds__(512) void w4_gemm_i8_kernel(W4I8Args a) {
     const uint32_t flast = f1 > f0 ? f1 - 1 : f0 ? f0 - 1 : 0;
     const uint32_t lane_w = 2 * b * a.n + colc;                    // lane part of a packed-word address
 
-    STAMP(0);
     uint32_t braw[U][CS][2][Q], msc[U][Q], mzp[U][Q];
     auto fetch_b = [&](int slot, uint32_t chunk) {
         const uint32_t fc = min(chunk, flast);                       // past the wave's share: fetched again, adds 0
@@ -337,7 +308,6 @@ __global__ __launch_bounds__(512) void w4_gemm_i8_kernel(W4I8Args a) {
     fetch_a(0, f0, 0);
 #pragma unroll
     for (int u = 0; u < U; u++) fetch_b(u, f0 + u);
-    STAMP(1);
 
     // Whole rounds of U chunks, straight-line code: a chunk past the wave's share is computed on the last
     // chunk's data again (addresses are clamped) with its scale and zero-point set to 0, so it adds 0.
@@ -405,9 +375,6 @@ __global__ __launch_bounds__(512) void w4_gemm_i8_kernel(W4I8Args a) {
                         accf[t][q][i] = fmaf(sc[q], tot, accf[t][q][i]);
                     }
             }
-#ifdef RUMUS_TIMERS
-            if (base == f0 && u == 0) { __builtin_amdgcn_sched_barrier(0); if (accf[0][0][0] != 1e30f) STAMP(2); }
-#endif
         }
         // - scale * zp * (sum of X over the chunk), the round's chunks at once: [16 rows x 4 chunks] x [4 chunks x 16 columns]
 #pragma unroll
@@ -415,7 +382,6 @@ __global__ __launch_bounds__(512) void w4_gemm_i8_kernel(W4I8Args a) {
 #pragma unroll
             for (int q = 0; q < Q; q++) accf[t][q] = __builtin_amdgcn_mfma_f32_16x16x4f32(sm[t], szq[q], accf[t][q], 0, 0, 0);
     }
-    STAMP(3);
 
     // back to the activations' scale (this wave's share of K has its own), then the eight shares meet in LDS;
     // wave w adds them up, in a fixed order, for rows 4b + w % 4 of row tile w / 4 and stores
@@ -429,7 +395,6 @@ __global__ __launch_bounds__(512) void w4_gemm_i8_kernel(W4I8Args a) {
             for (int i = 0; i < 4; i++) red[wk][(t * Q + q) * 4 + i][lane] = f1 > f0 ? accf[t][q][i] * r4[i] : 0.0f;
     }
     __syncthreads();
-    STAMP(4);
     if (wk >= RT * 4) return;
     const uint32_t t = wk >> 2, i = wk & 3;
     const uint32_t row = (rb * RT + t) * 16 + 4 * b + i;

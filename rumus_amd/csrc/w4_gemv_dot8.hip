@@ -69,24 +69,6 @@ __device__ __forceinline__ float reduce_row_lanes(float v) {
     return v;
 }
 
-#ifdef RUMUS_TIMERS
-// instrumented build only (-DRUMUS_TIMERS): wall-clock stamps (10 ns ticks) of every wave of the first 256
-// workgroups at fixed points, [workgroup][wave][stamp].  A stamp is taken once `after` is known (the branch
-// on its bits makes the clock read depend on it).
-constexpr uint32_t kD8StampWorkgroups = 256;
-__device__ unsigned long long g_d8_stamps[kD8StampWorkgroups * 8 * 8];
-extern "C" int rumus_dbg_d8_stamps(unsigned long long* host, size_t count) {
-    if (count > kD8StampWorkgroups * 8 * 8) return 1;
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_d8_stamps), count * 8);
-}
-#define D8_STAMP(i, after) do { __builtin_amdgcn_sched_barrier(0);                                         \
-        if ((threadIdx.x & 63) == 0 && blockIdx.x < kD8StampWorkgroups && (threadIdx.x >> 6) < 8 &&        \
-            __float_as_uint(after) != 0x7fabcdefu)                                                         \
-            g_d8_stamps[(blockIdx.x * 8 + (threadIdx.x >> 6)) * 8 + (i)] = wall_clock64();                 \
-        __builtin_amdgcn_sched_barrier(0); } while (0)
-#else
-#define D8_STAMP(i, after)
-#endif
 
 // Kernel arguments are passed flat.  This file is built with the first two
 // arguments (the pointers to the packed words and the scales) preloaded into
@@ -116,15 +98,17 @@ __device__ __forceinline__ float* d8_sq_lds() {
 // (a workgroup's lanes load each element of the row exactly once), the sums of squares travel with the wave sums
 // through LDS, and rsqrt(...) multiplies the result.  `resid` (or null): y = ... + resid[m][n], the residual add of
 // the decoder block, in the epilogue.
+// `resid` may be the output itself (each element is read by the thread that then stores it), so neither of the
+// two pointers is declared restrict.
 // BLOCK: the kernel looks at norm_w / eps / resid at all; the plain kernels are launched with nulls there and
 // compile to what they were without these arguments.
 template <int M, int T, int OCT, bool FASTX, bool ZP4, bool TILED, bool GLU = false, bool NORM = false, bool BLOCK = false>
 __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
     const uint32_t* __restrict__ packed, const float* __restrict__ scales,
-    const float* __restrict__ zps, const float* __restrict__ xin, float* __restrict__ yout,
+    const float* __restrict__ zps, const float* __restrict__ xin, float* yout,
     uint32_t n, uint32_t k, uint32_t padded_k, uint32_t group_size,
     const float* __restrict__ bias, const int32_t* __restrict__ perm,
-    const float* __restrict__ norm_w, float eps, const float* __restrict__ resid) {
+    const float* __restrict__ norm_w, float eps, const float* resid) {
     static_assert(!NORM || BLOCK, "the norm is one of the block's forms");
     static_assert(OCT == 4 || OCT == 8, "a quad shares 4 or 8 word rows");
     static_assert(!NORM || (FASTX && !GLU), "the fused norm reads plain rows with 128-bit loads");
@@ -152,7 +136,6 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
 #pragma unroll
         for (int m = 0; m < M; m++) ssq[m] = 0.0f;
     }
-    D8_STAMP(0, acc[0][0]);
 
     // every quad runs the same number of sweeps; a dead quad carries scale 0
     for (uint32_t base = 0; base < nchunks; base += RL) {
@@ -324,7 +307,6 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
                     pl[3 * OPL + t][i] = quad_bcast<3>(own[t][i]);
                 }
 
-            D8_STAMP(1, __uint_as_float(pl[OCT - 1][4]));      // planes built (last sweep, last row of x)
             // ---- 3. dot products -------------------------------------------------
             // word row by word row, in the order the loads were issued and retire: the rows that have
             // arrived are multiplied while the later ones are still on their way, and only the last
@@ -355,7 +337,6 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
         }
     }
 
-    D8_STAMP(2, acc[M - 1][3]);                                // every weight arrived and multiplied
     // ---- 4. reduce over the quads of a wave, then over the waves -----------------
     const uint32_t lane = tid & 63, wave = tid >> 6;
 #pragma unroll
@@ -379,9 +360,7 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
             if (lane == 15) d8_sq_lds<WAVES, M>()[wave * M + m] = q;
         }
     }
-    D8_STAMP(3, acc[M - 1][3]);                                // reduced over the wave, written to LDS
     __syncthreads();
-    D8_STAMP(4, acc[M - 1][3]);                                // barrier passed
     if (tid < M * kD8Cols) {
         const uint32_t m = tid / kD8Cols, c = tid % kD8Cols;
         const uint32_t oc = cchunk * kD8Cols + c;
@@ -402,7 +381,6 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
             yout[(uint64_t)m * n + oc] = v;
         }
     }
-    D8_STAMP(5, acc[M - 1][3]);                                // result stored (the waves that store: issued)
 }
 
 // Launch geometry: threads per workgroup and word rows per quad.

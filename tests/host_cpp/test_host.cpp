@@ -253,9 +253,20 @@ static void test_block(const std::string& dir) {
     spill(dir + "/block_y.bin", hy.data(), hy.size() * 4);
     spill(dir + "/block_y1.bin", hy1.data(), hy1.size() * 4);
     spill(dir + "/block_k.bin", hk.data(), hk.size() * 4);
+    // the same two calls on temporaries the caller keeps (no allocation, no wait inside): same bits, twice in a row
+    DecoderBlockW4::Scratch scratch(blk, batch * n);
+    DeviceBuffer<float> y2(hx.size()), y3(hx1.size());
+    blk.forward(x.data(), batch, n, y2.data(), kc.data(), vc.data(), cache_len, 0, scratch);
+    for (int rep = 0; rep < 2; rep++) blk.forward(x1.data(), batch, 1, y3.data(), kc.data(), vc.data(), cache_len, n, scratch);
+    check(rumus_hip_sync(nullptr));
+    CHECK(y2.download() == hy && y3.download() == hy1 && kc.download() == hk, "block on a kept Scratch differs");
     bool threw = false;
     try { blk.forward(x.data(), batch, n, y.data(), kc.data(), vc.data(), cache_len, 1); } catch (const Error& e) { threw = e.code == RUMUS_HIP_EINVAL; }
     CHECK(threw, "several tokens at pos > 0 must be rejected");
+    threw = false;
+    DecoderBlockW4::Scratch small(blk, 1);
+    try { blk.forward(x.data(), batch, n, y.data(), kc.data(), vc.data(), cache_len, 0, small); } catch (const Error& e) { threw = e.code == RUMUS_HIP_EINVAL; }
+    CHECK(threw || batch * n <= 1, "a Scratch of fewer rows must be rejected");
 }
 
 static void test_errors() {

@@ -190,11 +190,14 @@ def test_kv_append_is_an_exact_copy(ops, layout, b, h, n, pos, cache_len):
 
 @pytest.mark.parametrize("layout", ["token_major", "reference"])
 @pytest.mark.parametrize("b,h,pos,cache_len", [(1, 32, 2047, 2048), (3, 2, 0, 5), (2, 3, 255, 300), (2, 3, 256, 300),
-                                               (1, 4, 4, 5)])
+                                               (1, 4, 4, 5),
+                                               # slices of 256 keys (batch * heads * slices >= 512): the last slice
+                                               # full, and the last slice holding the new key alone
+                                               (2, 32, 2047, 2048), (2, 32, 1792, 1800)])
 def test_attention_decode_append_is_append_then_attention(ops, layout, b, h, pos, cache_len):
     """One call for the cache write of the newest token and the attention of its query: the same bits in the output
     and in the caches as kv_append followed by attention, on both cache layouts, at the first and the last
-    position and across a slice boundary of the decode kernel (256 keys)."""
+    position, across a slice boundary of the decode kernel and with slices of 64, 128 and 256 keys."""
     say(f"attention_decode_append {layout} b={b} h={h} pos={pos} T={cache_len}")
     rng = np.random.default_rng(7 * b + h + pos)
     qkv = rng.normal(0, 1, (b, 1, 3, h, 128)).astype(np.float32)

@@ -29,10 +29,12 @@ def test_static_scratch_entry_point_matches_the_allocating_one(ops):
     ps, perm = ops.w4_actorder_prepare(dev(packed), dev(g_idx), g)
     sd, zd = dev(scales), dev(zp)
     bias = dev(rng.normal(0, 0.01, n).astype(np.float32))
-    # first the largest call (128 rows: converted activations + partial tiles of the K shares), then smaller
-    # ones that reuse the array with the first call's contents still in it, one with another weight shape
+    # Calls in a row that share the array, each with the contents the one before left in it.  128, 16 and 48 rows
+    # run the int8-path kernels (digit planes, chunk sums and row scales in the array); 192 and 300 rows the f16
+    # tiles with K shared over three and two workgroups per tile, whose partial tiles (25-26 MB) fill most of the
+    # array behind the converted activations; 1024 rows the f16 tiles without partial tiles (18 MB of activations).
     outs = []
-    for m in (128, 16, 48, 16):
+    for m in (128, 192, 16, 300, 48, 1024, 16):
         say(f"qmatmul_int4_perm_static m={m} k={k} n={n} act-order")
         x = dev(rng.normal(0, 1, (m, k)).astype(np.float32))
         y = torch.empty((m, n), dtype=torch.float32, device="cuda")
@@ -42,7 +44,7 @@ def test_static_scratch_entry_point_matches_the_allocating_one(ops):
         outs.append((host(x), host(y)))
     # and against the CPU restatement on a few rows of the first and the last call
     unsorted_w = dict(packed=packed, scales=scales, zp=zp)
-    for xs, ys in (outs[0], outs[-1]):
+    for xs, ys in (outs[0], outs[1], outs[3], outs[-1]):
         rows = [0, xs.shape[0] - 1]
         want = oracle.qmatmul_int4(xs[rows], unsorted_w["packed"], unsorted_w["scales"], unsorted_w["zp"], k, g,
                                    bias=host(bias), g_idx=g_idx, threads=8)
