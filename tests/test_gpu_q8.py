@@ -210,7 +210,7 @@ def test_q8_dense_rejects(ops):
     with pytest.raises(ValueError):                        # blocks smaller than a column have no dense form
         nn.Q8Tensor(dev(oracle.tensor_quantize(np.ones((64, 8), np.float32), 32)), (64, 8), 32).prepare()
     with pytest.raises(ops.RumusError):                    # more columns than the layout kernel's grid takes
-        ops.q8_dense_layout(torch.zeros(8, dtype=torch.int32, device="cuda"), 16, 70000, 16)
+        ops.q8_dense_layout(torch.zeros(70000 * 5, dtype=torch.int32, device="cuda"), 16, 70000, 16)
     words = dev(oracle.tensor_quantize(np.ones((64, 8), np.float32), 32))
     with pytest.raises(ops.RumusError):                    # two blocks per column
         ops.q8_dense_layout(words, 64, 8, 32)
