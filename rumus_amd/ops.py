@@ -95,9 +95,8 @@ def matmul_q8(a: torch.Tensor, words: torch.Tensor, k: int, n: int, block_size: 
 def q8_dense_layout(words: torch.Tensor, k: int, n: int, block_size: int):
     """A Q8 buffer with one block per column (``block_size >= k``) as dense int8 ``[n, k]`` plus the ``n`` block
     scales: the operands of :func:`matmul_q8_dense`, made once per weight."""
-    if block_size <= 0 or block_size < k:
-        raise ValueError("q8_dense_layout: one block per column wanted (block_size >= k)")
-    if words.numel() < n * ((4 + block_size + 3) // 4):
+    # (block_size < k, several blocks per column, is refused by the library itself)
+    if block_size <= 0 or words.numel() < n * (-(-k // block_size)) * ((4 + block_size + 3) // 4):
         raise ValueError("q8_dense_layout: the Q8 buffer is shorter than n blocks")
     wq = torch.empty((n, k), dtype=torch.int8, device=words.device)
     sw = torch.empty(n, dtype=torch.float32, device=words.device)
