@@ -42,17 +42,23 @@ WEIGHT_SETS = 64
 # HBM bytes per GEMV launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by a 256 MiB copy
 # (profiles/w4_gemv_dot8_1x4096x4096_hbm_traffic.txt); a counter result, not measured by this script
 GEMV_TRAFFIC_BYTES = 9650224
+# untimed replays before a long matrix-core kernel is timed (see time_graph)
+SETTLE_S = 0.06
 
 
 def log(msg):
     print(msg, file=sys.stderr, flush=True)
 
 
-def time_graph(torch, launch_all, launches_per_replay, replays, warmup_replays):
+def time_graph(torch, launch_all, launches_per_replay, replays, warmup_replays, settle_s=0.0):
     """Capture `launch_all` (a burst of `launches_per_replay` launches) in a HIP graph and time exactly
     `replays` replays after `warmup_replays` untimed ones, every replay between its own pair of HIP
     events on the stream the kernels run on.  Returns a dict: seconds per LAUNCH as median / mean / min /
-    max over the replays, the replay count and whether a graph was used."""
+    max over the replays, the replay count and whether a graph was used.
+    `settle_s`: the untimed replays go on for at least this long.  A kernel that loads the matrix cores runs its
+    first few hundred launches after a quieter phase 10-25 % slower (the board's power management settles over
+    about 40 ms: 2048 x 4096 x 11008 int8 measured 107, 131, 121, 114, 107 ... 103 us per launch in successive
+    bursts of ten), so the long kernels are timed once that has passed."""
     stream = torch.cuda.current_stream()
     graph = None
     try:
@@ -74,6 +80,11 @@ def time_graph(torch, launch_all, launches_per_replay, replays, warmup_replays):
     for _ in range(max(0, int(warmup_replays))):
         run()
     torch.cuda.synchronize()
+    t_settle = time.perf_counter()
+    while time.perf_counter() - t_settle < settle_s:
+        for _ in range(4):
+            run()
+        torch.cuda.synchronize()
     marks = [torch.cuda.Event(enable_timing=True) for _ in range(replays + 1)]
     marks[0].record()
     for i in range(replays):
@@ -157,7 +168,7 @@ def bench_i8_gemm(torch, ops, replays=12, warmup=3):
         for _ in range(per_graph):
             ops.i8_gemm(xq, wq, sx, sw, None, out=y)
 
-    t = time_graph(torch, burst, per_graph, replays, warmup)
+    t = time_graph(torch, burst, per_graph, replays, warmup, SETTLE_S)
     sec = t["median"]
     ops_per = 2.0 * m * k * n
 
@@ -183,7 +194,7 @@ def bench_i8_gemm(torch, ops, replays=12, warmup=3):
             for _ in range(per_graph):
                 torch._int_mm(xq, wt)
 
-        vendor = ops_per / time_graph(torch, burst_vendor, per_graph, replays, warmup)["median"] / 1e12
+        vendor = ops_per / time_graph(torch, burst_vendor, per_graph, replays, warmup, SETTLE_S)["median"] / 1e12
     except Exception as exc:   # informational only
         log(f"[bench] vendor int8 GEMM not timed: {exc}")
     # The same kernel on operands without bit activity (all ones: every product and sum is still computed, the
@@ -197,7 +208,7 @@ def bench_i8_gemm(torch, ops, replays=12, warmup=3):
             for _ in range(per_graph):
                 ops.i8_gemm(xq1, wq1, sx, sw, None, out=y)
 
-        tq = time_graph(torch, burst_quiet, per_graph, replays, warmup)["median"]
+        tq = time_graph(torch, burst_quiet, per_graph, replays, warmup, SETTLE_S)["median"]
         quiet = {"operands": "all ones", "ms_per_launch": tq * 1e3, "tops": ops_per / tq / 1e12,
                  "frac": ops_per / tq / 1e12 / I8_PEAK_TOPS}
         wt1 = wq1.t()
@@ -206,7 +217,7 @@ def bench_i8_gemm(torch, ops, replays=12, warmup=3):
             for _ in range(per_graph):
                 torch._int_mm(xq1, wt1)
 
-        quiet["vendor_int_mm_tops"] = ops_per / time_graph(torch, burst_vendor_quiet, per_graph, replays, warmup)["median"] / 1e12
+        quiet["vendor_int_mm_tops"] = ops_per / time_graph(torch, burst_vendor_quiet, per_graph, replays, warmup, SETTLE_S)["median"] / 1e12
         del xq1, wq1, wt1
     except Exception as exc:   # informational only
         log(f"[bench] constant-operand run not timed: {exc}")
@@ -355,8 +366,9 @@ def bench_w4_gemm(torch, ops, m, replays=10, warmup=2):
         for _ in range(10):
             ops.qmatmul_int4_perm(x, packed_sorted, scales, zp, k, G, perm=perm, out=y)
 
-    sec = time_graph(torch, burst, len(copies), replays, warmup)["median"]
-    sec_res = time_graph(torch, burst_resident, 10, replays, warmup)["median"]
+    settle = SETTLE_S if m >= 512 else 0.0
+    sec = time_graph(torch, burst, len(copies), replays, warmup, settle)["median"]
+    sec_res = time_graph(torch, burst_resident, 10, replays, warmup, settle)["median"]
     del copies
     flops = 2.0 * m * k * n
     return {"workload": f"w4_gemm_actorder_{m}x4096x11008_g128", "hip_graph": True, "weight_copies_rotated": ncopy,
@@ -402,7 +414,7 @@ def bench_i8_mid(torch, ops, replays=10, warmup=2):
             for _ in range(4):
                 ops.i8_gemm(xq, wq, sx, sw, None, out=y)
 
-        sec = time_graph(torch, burst, 4, replays, warmup)["median"]
+        sec = time_graph(torch, burst, 4, replays, warmup, SETTLE_S)["median"]
         row = {"workload": f"int8_gemm_{m}x{k}x{n}", "ms_per_launch": sec * 1e3, "tops": 2.0 * m * k * n / sec / 1e12}
         try:
             wt = wq.t()
@@ -411,7 +423,7 @@ def bench_i8_mid(torch, ops, replays=10, warmup=2):
                 for _ in range(4):
                     torch._int_mm(xq, wt)
 
-            row["vendor_int_mm_tops"] = 2.0 * m * k * n / time_graph(torch, vendor, 4, replays, warmup)["median"] / 1e12
+            row["vendor_int_mm_tops"] = 2.0 * m * k * n / time_graph(torch, vendor, 4, replays, warmup, SETTLE_S)["median"] / 1e12
         except Exception as e:                      # not every torch build can capture it
             row["vendor_int_mm_tops"] = None
             log(f"vendor int_mm skipped: {e}")
@@ -441,7 +453,7 @@ def bench_grad_x(torch, ops, replays=10, warmup=2):
             for p, s_, z in sets:
                 ops.qmatmul_int4_t(gy, p, s_, z, k, G, out=out)
 
-        sec = time_graph(torch, burst, len(sets), replays, warmup)["median"]
+        sec = time_graph(torch, burst, len(sets), replays, warmup, SETTLE_S if m >= 512 else 0.0)["median"]
         rows.append({"workload": f"w4_grad_x_{m}x4096x11008_g128", "ms_per_call": sec * 1e3,
                      "weight_copies_rotated": len(sets) if m <= 128 else 1,
                      "tflops": 2.0 * m * k * n / sec / 1e12,
@@ -470,7 +482,7 @@ def bench_q8_matmul(torch, ops, replays=10, warmup=2):
                 for wds in sets:
                     ops.matmul_q8(a, wds, k, n, bs, out=c)
 
-            sec = time_graph(torch, burst, len(sets), replays, warmup)["median"]
+            sec = time_graph(torch, burst, len(sets), replays, warmup, SETTLE_S if m >= 512 else 0.0)["median"]
             rows.append({"workload": f"matmul_q8_{m}x4096x11008_bs{bs}", "ms_per_call": sec * 1e3,
                          "weight_copies_rotated": len(sets) if m <= 32 else 1,
                          "tflops": 2.0 * m * k * n / sec / 1e12,
@@ -485,7 +497,7 @@ def bench_q8_matmul(torch, ops, replays=10, warmup=2):
                     for _ in range(4):
                         ops.matmul_q8_dense(a, wq, sw, out=c)
 
-                sec = time_graph(torch, burst, 4, replays, warmup)["median"]
+                sec = time_graph(torch, burst, 4, replays, warmup, SETTLE_S)["median"]
                 rows.append({"workload": f"matmul_q8_dense_{m}x4096x11008", "ms_per_call": sec * 1e3,
                              "tflops": 2.0 * m * k * n / sec / 1e12, "weight_gbs": (k * n + 4 * n) / sec / 1e9})
             del wq, sw
@@ -604,7 +616,9 @@ def bench_decoder_block(torch, ops):
 
 def cpu_baseline(x, w, budget_s=12.0):
     """The CPU restatement of the reference kernels on the host cores: single thread (the
-    reference CpuBackend's contract) for `value`, all cores as an extra figure."""
+    reference CpuBackend's contract) for `value`, all cores as an extra figure.  Runs before the process touches
+    the GPU: the runtime's helper threads otherwise share the cores with the timed loops (the all-core figure
+    then scattered between 1.4 and 12 ms)."""
     import oracle
     t0 = time.perf_counter()
     packed, scales, zp = oracle.w4_from_f32(w, G)
@@ -657,6 +671,13 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this build targets one GPU; --gpus above 1 is not supported "
                  "(no collectives or sharding are part of it)")
+
+    cb = y_cpu = None
+    if not args.no_cpu:
+        from rumus_amd import workloads
+        w_cpu, x_cpu = workloads.w4_gemv(0)
+        cb, y_cpu = cpu_baseline(x_cpu, w_cpu)
+        del w_cpu, x_cpu
 
     import torch
     if not torch.cuda.is_available():
@@ -743,7 +764,6 @@ def main():
         out["decoder_block"] = bench_decoder_block(torch, ops)
 
     if not args.no_cpu:
-        cb, y_cpu = cpu_baseline(r["x"], r["w"])
         out["cpu_baseline"] = cb
         err = np.abs(r["y0"] - y_cpu)
         tol = 1e-4 + 1e-3 * np.abs(y_cpu)
