@@ -469,10 +469,12 @@ static int launch_i8_q(const W4I8Args& k, bool zp4, uint32_t row_blocks, hipStre
 int w4_launch_gemm_i8(const W4Args& a, hipStream_t s) {
     const uint32_t cs = a.group_size % 128 == 0 ? 2 : 1;             // chunk = 128 or 64 k: never across a group end
     const uint32_t steps = a.padded_k / 64, chunks = steps / cs, per = ceil_div(chunks, (uint32_t)kI8WK);
-    // up to 64 rows in one workgroup per column block, so that the weights are streamed once (48 rows 26.2 -> 23.7 us,
-    // 64 rows 26.7 -> 24.3 us against two blocks of 32 rows); beyond, blocks of 32 rows: eight row tiles per
-    // workgroup spill registers and run one long round (128 rows 40.0 -> 43.8 us)
-    const uint32_t rt_per = a.m <= 16 ? 1 : a.m <= 32 || a.m > 64 ? 2 : 4, row_blocks = ceil_div(a.m, 16 * rt_per), rts = row_blocks * rt_per;
+    // Rows per workgroup.  The weights are streamed once per block of rows, so blocks of 64 rows (four row tiles)
+    // where they are well filled: 48 rows 26.2 -> 23.7 us, 64 rows 26.7 -> 24.3 us, 128 rows 40.8 -> 37.5 us against
+    // blocks of 32; 65 to 96 rows stay on blocks of 32 (80 rows: 36.8 against 37.6 us with a second, mostly empty
+    // block of 64).  Eight row tiles per workgroup spill registers and run one long round (128 rows 43.8 us).
+    const uint32_t rt_per = a.m <= 16 ? 1 : a.m <= 32 || (a.m > 64 && a.m <= 96) ? 2 : 4;
+    const uint32_t row_blocks = ceil_div(a.m, 16 * rt_per), rts = row_blocks * rt_per;
     RUMUS_REQUIRE(row_blocks <= 65535, "qmatmul_int4: m %u is beyond the grid limit", a.m);
     auto up = [](size_t v) { return (v + 255) & ~size_t(255); };
     const size_t planes_bytes = (size_t)rts * steps * 3 * 1024;
