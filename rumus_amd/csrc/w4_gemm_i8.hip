@@ -35,6 +35,7 @@ typedef uint32_t u3a4 __attribute__((ext_vector_type(3), aligned(4)));
 
 constexpr int kI8WK = 8;                   // waves of a workgroup = shares of K
 constexpr uint32_t kI8MaxRows = 128;       // beyond, the f16 tile kernel's larger tiles win
+constexpr int kI8Outliers = 16;            // elements per (row, share of K) that may leave the fixed point
 
 struct W4I8Args {
     const uint32_t* packed;
@@ -45,6 +46,9 @@ struct W4I8Args {
     const uint8_t* planes;    // [row tile][step][digit][64 lanes x 16 bytes]
     const float* rscale;      // [row tile][share][16 rows]: 2^-e (NaN: that part of the row holds a NaN or an infinity)
     const int32_t* csum;      // [row tile][chunk][16 rows]: sum of the chunk's X
+    const int32_t* out_n;     // [row][share]: elements of that part of the row that are multiplied on their own
+    const int32_t* out_k;     // [row][share][kI8Outliers]: their positions (rows of the packed matrix) ...
+    const float* out_x;       // ... and values
     float* y;
     uint32_t m, n, steps, chunks, steps_per_group, per;   // per: chunks per share
 };
@@ -88,8 +92,8 @@ __device__ __forceinline__ int group_sum(int v) {
 template <int CS, bool VEC, bool STAGED>
 __global__ __launch_bounds__(STAGED ? 64 * kI8WK : 64) void w4_i8_prepare_kernel(
     const float* __restrict__ x, const int32_t* __restrict__ perm, uint8_t* __restrict__ planes,
-    float* __restrict__ rscale, int32_t* __restrict__ csum, uint32_t m, uint32_t k, uint32_t steps, uint32_t chunks,
-    uint32_t per) {
+    float* __restrict__ rscale, int32_t* __restrict__ csum, int32_t* __restrict__ out_n, int32_t* __restrict__ out_k,
+    float* __restrict__ out_x, uint32_t m, uint32_t k, uint32_t steps, uint32_t chunks, uint32_t per) {
     static_assert(!(VEC && STAGED), "staging is for the gather");
     extern __shared__ __attribute__((aligned(16))) float lds_row[];
     constexpr int CACHE = 4;
@@ -186,6 +190,47 @@ __global__ __launch_bounds__(STAGED ? 64 * kI8WK : 64) void w4_i8_prepare_kernel
         mb = max(mb, max_bits(v));
     }
     mb = wave_max(mb);
+    // Elements that tower over the rest of their part would set the fixed point for all of it and cost the others
+    // their low bits (22 bits below the LARGEST magnitude).  When only a few elements lie within 2^-8 of the largest
+    // - few enough for the slots left - they leave the fixed point: position and value go to the matmul, which
+    // multiplies them in f32 on their own, x * ((q - zp) * scale) as the reference's loop does with every element,
+    // and the part is scaled by what remains (looked at once more: towers of two heights).  Ordinary data has
+    // hundreds of elements that close to the largest and passes with one count.  Only where the whole part sits
+    // in registers (shares up to 2048 k).
+    uint32_t n_out = 0;
+    if (k_end - k_begin <= 64 * 8 * CACHE) {
+        for (int level = 0; level < 2; level++) {
+            if (mb == 0 || mb >= 0x7f800000u) break;                   // nothing there, or a NaN / an infinity: poisoned below
+            const uint32_t near_top = mb > (8u << 23) ? mb - (8u << 23) : 1u;   // the largest / 256, on the bit patterns
+            int near = 0;
+#pragma unroll
+            for (int i = 0; i < CACHE; i++)
+#pragma unroll
+                for (int j = 0; j < 8; j++) near += (__float_as_uint(cache[i][j]) & 0x7fffffffu) >= near_top ? 1 : 0;
+            near = wave_sum(near);
+            if ((uint32_t)near > (uint32_t)kI8Outliers - n_out) break;
+#pragma unroll
+            for (int i = 0; i < CACHE; i++)
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const bool hit = (__float_as_uint(cache[i][j]) & 0x7fffffffu) >= near_top;
+                    const uint64_t hits = __ballot(hit);
+                    if (hit) {
+                        const uint64_t slot = ((uint64_t)row * kI8WK + share) * kI8Outliers + n_out +
+                                              (uint32_t)__builtin_popcountll(hits & ((1ull << lane) - 1ull));
+                        out_k[slot] = (int32_t)(k_begin + (lane + 64 * i) * 8 + j);
+                        out_x[slot] = cache[i][j];
+                        cache[i][j] = 0.0f;
+                    }
+                    n_out += (uint32_t)__builtin_popcountll(hits);
+                }
+            mb = 0;
+#pragma unroll
+            for (int i = 0; i < CACHE; i++) mb = max(mb, max_bits(cache[i]));
+            mb = wave_max(mb);
+        }
+    }
+    if (lane == 0) out_n[(uint64_t)row * kI8WK + share] = (int32_t)n_out;
     // 2^e with max * 2^e in [2^21, 2^22); e stops at 126, where 2^-e is the smallest normal number, so parts whose
     // largest magnitude lies below 2^-107 keep fewer than 20 bits.  A
     // non-finite activation poisons its row: the scale becomes NaN (the digits are then whatever the
@@ -385,6 +430,42 @@ __global__ __launch_bounds__(512) void w4_gemm_i8_kernel(W4I8Args a) {
             for (int q = 0; q < Q; q++) accf[t][q] = __builtin_amdgcn_mfma_f32_16x16x4f32(sm[t], szq[q], accf[t][q], 0, 0, 0);
     }
 
+    // Elements that left the fixed point (w4_i8_prepare_kernel): x * ((q - zp) * scale) in f32, the reference's own
+    // expression, added in the accumulators' units (x / rscale: a power of two, exact).  Lane (c, b) holds rows
+    // 4b .. 4b + 3 and columns colc .. colc + Q - 1 of a tile.
+#pragma unroll
+    for (int t = 0; t < RT; t++) {
+        const uint32_t row0 = (rb * RT + t) * 16;
+        const int cnt = a.out_n[(uint64_t)(row0 + c) * WK + wk];
+        uint32_t rows_with = (uint32_t)(__ballot(cnt > 0) & 0xFFFFu);
+        while (rows_with) {                                            // wave-uniform
+            const uint32_t r = (uint32_t)__builtin_ctz(rows_with);
+            rows_with &= rows_with - 1;
+            const uint32_t n_r = (uint32_t)__builtin_amdgcn_readlane(cnt, r);
+            const float unit = 1.0f / a.rscale[((uint64_t)(rb * RT + t) * WK + wk) * 16 + r];
+            for (uint32_t o = 0; o < n_r; o++) {
+                const uint64_t slot = ((uint64_t)(row0 + r) * WK + wk) * kI8Outliers + o;
+                const uint32_t ko = (uint32_t)a.out_k[slot];
+                const float xo = a.out_x[slot] * unit;
+                const uint32_t g = (ko / 64) / a.steps_per_group;
+                uint32_t wq[Q], sq[Q], zq[Q];
+                load_q<Q>(a.packed + (uint64_t)(ko / 8) * a.n + colc, wq);
+                load_q<Q>(reinterpret_cast<const uint32_t*>(a.scales) + (uint64_t)g * a.n + colc, sq);
+                if (ZP4) zq[0] = a.zp4[(uint64_t)g * (a.n / 8) + colc / 8];
+                else load_q<Q>(reinterpret_cast<const uint32_t*>(a.zp) + (uint64_t)g * a.n + colc, zq);
+#pragma unroll
+                for (int q = 0; q < Q; q++) {
+                    const float nib = (float)((wq[q] >> (4 * (ko & 7u))) & 15u);
+                    const float z = ZP4 ? (float)((zq[0] >> (4 * ((colc & 7u) + q))) & 15u) : __uint_as_float(zq[q]);
+                    const float w = (nib - z) * __uint_as_float(sq[q]);
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        accf[t][q][i] = (b == r / 4 && (uint32_t)i == r % 4) ? fmaf(xo, w, accf[t][q][i]) : accf[t][q][i];
+                }
+            }
+        }
+    }
+
     // back to the activations' scale (this wave's share of K has its own), then the eight shares meet in LDS, two
     // row tiles per round; wave w adds them up, in a fixed order, for rows 4b + w % 4 of the round's row tile w / 4
     // and stores
@@ -478,13 +559,17 @@ int w4_launch_gemm_i8(const W4Args& a, hipStream_t s) {
     RUMUS_REQUIRE(row_blocks <= 65535, "qmatmul_int4: m %u is beyond the grid limit", a.m);
     auto up = [](size_t v) { return (v + 255) & ~size_t(255); };
     const size_t planes_bytes = (size_t)rts * steps * 3 * 1024;
-    const size_t csum_bytes = up((size_t)rts * chunks * 16 * sizeof(int32_t)), rscale_bytes = (size_t)rts * kI8WK * 16 * sizeof(float);
+    const size_t csum_bytes = up((size_t)rts * chunks * 16 * sizeof(int32_t)), rscale_bytes = up((size_t)rts * kI8WK * 16 * sizeof(float));
+    const size_t outn_bytes = up((size_t)rts * 16 * kI8WK * sizeof(int32_t)), outk_bytes = outn_bytes * kI8Outliers;
     void* ws = nullptr;
     WorkspaceLease lease;                                            // until both kernels are queued
-    if (int rc = workspace_get(s, planes_bytes + csum_bytes + rscale_bytes, &ws, lease)) return rc;
+    if (int rc = workspace_get(s, planes_bytes + csum_bytes + rscale_bytes + outn_bytes + 2 * outk_bytes, &ws, lease)) return rc;
     uint8_t* planes = static_cast<uint8_t*>(ws);
     int32_t* csum = reinterpret_cast<int32_t*>(planes + planes_bytes);
     float* rscale = reinterpret_cast<float*>(planes + planes_bytes + csum_bytes);
+    int32_t* out_n = reinterpret_cast<int32_t*>(planes + planes_bytes + csum_bytes + rscale_bytes);
+    int32_t* out_k = reinterpret_cast<int32_t*>(planes + planes_bytes + csum_bytes + rscale_bytes + outn_bytes);
+    float* out_x = reinterpret_cast<float*>(planes + planes_bytes + csum_bytes + rscale_bytes + outn_bytes + outk_bytes);
     const bool vec = !a.perm && a.k % 4 == 0 && (reinterpret_cast<uintptr_t>(a.x) & 15) == 0;
     const bool staged = a.perm && (size_t)a.k * sizeof(float) <= 64 * 1024 && a.k % 8 == 0 &&
                         ((reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.perm)) & 15) == 0;
@@ -494,19 +579,19 @@ int w4_launch_gemm_i8(const W4Args& a, hipStream_t s) {
     do {                                                                                                               \
         if (staged)                                                                                                    \
             hipLaunchKernelGGL((w4_i8_prepare_kernel<CS, false, true>), dim3(rts * 16), dim3(64 * kI8WK), row_bytes, s, \
-                               a.x, a.perm, planes, rscale, csum, a.m, a.k, steps, chunks, per);                       \
+                               a.x, a.perm, planes, rscale, csum, out_n, out_k, out_x, a.m, a.k, steps, chunks, per); \
         else if (vec)                                                                                                  \
             hipLaunchKernelGGL((w4_i8_prepare_kernel<CS, true, false>), pgrid, dim3(64), 0, s, a.x, a.perm, planes,    \
-                               rscale, csum, a.m, a.k, steps, chunks, per);                                            \
+                               rscale, csum, out_n, out_k, out_x, a.m, a.k, steps, chunks, per);                      \
         else                                                                                                           \
             hipLaunchKernelGGL((w4_i8_prepare_kernel<CS, false, false>), pgrid, dim3(64), 0, s, a.x, a.perm, planes,   \
-                               rscale, csum, a.m, a.k, steps, chunks, per);                                            \
+                               rscale, csum, out_n, out_k, out_x, a.m, a.k, steps, chunks, per);                      \
     } while (0)
     if (cs == 2) RUMUS_I8_PREPARE(2);
     else RUMUS_I8_PREPARE(1);
 #undef RUMUS_I8_PREPARE
     if (int rc = check_launch("w4_i8_prepare_kernel")) return rc;
-    const W4I8Args k{a.packed, a.scales, a.zp, a.zp4, a.bias, planes, rscale, csum, a.y,
+    const W4I8Args k{a.packed, a.scales, a.zp, a.zp4, a.bias, planes, rscale, csum, out_n, out_k, out_x, a.y,
                      a.m, a.n, steps, chunks, a.group_size / 64, per};
     const bool zp4 = a.zp4 != nullptr;
     // a wave's whole share in flight when it is up to four chunks (two for two row tiles: registers)

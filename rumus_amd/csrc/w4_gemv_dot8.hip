@@ -218,14 +218,14 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
         const uint32_t* p = TILED ? packed + ((uint64_t)cchunk * (padded_k / 8) + (uint64_t)ch * OCT) * kD8Cols + 4 * cq
                                   : packed + (uint64_t)ch * OCT * n + col_c;
         const uint64_t wstride = TILED ? kD8Cols : n;
-        float4 sc, zp;
+        float4 sc, zp;          // zp: the four zero-points, or with ZP4 their packed word in .x (unpacked where it is used)
         auto load_meta = [&]() __attribute__((always_inline)) {
             sc = *reinterpret_cast<const float4*>(scales + mo);
             // ZP4 + TILED: the two zero-point words of a tile's 16 columns sit side by side per group
-            zp = !ZP4 ? *reinterpret_cast<const float4*>(zps + mo)
-                 : TILED ? w4_zp4_unpack4(reinterpret_cast<const uint32_t*>(zps)[
-                               ((uint64_t)cchunk * (padded_k / group_size) + g) * 2 + (cq >> 1)] >> ((cq & 1) * 16))
-                         : w4_zp4_load4(reinterpret_cast<const uint32_t*>(zps), g, n, col_c);
+            if (!ZP4) zp = *reinterpret_cast<const float4*>(zps + mo);
+            else zp.x = __uint_as_float(TILED ? reinterpret_cast<const uint32_t*>(zps)[
+                                                    ((uint64_t)cchunk * (padded_k / group_size) + g) * 2 + (cq >> 1)] >> ((cq & 1) * 16)
+                                              : reinterpret_cast<const uint32_t*>(zps)[(uint64_t)g * (n / 8) + col_c / 8] >> ((col_c & 4u) * 4u));
         };
 #pragma unroll
         for (int u = 0; u < OCT; u++) w[u] = *reinterpret_cast<const uint4*>(p + (uint64_t)u * wstride);
@@ -236,7 +236,12 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
 #pragma unroll
         for (int u = 0; u < OCT; u++) { wv[u][0] = w[u].x; wv[u][1] = w[u].y; wv[u][2] = w[u].z; wv[u][3] = w[u].w; }
         const float scv[4] = {sc.x, sc.y, sc.z, sc.w};
-        const float zv[4] = {zp.x, zp.y, zp.z, zp.w};
+        // the zero-points in f32, computed where they are used (after the dot products): unpacked here, the wait for
+        // their word - the last load - would come ahead of every dot product
+        auto zero_points = [&](float (&zv)[4]) __attribute__((always_inline)) {
+            const float4 z = ZP4 ? w4_zp4_unpack4(__float_as_uint(zp.x)) : zp;
+            zv[0] = z.x; zv[1] = z.y; zv[2] = z.z; zv[3] = z.w;
+        };
 
 #pragma unroll
         for (int m = 0; m < M; m++) {
@@ -248,8 +253,19 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
             for (int t = 0; t < OPL; t++)
 #pragma unroll
                 for (int j = 0; j < 8; j++) amax = max(amax, __float_as_uint(xv[m][t][j]) & 0x7FFFFFFFu);
+            const uint32_t lane_max = amax;                // of this lane's OPL octets
             amax = max(amax, (uint32_t)RUMUS_DPP_I(amax, kDppXor1));
             amax = max(amax, (uint32_t)RUMUS_DPP_I(amax, kDppXor2));
+            // A chunk whose largest element towers over one of its four octets of 8 consecutive k (that octet's
+            // largest more than 2^8 below it) would cost that octet its low bits in the fixed point below.  Such a
+            // chunk is multiplied in f32 instead, element by element, at the end of this round (`wild`).  The
+            // octets' maxima are the lanes' own (OPL == 1) on the way to amax; ordinary data never has such a chunk.
+            uint32_t omin = lane_max;
+            omin = min(omin, (uint32_t)RUMUS_DPP_I(omin, kDppXor1));
+            omin = min(omin, (uint32_t)RUMUS_DPP_I(omin, kDppXor2));
+            // (not with packed zero-points: there the same code costs 0.3 us per launch at 1 x 4096 x 4096, as the raised
+            // priority above does, for reasons not found; that format keeps the plain fixed point)
+            const bool wild = !ZP4 && omin + (8u << 23) < amax && amax < 0x7F800000u;
             // amax = a * 2^E (1 <= a < 2): scale by just under 2^(18-E) so that |x * f| < 2^19 - 1/2
             const uint32_t ebits = amax >> 23;             // biased exponent
             // the factor 1 - 2^-20 keeps rint(amax * f) at 2^19 - 1 or below
@@ -263,6 +279,7 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
                 f = 0.0f;
                 finv = __uint_as_float(0x7FC00000u);
             }
+            finv = wild ? 0.0f : finv;     // a wild chunk's fixed point adds nothing; it is multiplied in f32 below
             uint32_t own[OPL][5];
             int xsum = 0;
 #pragma unroll
@@ -326,6 +343,8 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
 #pragma unroll
                     for (int i = 0; i < 5; i++) d[c][i] = udot8(wv[u][c], pl[u][i], d[c][i]);
                 }
+            float zv[4];
+            zero_points(zv);
 #pragma unroll
             for (int c = 0; c < 4; c++) {
                 // D < 2^31: 8*OCT*225 * (16^5 - 1) / 15
@@ -333,6 +352,35 @@ __global__ __launch_bounds__(T) void w4_gemv_dot8_kernel(
                 const int I = (int)D - (int)(qsum[c] << 19);
                 const float part = (float)I * finv;
                 acc[m][c] = fmaf(scv[c], fmaf(-zv[c], xs, part), acc[m][c]);
+            }
+            if (__builtin_expect(wild, 0)) {
+                // (the fixed point added nothing: finv was zeroed)  The reference's loop over this chunk:
+                // sum += x * ((q - zp) * scale), ascending k.  The activations are read again (the lanes of a quad
+                // ask for the same address) rather than kept in registers for a case that ordinary data never has.
+                float exact[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int u = 0; u < OCT; u++)
+#pragma unroll
+                    for (int j = 0; j < 8; j++) {
+                        const uint32_t kk = (ch * OCT + u) * 8 + j;
+                        const bool in = kk < k;
+                        const uint32_t kc = in ? kk : 0;
+                        float xe;
+                        if (FASTX) {
+                            const float* xrow = xin + (uint64_t)m * (GLU ? 2 * k : k) + kc;
+                            xe = xrow[0];
+                            if (GLU) xe = silu_mul(xe, xrow[k]);
+                            if constexpr (NORM) xe *= norm_w[kc];
+                        } else {
+                            xe = xin[(uint64_t)m * k + (perm ? (uint32_t)perm[kc] : kc)];
+                        }
+                        xe = in ? xe : 0.0f;
+#pragma unroll
+                        for (int c = 0; c < 4; c++)
+                            exact[c] = fmaf(xe, ((float)((wv[u][c] >> (4 * j)) & 15u) - zv[c]) * scv[c], exact[c]);
+                    }
+#pragma unroll
+                for (int c = 0; c < 4; c++) acc[m][c] += exact[c];
             }
         }
     }

@@ -88,8 +88,8 @@ def test_rows_of_any_magnitude(ops, m, k, n, g, act_order):
 def test_few_rows_of_any_magnitude(ops, m, act_order):
     """Up to 128 rows the kernels turn x into fixed point, 20 bits below the largest magnitude of a part of the row
     (32 consecutive k for up to 8 rows, an eighth of K beyond): uniformly scaled rows, 1e-30 to 3e33, are as
-    accurate as ordinary ones; in a part that one element dominates the others are rounded to that element's
-    2^-20, so the error there is bounded by max|x| 2^-19 sum|w| rather than by the summed terms."""
+    accurate as ordinary ones; a row with one element that dominates its part stays within the bound
+    max|x| 2^-19 sum|w| (such an element is multiplied in f32 on its own: test_outlier_columns_keep_the_tolerance)."""
     say(f"w4 forward row scaling m={m} act_order={act_order}")
     k, n, g = 1024, 1024, 128
     rng = np.random.default_rng(100 + m)
@@ -159,3 +159,43 @@ def test_q8_matmul_rows_of_any_magnitude(ops, m, bs):
     assert rel[plain].max() < 2e-6
     if m > 3:                                            # the dominated row: digit planes below the row part's maximum
         assert rel[3].max() < 2e-4
+
+
+@pytest.mark.parametrize("m", [1, 4, 16, 128])
+@pytest.mark.parametrize("act_order", [False, True])
+@pytest.mark.parametrize("big", [1000.0, 3000.0])
+def test_outlier_columns_keep_the_tolerance(ops, m, act_order, big):
+    """N(0,1) activations with outlier channels a thousand times larger, the way the hidden states of language
+    models have them (4096 -> 1024, three lone channels per row and, in row 2, a run of six neighbours): up to 128
+    rows the kernels hold x in fixed point below the largest magnitude of a part of the row, and such elements
+    would cost their neighbours the low bits.  They leave the fixed point instead - the decode kernel multiplies a
+    chunk with a towering element in f32, element by element; the int8-path kernels multiply the towering elements
+    on their own - so every output stays within rel 1e-3 / abs 1e-4 of the float64 product."""
+    say(f"w4 forward with outlier channels m={m} act_order={act_order} big={big}")
+    k, n, g = 4096, 1024, 128
+    rng = np.random.default_rng(7000 + m)
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    x = rng.normal(0, 1, (m, k)).astype(np.float32)
+    x[:, 7] = big
+    x[:, 1234] = -3 * big
+    x[:, 4000] = 0.5 * big
+    if m > 2:
+        x[2, 8:14] = np.array([2, -1, 1, 1, -2, 1], np.float32) * big
+    packed, scales, zp = oracle.w4_from_f32(w, g)
+    d = [dev(a) for a in (packed, scales, zp)]
+    if act_order:
+        perm_np = rng.permutation(k).astype(np.int32)
+        xs = x[:, perm_np]
+        got = host(ops.qmatmul_int4_perm(dev(x), *d, k, g, perm=dev(perm_np)))
+    else:
+        xs = x
+        got = host(ops.qmatmul_int4(dev(x), *d, k, g))
+    exact = xs.astype(np.float64) @ oracle.w4_dequant(packed, scales, zp, k, g).astype(np.float64)
+    err = np.abs(got - exact)
+    tol = 1e-4 + 1e-3 * np.abs(exact)
+    assert (err <= tol).all(), f"worst error / tolerance {np.max(err / tol):.2f}"
+    # for scale: the reference's own loop (f32, one element after the other) on two rows - at 3000 sigma it misses
+    # this tolerance itself on outputs near zero, the kernels above do not
+    rows = [0, min(2, m - 1)]
+    ref = oracle.qmatmul_int4(xs[rows], packed, scales, zp, k, g).astype(np.float64)
+    say(f"    kernels: worst error / tolerance {np.max(err / tol):.2f}; the f32 loop: {np.max(np.abs(ref - exact[rows]) / tol[rows]):.2f}")
