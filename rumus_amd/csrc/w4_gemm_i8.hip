@@ -46,7 +46,7 @@ struct W4I8Args {
     const uint8_t* planes;    // [row tile][step][digit][64 lanes x 16 bytes]
     const float* rscale;      // [row tile][share][16 rows]: 2^-e (NaN: that part of the row holds a NaN or an infinity)
     const int32_t* csum;      // [row tile][chunk][16 rows]: sum of the chunk's X
-    const int32_t* out_n;     // [row][share]: elements of that part of the row that are multiplied on their own
+    const uint8_t* out_n;     // [row tile][share][16 rows]: elements of that part of the row that are multiplied on their own
     const int32_t* out_k;     // [row][share][kI8Outliers]: their positions (rows of the packed matrix) ...
     const float* out_x;       // ... and values
     float* y;
@@ -92,7 +92,7 @@ __device__ __forceinline__ int group_sum(int v) {
 template <int CS, bool VEC, bool STAGED>
 __global__ __launch_bounds__(STAGED ? 64 * kI8WK : 64) void w4_i8_prepare_kernel(
     const float* __restrict__ x, const int32_t* __restrict__ perm, uint8_t* __restrict__ planes,
-    float* __restrict__ rscale, int32_t* __restrict__ csum, int32_t* __restrict__ out_n, int32_t* __restrict__ out_k,
+    float* __restrict__ rscale, int32_t* __restrict__ csum, uint8_t* __restrict__ out_n, int32_t* __restrict__ out_k,
     float* __restrict__ out_x, uint32_t m, uint32_t k, uint32_t steps, uint32_t chunks, uint32_t per) {
     static_assert(!(VEC && STAGED), "staging is for the gather");
     extern __shared__ __attribute__((aligned(16))) float lds_row[];
@@ -189,6 +189,7 @@ __global__ __launch_bounds__(STAGED ? 64 * kI8WK : 64) void w4_i8_prepare_kernel
         load8(k0, v);
         mb = max(mb, max_bits(v));
     }
+    const uint32_t lane_top = mb;                                  // this lane's largest
     mb = wave_max(mb);
     // Elements that tower over the rest of their part would set the fixed point for all of it and cost the others
     // their low bits (22 bits below the LARGEST magnitude).  When only a few elements lie within 2^-8 of the largest
@@ -199,38 +200,51 @@ __global__ __launch_bounds__(STAGED ? 64 * kI8WK : 64) void w4_i8_prepare_kernel
     // in registers (shares up to 2048 k).
     uint32_t n_out = 0;
     if (k_end - k_begin <= 64 * 8 * CACHE) {
-        for (int level = 0; level < 2; level++) {
-            if (mb == 0 || mb >= 0x7f800000u) break;                   // nothing there, or a NaN / an infinity: poisoned below
-            const uint32_t near_top = mb > (8u << 23) ? mb - (8u << 23) : 1u;   // the largest / 256, on the bit patterns
-            int near = 0;
+        // first a test that ordinary data fails at once: does any lane hold nothing within 2^-8 of the largest?  (If
+        // every lane does, 64 elements are that close: more than the slots.)
+        const uint32_t lowest_top = ~wave_max(~lane_top);
+        if (lowest_top + (8u << 23) < mb && mb < 0x7f800000u) {
+            for (int level = 0; level < 2; level++) {
+                if (mb == 0 || mb >= 0x7f800000u) break;               // nothing there, or a NaN / an infinity: poisoned below
+                const uint32_t near_top = mb > (8u << 23) ? mb - (8u << 23) : 1u;   // the largest / 256, on the bit patterns
+                int near = 0;
 #pragma unroll
-            for (int i = 0; i < CACHE; i++)
+                for (int i = 0; i < CACHE; i++)
 #pragma unroll
-                for (int j = 0; j < 8; j++) near += (__float_as_uint(cache[i][j]) & 0x7fffffffu) >= near_top ? 1 : 0;
-            near = wave_sum(near);
-            if ((uint32_t)near > (uint32_t)kI8Outliers - n_out) break;
+                    for (int j = 0; j < 8; j++) near += (__float_as_uint(cache[i][j]) & 0x7fffffffu) >= near_top ? 1 : 0;
+                int left = wave_sum(near);
+                if ((uint32_t)left > (uint32_t)kI8Outliers - n_out) break;
+                // one element at a time: the first lane that still has one hands over its first
+                while (left > 0) {
+                    int at = -1;
 #pragma unroll
-            for (int i = 0; i < CACHE; i++)
+                    for (int i = CACHE - 1; i >= 0; i--)
 #pragma unroll
-                for (int j = 0; j < 8; j++) {
-                    const bool hit = (__float_as_uint(cache[i][j]) & 0x7fffffffu) >= near_top;
-                    const uint64_t hits = __ballot(hit);
-                    if (hit) {
-                        const uint64_t slot = ((uint64_t)row * kI8WK + share) * kI8Outliers + n_out +
-                                              (uint32_t)__builtin_popcountll(hits & ((1ull << lane) - 1ull));
-                        out_k[slot] = (int32_t)(k_begin + (lane + 64 * i) * 8 + j);
-                        out_x[slot] = cache[i][j];
-                        cache[i][j] = 0.0f;
+                        for (int j = 7; j >= 0; j--)
+                            if ((__float_as_uint(cache[i][j]) & 0x7fffffffu) >= near_top) at = i * 8 + j;
+                    const uint32_t owner = (uint32_t)__builtin_ctzll(__ballot(at >= 0));
+                    if (lane == owner) {
+                        float v = 0.0f;
+#pragma unroll
+                        for (int i = 0; i < CACHE; i++)
+#pragma unroll
+                            for (int j = 0; j < 8; j++)
+                                if (at == i * 8 + j) { v = cache[i][j]; cache[i][j] = 0.0f; }
+                        const uint64_t slot = ((uint64_t)row * kI8WK + share) * kI8Outliers + n_out;
+                        out_k[slot] = (int32_t)(k_begin + (lane + 64 * (at >> 3)) * 8 + (at & 7));
+                        out_x[slot] = v;
                     }
-                    n_out += (uint32_t)__builtin_popcountll(hits);
+                    n_out++;
+                    left--;
                 }
-            mb = 0;
+                mb = 0;
 #pragma unroll
-            for (int i = 0; i < CACHE; i++) mb = max(mb, max_bits(cache[i]));
-            mb = wave_max(mb);
+                for (int i = 0; i < CACHE; i++) mb = max(mb, max_bits(cache[i]));
+                mb = wave_max(mb);
+            }
         }
     }
-    if (lane == 0) out_n[(uint64_t)row * kI8WK + share] = (int32_t)n_out;
+    if (lane == 0) out_n[((uint64_t)rt * kI8WK + share) * 16 + row_l] = (uint8_t)n_out;
     // 2^e with max * 2^e in [2^21, 2^22); e stops at 126, where 2^-e is the smallest normal number, so parts whose
     // largest magnitude lies below 2^-107 keep fewer than 20 bits.  A
     // non-finite activation poisons its row: the scale becomes NaN (the digits are then whatever the
@@ -350,6 +364,13 @@ __global__ __launch_bounds__(512) void w4_gemm_i8_kernel(W4I8Args a) {
 #pragma unroll
         for (int q = 0; q < Q; q++) accf[t][q] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 
+    // whether any element of this share of the rows of each tile left the fixed point (see the end of the kernel):
+    // sixteen byte counts at a wave-uniform address, a scalar load asked for now and looked at when the loop is done
+    uint4 out_bytes[RT];
+#pragma unroll
+    for (int t = 0; t < RT; t++)
+        out_bytes[t] = *reinterpret_cast<const uint4*>(a.out_n + ((uint64_t)(rb * RT + t) * WK + wk) * 16);
+
     // Loads retire in order, so what is issued last is waited for last: activation fragments (needed
     // first, they come out of the L2) always go ahead of the weight loads that are needed later.
     fetch_a(0, f0, 0);
@@ -435,10 +456,15 @@ __global__ __launch_bounds__(512) void w4_gemm_i8_kernel(W4I8Args a) {
     // 4b .. 4b + 3 and columns colc .. colc + Q - 1 of a tile.
 #pragma unroll
     for (int t = 0; t < RT; t++) {
+        // (the words stay opaque until the loop's results exist: looked at earlier, the wait for them would stand at
+        // the top of the kernel)
+        uint32_t any = out_bytes[t].x | out_bytes[t].y | out_bytes[t].z | out_bytes[t].w;
+        asm volatile("" : "+s"(any) : "v"(accf[t][0][0]));
+        if (any == 0) continue;                                        // wave-uniform; ordinary data ends here
         const uint32_t row0 = (rb * RT + t) * 16;
-        const int cnt = a.out_n[(uint64_t)(row0 + c) * WK + wk];
+        const int cnt = a.out_n[((uint64_t)(rb * RT + t) * WK + wk) * 16 + c];
         uint32_t rows_with = (uint32_t)(__ballot(cnt > 0) & 0xFFFFu);
-        while (rows_with) {                                            // wave-uniform
+        while (rows_with) {
             const uint32_t r = (uint32_t)__builtin_ctz(rows_with);
             rows_with &= rows_with - 1;
             const uint32_t n_r = (uint32_t)__builtin_amdgcn_readlane(cnt, r);
@@ -560,14 +586,14 @@ int w4_launch_gemm_i8(const W4Args& a, hipStream_t s) {
     auto up = [](size_t v) { return (v + 255) & ~size_t(255); };
     const size_t planes_bytes = (size_t)rts * steps * 3 * 1024;
     const size_t csum_bytes = up((size_t)rts * chunks * 16 * sizeof(int32_t)), rscale_bytes = up((size_t)rts * kI8WK * 16 * sizeof(float));
-    const size_t outn_bytes = up((size_t)rts * 16 * kI8WK * sizeof(int32_t)), outk_bytes = outn_bytes * kI8Outliers;
+    const size_t outn_bytes = up((size_t)rts * 16 * kI8WK), outk_bytes = up((size_t)rts * 16 * kI8WK * kI8Outliers * sizeof(int32_t));
     void* ws = nullptr;
     WorkspaceLease lease;                                            // until both kernels are queued
     if (int rc = workspace_get(s, planes_bytes + csum_bytes + rscale_bytes + outn_bytes + 2 * outk_bytes, &ws, lease)) return rc;
     uint8_t* planes = static_cast<uint8_t*>(ws);
     int32_t* csum = reinterpret_cast<int32_t*>(planes + planes_bytes);
     float* rscale = reinterpret_cast<float*>(planes + planes_bytes + csum_bytes);
-    int32_t* out_n = reinterpret_cast<int32_t*>(planes + planes_bytes + csum_bytes + rscale_bytes);
+    uint8_t* out_n = planes + planes_bytes + csum_bytes + rscale_bytes;
     int32_t* out_k = reinterpret_cast<int32_t*>(planes + planes_bytes + csum_bytes + rscale_bytes + outn_bytes);
     float* out_x = reinterpret_cast<float*>(planes + planes_bytes + csum_bytes + rscale_bytes + outn_bytes + outk_bytes);
     const bool vec = !a.perm && a.k % 4 == 0 && (reinterpret_cast<uintptr_t>(a.x) & 15) == 0;
