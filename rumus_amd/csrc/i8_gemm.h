@@ -38,6 +38,10 @@ int i8_launch_gemv(const int8_t* xq, const int8_t* wq, const float* sx, const fl
                    float* y, uint32_t m, uint32_t k, uint32_t n, hipStream_t s);
 
 // 5 to 32 rows, K % 256 == 0: MFMA tiles fed straight from global memory (i8_gemv.hip).
+// 5..64 rows with the activations resident in registers, where i8_resident_takes says so
+bool i8_resident_takes(uint32_t m, uint32_t k, uint32_t n);
+int i8_launch_resident(const int8_t* xq, const int8_t* wq, const float* sx, const float* sw, const float* bias, int32_t* acc,
+                       float* y, uint32_t m, uint32_t k, uint32_t n, hipStream_t s);
 int i8_launch_stream(const int8_t* xq, const int8_t* wq, const float* sx, const float* sw, const float* bias, int32_t* acc,
                      float* y, uint32_t m, uint32_t k, uint32_t n, hipStream_t s);
 

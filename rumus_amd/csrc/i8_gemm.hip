@@ -458,16 +458,20 @@ static I8Plan i8_plan_single(uint32_t m, uint32_t n) {
 
 // Which kernel takes an m x k x n product.  Pure host arithmetic: rumus_hip_i8_gemm launches what this returns,
 // and rumus_hip_i8_gemm_workspace_size replays it to size the workspace.
-enum class I8Route { Gemv, Stream, SplitRows, Wide, Dma256, Reg4x2, Mid, Small, Reg2x2, Reg1x1 };
+enum class I8Route { Gemv, Resident, Stream, SplitRows, Wide, Dma256, Reg4x2, Mid, Small, Reg2x2, Reg1x1 };
 struct I8Choice { I8Route route; uint32_t split_rows; int wide; };
 
 static I8Choice i8_choose(uint32_t m, uint32_t k, uint32_t n) {
     // decode: up to 4 rows on v_dot4_i32_i8 (4096 x 11008 from a HIP graph over rotating weight copies: 9.3, 10.0,
     // 12.7 us for 1, 2, 4 rows against 18.3 us for 8 rows on the one-wave MFMA tiles)
     if (m <= 4) return {I8Route::Gemv, 0, 0};
-    // 5 to 16 rows (to 32 on smaller weights): MFMA tiles fed straight from global memory, a workgroup per 16 columns
-    // (from HBM, 8 rows: 4096 x 11008 14.5 us against 18.1 us for the LDS-staged tiles below, 4096 x 4096 7.4 against 12.8;
-    // 32 rows: 22.5 against 20.6 and 10.8 against 14.6)
+    // 5 to 64 rows over K of 3072 to 4096 (to 8192 up to 32 rows, to 12288 up to 16): the activations stay in registers
+    // and a workgroup walks over its column tiles (from HBM, 4096 x 11008 at 5, 16, 32, 64 rows: 13.0, 14.5, 16.2, 20.6 us
+    // against 14.0, 17.6, 22.4, 26.7 for the routes below; 3072 x 8192: 8.5, 9.3, 11.4, 15.4 against 10.6, 12.9, 17.8, 20.1)
+    if (i8_resident_takes(m, k, n)) return {I8Route::Resident, 0, 0};
+    // other K, 5 to 16 rows (to 32 on smaller weights): MFMA tiles fed straight from global memory, a workgroup per 16
+    // columns (from HBM, 8 rows: 4096 x 11008 14.5 us against 18.1 us for the LDS-staged tiles below, 4096 x 4096 7.4
+    // against 12.8; 32 rows: 22.5 against 20.6 and 10.8 against 14.6)
     if (k % 256 == 0 && (m <= 16 || (m <= 32 && (uint64_t)n * k <= (32ull << 20)))) return {I8Route::Stream, 0, 0};
     // Largest tile that still gives every CU a workgroup.
     const uint64_t big = (uint64_t)ceil_div(m, 256) * ceil_div(n, 128);
@@ -575,6 +579,7 @@ extern "C" int rumus_hip_i8_gemm(const int8_t* xq, const int8_t* wq, const float
     const I8Choice c = i8_choose(m, k, n);
     switch (c.route) {
         case I8Route::Gemv: return i8_launch_gemv(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
+        case I8Route::Resident: return i8_launch_resident(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
         case I8Route::Stream: return i8_launch_stream(xq, wq, sx, sw, bias, acc, y, m, k, n, s);
         case I8Route::SplitRows: {
             const uint32_t m1 = c.split_rows;

@@ -198,3 +198,24 @@ def test_i8_many_tiles(ops, case):
     acc_want = oracle.i8_gemm_i32(xq, wq, threads=8)
     np.testing.assert_array_equal(host(acc), acc_want)
     assert_close(host(y), oracle.i8_rescale_bias(acc_want, sx, sw, bias))
+
+
+# Few rows over long K: the kernel that keeps the activations in registers (5..64 rows, K steps shared by eight waves,
+# up to three chunks of K per column tile) and its neighbours on either side of every limit.
+@pytest.mark.parametrize("k", [3008, 3072, 3136, 4096, 4160, 8192, 8256, 11008, 12288, 12352])
+def test_i8_few_rows_long_k(ops, k):
+    import torch
+    rng = np.random.default_rng(7000 + k)
+    wq_all = rng.integers(-127, 128, (4100, k)).astype(np.int8)
+    sw_all = rng.uniform(0.001, 0.1, 4100).astype(np.float32)
+    bias_all = rng.normal(0, 0.01, 4100).astype(np.float32)
+    for m, n in ((5, 4100), (16, 8), (17, 100), (31, 352), (32, 4100), (33, 16), (48, 1000), (49, 40), (64, 4100), (65, 352)):
+        say(f"sweep i8 few rows m={m} k={k} n={n}")
+        xq = rng.integers(-127, 128, (m, k)).astype(np.int8)
+        sx = rng.uniform(0.001, 0.1, m).astype(np.float32)
+        wq, sw, bias = wq_all[:n], sw_all[:n], bias_all[:n] if (m + n) % 2 else None
+        y, acc = ops.i8_gemm(torch.from_numpy(xq).cuda(), torch.from_numpy(np.ascontiguousarray(wq)).cuda(), dev(sx), dev(sw),
+                             None if bias is None else dev(bias), want_acc=True)
+        acc_want = oracle.i8_gemm_i32(xq, wq, threads=8)
+        np.testing.assert_array_equal(host(acc), acc_want)
+        assert_close(host(y), oracle.i8_rescale_bias(acc_want, sx, sw, bias))

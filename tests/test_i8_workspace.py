@@ -28,14 +28,21 @@ def test_workspace_size_never_exceeds_the_documented_bound(library):
 
 
 def test_row_split_remainders_are_counted(library):
-    # 2080 rows x 11008 columns: 2048 rows of wide blocks (no workspace) + 32 rows that share K over workgroups;
-    # the size of the whole is the size of the remainder, not 0
-    assert library.rumus_hip_i8_gemm_workspace_size(2048, 4096, 11008) == 0
-    rest = library.rumus_hip_i8_gemm_workspace_size(32, 4096, 11008)
+    # 2080 rows x 11008 columns, K = 11008: 2048 rows of wide blocks (no workspace) + 32 rows that share K over
+    # workgroups; the size of the whole is the size of the remainder, not 0
+    assert library.rumus_hip_i8_gemm_workspace_size(2048, 11008, 11008) == 0
+    rest = library.rumus_hip_i8_gemm_workspace_size(32, 11008, 11008)
     assert rest > 0
-    assert library.rumus_hip_i8_gemm_workspace_size(2080, 4096, 11008) == rest
+    assert library.rumus_hip_i8_gemm_workspace_size(2080, 11008, 11008) == rest
     for m in (2068, 2072, 2076, 2080):
-        assert library.rumus_hip_i8_gemm_workspace_size(m, 4096, 11008) > 0
+        assert library.rumus_hip_i8_gemm_workspace_size(m, 11008, 11008) > 0
+
+
+def test_resident_activation_kernel_needs_nothing(library):
+    # 5 to 64 rows with K of 3072 to 4096 (to 8192 up to 32 rows, to 12288 up to 16): one launch, no partial sums in memory
+    for m, k in ((5, 4096), (32, 4096), (64, 3072), (64, 4096), (32, 8192), (16, 11008), (16, 12288)):
+        assert library.rumus_hip_i8_gemm_workspace_size(m, k, 11008) == 0, (m, k)
+    assert library.rumus_hip_i8_gemm_workspace_size(2080, 4096, 11008) == 0   # 2048 rows of wide blocks + 32 resident
 
 
 def test_degenerate_shapes_need_nothing(library):
