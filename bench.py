@@ -664,6 +664,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10, help="untimed passes before them")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-gemv", action="store_true", help="skip the secondary workloads")
+    ap.add_argument("--with-i8-gemm", action="store_true",
+                    help="with --only-gemv: run the INT8 GEMM leg as well (the two kernels whose HBM traffic is "
+                         "taken from counters)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run plain 256 MiB device copies (reference kernel of known traffic for "
                          "scaling FETCH_SIZE / WRITE_SIZE counters)")
@@ -751,6 +754,8 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    if args.only_gemv and args.with_i8_gemm:
+        out["secondary"] = bench_i8_gemm(torch, ops)
     if not args.only_gemv:
         out["secondary"] = bench_i8_gemm(torch, ops)
         out["w4_gemv_wider"] = bench_gemv_shapes(torch, ops)

@@ -243,6 +243,31 @@ int rumus_hip_qmatmul_int4(const float* x, const uint32_t* packed,
                            uint32_t group_size, uint32_t num_groups,
                            rumus_hip_stream_t stream);
 
+/* The two quantized matmuls with half-precision activations.  The reference's
+ * kernels are typed `scalar` = f32 or f16 as the activations are
+ * (rumus/src/backend/gpu/shaders/matmul_q8.wgsl:1-5,26-28,
+ * rumus-vision/src/shaders/qmatmul_int4.wgsl:33-38; the type is picked at
+ * rumus/src/ext/mod.rs:132-150): in f16 mode activations, output and the
+ * running sum are f16.  Here a / x and c / y are IEEE half (uint16_t bits),
+ * the product runs in the f32 kernels of rumus_hip_matmul_q8 /
+ * rumus_hip_qmatmul_int4 on the widened activations (same arguments, same
+ * checks, same accuracy) and the result is rounded to f16 once, to nearest
+ * even.  Scales, zero-points and bias stay f32 (convert stored f16 metadata
+ * once with rumus_hip_f16_to_f32).  The f32 copies live in a staging buffer
+ * per (device, stream) of 4 * m * (k + n) + 512 bytes, grown inside the call
+ * like the workspace; rumus_hip_f16_staging_reserve sizes it up front for
+ * callers that must not allocate later; rumus_hip_shutdown frees it. */
+int rumus_hip_matmul_q8_f16(const uint16_t* a, const uint32_t* b, uint16_t* c,
+                            uint32_t m, uint32_t k, uint32_t n, uint32_t block_size,
+                            rumus_hip_stream_t stream);
+int rumus_hip_qmatmul_int4_f16(const uint16_t* x, const uint32_t* packed,
+                               const float* scales, const float* zero_points,
+                               const float* bias, const int32_t* g_idx, uint16_t* y,
+                               uint32_t m, uint32_t k, uint32_t n, uint32_t padded_k,
+                               uint32_t group_size, uint32_t num_groups,
+                               rumus_hip_stream_t stream);
+int rumus_hip_f16_staging_reserve(rumus_hip_stream_t stream, uint64_t bytes);
+
 /* rumus_hip_qmatmul_int4_perm for callers that cannot allocate (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No
  * counterpart in the reference.  Same arguments, same kernels and the same

@@ -59,6 +59,9 @@ PROTOTYPES = {
     "rumus_hip_w4_quantize_pack_sym": (_i32, [_vp, _u32, _u32, _u32, _vp, _vp, _vp, _vp]),
     "rumus_hip_w4_quantize_pack_awq": (_i32, [_vp, _u32, _u32, _u32, _vp, _vp, _vp, _vp]),
     "rumus_hip_f16_to_f32": (_i32, [_vp, _vp, _u64, _vp]),
+    "rumus_hip_matmul_q8_f16": (_i32, [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
+    "rumus_hip_qmatmul_int4_f16": (_i32, [_vp] * 7 + [_u32] * 6 + [_vp]),
+    "rumus_hip_f16_staging_reserve": (_i32, [_vp, _u64]),
     "rumus_hip_w4_qzeros_unpack": (_i32, [_vp, _u32, _u32, _vp, _vp]),
     "rumus_hip_w4_decode_layout": (_i32, [_vp, _vp, _vp, _u32, _u32, _u32, _vp, _vp, _vp, _vp]),
     "rumus_hip_qmatmul_int4_decode": (_i32, [_vp] * 7 + [_u32] * 6 + [_vp]),

@@ -27,13 +27,17 @@ class WorkspaceLease {
     WorkspaceLease(const WorkspaceLease&) = delete;
     WorkspaceLease& operator=(const WorkspaceLease&) = delete;
   private:
-    friend int workspace_get(hipStream_t, size_t, void**, WorkspaceLease&);
+    friend int arena_get(int, hipStream_t, size_t, void**, WorkspaceLease&);
     void* arena_ = nullptr;
 };
 
 // Device workspace of at least `bytes` for work queued on `stream` (runtime.hip); `lease` then holds the
 // stream's workspace lock.
 int workspace_get(hipStream_t stream, size_t bytes, void** out, WorkspaceLease& lease);
+// A second buffer per (device, stream), for entry points that wrap another entry point between two conversions
+// (the half-precision ones): what they stage must outlive the inner call, whose workspace may grow - that is, be
+// freed - under it.  Never nested, never replaced by a fixed buffer.
+int staging_get(hipStream_t stream, size_t bytes, void** out, WorkspaceLease& lease);
 // A call that holds workspace memory and then calls another entry point that takes workspace of its own on the
 // same stream (the Q8 matmul around the int8 GEMM) asks for both sizes at once and keeps one of these alive over
 // the inner call: workspace_get then hands out the part of the buffer behind `offset`, and fails instead of

@@ -39,11 +39,12 @@ struct Arena {
 struct ArenaKey {
     int device;
     hipStream_t stream;
-    bool operator==(const ArenaKey& o) const { return device == o.device && stream == o.stream; }
+    int kind;                        // 0: the workspace of the kernels, 1: staging buffers of the half-precision entry points
+    bool operator==(const ArenaKey& o) const { return device == o.device && stream == o.stream && kind == o.kind; }
 };
 struct ArenaKeyHash {
     size_t operator()(const ArenaKey& k) const {
-        return std::hash<const void*>()(k.stream) ^ (std::hash<int>()(k.device) * 0x9e3779b97f4a7c15ull);
+        return std::hash<const void*>()(k.stream) ^ (std::hash<int>()(k.device * 2 + k.kind) * 0x9e3779b97f4a7c15ull);
     }
 };
 std::mutex g_arena_mutex;
@@ -69,7 +70,17 @@ WorkspaceFixed::~WorkspaceFixed() {
     g_fixed_bytes = prev_bytes_;
 }
 
+int arena_get(int kind, hipStream_t stream, size_t bytes, void** out, WorkspaceLease& lease);
+
 int workspace_get(hipStream_t stream, size_t bytes, void** out, WorkspaceLease& lease) {
+    return arena_get(0, stream, bytes, out, lease);
+}
+
+int staging_get(hipStream_t stream, size_t bytes, void** out, WorkspaceLease& lease) {
+    return arena_get(1, stream, bytes, out, lease);
+}
+
+int arena_get(int kind, hipStream_t stream, size_t bytes, void** out, WorkspaceLease& lease) {
     int device = 0;
     if (int rc = check_hip(hipGetDevice(&device), "hipGetDevice")) return rc;
     if (lease.arena_) return set_error(RUMUS_HIP_EINVAL, "workspace lease used twice");
@@ -77,12 +88,12 @@ int workspace_get(hipStream_t stream, size_t bytes, void** out, WorkspaceLease& 
     {
         // the table lock covers the lookup only; entries of an unordered_map do not move
         std::lock_guard<std::mutex> lock(g_arena_mutex);
-        found = &g_arenas[ArenaKey{device, stream}];
+        found = &g_arenas[ArenaKey{device, stream, kind}];
     }
     found->in_use.lock();            // from here on this thread alone queues work that uses the buffer
     lease.arena_ = found;
     Arena& a = *found;
-    if (g_fixed_ptr) {               // a buffer of fixed size stands in for the stream's own: nothing is allocated
+    if (kind == 0 && g_fixed_ptr) {  // a buffer of fixed size stands in for the stream's own: nothing is allocated
         const size_t offset = g_nest_offset;
         if (offset + bytes > g_fixed_bytes)
             return set_error(RUMUS_HIP_EINVAL, "this call needs %zu bytes of scratch memory, the fixed buffer holds %zu",
@@ -90,7 +101,7 @@ int workspace_get(hipStream_t stream, size_t bytes, void** out, WorkspaceLease& 
         *out = static_cast<uint8_t*>(g_fixed_ptr) + offset;
         return RUMUS_HIP_OK;
     }
-    if (const size_t offset = g_nest_offset) {
+    if (const size_t offset = kind == 0 ? g_nest_offset : 0) {
         if (a.bytes < offset + bytes)
             return set_error(RUMUS_HIP_EINVAL, "nested workspace of %zu bytes behind %zu does not fit the %zu reserved", bytes,
                              offset, a.bytes);
@@ -101,8 +112,9 @@ int workspace_get(hipStream_t stream, size_t bytes, void** out, WorkspaceLease& 
         hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
         if (stream && hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
             return set_error(RUMUS_HIP_EINVAL,
-                             "workspace of %zu bytes needed while the stream is capturing: call "
-                             "rumus_hip_workspace_reserve before the capture", bytes);
+                             "%s of %zu bytes needed while the stream is capturing: call %s before the capture",
+                             kind ? "staging memory" : "workspace", bytes,
+                             kind ? "rumus_hip_f16_staging_reserve" : "rumus_hip_workspace_reserve");
         if (a.ptr) {
             if (int rc = check_hip(hipStreamSynchronize(stream), "hipStreamSynchronize")) return rc;
             if (int rc = check_hip(hipFree(a.ptr), "hipFree(workspace)")) return rc;
@@ -141,6 +153,13 @@ int rumus_hip_workspace_reserve(rumus_hip_stream_t stream, uint64_t bytes) {
     if (bytes == 0) return RUMUS_HIP_OK;
     rumus::WorkspaceLease lease;
     return rumus::workspace_get(rumus::as_stream(stream), (size_t)bytes, &p, lease);
+}
+
+int rumus_hip_f16_staging_reserve(rumus_hip_stream_t stream, uint64_t bytes) {
+    void* p = nullptr;
+    if (bytes == 0) return RUMUS_HIP_OK;
+    rumus::WorkspaceLease lease;
+    return rumus::staging_get(rumus::as_stream(stream), (size_t)bytes, &p, lease);
 }
 
 int rumus_hip_shutdown(void) { return rumus::workspace_release_all(); }

@@ -115,6 +115,12 @@ class QLinear:
     def forward(self, x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``y = x @ dequant(W) + bias`` in one launch (the reference runs a second add_bias pass)."""
         w = self.weight
+        if x.dtype == torch.float16:
+            # the reference's kernels take f16 activations as they take f32 ones (qmatmul_int4.wgsl:33-38)
+            if w.perm is not None:
+                raise NotImplementedError("f16 activations with act-order weights")
+            return ops.qmatmul_int4_f16(x, w.packed_tensor, w.scales_tensor, w.zp_tensor, w.k, w.group_size,
+                                        bias=self.bias, out=out)
         if x.shape[0] <= w.decode_rows:
             return ops.qmatmul_int4_decode(x, *w.decode, w.k, w.group_size, bias=self.bias, perm=w.perm, out=out)
         return ops.qmatmul_int4_perm(x, w.packed_tensor, w.scales_tensor, w.zp_tensor, w.k,
@@ -202,6 +208,8 @@ def matmul(lhs: torch.Tensor, rhs) -> torch.Tensor:
         raise ValueError("matmul: this path handles Q8 weights only")
     if lhs.dim() != 2 or lhs.shape[1] != rhs.shape[0]:
         raise ValueError("matmul: inner dimension mismatch")
+    if lhs.dtype == torch.float16:      # matmul_q8.wgsl:1-5: A and C are `scalar`, f32 or f16
+        return ops.matmul_q8_f16(lhs.contiguous(), rhs.buffer, rhs.shape[0], rhs.shape[1], rhs.block_size)
     dense = getattr(rhs, "_dense", None)
     if dense is not None and lhs.shape[0] >= Q8_DENSE_MIN_ROWS:
         return ops.matmul_q8_dense(lhs.contiguous(), *dense)
@@ -215,6 +223,8 @@ Q8_DENSE_MIN_ROWS = 384
 def linear_forward(linear: Linear, x: torch.Tensor, weight_q8: Q8Tensor) -> torch.Tensor:
     """``Linear::forward`` (nn/linear.rs:76-103) with the weight replaced by its Q8 form."""
     out = matmul(x, weight_q8)
+    if linear.bias is not None and out.dtype != torch.float32:
+        raise NotImplementedError("linear_forward: the bias pass is f32 only")
     return ops.add_bias(out, linear.bias) if linear.bias is not None else out
 
 

@@ -14,7 +14,7 @@ from ._lib import RumusError, call
 
 __all__ = [
     "q8_buf_size", "q8_quantize", "q8_dequantize", "q8_dequantize_kn", "matmul_q8", "q8_dense_layout", "matmul_q8_dense", "add_bias", "transpose_f32",
-    "i8_quantize_rows", "i8_quantize_cols_t", "i8_gemm", "w4_quantize_pack", "qmatmul_int4",
+    "i8_quantize_rows", "i8_quantize_cols_t", "i8_gemm", "w4_quantize_pack", "qmatmul_int4", "matmul_q8_f16", "qmatmul_int4_f16",
     "qmatmul_int4_t", "w4_actorder_prepare", "qmatmul_int4_perm", "w4_geometry", "RumusError",
 ]
 
@@ -88,6 +88,22 @@ def matmul_q8(a: torch.Tensor, words: torch.Tensor, k: int, n: int, block_size: 
     if c.shape != (m, n) or c.dtype != torch.float32 or not c.is_contiguous():
         raise ValueError("matmul: out must be a contiguous f32 [m, n] tensor")
     call("rumus_hip_matmul_q8", _dev(a, torch.float32, "a"), _dev(words, torch.int32, "b"),
+         c.data_ptr(), m, k, n, block_size, _stream())
+    return c
+
+
+def matmul_q8_f16(a: torch.Tensor, words: torch.Tensor, k: int, n: int, block_size: int, out=None) -> torch.Tensor:
+    """:func:`matmul_q8` on half-precision activations: ``a`` and the result are ``torch.float16``; the product runs in
+    the f32 kernels and is rounded to f16 once."""
+    m = a.shape[0]
+    if a.dim() != 2 or a.shape[1] != k:
+        raise ValueError("matmul: inner dimension mismatch")
+    if block_size <= 0 or words.numel() < n * (-(-k // block_size)) * ((4 + block_size + 3) // 4):
+        raise ValueError("matmul: the Q8 buffer is shorter than n columns of whole blocks (k % block_size != 0?)")
+    c = torch.empty((m, n), dtype=torch.float16, device=a.device) if out is None else out
+    if c.shape != (m, n) or c.dtype != torch.float16 or not c.is_contiguous():
+        raise ValueError("matmul: out must be a contiguous f16 [m, n] tensor")
+    call("rumus_hip_matmul_q8_f16", _dev(a, torch.float16, "a"), _dev(words, torch.int32, "b"),
          c.data_ptr(), m, k, n, block_size, _stream())
     return c
 
@@ -332,7 +348,8 @@ def qmatmul_int4_zp4(x, packed, scales, qzeros, k, group_size, bias=None, perm=N
     return y
 
 
-def _w4_sizes(who, packed, scales, zp, k, group_size, rows, bias=None, index=None, out=None, out_cols=None, zp4=False):
+def _w4_sizes(who, packed, scales, zp, k, group_size, rows, bias=None, index=None, out=None, out_cols=None, zp4=False,
+              out_dtype=torch.float32):
     """The kernels take raw pointers: a short array would be read past its end on the device.  Checks the element
     counts the geometry implies (the library itself rejects a bad group size or alignment)."""
     if group_size <= 0 or packed.dim() != 2:
@@ -348,27 +365,33 @@ def _w4_sizes(who, packed, scales, zp, k, group_size, rows, bias=None, index=Non
         raise ValueError(f"{who}: g_idx / perm must hold k = {k} entries")
     if out is not None:
         cols = n if out_cols is None else out_cols
-        if tuple(out.shape) != (rows, cols) or out.dtype != torch.float32 or not out.is_contiguous():
-            raise ValueError(f"{who}: out must be a contiguous f32 [{rows}, {cols}] tensor")
+        if tuple(out.shape) != (rows, cols) or out.dtype != out_dtype or not out.is_contiguous():
+            raise ValueError(f"{who}: out must be a contiguous {out_dtype} [{rows}, {cols}] tensor")
 
 
-def _w4_call(name, x, packed, scales, zp, bias, extra, k, group_size, out=None):
+def _w4_call(name, x, packed, scales, zp, bias, extra, k, group_size, out=None, act=torch.float32):
     m = x.shape[0]
     n = packed.shape[1]
     if x.dim() != 2 or x.shape[1] != k:
         raise ValueError("qmatmul_int4: x must be [m, k]")
-    _w4_sizes(name, packed, scales, zp, k, group_size, m, bias, extra, out)
+    _w4_sizes(name, packed, scales, zp, k, group_size, m, bias, extra, out, out_dtype=act)
     padded_k, groups = w4_geometry(k, group_size) if group_size > 0 else (k, 0)
-    y = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=x.device)
-    call(name, _dev(x, torch.float32, "x"), _dev(packed, torch.int32, "packed"),
+    y = out if out is not None else torch.empty((m, n), dtype=act, device=x.device)
+    call(name, _dev(x, act, "x"), _dev(packed, torch.int32, "packed"),
          _dev(scales, torch.float32, "scales"), _dev(zp, torch.float32, "zero_points"),
          _opt(bias, torch.float32, "bias"), _opt(extra, torch.int32, "g_idx/perm"),
-         _dev(y, torch.float32, "y"), m, k, n, padded_k, group_size, groups, _stream())
+         _dev(y, act, "y"), m, k, n, padded_k, group_size, groups, _stream())
     return y
 
 
 def qmatmul_int4(x, packed, scales, zp, k, group_size, bias=None, g_idx=None, out=None):
     return _w4_call("rumus_hip_qmatmul_int4", x, packed, scales, zp, bias, g_idx, k, group_size, out)
+
+
+def qmatmul_int4_f16(x, packed, scales, zp, k, group_size, bias=None, g_idx=None, out=None):
+    """:func:`qmatmul_int4` on half-precision activations: ``x`` and the result are ``torch.float16``; scales,
+    zero-points and bias stay f32.  The product runs in the f32 kernels and is rounded to f16 once."""
+    return _w4_call("rumus_hip_qmatmul_int4_f16", x, packed, scales, zp, bias, g_idx, k, group_size, out, torch.float16)
 
 
 def qmatmul_int4_perm(x, packed_sorted, scales, zp, k, group_size, bias=None, perm=None, out=None):

@@ -44,6 +44,12 @@ extern "C" {
     pub fn rumus_hip_w4_quantize_pack_awq(w: *const f32, k: u32, n: u32, group_size: u32, packed: *mut u32,
                                           scales: *mut f32, qzeros: *mut u32, s: Stream) -> c_int;
     pub fn rumus_hip_f16_to_f32(input: *const u16, out: *mut f32, numel: u64, s: Stream) -> c_int;
+    pub fn rumus_hip_matmul_q8_f16(a: *const u16, b: *const u32, c: *mut u16, m: u32, k: u32, n: u32, block_size: u32,
+                                   s: Stream) -> c_int;
+    pub fn rumus_hip_qmatmul_int4_f16(x: *const u16, packed: *const u32, scales: *const f32, zero_points: *const f32,
+                                      bias: *const f32, g_idx: *const i32, y: *mut u16, m: u32, k: u32, n: u32,
+                                      padded_k: u32, group_size: u32, num_groups: u32, s: Stream) -> c_int;
+    pub fn rumus_hip_f16_staging_reserve(s: Stream, bytes: u64) -> c_int;
     pub fn rumus_hip_w4_qzeros_unpack(qzeros: *const u32, num_groups: u32, n: u32, zero_points: *mut f32,
                                       s: Stream) -> c_int;
     pub fn rumus_hip_w4_decode_layout(packed: *const u32, scales: *const f32, zero_points: *const f32,

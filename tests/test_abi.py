@@ -88,6 +88,16 @@ def test_empty_calls_succeed_without_arrays_and_full_ones_need_them(library):
     assert L.rumus_hip_matmul_q8(None, None, None, 1, 64, 8, 32, None) == _lib.EINVAL
     assert L.rumus_hip_matmul_q8(None, None, None, 0, 64, 8, 6, None) == _lib.EINVAL
     assert L.rumus_hip_matmul_q8_dense(None, None, None, None, 0, 64, 8, None) == 0
+    # the half-precision entry points answer like the f32 ones they wrap
+    assert L.rumus_hip_matmul_q8_f16(None, None, None, 0, 64, 8, 32, None) == 0
+    assert L.rumus_hip_matmul_q8_f16(None, None, None, 1, 64, 8, 32, None) == _lib.EINVAL
+    assert L.rumus_hip_matmul_q8_f16(None, None, None, 0, 64, 8, 6, None) == _lib.EINVAL
+    assert L.rumus_hip_qmatmul_int4_f16(None, None, None, None, None, None, None, 0, 128, 64, 128, 64, 2, None) == 0
+    assert L.rumus_hip_qmatmul_int4_f16(None, None, None, None, None, None, None, 2, 128, 64, 128, 64, 2, None) == _lib.EINVAL
+    assert b"null buffer" in L.rumus_hip_last_error()
+    assert L.rumus_hip_qmatmul_int4_f16(None, None, None, None, None, None, None, 2, 100, 4, 128, 64, 3, None) == _lib.EINVAL
+    assert b"padded_k" in L.rumus_hip_last_error()
+    assert L.rumus_hip_f16_staging_reserve(None, 0) == 0
     assert L.rumus_hip_q8_quantize(None, None, 0, 32, None) == 0
     assert L.rumus_hip_q8_dequantize(None, None, 0, 32, None) == 0
     assert L.rumus_hip_i8_quantize_rows(None, None, None, 0, 64, None) == 0
