@@ -41,7 +41,9 @@ BYTES_U4_ZP = K * N // 2 + GROUPS * N * 4 + GROUPS * N // 2 + K * 4 + N * 4  # 9
 WEIGHT_SETS = 64
 # HBM bytes per GEMV launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by a 256 MiB copy
 # (profiles/w4_gemv_dot8_1x4096x4096_hbm_traffic.txt); a counter result, not measured by this script
-GEMV_TRAFFIC_BYTES = 9650224
+GEMV_TRAFFIC_BYTES = 9659300
+# the same for the INT8 GEMM 2048 x 4096 x 11008 (112,742,523 B read + 90,177,536 B written), same file
+I8_GEMM_TRAFFIC_BYTES = 202920059
 # untimed replays before a long matrix-core kernel is timed (see time_graph)
 SETTLE_S = 0.06
 
@@ -227,7 +229,9 @@ def bench_i8_gemm(torch, ops, replays=12, warmup=3):
         "same_kernel_constant_operands": quiet,
         "timing": spread(t),
         "roofline": {"bound": "mfma", "achieved": tops, "peak": I8_PEAK_TOPS, "unit": "TOP/s",
-                     "frac": tops / I8_PEAK_TOPS, "traffic": None},
+                     "frac": tops / I8_PEAK_TOPS, "traffic": I8_GEMM_TRAFFIC_BYTES,
+                     "traffic_from": "profiles/w4_gemv_dot8_1x4096x4096_hbm_traffic.txt (rocprofv3 FETCH_SIZE + WRITE_SIZE "
+                                     "of a counter run of this kernel, not measured by this script)"},
         "mfma_only_random_operands": ceiling,
         "frac_of_mfma_only": (tops / ceiling["tops"]) if ceiling else None,
         "vendor_int_mm_tops": vendor,
