@@ -235,7 +235,18 @@ int rumus_hip_f16_to_f32(const uint16_t* in, float* out, uint64_t numel,
  * bias may be NULL.  EXTENSION: g_idx (device int32[k], may be NULL) replaces
  * g by g_idx[row] (act-order).
  * EINVAL unless group_size % 8 == 0, padded_k == num_groups*group_size,
- * k <= padded_k < k+group_size. */
+ * k <= padded_k < k+group_size.
+ * Numerics: within rel 1e-3 / abs 1e-4 of the reference's f32 loop; rows of
+ * any magnitude; a NaN or an infinity in x poisons its own row only.  Up to
+ * 128 rows x is held in fixed point below the largest magnitude of a part of
+ * the row (20 bits per 32 k up to decode_max_rows rows, 22 bits per eighth of
+ * K beyond): |error| <= max|x| * 2^-19 * sum|w| over that part.  Elements
+ * that tower over their part by 2^8 or more are multiplied in f32 on their
+ * own (all of a chunk of 32 k in the few-row kernel; up to 16 elements per
+ * row and eighth of K beyond), so single outlier channels of thousands of
+ * sigma keep the tolerance.  The u4-zero-point decode entry point
+ * (rumus_hip_qmatmul_int4_decode_zp4) does not make that exception and keeps
+ * the plain bound.  Beyond 128 rows every element keeps 22 bits of its own. */
 int rumus_hip_qmatmul_int4(const float* x, const uint32_t* packed,
                            const float* scales, const float* zero_points,
                            const float* bias, const int32_t* g_idx, float* y,
