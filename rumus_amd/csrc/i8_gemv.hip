@@ -197,83 +197,6 @@ __global__ __launch_bounds__(256) void i8_stream_kernel(
     }
 }
 
-// 17..32 rows over weights too large for the last-level cache: two row tiles by two column tiles per workgroup (each
-// activation load serves two weight loads, where two row tiles by one column tile ask for two activation loads per weight
-// load), and eight waves that take the K steps of 64 in turn (wave w: steps w, w + 8, ...), so that the launch holds
-// as many waves as the four-wave form with one column tile.  All eight waves share the final sum.
-__global__ __launch_bounds__(512) void i8_stream8_kernel(
-    const int8_t* __restrict__ xq, const int8_t* __restrict__ wq, const float* __restrict__ sx,
-    const float* __restrict__ sw, const float* __restrict__ bias, int32_t* __restrict__ acc_out,
-    float* __restrict__ y, uint32_t M, uint32_t K, uint32_t N) {
-    __shared__ int32_t part[8][4][4][64];                      // [wave][row tile, column tile][register][lane]
-    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t c = lane & 15, q = lane >> 4;
-    const uint32_t n0 = blockIdx.x * 32;
-    const uint32_t steps = K / 64;
-    const uint32_t mine = (steps + 7 - wave) / 8;              // K steps of this wave (0 for waves 4..7 when K == 256)
-    const int8_t* bp[2];
-    const int8_t* ap[2];
-#pragma unroll
-    for (int j = 0; j < 2; j++) bp[j] = wq + (uint64_t)min(n0 + 16 * j + c, N - 1) * K + 16 * q;
-#pragma unroll
-    for (int t = 0; t < 2; t++) ap[t] = xq + (uint64_t)min(16 * t + c, M - 1) * K + 16 * q;
-    v4i acc[2][2];
-#pragma unroll
-    for (int t = 0; t < 2; t++)
-#pragma unroll
-        for (int j = 0; j < 2; j++) acc[t][j] = v4i{0, 0, 0, 0};
-    for (uint32_t i0 = 0; i0 < mine; i0 += 8) {                // 8 K steps per round, the last round maybe shorter
-        v4i b[8][2], a[8][2];
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const uint32_t kk = 64 * (wave + 8 * min(i0 + i, mine - 1));   // past the end: the last step again, not multiplied
-#pragma unroll
-            for (int j = 0; j < 2; j++) b[i][j] = *reinterpret_cast<const v4i*>(bp[j] + kk);
-#pragma unroll
-            for (int t = 0; t < 2; t++) a[i][t] = *reinterpret_cast<const v4i*>(ap[t] + kk);
-        }
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            if (i0 + i < mine) {
-#pragma unroll
-                for (int t = 0; t < 2; t++)
-#pragma unroll
-                    for (int j = 0; j < 2; j++)
-                        acc[t][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i][t], b[i][j], acc[t][j], 0, 0, 0);
-            }
-        }
-    }
-#pragma unroll
-    for (int t = 0; t < 2; t++)
-#pragma unroll
-        for (int j = 0; j < 2; j++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) part[wave][t * 2 + j][r][lane] = acc[t][j][r];
-    __syncthreads();
-    // register r of lane l: row 4 (l / 16) + r, column l % 16 of the 16 x 16 tile; wave w adds up registers
-    // 2 (w % 2) and 2 (w % 2) + 1 of tile w / 2
-    const uint32_t u = wave >> 1, t = u >> 1, j = u & 1;
-    const uint32_t col = n0 + 16 * j + c;
-    if (col >= N) return;
-    const float swc = y ? sw[col] : 0.0f, bc = (y && bias) ? bias[col] : 0.0f;
-#pragma unroll
-    for (int e = 0; e < 2; e++) {
-        const uint32_t r = 2 * (wave & 1) + e;
-        const uint32_t row = 16 * t + 4 * q + r;
-        if (row >= M) continue;
-        int32_t v = 0;
-#pragma unroll
-        for (int w = 0; w < 8; w++) v += part[w][u][r][lane];
-        const uint64_t o = (uint64_t)row * N + col;
-        if (acc_out) acc_out[o] = v;
-        if (y) {
-            float f = __fmul_rn(__fmul_rn((float)v, sx[row]), swc);
-            if (bias) f = __fadd_rn(f, bc);
-            y[o] = f;
-        }
-    }
-}
-
 // 5 to 64 rows with the activations resident in registers.  Eight waves, each an eighth of the K steps of 64 (the
 // last waves maybe fewer), load their part of the 16 RT activation rows once (8 CH steps at most: 32 RT CH registers)
 // and then walk over the workgroup's column tiles of 16 (blockIdx.x, + gridDim.x, ...) in chunks of 8 K steps, the
@@ -424,10 +347,6 @@ int i8_launch_stream(const int8_t* xq, const int8_t* wq, const float* sx, const 
         hipLaunchKernelGGL((i8_stream_kernel<1, 2>), dim3(ceil_div(n, 32)), dim3(256), 0, s, xq, wq, sx, sw, bias, acc, y, m, k, n);
     else if (m <= 16)
         hipLaunchKernelGGL((i8_stream_kernel<1, 1>), dim3(ceil_div(n, 16)), dim3(256), 0, s, xq, wq, sx, sw, bias, acc, y, m, k, n);
-    else if (getenv("RUMUS_I8_32") && atoi(getenv("RUMUS_I8_32")) == 1)
-        hipLaunchKernelGGL(i8_stream8_kernel, dim3(ceil_div(n, 32)), dim3(512), 0, s, xq, wq, sx, sw, bias, acc, y, m, k, n);
-    else if (getenv("RUMUS_I8_32") && atoi(getenv("RUMUS_I8_32")) == 2)
-        hipLaunchKernelGGL((i8_stream_kernel<2, 2>), dim3(ceil_div(n, 32)), dim3(256), 0, s, xq, wq, sx, sw, bias, acc, y, m, k, n);
     else
         hipLaunchKernelGGL((i8_stream_kernel<2, 1>), dim3(ceil_div(n, 16)), dim3(256), 0, s, xq, wq, sx, sw, bias, acc, y, m, k, n);
     return check_launch("i8_stream_kernel");
