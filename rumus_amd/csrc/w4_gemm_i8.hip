@@ -313,7 +313,7 @@ __global__ __launch_bounds__(512) void w4_gemm_i8_kernel(W4I8Args a) {
     constexpr int WK = kI8WK;
     static_assert((U * RT) % 2 == 0, "the two activation slots alternate with a fixed phase per unrolled position");
     static_assert(U <= 4, "a round's chunks are the four k slots of the zero-point MFMA");
-    constexpr int RP = RT >= 2 ? 2 : 1;                            // row tiles per round of the final sum over the shares
+    constexpr int RP = RT % 2 == 0 ? 2 : 1;                        // row tiles per round of the final sum over the shares
     static_assert(RT % RP == 0, "whole rounds");
     __shared__ float red[WK][RP * Q * 4][64];
     const uint32_t lane = threadIdx.x & 63, wk = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -576,11 +576,12 @@ static int launch_i8_q(const W4I8Args& k, bool zp4, uint32_t row_blocks, hipStre
 int w4_launch_gemm_i8(const W4Args& a, hipStream_t s) {
     const uint32_t cs = a.group_size % 128 == 0 ? 2 : 1;             // chunk = 128 or 64 k: never across a group end
     const uint32_t steps = a.padded_k / 64, chunks = steps / cs, per = ceil_div(chunks, (uint32_t)kI8WK);
-    // Rows per workgroup.  The weights are streamed once per block of rows, so blocks of 64 rows (four row tiles)
-    // where they are well filled: 48 rows 26.2 -> 23.7 us, 64 rows 26.7 -> 24.3 us, 128 rows 40.8 -> 37.5 us against
-    // blocks of 32; 65 to 96 rows stay on blocks of 32 (80 rows: 36.8 against 37.6 us with a second, mostly empty
-    // block of 64).  Eight row tiles per workgroup spill registers and run one long round (128 rows 43.8 us).
-    const uint32_t rt_per = a.m <= 16 ? 1 : a.m <= 32 || (a.m > 64 && a.m <= 96) ? 2 : 4;
+    // Rows per workgroup.  The weights are streamed once per block of rows, so the blocks are as tall as the registers
+    // allow (four row tiles: 64 rows 26.7 -> 22.8 us, 128 rows 40.8 -> 36.8 us against blocks of 32) but not taller than
+    // the rows that exist: 33 to 48 rows take one block of 48 (40 rows 21.7 -> 19.8 us against a block of 64 with an
+    // empty tile), 65 to 96 rows two blocks of 48 (80 rows 34.2 -> 31.7 us against three blocks of 32).  Eight row tiles
+    // per workgroup spill registers and run one long round (128 rows 43.8 us).
+    const uint32_t rt_per = a.m <= 16 ? 1 : a.m <= 32 ? 2 : a.m <= 48 || (a.m > 64 && a.m <= 96) ? 3 : 4;
     const uint32_t row_blocks = ceil_div(a.m, 16 * rt_per), rts = row_blocks * rt_per;
     RUMUS_REQUIRE(row_blocks <= 65535, "qmatmul_int4: m %u is beyond the grid limit", a.m);
     auto up = [](size_t v) { return (v + 255) & ~size_t(255); };
@@ -623,6 +624,7 @@ int w4_launch_gemm_i8(const W4Args& a, hipStream_t s) {
     // a wave's whole share in flight when it is up to four chunks (two for two row tiles: registers)
     if (rt_per == 1) return cs == 2 ? launch_i8_q<1, 2, 4>(k, zp4, row_blocks, s) : launch_i8_q<1, 1, 4>(k, zp4, row_blocks, s);
     if (rt_per == 2) return cs == 2 ? launch_i8_q<2, 2, 2>(k, zp4, row_blocks, s) : launch_i8_q<2, 1, 2>(k, zp4, row_blocks, s);
+    if (rt_per == 3) return cs == 2 ? launch_i8_q<3, 2, 2>(k, zp4, row_blocks, s) : launch_i8_q<3, 1, 2>(k, zp4, row_blocks, s);
     return cs == 2 ? launch_i8_q<4, 2, 2>(k, zp4, row_blocks, s) : launch_i8_q<4, 1, 2>(k, zp4, row_blocks, s);
 }
 
