@@ -763,7 +763,8 @@ def main():
     if not args.only_gemv:
         out["secondary"] = bench_i8_gemm(torch, ops)
         out["w4_gemv_wider"] = bench_gemv_shapes(torch, ops)
-        out["w4_gemm"] = [bench_w4_gemm(torch, ops, 16), bench_w4_gemm(torch, ops, 128),
+        out["w4_gemm"] = [bench_w4_gemm(torch, ops, 16), bench_w4_gemm(torch, ops, 128), bench_w4_gemm(torch, ops, 256),
+                          bench_w4_gemm(torch, ops, 512),
                           bench_w4_gemm(torch, ops, 1024), bench_w4_gemm(torch, ops, 2048)]
         out["f16_mfma_only"] = probe_f16_mfma_ceiling()
         out["q8_matmul"] = bench_q8_matmul(torch, ops)

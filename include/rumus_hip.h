@@ -238,15 +238,18 @@ int rumus_hip_f16_to_f32(const uint16_t* in, float* out, uint64_t numel,
  * k <= padded_k < k+group_size.
  * Numerics: within rel 1e-3 / abs 1e-4 of the reference's f32 loop; rows of
  * any magnitude; a NaN or an infinity in x poisons its own row only.  Up to
- * 128 rows x is held in fixed point below the largest magnitude of a part of
- * the row (20 bits per 32 k up to decode_max_rows rows, 22 bits per eighth of
- * K beyond): |error| <= max|x| * 2^-19 * sum|w| over that part.  Elements
+ * 128 rows (up to 512 where the integer matrix-core kernel is the faster one:
+ * group_size % 64 == 0 and enough columns to fill the chip) x is held in fixed
+ * point below the largest magnitude of a part of the row (20 bits per 32 k up
+ * to decode_max_rows rows, 22 bits per eighth of K beyond):
+ * |error| <= max|x| * 2^-19 * sum|w| over that part.  Elements
  * that tower over their part by 2^8 or more are multiplied in f32 on their
  * own (all of a chunk of 32 k in the few-row kernel; up to 16 elements per
  * row and eighth of K beyond), so single outlier channels of thousands of
  * sigma keep the tolerance.  The u4-zero-point decode entry point
  * (rumus_hip_qmatmul_int4_decode_zp4) does not make that exception and keeps
- * the plain bound.  Beyond 128 rows every element keeps 22 bits of its own. */
+ * the plain bound.  Larger batches, and those the f16 tile kernel takes, keep
+ * 22 bits of every element. */
 int rumus_hip_qmatmul_int4(const float* x, const uint32_t* packed,
                            const float* scales, const float* zero_points,
                            const float* bias, const int32_t* g_idx, float* y,
@@ -289,10 +292,11 @@ int rumus_hip_f16_staging_reserve(rumus_hip_stream_t stream, uint64_t bytes);
  * until the process ends; nothing is allocated or freed, on any call.
  * EINVAL ("needs ... bytes of scratch memory") when the shape needs more than
  * the array holds; the need is the qmatmul_int4 line of the workspace bounds
- * above and does not grow evenly with m: with k = 4096, n = 11008 calls of
- * 318 to 512 rows are refused (their partial sums, kept while the output has
- * few tiles, do not fit), calls of up to 317 rows and of 513 to about 1900
- * rows run.
+ * above and does not grow evenly with m: batches that share K over
+ * workgroups of the f16 tile kernel (few output tiles) need room for their
+ * partial sums.  With k = 4096, n = 11008 and groups of 128 every call up to
+ * about 1900 rows runs; with groups of 32 (which the integer kernel for up to
+ * 512 rows does not take) calls of 318 to 383 rows are refused.
  * All calls on one GPU share the one array, whatever their stream: calls that
  * overlap in time on one GPU race (calls on one stream do not overlap).
  * Nothing in the array has to start at zero: every byte a kernel reads from

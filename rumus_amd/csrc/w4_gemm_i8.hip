@@ -34,7 +34,9 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef uint32_t u3a4 __attribute__((ext_vector_type(3), aligned(4)));
 
 constexpr int kI8WK = 8;                   // waves of a workgroup = shares of K
-constexpr uint32_t kI8MaxRows = 128;       // beyond, the f16 tile kernel's larger tiles win
+constexpr uint32_t kI8AlwaysRows = 128;    // batches up to here always come here ...
+constexpr uint32_t kI8MaxRows = 512;       // ... and up to here where the rounds of workgroups are well filled; beyond, the
+                                           // f16 tile kernel's larger tiles win
 constexpr int kI8Outliers = 16;            // elements per (row, share of K) that may leave the fixed point
 
 struct W4I8Args {
@@ -532,12 +534,30 @@ __global__ __launch_bounds__(512) void w4_gemm_i8_kernel(W4I8Args a) {
     }
 }
 
+static int pick_q(uint32_t n, uint32_t row_blocks, bool zp4);
+
+// 129 to 512 rows: the workgroups (a block of 64 rows by 16 Q columns each) run one per compute unit, in rounds of 256
+// that last the same full or not.  Where the rounds are at least three quarters full, with three or four columns per
+// lane, this kernel beats the f16 tiles (4096 -> 11008: 129 rows 55.8 -> 47.8 us, 256 rows 75.4 -> 60.1, 384 rows 118 -> 98,
+// 512 rows 120 -> 118; 4096 -> 4096 at 512 rows 56.2 -> 45.6; 8192 -> 8192 at 384 rows 132 -> 107); where the column count
+// only fills the rounds with two columns per lane it loses (11008 -> 4096 at 384 rows 91 -> 101 us, 8192 -> 8192 at 160
+// rows 68 -> 72) and the f16 tiles keep the batch.
+static bool i8_rounds_filled(uint32_t m, uint32_t n, bool zp4) {
+    const uint32_t row_blocks = ceil_div(m, 64);
+    const uint32_t q = (uint32_t)pick_q(n, row_blocks, zp4);
+    const uint64_t wgs = (uint64_t)ceil_div(n, 16 * q) * row_blocks;
+    const uint64_t rounds = (wgs + 255) / 256;
+    return q >= 3 && wgs * 4 >= rounds * 256 * 3;
+}
+
 bool w4_gemm_i8_supported(const W4Args& a) {
     const uintptr_t bits = reinterpret_cast<uintptr_t>(a.packed) | reinterpret_cast<uintptr_t>(a.scales) |
                            reinterpret_cast<uintptr_t>(a.zp) | reinterpret_cast<uintptr_t>(a.y) |
                            (a.bias ? reinterpret_cast<uintptr_t>(a.bias) : 0);
-    return a.m > 0 && a.m <= kI8MaxRows && a.group_size % 64 == 0 && a.n % 4 == 0 && a.n >= 4 && (bits & 15) == 0 &&
-           !a.g_idx && !a.tiled && !a.glu && (!a.zp4 || a.n % 8 == 0);
+    if (!(a.m > 0 && a.m <= kI8MaxRows && a.group_size % 64 == 0 && a.n % 4 == 0 && a.n >= 4 && (bits & 15) == 0 &&
+          !a.g_idx && !a.tiled && !a.glu && (!a.zp4 || a.n % 8 == 0)))
+        return false;
+    return a.m <= kI8AlwaysRows || i8_rounds_filled(a.m, a.n, a.zp4 != nullptr);
 }
 
 template <int Q, int RT, int CS, int U>

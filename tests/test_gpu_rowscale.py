@@ -161,18 +161,19 @@ def test_q8_matmul_rows_of_any_magnitude(ops, m, bs):
         assert rel[3].max() < 2e-4
 
 
-@pytest.mark.parametrize("m", [1, 4, 16, 128])
+@pytest.mark.parametrize("m,n", [(1, 1024), (4, 1024), (16, 1024), (128, 1024), (256, 4096), (512, 4096)])
 @pytest.mark.parametrize("act_order", [False, True])
 @pytest.mark.parametrize("big", [1000.0, 3000.0])
-def test_outlier_columns_keep_the_tolerance(ops, m, act_order, big):
+def test_outlier_columns_keep_the_tolerance(ops, m, n, act_order, big):
     """N(0,1) activations with outlier channels a thousand times larger, the way the hidden states of language
-    models have them (4096 -> 1024, three lone channels per row and, in row 2, a run of six neighbours): up to 128
-    rows the kernels hold x in fixed point below the largest magnitude of a part of the row, and such elements
+    models have them (4096 -> 1024, three lone channels per row and, in row 2, a run of six neighbours; 4096 -> 4096 at
+    256 and 512 rows, which the int8-path kernels take where the columns fill the chip): up to 128 rows, and in those
+    larger batches, the kernels hold x in fixed point below the largest magnitude of a part of the row, and such elements
     would cost their neighbours the low bits.  They leave the fixed point instead - the decode kernel multiplies a
     chunk with a towering element in f32, element by element; the int8-path kernels multiply the towering elements
     on their own - so every output stays within rel 1e-3 / abs 1e-4 of the float64 product."""
-    say(f"w4 forward with outlier channels m={m} act_order={act_order} big={big}")
-    k, n, g = 4096, 1024, 128
+    say(f"w4 forward with outlier channels m={m} n={n} act_order={act_order} big={big}")
+    k, g = 4096, 128
     rng = np.random.default_rng(7000 + m)
     w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
     x = rng.normal(0, 1, (m, k)).astype(np.float32)

@@ -29,10 +29,9 @@ def test_static_scratch_entry_point_matches_the_allocating_one(ops):
     ps, perm = ops.w4_actorder_prepare(dev(packed), dev(g_idx), g)
     sd, zd = dev(scales), dev(zp)
     bias = dev(rng.normal(0, 0.01, n).astype(np.float32))
-    # Calls in a row that share the array, each with the contents the one before left in it.  128, 16 and 48 rows
-    # run the int8-path kernels (digit planes, chunk sums and row scales in the array); 192 and 300 rows the f16
-    # tiles with K shared over three and two workgroups per tile, whose partial tiles (25-26 MB) fill most of the
-    # array behind the converted activations; 1024 rows the f16 tiles without partial tiles (18 MB of activations).
+    # Calls in a row that share the array, each with the contents the one before left in it.  Up to 300 rows run the
+    # int8-path kernels (digit planes, chunk sums, row scales and the lists of towering elements in the array); 1024
+    # rows the f16 tiles without partial tiles (18 MB of converted activations).
     outs = []
     for m in (128, 192, 16, 300, 48, 1024, 16):
         say(f"qmatmul_int4_perm_static m={m} k={k} n={n} act-order")
@@ -49,6 +48,20 @@ def test_static_scratch_entry_point_matches_the_allocating_one(ops):
         want = oracle.qmatmul_int4(xs[rows], unsorted_w["packed"], unsorted_w["scales"], unsorted_w["zp"], k, g,
                                    bias=host(bias), g_idx=g_idx, threads=8)
         assert_close(ys[rows], want)
+    # Groups of 32 are not for the int8 path: 192 and 300 rows run the f16 tiles with K shared over three and two
+    # workgroups per tile, whose partial tiles (25-26 MB) fill most of the array behind the converted activations -
+    # after calls that left other contents there.
+    p32, s32, z32 = oracle.w4_from_f32(w, 32)
+    pd, sd32, zd32 = dev(p32), dev(s32), dev(z32)
+    for m in (192, 16, 300):
+        say(f"qmatmul_int4_perm_static m={m} k={k} n={n} g=32")
+        x = dev(rng.normal(0, 1, (m, k)).astype(np.float32))
+        y = torch.empty((m, n), dtype=torch.float32, device="cuda")
+        ops.qmatmul_int4_perm_static(x, pd, sd32, zd32, k, 32, bias=bias, out=y)
+        want = ops.qmatmul_int4_perm(x, pd, sd32, zd32, k, 32, bias=bias)
+        np.testing.assert_array_equal(host(y), host(want), err_msg=f"g=32 m={m}")
+        rows = [0, m - 1]
+        assert_close(host(y)[rows], oracle.qmatmul_int4(host(x)[rows], p32, s32, z32, k, 32, bias=host(bias), threads=8))
     say("qmatmul_int4_perm_static small weight, plain order, few rows (no scratch needed)")
     k2, n2 = 512, 256
     w2 = rng.normal(0, 0.02, (k2, n2)).astype(np.float32)
