@@ -238,7 +238,7 @@ int rumus_hip_f16_to_f32(const uint16_t* in, float* out, uint64_t numel,
  * k <= padded_k < k+group_size.
  * Numerics: within rel 1e-3 / abs 1e-4 of the reference's f32 loop; rows of
  * any magnitude; a NaN or an infinity in x poisons its own row only.  Up to
- * 128 rows (up to 512 where the integer matrix-core kernel is the faster one:
+ * 128 rows (up to 1024 where the integer matrix-core kernel is the faster one:
  * group_size % 64 == 0 and enough columns to fill the chip) x is held in fixed
  * point below the largest magnitude of a part of the row (20 bits per 32 k up
  * to decode_max_rows rows, 22 bits per eighth of K beyond):
@@ -295,8 +295,8 @@ int rumus_hip_f16_staging_reserve(rumus_hip_stream_t stream, uint64_t bytes);
  * above and does not grow evenly with m: batches that share K over
  * workgroups of the f16 tile kernel (few output tiles) need room for their
  * partial sums.  With k = 4096, n = 11008 and groups of 128 every call up to
- * about 1900 rows runs; with groups of 32 (which the integer kernel for up to
- * 512 rows does not take) calls of 318 to 383 rows are refused.
+ * about 1900 rows runs; with groups of 32 (which the integer kernel does not
+ * take) calls of 318 to 383 rows are refused.
  * All calls on one GPU share the one array, whatever their stream: calls that
  * overlap in time on one GPU race (calls on one stream do not overlap).
  * Nothing in the array has to start at zero: every byte a kernel reads from

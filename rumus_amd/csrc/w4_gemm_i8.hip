@@ -25,6 +25,8 @@
 // by side.  Weights go global -> registers -> MFMA, a wave's whole share in flight when it is four
 // chunks or fewer; the activation planes come out of the L2 (every workgroup reads all of them, 3 bytes
 // per element).
+#include <algorithm>
+
 #include "w4.h"
 
 namespace rumus {
@@ -35,8 +37,9 @@ typedef uint32_t u3a4 __attribute__((ext_vector_type(3), aligned(4)));
 
 constexpr int kI8WK = 8;                   // waves of a workgroup = shares of K
 constexpr uint32_t kI8AlwaysRows = 128;    // batches up to here always come here ...
-constexpr uint32_t kI8MaxRows = 512;       // ... and up to here where the rounds of workgroups are well filled; beyond, the
-                                           // f16 tile kernel's larger tiles win
+constexpr uint32_t kI8FilledRows = 512;    // ... up to here where the rounds of workgroups are well filled ...
+constexpr uint32_t kI8MaxRows = 1024;      // ... and up to here where the f16 tile kernel's rounds are badly filled; beyond,
+                                           // its larger tiles win
 constexpr int kI8Outliers = 16;            // elements per (row, share of K) that may leave the fixed point
 
 struct W4I8Args {
@@ -550,6 +553,25 @@ static bool i8_rounds_filled(uint32_t m, uint32_t n, bool zp4) {
     return q >= 3 && wgs * 4 >= rounds * 256 * 3;
 }
 
+// 513 to 1024 rows (k, n >= 4096): both kernels run in rounds, and the f16 tiles of 64 x 512 make few of them: where this
+// kernel's estimate is under 0.8 of theirs it wins by 4 to 24 % (4096 -> 11008 at 768 rows 215 -> 179 us: 264 tiles are
+// two rounds of the f16 kernel; 4096 -> 4096 at 768 rows 90 -> 70; 8192 -> 8192 at 576 rows 253 -> 171), elsewhere the two
+// are within a few percent of each other or the f16 tiles are ahead (5120 -> 13824 at 576 rows 179 against 212 us).
+// Estimates in microseconds at k = 4096 (both scale with k): workgroups here cost 8.5 + 3.2 Q each, a round of the
+// eight-wave f16 tiles 120, its four-wave form as w4_launch_gemm prices it.
+static bool i8_beats_f16_rounds(uint32_t m, uint32_t n, bool zp4) {
+    const uint32_t row_blocks = ceil_div(m, 64);
+    const uint32_t q = (uint32_t)pick_q(n, row_blocks, zp4);
+    if (q < 3) return false;
+    const double wgs = (double)ceil_div(n, 16 * q) * row_blocks;
+    const double est_i8 = (wgs / 256.0 + 0.5) * (8.5 + 3.2 * q) * (14.3 / 18.1);
+    const uint64_t tiles = (uint64_t)row_blocks * ceil_div(n, 512), full = (tiles + 255) / 256;
+    const uint64_t halves = ((uint64_t)row_blocks * ceil_div(n, 256) + 255) / 256;
+    double units = 0.97 * (double)full;
+    if (tiles >= 192) units = std::min(units, (double)(halves / 2) * 1.05 + (double)(halves % 2) * 0.75);
+    return est_i8 <= 0.8 * units * 120.0;
+}
+
 bool w4_gemm_i8_supported(const W4Args& a) {
     const uintptr_t bits = reinterpret_cast<uintptr_t>(a.packed) | reinterpret_cast<uintptr_t>(a.scales) |
                            reinterpret_cast<uintptr_t>(a.zp) | reinterpret_cast<uintptr_t>(a.y) |
@@ -557,7 +579,9 @@ bool w4_gemm_i8_supported(const W4Args& a) {
     if (!(a.m > 0 && a.m <= kI8MaxRows && a.group_size % 64 == 0 && a.n % 4 == 0 && a.n >= 4 && (bits & 15) == 0 &&
           !a.g_idx && !a.tiled && !a.glu && (!a.zp4 || a.n % 8 == 0)))
         return false;
-    return a.m <= kI8AlwaysRows || i8_rounds_filled(a.m, a.n, a.zp4 != nullptr);
+    if (a.m <= kI8AlwaysRows) return true;
+    if (a.m <= kI8FilledRows) return i8_rounds_filled(a.m, a.n, a.zp4 != nullptr);
+    return a.k >= 4096 && a.n >= 4096 && i8_beats_f16_rounds(a.m, a.n, a.zp4 != nullptr);
 }
 
 template <int Q, int RT, int CS, int U>

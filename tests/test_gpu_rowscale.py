@@ -161,13 +161,13 @@ def test_q8_matmul_rows_of_any_magnitude(ops, m, bs):
         assert rel[3].max() < 2e-4
 
 
-@pytest.mark.parametrize("m,n", [(1, 1024), (4, 1024), (16, 1024), (128, 1024), (256, 4096), (512, 4096)])
+@pytest.mark.parametrize("m,n", [(1, 1024), (4, 1024), (16, 1024), (128, 1024), (256, 4096), (512, 4096), (768, 4096)])
 @pytest.mark.parametrize("act_order", [False, True])
 @pytest.mark.parametrize("big", [1000.0, 3000.0])
 def test_outlier_columns_keep_the_tolerance(ops, m, n, act_order, big):
     """N(0,1) activations with outlier channels a thousand times larger, the way the hidden states of language
     models have them (4096 -> 1024, three lone channels per row and, in row 2, a run of six neighbours; 4096 -> 4096 at
-    256 and 512 rows, which the int8-path kernels take where the columns fill the chip): up to 128 rows, and in those
+    256, 512 and 768 rows, which the int8-path kernels take where the columns fill the chip): up to 128 rows, and in those
     larger batches, the kernels hold x in fixed point below the largest magnitude of a part of the row, and such elements
     would cost their neighbours the low bits.  They leave the fixed point instead - the decode kernel multiplies a
     chunk with a towering element in f32, element by element; the int8-path kernels multiply the towering elements
