@@ -249,7 +249,10 @@ int rumus_hip_f16_to_f32(const uint16_t* in, float* out, uint64_t numel,
  * sigma keep the tolerance.  The u4-zero-point decode entry point
  * (rumus_hip_qmatmul_int4_decode_zp4) does not make that exception and keeps
  * the plain bound.  Larger batches, and those the f16 tile kernel takes, keep
- * 22 bits of every element. */
+ * 22 bits of every element and add in f32.  That kernel is faster on tables
+ * of integer zero-points (what AWQ and GPTQ checkpoints hold; it looks before
+ * it multiplies): an eighth of its work at groups of 128, more at smaller
+ * groups, exists only for their fractional part. */
 int rumus_hip_qmatmul_int4(const float* x, const uint32_t* packed,
                            const float* scales, const float* zero_points,
                            const float* bias, const int32_t* g_idx, float* y,

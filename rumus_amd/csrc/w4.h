@@ -37,6 +37,9 @@ struct W4Args {
     // [2^14, 2^15) before the split into f16 planes (rinv), and its reciprocal for the results (rfac)
     const float* rinv = nullptr;
     const float* rfac = nullptr;
+    // w4_gemm_tile only (set by its launcher; f32 zero-points): kZpFlagWords words, nonzero where a part of the
+    // zero-point table holds a value that is no integer (w4_zp_scan_kernel)
+    const uint32_t* zflags = nullptr;
 };
 
 // zero-points of 4 (col % 4 == 0) or 2 (col % 2 == 0) adjacent columns from the packed form

@@ -60,21 +60,23 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 constexpr int kTileCols = 512;   // columns per workgroup of eight waves
 constexpr int kStageK = 128;     // rows of K staged per barrier (8 MFMA steps of 16)
 constexpr int kMaxSplits = 16;
+constexpr uint32_t kZpFlagWords = 256;   // blocks of w4_zp_scan_kernel, one flag word each
 
-// one packed word -> B fragment, k order 0,4,1,5,2,6,3,7
-__device__ __forceinline__ v8h nibbles_to_f16(uint32_t w) {
-    const v2h k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
-    const v2h k64 = {(_Float16)-64.0f, (_Float16)-64.0f};
+// one packed word -> B fragment, k order 0,4,1,5,2,6,3,7, with the column's integer zero-point z taken off on the way:
+// the magic-number conversion ends in a subtraction anyway (1024 + n - 1024, and (1024 + 16 n) / 16 - 64 for the nibbles
+// that sit four bits higher), so 1024 + z and 64 + z in place of the constants cost nothing.  n - z is an exact f16.
+// big = {1024 + z, 1024 + z}, small = {-(64 + z), -(64 + z)}.
+__device__ __forceinline__ v8h nibbles_to_f16(uint32_t w, v2h big, v2h small) {
     const v2h k16th = {(_Float16)0.0625f, (_Float16)0.0625f};
     const uint32_t t0 = (w & 0x000F000Fu) | 0x64006400u;          // 1024 + n0, 1024 + n4
     const uint32_t t1 = (w & 0x00F000F0u) | 0x64006400u;          // 1024 + 16 n1, 1024 + 16 n5
     const uint32_t w8 = w >> 8;
     const uint32_t t2 = (w8 & 0x000F000Fu) | 0x64006400u;         // n2, n6
     const uint32_t t3 = (w8 & 0x00F000F0u) | 0x64006400u;         // 16 n3, 16 n7
-    const v2h h0 = __builtin_bit_cast(v2h, t0) - k1024;
-    const v2h h1 = __builtin_elementwise_fma(__builtin_bit_cast(v2h, t1), k16th, k64);   // exact: (1024+16n)/16 - 64
-    const v2h h2 = __builtin_bit_cast(v2h, t2) - k1024;
-    const v2h h3 = __builtin_elementwise_fma(__builtin_bit_cast(v2h, t3), k16th, k64);
+    const v2h h0 = __builtin_bit_cast(v2h, t0) - big;
+    const v2h h1 = __builtin_elementwise_fma(__builtin_bit_cast(v2h, t1), k16th, small);   // exact: (1024+16n)/16 - 64 - z
+    const v2h h2 = __builtin_bit_cast(v2h, t2) - big;
+    const v2h h3 = __builtin_elementwise_fma(__builtin_bit_cast(v2h, t3), k16th, small);
     return v8h{h0[0], h0[1], h1[0], h1[1], h2[0], h2[1], h3[0], h3[1]};
 }
 
@@ -156,6 +158,13 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
     const uint32_t word_rows = a.padded_k / 8;
     const uint32_t k_end = min(a.padded_k, st_end * kStageK);
     if (tid < BM) lds_rf[tid] = a.rfac[min(m0 + tid, a.m - 1)];          // read after the stages' barriers
+
+    // Whether any zero-point of the table has a rest at all (found by w4_zp_scan_kernel before this launch):
+    // checkpoints store integers (as f32 here, or packed), and then the rank-1 updates - an eighth of the
+    // matrix-core time at groups of 128 - are left out.  Requested here, looked at before the first stage.
+    uint4 zflag = make_uint4(0, 0, 0, 0);
+    if constexpr (!ZP4) zflag = reinterpret_cast<const uint4*>(a.zflags)[lane];
+    static_assert(kZpFlagWords == 256, "four flag words per lane");
 
     // ---- staging role: thread t converts 16 consecutive k (MFMA step t%8) of row t/8 -----
     const uint32_t s_row = tid >> 3, s_step = tid & 7;
@@ -298,6 +307,25 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
     floats_t sc_cur, zp_cur, sc_after[DEPTH][NF], zp_after[DEPTH][NF];
     meta_load(g_cur, sc_cur, zp_cur);
     sc_cur = nonzero(sc_cur);
+    // The zero-point of the current group, split: its nearest integer z (kept within what 1024 + z holds exactly in
+    // f16) leaves the weights in the conversion, so that the matrix cores sum x (q - z) - an element that towers over
+    // its row then weighs in with its own small product where q is near the zero-point, not with two large sums that
+    // cancel -, and the rest, zp - z, stays in the rank-1 update below.
+    v2h z_big[TN], z_small[TN];
+    float z_rest[TN];
+    auto split_zero = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const float zp = flt_of(zp_cur, j);
+            float z = fminf(fmaxf(rintf(zp), -1008.0f), 1008.0f);
+            z = zp == zp ? z : 0.0f;                          // a NaN zero-point stays whole in the rank-1 term
+            z_rest[j] = zp - z;
+            const _Float16 b = (_Float16)(1024.0f + z), sm = (_Float16)(-64.0f - z);
+            z_big[j] = v2h{b, b};
+            z_small[j] = v2h{sm, sm};
+        }
+    };
+    split_zero();
 
     // metadata of the groups that follow the settlement points of stage `st`
     auto stage_meta_load = [&](uint32_t st, int set) __attribute__((always_inline)) {
@@ -306,21 +334,24 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
             meta_load((st * kStageK + (f + 1) * FOLD * 16) / a.group_size, sc_after[set][f], zp_after[set][f]);
     };
 
-    auto fold = [&](uint32_t buf, int s_last, uint32_t kend, int set, int f) __attribute__((always_inline)) {
-        // rank-1 update acc[i][j] += X[i] (x) (-zp[j]) on the f32 matrix core: operand slot k=0
-        // carries the values (lanes 0..31), slot k=1 (lanes 32..63) is zero
-        float zb[TN];
+    auto fold = [&](uint32_t buf, int s_last, uint32_t kend, int set, int f, auto rest_tag) __attribute__((always_inline)) {
+        // rank-1 update acc[i][j] += X[i] (x) (-(zp[j] - z[j])) on the f32 matrix core: operand slot k=0
+        // carries the values (lanes 0..31), slot k=1 (lanes 32..63) is zero; compiled out of the loop that runs when
+        // every zero-point is an integer
+        if constexpr (decltype(rest_tag)::value) {
+            float zb[TN];
 #pragma unroll
-        for (int j = 0; j < TN; j++) zb[j] = kb == 0 ? -flt_of(zp_cur, j) : 0.0f;
+            for (int j = 0; j < TN; j++) zb[j] = kb == 0 ? -z_rest[j] : 0.0f;
 #pragma unroll
-        for (int i = 0; i < RT; i++) {
-            float xs = 0.0f;
+            for (int i = 0; i < RT; i++) {
+                float xs = 0.0f;
 #pragma unroll
-            for (int cc = 0; cc < FOLD; cc++) xs += lds_xs[buf][s_last - cc][(wm * RT + i) * 32 + l32];
-            xs = kb == 0 ? xs : 0.0f;
+                for (int cc = 0; cc < FOLD; cc++) xs += lds_xs[buf][s_last - cc][(wm * RT + i) * 32 + l32];
+                xs = kb == 0 ? xs : 0.0f;
 #pragma unroll
-            for (int j = 0; j < TN; j++)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(xs, zb[j], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(xs, zb[j], acc[i][j], 0, 0, 0);
+            }
         }
         const uint32_t g_after = kend / a.group_size;
         if (kend < k_end && g_after != g_cur) {           // uniform: a new group starts
@@ -337,6 +368,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
             g_cur = g_after;
             sc_cur = sn;
             zp_cur = zp_after[set][f];
+            split_zero();
         }
     };
 
@@ -356,7 +388,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
 
     // Multiply stage `st` from LDS buffer `buf`; refill the weight registers for stage
     // st+DEPTH and convert the activations of stage st+1 into the other buffer.
-    auto compute = [&](uint32_t st, uint32_t buf, auto set_tag) __attribute__((always_inline)) {
+    auto compute = [&](uint32_t st, uint32_t buf, auto set_tag, auto rest_tag) __attribute__((always_inline)) {
         constexpr int SET = decltype(set_tag)::value;
         if (PREFETCH) read_frags(buf, 0, 0);
 #pragma unroll
@@ -371,7 +403,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
             }
             v8h bfr[TN];
 #pragma unroll
-            for (int j = 0; j < TN; j++) bfr[j] = nibbles_to_f16(word_of(wq[SET][s], j));
+            for (int j = 0; j < TN; j++) bfr[j] = nibbles_to_f16(word_of(wq[SET][s], j), z_big[j], z_small[j]);
             weight_load(st + DEPTH, SET, s);
             // all hi products, then all lo products: dependent MFMAs are TN*RT apart
 #pragma unroll
@@ -384,7 +416,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
 #pragma unroll
                 for (int j = 0; j < TN; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[cur][i], bfr[j], acc[i][j], 0, 0, 0);
-            if ((s + 1) % FOLD == 0) fold(buf, s, st * kStageK + (s + 1) * 16, SET, s / FOLD);
+            if ((s + 1) % FOLD == 0) fold(buf, s, st * kStageK + (s + 1) * 16, SET, s / FOLD, rest_tag);
             if (s >= 8 - PIECES) stage_store_piece(st + 1, buf ^ 1, s - (8 - PIECES), DEPTH - 1 - SET);
         }
         stage_meta_load(st + DEPTH, SET);
@@ -403,18 +435,27 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
     if (DEPTH == 2) stage_load(st_begin + 1, DEPTH - 1);
 #pragma unroll
     for (int piece = 0; piece < PIECES; piece++) stage_store_piece(st_begin, 0, piece, 0);
-    uint32_t buf = 0;
-    for (uint32_t st = st_begin; st < st_end; st += DEPTH) {
-        lds_barrier();                                // buffer `buf` staged; the other one is free
-        stage_load(st + DEPTH, 0);
-        compute(st, buf, std::integral_constant<int, 0>{});
-        buf ^= 1;
-        if (DEPTH == 2 && st + 1 < st_end) {
-            lds_barrier();
-            stage_load(st + 1 + DEPTH, DEPTH - 1);
-            compute(st + 1, buf, std::integral_constant<int, DEPTH - 1>{});
+    // The loop exists twice, with and without the rank-1 updates.
+    auto stages = [&](auto rest_tag) __attribute__((always_inline)) {
+        uint32_t buf = 0;
+        for (uint32_t st = st_begin; st < st_end; st += DEPTH) {
+            lds_barrier();                                // buffer `buf` staged; the other one is free
+            stage_load(st + DEPTH, 0);
+            compute(st, buf, std::integral_constant<int, 0>{}, rest_tag);
             buf ^= 1;
+            if (DEPTH == 2 && st + 1 < st_end) {
+                lds_barrier();
+                stage_load(st + 1 + DEPTH, DEPTH - 1);
+                compute(st + 1, buf, std::integral_constant<int, DEPTH - 1>{}, rest_tag);
+                buf ^= 1;
+            }
         }
+    };
+    if constexpr (ZP4) {
+        stages(std::false_type{});
+    } else {
+        if (__builtin_amdgcn_ballot_w64((zflag.x | zflag.y | zflag.z | zflag.w) != 0) != 0) stages(std::true_type{});
+        else stages(std::false_type{});
     }
 
     // ---- store: for each row a lane holds TN adjacent columns ----------------------------
@@ -484,6 +525,28 @@ static uint32_t pick_splits(uint32_t tiles, uint32_t nstages, uint32_t* stages_p
     const uint32_t sps = ceil_div(nstages, want);
     *stages_per_split = sps;
     return ceil_div(nstages, sps);                       // no empty split
+}
+
+// flags[block] = 1 when the block's share of the zero-point table (count4 float4) holds a value that is no integer
+// within the range that the tile kernel takes off inside its f16 conversion, else 0.  Every word is written by every
+// launch: nothing to clear.
+__global__ __launch_bounds__(256) void w4_zp_scan_kernel(const float4* __restrict__ zp, uint32_t count4,
+                                                         uint32_t* __restrict__ flags) {
+    bool mine = false;
+    const uint32_t step = kZpFlagWords * 256;
+    for (uint32_t i = blockIdx.x * 256 + threadIdx.x; i < count4; i += 4 * step) {
+        float4 z[4];
+#pragma unroll
+        for (uint32_t u = 0; u < 4; u++) z[u] = zp[min(i + u * step, count4 - 1)];
+#pragma unroll
+        for (uint32_t u = 0; u < 4; u++) {
+            const float v[4] = {z[u].x, z[u].y, z[u].z, z[u].w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) mine = mine || !(v[j] == rintf(v[j]) && fabsf(v[j]) <= 1008.0f);   // a NaN counts
+        }
+    }
+    const int any = __syncthreads_or(mine);
+    if (threadIdx.x == 0) flags[blockIdx.x] = any ? 1u : 0u;
 }
 
 // xp[r][j] = x[r][perm[j]] (perm null: j) for j < k, 0 for k <= j < k4: the act-order column
@@ -770,14 +833,22 @@ static int launch_tile(const W4Args& a_in, hipStream_t s) {
     const size_t x_bytes = PRE ? 2 * plane_bytes + sums_bytes
                                : prepare ? (((size_t)a.m * k4 * sizeof(float) + 255) & ~size_t(255)) : 0;
     const size_t part_bytes = splits > 1 ? (size_t)splits * a.m * a.n * sizeof(float) : 0;
-    const size_t fac_bytes = ((size_t)2 * a.m * sizeof(float) + 255) & ~size_t(255);   // rinv[m], rfac[m]
+    const size_t flag_bytes = kZpFlagWords * sizeof(uint32_t);
+    const size_t fac_bytes = flag_bytes + (((size_t)2 * a.m * sizeof(float) + 255) & ~size_t(255));   // flags, rinv[m], rfac[m]
     float* out = a.y;
     WorkspaceLease lease;                                    // until the last kernel of this call is queued
     {
         void* ws = nullptr;
         if (int rc = workspace_get(s, fac_bytes + x_bytes + part_bytes, &ws, lease)) return rc;
-        float* fac = static_cast<float*>(ws);
+        uint32_t* zflags = static_cast<uint32_t*>(ws);
+        float* fac = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + flag_bytes);
         ws = static_cast<uint8_t*>(ws) + fac_bytes;
+        if (!a.zp4) {
+            hipLaunchKernelGGL(w4_zp_scan_kernel, dim3(kZpFlagWords), dim3(256), 0, s, reinterpret_cast<const float4*>(a.zp),
+                               (uint32_t)((uint64_t)a.num_groups * a.n / 4), zflags);
+            if (int rc = check_launch("w4_zp_scan_kernel")) return rc;
+            a.zflags = zflags;
+        }
         a.rinv = fac;
         a.rfac = fac + a.m;
         // the pre-converting kernels that hold whole rows (in LDS for the gather, in registers for plain x) find

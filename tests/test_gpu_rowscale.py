@@ -26,9 +26,8 @@ def ops():
 def test_rows_of_any_magnitude(ops, m, k, n, g, act_order):
     """Batches beyond 128 rows split x into two f16 planes: every row is first scaled by a power of two into
     f16's range, so rows of 1e-12, rows of 1e9 and a row with one element of 2e5 (beyond f16's 65504) come
-    out as accurate as ordinary ones, in units of the summed terms (of the two sums the kernels keep, for the
-    dominated row); multiplying x by 2^40 multiplies y by
-    2^40 exactly; an infinity or a NaN poisons its own row only."""
+    out as accurate as ordinary ones, in units of the summed terms (for the dominated row: plus half a quantization
+    step per term); multiplying x by 2^40 multiplies y by 2^40 exactly; an infinity or a NaN poisons its own row only."""
     say(f"w4 forward row scaling m={m} k={k} n={n} g={g} act_order={act_order}")
     rng = np.random.default_rng(m + n)
     w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
@@ -58,12 +57,13 @@ def test_rows_of_any_magnitude(ops, m, k, n, g, act_order):
     assert np.isfinite(got).all()
     rel = np.abs(got - exact) / terms
     assert np.delete(rel, 3, axis=0).max() < 2e-6
-    # row 3: the kernels sum x q and x separately per group (scale (sum x q - zp sum x)), so where the dominating
-    # element meets a weight that dequantizes to almost nothing the two sums cancel: judged in units of
-    # |x| (q + zp) scale there
+    # row 3: the kernels sum x (q - z) with z the zero-point's nearest integer, and add (zp - z) sum x per group, so the
+    # dominating element weighs in with its own product plus at most half a step of its weight's scale: judged in
+    # units of |x| (|q - z| + |zp - z|) scale
     q = oracle.w4_unpack(packed, k).astype(np.float64)                      # [k, n] nibbles
     rows_of_group = np.repeat(np.arange(scales.shape[0]), g)[:k]
-    factored = np.abs(xs[3]).astype(np.float64) @ ((q + np.abs(zp[rows_of_group])) * scales[rows_of_group])
+    zr = np.rint(zp[rows_of_group]).astype(np.float64)
+    factored = np.abs(xs[3]).astype(np.float64) @ ((np.abs(q - zr) + np.abs(zp[rows_of_group] - zr)) * scales[rows_of_group])
     assert (np.abs(got[3] - exact[3]) / factored).max() < 2e-6
     np.testing.assert_array_equal(got[4], np.zeros(n, np.float32))
     say("  times 2^40")
@@ -81,6 +81,39 @@ def test_rows_of_any_magnitude(ops, m, k, n, g, act_order):
         out = host(call(dev(xb)))
         assert np.isnan(out[9]).all()
         np.testing.assert_array_equal(np.delete(out, 9, axis=0), np.delete(got, 9, axis=0))
+
+
+@pytest.mark.parametrize("m,k,n,g", [(160, 512, 1024, 128), (600, 1024, 2048, 32), (1100, 1024, 2048, 64)])
+def test_integer_zero_points_and_one_that_is_not(ops, m, k, n, g):
+    """The f16 kernel takes the nearest integer of a zero-point off inside its conversion of the weights and
+    leaves out the update for the rest when the whole table holds integers (a small kernel looks first).  One
+    entry that is no integer - anywhere in the table, here the last group's last column, then the first's first -,
+    one beyond the range the conversion holds exactly, and a NaN each bring the update back: judged against the
+    float64 product, in units of the summed terms; the NaN poisons its own column only."""
+    say(f"w4 forward integer zero-points m={m} k={k} n={n} g={g}")
+    rng = np.random.default_rng(m + g)
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    x = rng.normal(0, 1, (m, k)).astype(np.float32)
+    packed, scales, zp = oracle.w4_from_f32(w, g, symmetric=True)
+    assert (zp == np.rint(zp)).all()
+    zp = rng.integers(0, 16, zp.shape).astype(np.float32)            # integers, not all the same
+    cases = [("integers", None, None), ("last", (-1, -1), 7.25), ("first", (0, 0), 0.5), ("middle", (zp.shape[0] // 2, n // 2 + 1), -3.75),
+             ("large", (0, 5), 5000.0), ("large negative", (-1, 6), -70000.0), ("nan", (0, 9), np.nan)]
+    for name, at, value in cases:
+        z = zp.copy()
+        if at is not None:
+            z[at] = value
+        say(f"  {name}")
+        got = host(ops.qmatmul_int4(dev(x), dev(packed), dev(scales), dev(z), k, g))
+        deq = oracle.w4_dequant(packed, scales, z, k, g).astype(np.float64)
+        exact = x.astype(np.float64) @ deq
+        terms = np.abs(x).astype(np.float64) @ np.abs(deq) + 1e-300
+        if name == "nan":
+            col = at[1]
+            assert np.isnan(got[:, col]).all()
+            got, exact, terms = (np.delete(a, col, axis=1) for a in (got, exact, terms))
+        assert np.isfinite(got).all()
+        assert (np.abs(got - exact) / terms).max() < 2e-6
 
 
 @pytest.mark.parametrize("m", [1, 4, 8, 16, 64, 128])
