@@ -158,47 +158,66 @@ __global__ __launch_bounds__(64 * KW, 2) void w4t_gemm_kernel(
     //   last (and any slot left over): lanes 0..15 two f16 zero-point integers each (columns 2 lane,
     //         2 lane + 1); the other lanes fetch the same words again, into the unused tail of the stage
     const uint32_t l8 = lane >> 3, p8 = lane & 7;
-    const uint8_t* src[kTLoads];
-    uint32_t dst[kTLoads], colw[kTLoads], esz[kTLoads];        // colw: the lane's first column inside a step
-    bool wide[kTLoads], is_gy[kTLoads];                        // dst: offset inside the slot of its kind
+    // Address of a load = a base that is the same for the whole wave (array, tile, and the step's columns: scalar
+    // registers, advanced by scalar arithmetic) + a 32-bit offset per lane that never changes (row, column inside the
+    // step): no vector instruction per load and step.  Only a step that reaches past n (the last one when n % 32 != 0)
+    // works its addresses out lane by lane, to send the columns past n to column 0.
+    const uint8_t* ubase[kTLoads];                             // wave-uniform
+    uint32_t voff[kTLoads], colw[kTLoads];                     // per lane; colw: the lane's first column inside a step
+    uint32_t dst[kTLoads], esz[kTLoads];                       // dst: offset inside the slot of its kind
+    bool wide[kTLoads], is_gy[kTLoads];
+    const uint32_t zf_off = (uint32_t)(reinterpret_cast<const uint8_t*>(zf) - reinterpret_cast<const uint8_t*>(sp));   // one workspace: < 2^32
 #pragma unroll
     for (int i = 0; i < kTLoads; i++) {
         uint32_t q = KW * i + wave;
         if (HALF && q >= 4) q += 4;                            // no loads of rows 32..63 of grad_y
         is_gy[i] = q < 8;
         if (q < 8) {
-            const uint32_t row = min(m0 + 8 * q + l8, m - 1);
-            src[i] = reinterpret_cast<const uint8_t*>(gy + (uint64_t)row * n);
+            const uint32_t row = min(m0 + 8 * q + l8, m - 1) - m0;
+            ubase[i] = reinterpret_cast<const uint8_t*>(gy + (uint64_t)m0 * n);
             // rows two apart would put the conversion's 128-bit reads two to a bank: every other pair of rows
             // holds its 16-byte pieces swapped in twos (LDS piece p of row r = piece p ^ (r / 2 % 2) of the tile)
             dst[i] = q * 1024; colw[i] = 4 * (p8 ^ ((l8 >> 1) & 1)); wide[i] = true; esz[i] = 4;
+            voff[i] = (row * n + colw[i]) * 4;                 // < 64 n 4
         } else if (q < 8 + WS) {
             // the tile's 4 KW word rows (< padded_k / 8: whole groups exist in the arrays); lanes past them
             // fetch its last row again, into room the stage keeps for that
-            const uint32_t wr = k0 / 8 + min(8 * (q - 8) + l8, 4u * KW - 1);
-            src[i] = reinterpret_cast<const uint8_t*>(packed + (uint64_t)wr * n);
+            const uint32_t wr = min(8 * (q - 8) + l8, 4u * KW - 1);
+            ubase[i] = reinterpret_cast<const uint8_t*>(packed + (uint64_t)(k0 / 8) * n);
             dst[i] = (q - 8) * 1024; colw[i] = 4 * p8; wide[i] = true; esz[i] = 4;
+            voff[i] = (wr * n + colw[i]) * 4;
         } else if (q == 8 + WS) {
-            src[i] = reinterpret_cast<const uint8_t*>((lane < 32 ? sp : zf) + (uint64_t)g * n);
+            ubase[i] = reinterpret_cast<const uint8_t*>(sp + (uint64_t)g * n);   // zf lies zf_off behind sp
             dst[i] = kTRawW; colw[i] = lane & 31; wide[i] = false; esz[i] = 4;
+            voff[i] = colw[i] * 4 + (lane < 32 ? 0 : zf_off);
         } else {
-            src[i] = reinterpret_cast<const uint8_t*>(zo + (uint64_t)g * n);
+            ubase[i] = reinterpret_cast<const uint8_t*>(zo + (uint64_t)g * n);
             dst[i] = kTRawW + kTRawSz; colw[i] = 2 * (lane & 15); wide[i] = false; esz[i] = 2;
+            voff[i] = colw[i] * 2;
         }
     }
-    // columns past n are fetched from column 0: the conversion turns them into zeros
     auto issue = [&](uint32_t st, uint32_t gslot, uint32_t wslot) {
         uint8_t* const gbase = raw_gy + gslot * kTRawGy;
         uint8_t* const wbase = raw_wt + wslot * kTRawWt;
         const uint32_t c0 = min(st, st1 - 1) * 32;
+        if (c0 + 32 <= n) {
 #pragma unroll
-        for (int i = 0; i < kTLoads; i++) {
-            uint8_t* const base = is_gy[i] ? gbase : wbase;
-            const uint32_t col = c0 + colw[i] < n ? c0 + colw[i] : 0;
-            if (wide[i])
-                __builtin_amdgcn_global_load_lds((gptr_t)(src[i] + (uint64_t)col * esz[i]), (lptr_t)(base + dst[i]), 16, 0, 0);
-            else
-                __builtin_amdgcn_global_load_lds((gptr_t)(src[i] + (uint64_t)col * esz[i]), (lptr_t)(base + dst[i]), 4, 0, 0);
+            for (int i = 0; i < kTLoads; i++) {
+                uint8_t* const base = is_gy[i] ? gbase : wbase;
+                const uint8_t* const sb = ubase[i] + (uint64_t)c0 * esz[i];
+                if (wide[i]) __builtin_amdgcn_global_load_lds((gptr_t)(sb + voff[i]), (lptr_t)(base + dst[i]), 16, 0, 0);
+                else __builtin_amdgcn_global_load_lds((gptr_t)(sb + voff[i]), (lptr_t)(base + dst[i]), 4, 0, 0);
+            }
+        } else {
+            // columns past n are fetched from column 0: the conversion turns them into zeros
+#pragma unroll
+            for (int i = 0; i < kTLoads; i++) {
+                uint8_t* const base = is_gy[i] ? gbase : wbase;
+                const uint32_t col = c0 + colw[i] < n ? c0 + colw[i] : 0;
+                const uint8_t* const p = ubase[i] + (voff[i] - colw[i] * esz[i]) + (uint64_t)col * esz[i];
+                if (wide[i]) __builtin_amdgcn_global_load_lds((gptr_t)p, (lptr_t)(base + dst[i]), 16, 0, 0);
+                else __builtin_amdgcn_global_load_lds((gptr_t)p, (lptr_t)(base + dst[i]), 4, 0, 0);
+            }
         }
     };
 
@@ -236,7 +255,13 @@ __global__ __launch_bounds__(64 * KW, 2) void w4t_gemm_kernel(
             // to f16 in two different ways (v_fma_mixlo_f16 of the exact product here, a conversion of the
             // rounded f32 there), which on a tie differ by a whole f16 step that hi + lo then misses.
             const auto h2 = __builtin_amdgcn_cvt_pkrtz(a[e], a[e + 1]);
-            const auto l2 = __builtin_amdgcn_cvt_pkrtz(a[e] - (float)h2[0], a[e + 1] - (float)h2[1]);
+            // a - hi is exact (the low bits of a): one mixed-precision fma each (the f16 half read in place) instead of
+            // a conversion and a subtraction, which is what the compiler makes of the plain expression
+            const uint32_t h2b = __builtin_bit_cast(uint32_t, h2);
+            float r0, r1;
+            asm("v_fma_mix_f32 %0, %1, -1.0, %2 op_sel:[0,0,0] op_sel_hi:[1,0,0]" : "=v"(r0) : "v"(h2b), "v"(a[e]));
+            asm("v_fma_mix_f32 %0, %1, -1.0, %2 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r1) : "v"(h2b), "v"(a[e + 1]));
+            const auto l2 = __builtin_amdgcn_cvt_pkrtz(r0, r1);
             hi[e / 2] = __builtin_bit_cast(uint32_t, h2);
             lo[e / 2] = __builtin_bit_cast(uint32_t, l2);
         }
