@@ -68,11 +68,15 @@ constexpr uint32_t kZpFlagWords = 256;   // blocks of w4_zp_scan_kernel, one fla
 // big = {1024 + z, 1024 + z}, small = {-(64 + z), -(64 + z)}.
 __device__ __forceinline__ v8h nibbles_to_f16(uint32_t w, v2h big, v2h small) {
     const v2h k16th = {(_Float16)0.0625f, (_Float16)0.0625f};
-    const uint32_t t0 = (w & 0x000F000Fu) | 0x64006400u;          // 1024 + n0, 1024 + n4
-    const uint32_t t1 = (w & 0x00F000F0u) | 0x64006400u;          // 1024 + 16 n1, 1024 + 16 n5
+    // (w & mask) | 0x64006400 in one instruction each: v_and_or_b32 may read one scalar register only, so the masks
+    // live in vector registers (the compiler, left to itself, keeps both constants scalar and issues an AND and an OR)
+    const uint32_t m_lo = 0x000F000Fu, m_hi = 0x00F000F0u, magic = 0x64006400u;
     const uint32_t w8 = w >> 8;
-    const uint32_t t2 = (w8 & 0x000F000Fu) | 0x64006400u;         // n2, n6
-    const uint32_t t3 = (w8 & 0x00F000F0u) | 0x64006400u;         // 16 n3, 16 n7
+    uint32_t t0, t1, t2, t3;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(t0) : "v"(w), "v"(m_lo), "s"(magic));    // 1024 + n0, 1024 + n4
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(t1) : "v"(w), "v"(m_hi), "s"(magic));    // 1024 + 16 n1, 1024 + 16 n5
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(t2) : "v"(w8), "v"(m_lo), "s"(magic));   // n2, n6
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(t3) : "v"(w8), "v"(m_hi), "s"(magic));   // 16 n3, 16 n7
     const v2h h0 = __builtin_bit_cast(v2h, t0) - big;
     const v2h h1 = __builtin_elementwise_fma(__builtin_bit_cast(v2h, t1), k16th, small);   // exact: (1024+16n)/16 - 64 - z
     const v2h h2 = __builtin_bit_cast(v2h, t2) - big;
