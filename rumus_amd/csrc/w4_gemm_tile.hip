@@ -315,21 +315,26 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
     // f16) leaves the weights in the conversion, so that the matrix cores sum x (q - z) - an element that towers over
     // its row then weighs in with its own small product where q is near the zero-point, not with two large sums that
     // cancel -, and the rest, zp - z, stays in the rank-1 update below.
+    // The weights of a step are converted while the matrix cores work on the step before (b_next below), so the
+    // conversion's constants change one step ahead of the group: z_rest belongs to the group being multiplied,
+    // z_rest_next to the one being converted.
     v2h z_big[TN], z_small[TN];
-    float z_rest[TN];
-    auto split_zero = [&]() __attribute__((always_inline)) {
+    float z_rest[TN], z_rest_next[TN];
+    auto split_zero = [&](const floats_t& zps) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < TN; j++) {
-            const float zp = flt_of(zp_cur, j);
+            const float zp = flt_of(zps, j);
             float z = fminf(fmaxf(rintf(zp), -1008.0f), 1008.0f);
             z = zp == zp ? z : 0.0f;                          // a NaN zero-point stays whole in the rank-1 term
-            z_rest[j] = zp - z;
+            z_rest_next[j] = zp - z;
             const _Float16 b = (_Float16)(1024.0f + z), sm = (_Float16)(-64.0f - z);
             z_big[j] = v2h{b, b};
             z_small[j] = v2h{sm, sm};
         }
     };
-    split_zero();
+    split_zero(zp_cur);
+#pragma unroll
+    for (int j = 0; j < TN; j++) z_rest[j] = z_rest_next[j];
 
     // metadata of the groups that follow the settlement points of stage `st`
     auto stage_meta_load = [&](uint32_t st, int set) __attribute__((always_inline)) {
@@ -372,7 +377,8 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
             g_cur = g_after;
             sc_cur = sn;
             zp_cur = zp_after[set][f];
-            split_zero();
+#pragma unroll
+            for (int j = 0; j < TN; j++) z_rest[j] = z_rest_next[j];      // split when the group's first step was converted
         }
     };
 
@@ -392,8 +398,19 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
 
     // Multiply stage `st` from LDS buffer `buf`; refill the weight registers for stage
     // st+DEPTH and convert the activations of stage st+1 into the other buffer.
+    // B fragments of the step that comes next, converted while the matrix cores are busy with the current one: a wave
+    // cannot issue anything while it waits to issue an MFMA, so conversion and MFMAs of the same step one after
+    // the other leave the vector ALU idle during the MFMAs and the matrix cores idle during the conversion.
+    // (Not the four-wave shape: it has no registers for a second set of fragments and converts in place.)
+    constexpr bool PIPE = WAVES == 8 && FOLD >= 4;      // groups of 32 change their constants every other step: 5 % slower pipelined
+    v8h b_next[TN];
+    auto convert_words = [&](const words_t& wv) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) b_next[j] = nibbles_to_f16(word_of(wv, j), z_big[j], z_small[j]);
+    };
     auto compute = [&](uint32_t st, uint32_t buf, auto set_tag, auto rest_tag) __attribute__((always_inline)) {
         constexpr int SET = decltype(set_tag)::value;
+        constexpr int SETN = (SET + 1) % DEPTH;              // the set of the stage after this one
         if (PREFETCH) read_frags(buf, 0, 0);
 #pragma unroll
         for (int s = 0; s < 8; s++) {
@@ -406,9 +423,28 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
                 read_frags(buf, s, 0);
             }
             v8h bfr[TN];
+            const uint32_t kend = st * kStageK + (s + 1) * 16;
+            const bool group_ends = (s + 1) % FOLD == 0 && kend < k_end && kend / a.group_size != g_cur;
+            if constexpr (PIPE) {
 #pragma unroll
-            for (int j = 0; j < TN; j++) bfr[j] = nibbles_to_f16(word_of(wq[SET][s], j), z_big[j], z_small[j]);
-            weight_load(st + DEPTH, SET, s);
+                for (int j = 0; j < TN; j++) bfr[j] = b_next[j];
+                // the next step: of this stage, or the first of the next one (its words were requested a stage ago;
+                // past the end of K they are some valid words and the result is never used).  Where a group ends
+                // with this step, the next one is converted with the constants of the group that follows.
+                if (group_ends) split_zero(zp_after[SET][s / FOLD]);
+                if (s + 1 < 8) {
+                    convert_words(wq[SET][s + 1]);
+                    weight_load(st + DEPTH, SET, s + 1);
+                } else {
+                    convert_words(wq[SETN][0]);
+                    weight_load(st + 1 + DEPTH, SETN, 0);
+                }
+            } else {
+                convert_words(wq[SET][s]);
+                weight_load(st + DEPTH, SET, s);
+#pragma unroll
+                for (int j = 0; j < TN; j++) bfr[j] = b_next[j];
+            }
             // all hi products, then all lo products: dependent MFMAs are TN*RT apart
 #pragma unroll
             for (int i = 0; i < RT; i++)
@@ -420,7 +456,15 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
 #pragma unroll
                 for (int j = 0; j < TN; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[cur][i], bfr[j], acc[i][j], 0, 0, 0);
-            if ((s + 1) % FOLD == 0) fold(buf, s, st * kStageK + (s + 1) * 16, SET, s / FOLD, rest_tag);
+            if constexpr (PIPE) {                     // one MFMA, then its share of the conversion's vector instructions in its shadow
+#pragma unroll
+                for (int i = 0; i < 2 * RT * TN; i++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, (9 * TN + 6 + 2 * RT * TN - 1) / (2 * RT * TN), 0);
+                }
+            }
+            if (!PIPE && group_ends) split_zero(zp_after[SET][s / FOLD]);     // this step's words are converted: the next group's constants
+            if ((s + 1) % FOLD == 0) fold(buf, s, kend, SET, s / FOLD, rest_tag);
             if (s >= 8 - PIECES) stage_store_piece(st + 1, buf ^ 1, s - (8 - PIECES), DEPTH - 1 - SET);
         }
         stage_meta_load(st + DEPTH, SET);
@@ -439,6 +483,10 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
     if (DEPTH == 2) stage_load(st_begin + 1, DEPTH - 1);
 #pragma unroll
     for (int piece = 0; piece < PIECES; piece++) stage_store_piece(st_begin, 0, piece, 0);
+    if constexpr (PIPE) {
+        convert_words(wq[0][0]);
+        weight_load(st_begin + DEPTH, 0, 0);
+    }
     // The loop exists twice, with and without the rank-1 updates.
     auto stages = [&](auto rest_tag) __attribute__((always_inline)) {
         uint32_t buf = 0;
