@@ -71,7 +71,8 @@ int rumus_hip_sync(rumus_hip_stream_t stream);
  * bounds per call, in bytes:
  *   qmatmul_int4 / _perm / _zp4, m > 5: 5 * (m + 64) * (padded_k + 128) (activations
  *       in matrix-core order and a scale factor per row) + 64 * m * n (partial
- *       sums, only while the output has fewer than 192 tiles of 64 x 512) + 256;
+ *       sums, only while the output has fewer than 192 tiles of 64 x 512) + 1280
+ *       (the last kilobyte: flags of the look at the zero-point table);
  *   qmatmul_int4_t, m >= 8: 64 * m * k (partial sums, only below 512 tiles of
  *       64 x 128) + 10 * num_groups * n + 4 * (m + num_groups) + 2048;
  *   i8_gemm: rumus_hip_i8_gemm_workspace_size(m, k, n) exactly; at most
