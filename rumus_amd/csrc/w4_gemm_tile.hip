@@ -166,8 +166,9 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
     // Whether any zero-point of the table has a rest at all (found by w4_zp_scan_kernel before this launch):
     // checkpoints store integers (as f32 here, or packed), and then the rank-1 updates - an eighth of the
     // matrix-core time at groups of 128 - are left out.  Requested here, looked at before the first stage.
+    // (No flags - small batches, where the look costs more than it saves: the updates run.)
     uint4 zflag = make_uint4(0, 0, 0, 0);
-    if constexpr (!ZP4) zflag = reinterpret_cast<const uint4*>(a.zflags)[lane];
+    if constexpr (!ZP4) zflag = a.zflags ? reinterpret_cast<const uint4*>(a.zflags)[lane] : make_uint4(1, 0, 0, 0);
     static_assert(kZpFlagWords == 256, "four flag words per lane");
 
     // ---- staging role: thread t converts 16 consecutive k (MFMA step t%8) of row t/8 -----
@@ -895,7 +896,8 @@ static int launch_tile(const W4Args& a_in, hipStream_t s) {
         uint32_t* zflags = static_cast<uint32_t*>(ws);
         float* fac = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + flag_bytes);
         ws = static_cast<uint8_t*>(ws) + fac_bytes;
-        if (!a.zp4) {
+        // the look at the zero-points takes 2.5 to 3 us: from 128 rows on the updates it may save cost more
+        if (!a.zp4 && a.m >= 128) {
             hipLaunchKernelGGL(w4_zp_scan_kernel, dim3(kZpFlagWords), dim3(256), 0, s, reinterpret_cast<const float4*>(a.zp),
                                (uint32_t)((uint64_t)a.num_groups * a.n / 4), zflags);
             if (int rc = check_launch("w4_zp_scan_kernel")) return rc;
