@@ -37,9 +37,9 @@ typedef uint32_t u3a4 __attribute__((ext_vector_type(3), aligned(4)));
 
 constexpr int kI8WK = 8;                   // waves of a workgroup = shares of K
 constexpr uint32_t kI8AlwaysRows = 128;    // batches up to here always come here ...
-constexpr uint32_t kI8FilledRows = 512;    // ... up to here where the rounds of workgroups are well filled ...
-constexpr uint32_t kI8MaxRows = 1024;      // ... and up to here where the f16 tile kernel's rounds are badly filled; beyond,
-                                           // its larger tiles win
+constexpr uint32_t kI8MaxRows = 1024;      // ... up to here where an estimate says this kernel is the faster one (weights of at
+                                           // least 2048 x 4096); beyond, the larger tiles of the f16 kernel win ...
+constexpr uint32_t kI8FilledRows = 512;    // ... and for smaller weights up to here where the rounds of workgroups are well filled
 constexpr int kI8Outliers = 16;            // elements per (row, share of K) that may leave the fixed point
 
 struct W4I8Args {
@@ -539,7 +539,7 @@ __global__ __launch_bounds__(512) void w4_gemm_i8_kernel(W4I8Args a) {
 
 static int pick_q(uint32_t n, uint32_t row_blocks, bool zp4);
 
-// 129 to 512 rows: the workgroups (a block of 64 rows by 16 Q columns each) run one per compute unit, in rounds of 256
+// 129 to 512 rows on weights outside the range of the estimates below: the workgroups (a block of 64 rows by 16 Q columns each) run one per compute unit, in rounds of 256
 // that last the same full or not.  Where the rounds are at least three quarters full, with three or four columns per
 // lane, this kernel beats the f16 tiles (4096 -> 11008: 129 rows 55.8 -> 47.8 us, 256 rows 75.4 -> 60.1, 384 rows 118 -> 98,
 // 512 rows 120 -> 118; 4096 -> 4096 at 512 rows 56.2 -> 45.6; 8192 -> 8192 at 384 rows 132 -> 107); where the column count
@@ -553,23 +553,32 @@ static bool i8_rounds_filled(uint32_t m, uint32_t n, bool zp4) {
     return q >= 3 && wgs * 4 >= rounds * 256 * 3;
 }
 
-// 513 to 1024 rows (k, n >= 4096): both kernels run in rounds, and the f16 tiles of 64 x 512 make few of them: where this
-// kernel's estimate is under 0.8 of theirs it wins by 4 to 24 % (4096 -> 11008 at 768 rows 215 -> 179 us: 264 tiles are
-// two rounds of the f16 kernel; 4096 -> 4096 at 768 rows 90 -> 70; 8192 -> 8192 at 576 rows 253 -> 171), elsewhere the two
-// are within a few percent of each other or the f16 tiles are ahead (5120 -> 13824 at 576 rows 179 against 212 us).
-// Estimates in microseconds at k = 4096 (both scale with k): workgroups here cost 8.5 + 3.2 Q each, a round of the
-// eight-wave f16 tiles 120, its four-wave form as w4_launch_gemm prices it.
-static bool i8_beats_f16_rounds(uint32_t m, uint32_t n, bool zp4) {
+// 129 to 1024 rows, n >= 4096 and k >= 2048: both kernels run in rounds of workgroups over the 256 CUs, and which one
+// is faster depends on how the shape fills them.  Two estimates in microseconds, fitted to both kernels forced over ten
+// weight shapes (2048 x 8192 to 8192 x 28672) at nine batches each (within 8 % rms of this kernel's times and 6 % of the
+// f16 tiles'); the faster estimate takes the batch.  Measured against the better of the two on those 90 cases the
+// choice costs 1 % on average and 12 % at worst (the rules it replaced: 2 % and 30 %).
+//   here: W workgroups / 256 rounds of 3.4 + 3.9 Q each (Q columns per lane), less what the first round overlaps;
+//   f16 tiles: from 192 tiles of 64 x 512 on, rounds as w4_launch_gemm prices its two shapes, 109 per round; below,
+//       K is split over the workgroups and the time follows the tile count.
+// Both scale with K; 16 and 24 are what a call costs besides (activation planes, launches).
+static bool i8_beats_f16_estimate(uint32_t m, uint32_t k, uint32_t n, bool zp4) {
     const uint32_t row_blocks = ceil_div(m, 64);
     const uint32_t q = (uint32_t)pick_q(n, row_blocks, zp4);
-    if (q < 3) return false;
+    const double kf = (double)k / 4096.0;
     const double wgs = (double)ceil_div(n, 16 * q) * row_blocks;
-    const double est_i8 = (wgs / 256.0 + 0.5) * (8.5 + 3.2 * q) * (14.3 / 18.1);
+    const double est_i8 = (wgs / 256.0 - 0.14) * (3.4 + 3.9 * q) * kf + 16.0;
     const uint64_t tiles = (uint64_t)row_blocks * ceil_div(n, 512), full = (tiles + 255) / 256;
     const uint64_t halves = ((uint64_t)row_blocks * ceil_div(n, 256) + 255) / 256;
-    double units = 0.97 * (double)full;
-    if (tiles >= 192) units = std::min(units, (double)(halves / 2) * 1.05 + (double)(halves % 2) * 0.75);
-    return est_i8 <= 0.8 * units * 120.0;
+    double est_f16;
+    if (tiles >= 192) {
+        double units = 0.97 * (double)full;
+        units = std::min(units, (double)(halves / 2) * 1.05 + (double)(halves % 2) * 0.75);
+        est_f16 = units * 109.0 * kf + 24.0;
+    } else {
+        est_f16 = (156.0 * (double)tiles / 256.0 - 3.0) * kf + 24.0;
+    }
+    return est_i8 < est_f16;
 }
 
 bool w4_gemm_i8_supported(const W4Args& a) {
@@ -580,8 +589,8 @@ bool w4_gemm_i8_supported(const W4Args& a) {
           !a.g_idx && !a.tiled && !a.glu && (!a.zp4 || a.n % 8 == 0)))
         return false;
     if (a.m <= kI8AlwaysRows) return true;
-    if (a.m <= kI8FilledRows) return i8_rounds_filled(a.m, a.n, a.zp4 != nullptr);
-    return a.k >= 4096 && a.n >= 4096 && i8_beats_f16_rounds(a.m, a.n, a.zp4 != nullptr);
+    if (a.n >= 4096 && a.k >= 2048) return i8_beats_f16_estimate(a.m, a.k, a.n, a.zp4 != nullptr);
+    return a.m <= kI8FilledRows && i8_rounds_filled(a.m, a.n, a.zp4 != nullptr);
 }
 
 template <int Q, int RT, int CS, int U>
