@@ -2,6 +2,8 @@
 // and the rescale/bias epilogue.
 #pragma once
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace rumus {
@@ -102,26 +104,46 @@ __device__ __forceinline__ void i8_epilogue(const v16i (&acc)[TM][TN], const flo
 #pragma unroll
             for (int q = 0; q < 4; q++)
                 sxv[i][q] = *reinterpret_cast<const float4*>(sx + m0 + (wm * TM + i) * 32 + 8 * q + row_l);
+        // A store's address is a base that is the same for the whole wave (row tile, row of the quad: scalar registers)
+        // plus one 32-bit byte offset per lane and column tile (the lane's own row of four and its column), so that an
+        // element costs the conversion and its two multiplications and nothing for its address; the bias is a
+        // path of its own rather than a select per element.
+        const bool narrow = N < (1u << 27);                // the lane offsets, (4 N + column) floats at most, fit 32 bits
+        auto body = [&](auto bias_tag, auto narrow_tag) __attribute__((always_inline)) {
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
-            const uint32_t col = n0 + (wn * TN + j) * 32 + col_l;
-            if (n0 + (wn * TN + j) * 32 >= N) continue;    // uniform: this column tile lies past N
-            const float swc = sw[col];
-            const float bc = bias ? bias[col] : 0.0f;
+            for (int j = 0; j < TN; j++) {
+                const uint32_t col = n0 + (wn * TN + j) * 32 + col_l;
+                if (n0 + (wn * TN + j) * 32 >= N) continue;    // uniform: this column tile lies past N
+                const float swc = sw[col];
+                const float bc = decltype(bias_tag)::value ? bias[col] : 0.0f;
+                const uint32_t lane_off = (row_l * N + col) * (uint32_t)sizeof(float);
 #pragma unroll
-            for (int i = 0; i < TM; i++) {
+                for (int i = 0; i < TM; i++) {
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const uint32_t row = m0 + (wm * TM + i) * 32 + 8 * (r / 4) + row_l + (r % 4);
-                    const float4 s4 = sxv[i][r / 4];
-                    const float sr = (r % 4) == 0 ? s4.x : (r % 4) == 1 ? s4.y : (r % 4) == 2 ? s4.z : s4.w;
-                    float v = __fmul_rn(__fmul_rn((float)acc[i][j][r], sr), swc);
-                    if (bias) v = __fadd_rn(v, bc);
-                    // ordinary stores: the output stays in the Infinity Cache for whoever reads it next, and the
-                    // launch ends 1.5 % sooner than with the non-temporal hint (102.9 -> 101.3 us at 2048 x 4096 x 11008)
-                    y[(uint64_t)row * N + col] = v;
+                    for (int r = 0; r < 16; r++) {
+                        const uint32_t row_u = m0 + (wm * TM + i) * 32 + 8 * (r / 4) + (r % 4);      // uniform part of the row
+                        const float4 s4 = sxv[i][r / 4];
+                        const float sr = (r % 4) == 0 ? s4.x : (r % 4) == 1 ? s4.y : (r % 4) == 2 ? s4.z : s4.w;
+                        float v = __fmul_rn(__fmul_rn((float)acc[i][j][r], sr), swc);
+                        if (decltype(bias_tag)::value) v = __fadd_rn(v, bc);
+                        // ordinary stores: the output stays in the Infinity Cache for whoever reads it next, and the
+                        // launch ends 1.5 % sooner than with the non-temporal hint (102.9 -> 101.3 us at 2048 x 4096 x 11008)
+                        if constexpr (decltype(narrow_tag)::value) {
+                            uint8_t* const base = reinterpret_cast<uint8_t*>(y + (uint64_t)row_u * N);
+                            *reinterpret_cast<float*>(base + lane_off) = v;
+                        } else {
+                            y[(uint64_t)(row_u + row_l) * N + col] = v;
+                        }
+                    }
                 }
             }
+        };
+        if (bias) {
+            if (narrow) body(std::true_type{}, std::true_type{});
+            else body(std::true_type{}, std::false_type{});
+        } else {
+            if (narrow) body(std::false_type{}, std::true_type{});
+            else body(std::false_type{}, std::false_type{});
         }
         return;
     }
