@@ -105,6 +105,8 @@ __device__ __forceinline__ float4 nonzero(float4 s) {
     return make_float4(s.x == 0.0f ? 1e-30f : s.x, s.y == 0.0f ? 1e-30f : s.y, s.z == 0.0f ? 1e-30f : s.z,
                        s.w == 0.0f ? 1e-30f : s.w);
 }
+__device__ __forceinline__ float2 splat_of(float v, float2) { return make_float2(v, v); }
+__device__ __forceinline__ float4 splat_of(float v, float4) { return make_float4(v, v, v, v); }
 __device__ __forceinline__ float2 zp4_load(const uint32_t* zp4, uint32_t g, uint32_t n, uint32_t col, float2) {
     return w4_zp4_load2(zp4, g, n, col);
 }
@@ -344,6 +346,11 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
             meta_load((st * kStageK + (f + 1) * FOLD * 16) / a.group_size, sc_after[set][f], zp_after[set][f]);
     };
 
+    constexpr bool PIPE = WAVES == 8 && FOLD >= 4;      // groups of 32 change their constants every other step: 5 % slower pipelined
+    // PIPE: the factor that takes the accumulators from one group's scale to the next one's is applied tile by tile
+    // in front of the next step's first MFMAs (1 where no group ended), not in one block that has to wait for the
+    // last MFMA of this step and keeps the matrix cores waiting in turn.
+    floats_t rv_next = splat_of(1.0f, floats_t{});           // (a vector, not an array: arrays reached through the lambdas end up in scratch memory)
     auto fold = [&](uint32_t buf, int s_last, uint32_t kend, int set, int f, auto rest_tag) __attribute__((always_inline)) {
         // rank-1 update acc[i][j] += X[i] (x) (-(zp[j] - z[j])) on the f32 matrix core: operand slot k=0
         // carries the values (lanes 0..31), slot k=1 (lanes 32..63) is zero; compiled out of the loop that runs when
@@ -369,17 +376,23 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
             float rv[TN];
 #pragma unroll
             for (int j = 0; j < TN; j++) rv[j] = flt_of(sc_cur, j) / flt_of(sn, j);
+            if constexpr (PIPE) {
+                rv_next = sc_cur / sn;                          // the same quotients, component by component
+            } else {
 #pragma unroll
-            for (int i = 0; i < RT; i++)
+                for (int i = 0; i < RT; i++)
 #pragma unroll
-                for (int j = 0; j < TN; j++)
+                    for (int j = 0; j < TN; j++)
 #pragma unroll
-                    for (int r = 0; r < 16; r++) acc[i][j][r] *= rv[j];
+                        for (int r = 0; r < 16; r++) acc[i][j][r] *= rv[j];
+            }
             g_cur = g_after;
             sc_cur = sn;
             zp_cur = zp_after[set][f];
 #pragma unroll
             for (int j = 0; j < TN; j++) z_rest[j] = z_rest_next[j];      // split when the group's first step was converted
+        } else if constexpr (PIPE) {
+            rv_next = splat_of(1.0f, floats_t{});
         }
     };
 
@@ -403,7 +416,6 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
     // cannot issue anything while it waits to issue an MFMA, so conversion and MFMAs of the same step one after
     // the other leave the vector ALU idle during the MFMAs and the matrix cores idle during the conversion.
     // (Not the four-wave shape: it has no registers for a second set of fragments and converts in place.)
-    constexpr bool PIPE = WAVES == 8 && FOLD >= 4;      // groups of 32 change their constants every other step: 5 % slower pipelined
     v8h b_next[TN];
     auto convert_words = [&](const words_t& wv) __attribute__((always_inline)) {
 #pragma unroll
@@ -447,21 +459,46 @@ __global__ __launch_bounds__(64 * WAVES, 2) void w4_gemm_tile_kernel(W4Args a, f
                 for (int j = 0; j < TN; j++) bfr[j] = b_next[j];
             }
             // all hi products, then all lo products: dependent MFMAs are TN*RT apart
+            constexpr bool RESCALE = PIPE && true;
+            const bool after_fold = s % FOLD == 0;            // the step before settled a group (or the kernel starts: factor 1)
 #pragma unroll
             for (int i = 0; i < RT; i++)
 #pragma unroll
-                for (int j = 0; j < TN; j++)
+                for (int j = 0; j < TN; j++) {
+                    if (RESCALE && after_fold) {
+#pragma unroll
+                        for (int r = 0; r < 16; r++) acc[i][j][r] *= flt_of(rv_next, j);
+                    }
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[cur][i], bfr[j], acc[i][j], 0, 0, 0);
+                }
 #pragma unroll
             for (int i = 0; i < RT; i++)
 #pragma unroll
                 for (int j = 0; j < TN; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[cur][i], bfr[j], acc[i][j], 0, 0, 0);
             if constexpr (PIPE) {                     // one MFMA, then its share of the conversion's vector instructions in its shadow
-#pragma unroll
-                for (int i = 0; i < 2 * RT * TN; i++) {
+                constexpr int kConv = (9 * TN + 6 + 2 * RT * TN - 1) / (2 * RT * TN);
+                if (after_fold) {                     // (a tile's 16 multiplications stand in front of its first MFMA)
+                    __builtin_amdgcn_sched_group_barrier(0x002, 16, 0);
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x002, (9 * TN + 6 + 2 * RT * TN - 1) / (2 * RT * TN), 0);
+#pragma unroll
+                    for (int i = 1; i < RT * TN; i++) {
+                        __builtin_amdgcn_sched_group_barrier(0x002, 16 + kConv, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    }
+                    __builtin_amdgcn_sched_group_barrier(0x002, 2 * kConv, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+#pragma unroll
+                    for (int i = 1; i < RT * TN; i++) {
+                        __builtin_amdgcn_sched_group_barrier(0x002, kConv, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 2 * RT * TN; i++) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x002, kConv, 0);
+                    }
                 }
             }
             if (!PIPE && group_ends) split_zero(zp_after[SET][s / FOLD]);     // this step's words are converted: the next group's constants
