@@ -313,6 +313,10 @@ __global__ __launch_bounds__(64 * KW, 2) void w4t_gemm_kernel(
     RUMUS_WAIT_VMCNT((kTStages - 2) * kTLoads);               // step st0 has landed
     __builtin_amdgcn_s_barrier();
     convert(st0, 0, 0, 0);
+    // The B fragments of a step are cut out of its words while the MFMAs of the step before run (a wave issues
+    // nothing while it waits to issue an MFMA: fragments and MFMAs of the same step one after the other leave the
+    // vector ALU idle during the MFMAs and the matrix cores idle during the cutting).
+    t8h b0 = b_frag(0, 0), b1 = b_frag(1, 0);
     uint32_t cur = 0, gcur = 0;                                // slots of step st: weights and tables, grad_y
     for (uint32_t st = st0; st < st1; st++) {
         const int ab = (st - st0) & 1;
@@ -324,7 +328,7 @@ __global__ __launch_bounds__(64 * KW, 2) void w4t_gemm_kernel(
         RUMUS_WAIT_VMCNT((kTStages - 3) * kTLoads);
         __builtin_amdgcn_s_barrier();
         issue(st + (kTStages - 1), gcur, prv);
-        const t8h b0 = b_frag(0, cur), b1 = b_frag(1, cur);
+        const t8h nb0 = b_frag(0, nxt), nb1 = b_frag(1, nxt);   // step st+1 has landed (after the last step: that step's words again, unused)
         const uint8_t* abp = abuf + ab * kTAbuf;
 #pragma unroll
         for (int i = 0; i < RTILES; i++) {
@@ -335,7 +339,14 @@ __global__ __launch_bounds__(64 * KW, 2) void w4t_gemm_kernel(
             acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const t8h*>(hi + a_off[1]), b1, acc[i], 0, 0, 0);
             acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const t8h*>(lo + a_off[1]), b1, acc[i], 0, 0, 0);
         }
+#pragma unroll
+        for (int i = 0; i < 4 * RTILES; i++) {                 // an MFMA, then its share of the 40 instructions of the next fragments
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 40 / (4 * RTILES), 0);
+        }
         if (st + 1 < st1) convert(st + 1, gnxt, nxt, ab ^ 1);
+        b0 = nb0;
+        b1 = nb1;
         cur = nxt;
         gcur = gnxt;
     }
