@@ -342,18 +342,29 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void q8_gemm_blocks_f16_kernel(
         __builtin_amdgcn_s_barrier();
         issue(min(kt + (NS - 1), ksteps - 1), cur == 0 ? NS - 1 : cur - 1);
         const int8_t* base = lds + cur * STAGE;
+        // The bytes of the step's second pair become f16 while the MFMAs of its first pair run (a wave issues nothing
+        // while it waits to issue an MFMA, so conversion and MFMAs of the same pair one after the other leave the
+        // vector ALU idle during the MFMAs and the matrix cores idle during the conversion).
+        v8h bf[2][TN][2];
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const v4i w = *reinterpret_cast<const v4i*>(base + b_off[0] + j * 32 * kBK);
+            q8_bytes_to_f16(w, bf[0][j][0], bf[0][j][1]);
+        }
 #pragma unroll
         for (int s = 0; s < 2; s++) {
-            v8h af[P][2], bf[TN][2];
+            v8h af[P][2];
 #pragma unroll
             for (int p = 0; p < P; p++)
 #pragma unroll
                 for (int i = 0; i < 2; i++)
                     af[p][i] = *reinterpret_cast<const v8h*>(base + s * A_PAIR + a_off[i] + p * BM * kBK);
+            if (s == 0) {
 #pragma unroll
-            for (int j = 0; j < TN; j++) {
-                const v4i w = *reinterpret_cast<const v4i*>(base + b_off[s] + j * 32 * kBK);
-                q8_bytes_to_f16(w, bf[j][0], bf[j][1]);
+                for (int j = 0; j < TN; j++) {
+                    const v4i w = *reinterpret_cast<const v4i*>(base + b_off[1] + j * 32 * kBK);
+                    q8_bytes_to_f16(w, bf[1][j][0], bf[1][j][1]);
+                }
             }
             bool fold = EVERY;
             if (!EVERY) {
@@ -362,10 +373,17 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void q8_gemm_blocks_f16_kernel(
             }
 #pragma unroll
             for (int j = 0; j < TN; j++) {
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[0][0], bf[j][0], EVERY ? zero : acc[j], 0, 0, 0);
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[0][1], bf[j][1], acc[j], 0, 0, 0);
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[1][0], bf[j][0], acc[j], 0, 0, 0);
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[1][1], bf[j][1], acc[j], 0, 0, 0);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[0][0], bf[s][j][0], EVERY ? zero : acc[j], 0, 0, 0);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[0][1], bf[s][j][1], acc[j], 0, 0, 0);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[1][0], bf[s][j][0], acc[j], 0, 0, 0);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[1][1], bf[s][j][1], acc[j], 0, 0, 0);
+            }
+            if (s == 0) {
+#pragma unroll
+                for (int i = 0; i < 4 * TN; i++) {             // an MFMA, then its share of the second pair's conversion
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+                }
             }
             if (fold) {
                 left = period;
