@@ -343,15 +343,17 @@ def bench_gemv_shapes(torch, ops, replays=10, warmup=2):
     return rows
 
 
-def bench_w4_gemm(torch, ops, m, replays=10, warmup=2):
-    """W4 GEMM with act-order (GPTQ style), K=4096, N=11008, g128, symmetric zp=8.  The weights rotate over
+def bench_w4_gemm(torch, ops, m, replays=10, warmup=2, symmetric=True):
+    """W4 GEMM with act-order (GPTQ style), K=4096, N=11008, g128, symmetric zp=8 (stored as f32, as the reference
+    holds it; symmetric=False: the reference quantizer's own fractional zero-points, for which the large-batch kernel
+    keeps its extra pass).  The weights rotate over
     copies (> 600 MB in total, more than the 256 MB Infinity Cache) so that every launch reads them from HBM;
     the time on a single, cache-resident copy is reported beside it."""
     k, n = 4096, 11008
     dev = torch.device("cuda:0")
     gen = torch.Generator(device=dev).manual_seed(2)
     w = torch.randn((k, n), generator=gen, device=dev) * 0.02
-    packed, scales, zp = ops.w4_quantize_pack(w, G, symmetric=True)
+    packed, scales, zp = ops.w4_quantize_pack(w, G, symmetric=symmetric)
     del w
     g_idx = (torch.randperm(k, generator=gen, device=dev) // G).to(torch.int32)
     packed_sorted, perm = ops.w4_actorder_prepare(packed, g_idx, G)
@@ -375,7 +377,8 @@ def bench_w4_gemm(torch, ops, m, replays=10, warmup=2):
     sec_res = time_graph(torch, burst_resident, 10, replays, warmup, settle)["median"]
     del copies
     flops = 2.0 * m * k * n
-    return {"workload": f"w4_gemm_actorder_{m}x4096x11008_g128", "hip_graph": True, "weight_copies_rotated": ncopy,
+    return {"workload": f"w4_gemm_actorder_{m}x4096x11008_g128", "zero_points": "8.0 (f32)" if symmetric else "fractional (f32)",
+            "hip_graph": True, "weight_copies_rotated": ncopy,
             "ms_per_launch": sec * 1e3, "cache_resident_ms_per_launch": sec_res * 1e3,
             "gbs": nbytes / sec / 1e9, "hbm_frac": nbytes / sec / 1e9 / HBM_PEAK_GBS,
             "tflops": flops / sec / 1e12, "f16_mfma_frac": flops / sec / 1e12 / F16_PEAK_TFLOPS}
@@ -765,7 +768,8 @@ def main():
         out["w4_gemv_wider"] = bench_gemv_shapes(torch, ops)
         out["w4_gemm"] = [bench_w4_gemm(torch, ops, 16), bench_w4_gemm(torch, ops, 128), bench_w4_gemm(torch, ops, 256),
                           bench_w4_gemm(torch, ops, 512),
-                          bench_w4_gemm(torch, ops, 1024), bench_w4_gemm(torch, ops, 2048)]
+                          bench_w4_gemm(torch, ops, 1024), bench_w4_gemm(torch, ops, 2048),
+                          bench_w4_gemm(torch, ops, 2048, symmetric=False)]
         out["f16_mfma_only"] = probe_f16_mfma_ceiling()
         out["q8_matmul"] = bench_q8_matmul(torch, ops)
         out["w4_grad_x"] = bench_grad_x(torch, ops)
