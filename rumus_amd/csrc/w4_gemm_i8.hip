@@ -578,7 +578,7 @@ static bool i8_beats_f16_estimate(uint32_t m, uint32_t k, uint32_t n, bool zp4) 
     } else {
         est_f16 = (156.0 * (double)tiles / 256.0 - 3.0) * kf + 24.0;
     }
-    return est_i8 < est_f16;
+    return est_i8 < 0.97 * est_f16;                           // ties go to the f16 tiles (slightly fewer wrong choices on the fitted cases)
 }
 
 bool w4_gemm_i8_supported(const W4Args& a) {
